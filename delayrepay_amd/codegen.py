@@ -1,0 +1,563 @@
+"""HIP C++ source generation for fused expression kernels (gfx950).
+
+Takes the place of the reference's CUDA-C emitter (delayrepay/cuda.py:46-88,
+`CupyEmitter`, and `make_kernel`, :35-43).  The expression arrives as a
+`Program`: a flat SSA list produced by one memoised walk of the DAG
+(`hip.Tracer`), so a shared sub-expression is emitted once by construction;
+the reference re-walks shared nodes and removes duplicate statements
+afterwards (`dedup`, cuda.py:29-32).
+
+Differences in what is emitted:
+  * every value has its own C type (NumPy promotion), not one generic `T`;
+  * Python scalars are typed kernel parameters, not literals, so an f32
+    expression never computes in double and the kernel is reusable for any
+    scalar value (the reference inlines `str(val)`, cuda.py:84-85);
+  * names are positional (`l0`, `s1`, `v7`), so structurally equal
+    expressions produce identical source and hit the kernel cache (the
+    reference embeds a global serial number, delayarray.py:150-152).
+
+Kernel shapes (all 256-thread blocks = 4 wave64, grid-stride):
+  flat     contiguous operands, 128-bit loads/stores, several vectors in
+           flight per thread, optional non-temporal access, scalar tail;
+  nd       arbitrary strides / broadcasting, one element per thread-iteration;
+  stencil  2-D operands that are shifted views of one buffer: the union of the
+           shifted tiles is staged once through LDS (halo tile), tiles are
+           assigned to XCDs in contiguous bands;
+  + an optional reduction tail on flat/nd: per-thread accumulators, wave64
+    shuffle tree, LDS across the 4 waves, one partial per block, and a
+    one-block finalize kernel (no atomics, deterministic).
+"""
+import numpy as np
+
+BLOCK = 256          # threads per block: 4 wave64
+WAVE = 64
+N_XCD = 8            # accelerator dies with private L2 on MI355X
+
+# storage / arithmetic C type per dtype code
+CTYPE = {
+    "f4": "float",
+    "f8": "double",
+    "i4": "int",
+    "i8": "long long",
+    "u4": "unsigned int",
+    "u1": "unsigned char",
+    "b1": "unsigned char",
+}
+ITEMSIZE = {"f4": 4, "f8": 8, "i4": 4, "i8": 8, "u4": 4, "u1": 1, "b1": 1}
+# 16-byte vector type per dtype code (only 4- and 8-byte element types vectorise)
+VEC16 = {"f4": ("f4x4", 4), "f8": ("f8x2", 2), "i4": ("i4x4", 4), "i8": ("i8x2", 2),
+         "u4": ("u4x4", 4)}
+
+PREAMBLE = """\
+typedef float f4x4 __attribute__((ext_vector_type(4)));
+typedef double f8x2 __attribute__((ext_vector_type(2)));
+typedef int i4x4 __attribute__((ext_vector_type(4)));
+typedef long long i8x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u4x4 __attribute__((ext_vector_type(4)));
+"""
+
+
+def dtype_code(dtype):
+    dtype = np.dtype(dtype)
+    if dtype.kind == "b":
+        return "b1"
+    code = dtype.kind + str(dtype.itemsize)
+    if code not in CTYPE:
+        raise NotImplementedError(f"dtype {dtype} has no device representation")
+    return code
+
+
+def code_dtype(code):
+    return np.dtype({"b1": "bool"}.get(code, code))
+
+
+# ---- per-operation C expressions -------------------------------------------
+
+_FLOAT_FUNCS1 = {
+    "sin": "sin", "cos": "cos", "tan": "tan", "arcsin": "asin", "arccos": "acos",
+    "arctan": "atan", "sinh": "sinh", "cosh": "cosh", "tanh": "tanh", "exp": "exp",
+    "exp2": "exp2", "expm1": "expm1", "log": "log", "log2": "log2", "log10": "log10",
+    "log1p": "log1p", "sqrt": "sqrt", "cbrt": "cbrt", "erf": "erf", "erfc": "erfc",
+    "floor": "floor", "ceil": "ceil", "trunc": "trunc", "rint": "rint",
+}
+_FLOAT_FUNCS2 = {
+    "power": "pow", "arctan2": "atan2", "hypot": "hypot", "copysign": "copysign",
+    "fmod": "fmod", "fmax": "fmax", "fmin": "fmin",
+}
+_INFIX = {"add": "+", "subtract": "-", "multiply": "*", "divide": "/", "true_divide": "/"}
+_COMPARE = {"greater": ">", "less": "<", "greater_equal": ">=", "less_equal": "<=",
+            "equal": "==", "not_equal": "!="}
+
+SUPPORTED_UFUNCS = (set(_FLOAT_FUNCS1) | set(_FLOAT_FUNCS2) | set(_INFIX) | set(_COMPARE)
+                    | {"negative", "positive", "absolute", "fabs", "reciprocal", "maximum",
+                       "minimum", "square"})
+
+
+def _fn(name, dt):
+    """C math function for a float dtype: `sinf` for f4, `sin` for f8."""
+    return name + ("f" if dt == "f4" else "")
+
+
+def op_expr(name, dt, args):
+    """C expression computing ufunc `name` in arithmetic type `dt` on `args`
+    (C expressions already converted to `dt`)."""
+    is_float = dt in ("f4", "f8")
+    if name in _INFIX:
+        if name in ("divide", "true_divide") and not is_float:
+            raise NotImplementedError("integer division has no float result type here")
+        return f"{args[0]} {_INFIX[name]} {args[1]}"
+    if name in _COMPARE:
+        return f"(unsigned char)({args[0]} {_COMPARE[name]} {args[1]})"
+    if name == "negative":
+        return f"-{args[0]}"
+    if name == "positive":
+        return f"{args[0]}"
+    if name in ("absolute", "fabs"):
+        if is_float:
+            return f"{_fn('fabs', dt)}({args[0]})"
+        return f"({args[0]} < 0 ? -{args[0]} : {args[0]})"
+    if name == "reciprocal":
+        return f"({CTYPE[dt]})1 / {args[0]}"
+    if name == "maximum":   # NaN-propagating, like NumPy
+        a, b = args
+        return f"(({a} >= {b} || {a} != {a}) ? {a} : {b})"
+    if name == "minimum":
+        a, b = args
+        return f"(({a} <= {b} || {a} != {a}) ? {a} : {b})"
+    if name in _FLOAT_FUNCS1:
+        if not is_float:
+            raise NotImplementedError(f"{name} on a non-float type")
+        return f"{_fn(_FLOAT_FUNCS1[name], dt)}({args[0]})"
+    if name in _FLOAT_FUNCS2:
+        if not is_float:
+            raise NotImplementedError(f"{name} on a non-float type")
+        return f"{_fn(_FLOAT_FUNCS2[name], dt)}({args[0]}, {args[1]})"
+    raise NotImplementedError(f"ufunc {name!r} cannot be fused")
+
+
+class Program:
+    """Straight-line SSA form of an expression DAG.
+
+    leaves   list of dtype codes, one per distinct input array
+    scalars  list of dtype codes, one per scalar kernel parameter
+    ops      list of (name, compute dtype, result dtype, arg refs); a ref is
+             ('l', i) | ('s', i) | ('v', i); name 'cast' converts
+    roots    list of (ref, dtype code)
+    """
+
+    __slots__ = ("leaves", "scalars", "ops", "roots")
+
+    def __init__(self, leaves, scalars, ops, roots):
+        self.leaves = tuple(leaves)
+        self.scalars = tuple(scalars)
+        self.ops = tuple(ops)
+        self.roots = tuple(roots)
+
+    def key(self):
+        return (self.leaves, self.scalars, self.ops, self.roots)
+
+    def ref_dtype(self, ref):
+        kind, i = ref
+        if kind == "l":
+            return self.leaves[i]
+        if kind == "s":
+            return self.scalars[i]
+        return self.ops[i][2]
+
+
+def _conv(expr, src, dst):
+    if src == dst:
+        return expr
+    if dst == "b1":
+        return f"(unsigned char)({expr} != 0)"
+    return f"({CTYPE[dst]}){expr}"
+
+
+def emit_body(prog, out_dtypes, fname="dr_body"):
+    """Inline device function evaluating the whole program for one element.
+
+    Parameters: leaf values, scalar values, then one reference per root."""
+    params = [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
+    lines = [f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
+    for i, (name, cdt, rdt, args) in enumerate(prog.ops):
+        cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
+        if name == "cast":
+            expr = cargs[0]
+        else:
+            expr = op_expr(name, cdt, cargs)
+        lines.append(f"    const {CTYPE[rdt]} v{i} = {expr};")
+    for i, ((k, j), rdt) in enumerate(prog.roots):
+        lines.append(f"    r{i} = {_conv(f'{k}{j}', rdt, out_dtypes[i])};")
+    lines.append("}")
+    return "\n".join(lines)
+
+
+# ---- reduction pieces ------------------------------------------------------
+
+def _combine(op, a, b):
+    if op == "add":
+        return f"{a} + {b}"
+    return op_expr(op, "f8", [a, b])  # maximum/minimum expression is type-agnostic
+
+
+def _identity(op, dt):
+    if op == "add":
+        return f"({CTYPE[dt]})0"
+    if dt in ("f4", "f8"):
+        inf = "__builtin_inff()" if dt == "f4" else "__builtin_inf()"
+        return f"-{inf}" if op == "maximum" else inf
+    lim = {"i4": ("(-2147483647 - 1)", "2147483647"),
+           "i8": ("(-9223372036854775807LL - 1)", "9223372036854775807LL"),
+           "u4": ("0u", "4294967295u"), "u1": ("0", "255"), "b1": ("0", "1")}[dt]
+    return lim[0] if op == "maximum" else lim[1]
+
+
+def emit_block_reduce(op, dt):
+    """Device function: combine `v` over the block; valid in thread 0.
+
+    Wave64 shuffle-down tree, then the 4 wave leaders meet through LDS."""
+    ct = CTYPE[dt]
+    shfl = "__shfl_down(v, off, 64)"
+    if dt in ("u1", "b1"):
+        shfl = f"({ct})__shfl_down((int)v, off, 64)"
+    return f"""\
+__device__ __forceinline__ {ct} dr_block_reduce({ct} v)
+{{
+    __shared__ {ct} dr_wave_part[{BLOCK // WAVE}];
+#pragma unroll
+    for (int off = {WAVE // 2}; off > 0; off >>= 1) {{
+        const {ct} o = {shfl};
+        v = {_combine(op, 'v', 'o')};
+    }}
+    const int lane = threadIdx.x & {WAVE - 1};
+    const int wave = threadIdx.x >> 6;
+    if (lane == 0) dr_wave_part[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {{
+        v = dr_wave_part[0];
+#pragma unroll
+        for (int w = 1; w < {BLOCK // WAVE}; ++w) v = {_combine(op, 'v', 'dr_wave_part[w]')};
+    }}
+    return v;
+}}
+"""
+
+
+def emit_finalize(op, dt):
+    ct = CTYPE[dt]
+    return f"""\
+extern "C" __global__ __launch_bounds__({BLOCK})
+void dr_finalize(const {ct}* __restrict__ partial, {ct}* __restrict__ out, int count)
+{{
+    {ct} acc = {_identity(op, dt)};
+    for (int i = threadIdx.x; i < count; i += {BLOCK}) acc = {_combine(op, 'acc', 'partial[i]')};
+    acc = dr_block_reduce(acc);
+    if (threadIdx.x == 0) out[0] = acc;
+}}
+"""
+
+
+# ---- flat kernel -----------------------------------------------------------
+
+def _ld(nt, ptr):
+    return f"__builtin_nontemporal_load({ptr})" if nt else f"*({ptr})"
+
+
+def _st(nt, val, ptr):
+    return f"__builtin_nontemporal_store({val}, {ptr});" if nt else f"*({ptr}) = {val};"
+
+
+def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
+              reduce_op=None):
+    """Contiguous 1-D kernel.
+
+    leaf_class  per leaf 'c' (contiguous, same length as the output) or 'b'
+                (single element broadcast to every position)
+    vec         True: 16-byte vector accesses (all pointers 16-byte aligned and
+                all element types 4 or 8 bytes wide); False: one element per access
+    reduce_op   None, or 'add' | 'maximum' | 'minimum': the single root is
+                reduced instead of stored; the output is one partial per block
+    """
+    rs = "__restrict__ " if restrict else ""
+    n_leaf, n_out = len(prog.leaves), len(out_dtypes)
+    red_dt = out_dtypes[0] if reduce_op else None
+    if vec:
+        widths = [ITEMSIZE[dt] for dt, c in zip(prog.leaves, leaf_class) if c == "c"]
+        if not reduce_op:
+            widths += [ITEMSIZE[dt] for dt in out_dtypes]
+        E = 16 // min(widths) if widths else 4
+    else:
+        E = 1
+    src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    if reduce_op:
+        src.append(emit_block_reduce(reduce_op, red_dt))
+        src.append(emit_finalize(reduce_op, red_dt))
+
+    params = [f"const {CTYPE[dt]}* {rs}a{i}" for i, dt in enumerate(prog.leaves)]
+    if reduce_op:
+        params.append(f"{CTYPE[red_dt]}* {rs}partial")
+    else:
+        params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params.append("const long long n")
+
+    L = []
+    L.append(f'extern "C" __global__ __launch_bounds__({BLOCK})')
+    L.append(f"void dr_kernel({', '.join(params)})")
+    L.append("{")
+    for i, c in enumerate(leaf_class):
+        if c == "b":
+            L.append(f"    const {CTYPE[prog.leaves[i]]} b{i} = a{i}[0];")
+    if reduce_op:
+        for e in range(max(E, 1)):
+            L.append(f"    {CTYPE[red_dt]} acc{e} = {_identity(reduce_op, red_dt)};")
+    L.append(f"    const long long stride = (long long)gridDim.x * {BLOCK};")
+    L.append(f"    long long v = (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
+    scal = [f"s{i}" for i in range(len(prog.scalars))]
+
+    def step(tag, idx, indent):
+        """Code handling one vector (or element) at index expression `idx`:
+        (loads, compute+stores)."""
+        pad = " " * indent
+        loads, work = [], []
+        for i, (dt, c) in enumerate(zip(prog.leaves, leaf_class)):
+            if c != "c":
+                continue
+            if vec:
+                vt, per = VEC16[dt]
+                chunks = E // per
+                for ch in range(chunks):
+                    ptr = f"(const {vt}*)a{i} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
+                        else f"(const {vt}*)a{i} + ({idx})"
+                    loads.append(f"{pad}const {vt} L{i}_{ch}{tag} = {_ld(nt_load, ptr)};")
+            else:
+                loads.append(f"{pad}const {CTYPE[dt]} L{i}{tag} = "
+                             f"{_ld(nt_load, f'a{i} + ({idx})')};")
+        if vec and not reduce_op:
+            for o, dt in enumerate(out_dtypes):
+                vt, per = VEC16[dt]
+                for ch in range(E // per):
+                    work.append(f"{pad}{vt} R{o}_{ch}{tag};")
+        for e in range(E):
+            args = []
+            for i, (dt, c) in enumerate(zip(prog.leaves, leaf_class)):
+                if c == "b":
+                    args.append(f"b{i}")
+                elif vec:
+                    per = VEC16[dt][1]
+                    args.append(f"L{i}_{e // per}{tag}[{e % per}]")
+                else:
+                    args.append(f"L{i}{tag}")
+            outs = [f"t{o}" for o in range(n_out)]
+            decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+            call = f"dr_body({', '.join(args + scal + outs)});"
+            if reduce_op:
+                tail = f"acc{e} = {_combine(reduce_op, f'acc{e}', 't0')};"
+            elif vec:
+                tail = " ".join(f"R{o}_{e // VEC16[dt][1]}{tag}[{e % VEC16[dt][1]}] = t{o};"
+                                for o, dt in enumerate(out_dtypes))
+            else:
+                tail = " ".join(_st(nt_store, f"t{o}", f"o{o} + ({idx})") for o in range(n_out))
+            work.append(f"{pad}{{ {decl} {call} {tail} }}")
+        if vec and not reduce_op:
+            for o, dt in enumerate(out_dtypes):
+                vt, per = VEC16[dt]
+                chunks = E // per
+                for ch in range(chunks):
+                    ptr = f"({vt}*)o{o} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
+                        else f"({vt}*)o{o} + ({idx})"
+                    work.append(pad + _st(nt_store, f"R{o}_{ch}{tag}", ptr))
+        return loads, work
+
+    count = "nvec" if vec else "n"
+    if vec:
+        L.append(f"    const long long nvec = n / {E};")
+    if unroll > 1:
+        L.append(f"    for (; v + {unroll - 1} * stride < {count}; v += {unroll} * stride) {{")
+        all_loads, all_work = [], []
+        for u in range(unroll):
+            lo, wo = step(f"_u{u}", f"v + {u} * stride" if u else "v", 8)
+            all_loads += lo
+            all_work += wo
+        L += all_loads + all_work
+        L.append("    }")
+    L.append(f"    for (; v < {count}; v += stride) {{")
+    lo, wo = step("", "v", 8)
+    L += lo + wo
+    L.append("    }")
+    if vec and E > 1:
+        # scalar tail: the last n % E elements, by the first threads of block 0
+        L.append(f"    const long long t = nvec * {E} + (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
+        L.append("    if (t < n) {")
+        args = [f"b{i}" if c == "b" else f"a{i}[t]" for i, c in enumerate(leaf_class)]
+        decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+        outs = [f"t{o}" for o in range(n_out)]
+        L.append(f"        {decl} dr_body({', '.join(args + scal + outs)});")
+        if reduce_op:
+            L.append(f"        acc0 = {_combine(reduce_op, 'acc0', 't0')};")
+        else:
+            for o in range(n_out):
+                L.append(f"        o{o}[t] = t{o};")
+        L.append("    }")
+    if reduce_op:
+        accs = [f"acc{e}" for e in range(max(E, 1))]
+        while len(accs) > 1:   # pairwise: (acc0 + acc1) + (acc2 + acc3)
+            accs = [f"({_combine(reduce_op, accs[i], accs[i + 1])})" if i + 1 < len(accs)
+                    else accs[i] for i in range(0, len(accs), 2)]
+        L.append(f"    {CTYPE[red_dt]} total = {accs[0]};")
+        L.append("    total = dr_block_reduce(total);")
+        L.append("    if (threadIdx.x == 0) partial[blockIdx.x] = total;")
+    L.append("}")
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n", E
+
+
+# ---- general strided kernel ------------------------------------------------
+
+def emit_nd(prog, ndim, out_dtypes, index32, reduce_op=None):
+    """Arbitrary strides and broadcasting: each thread-iteration handles one
+    output element, decomposing its linear index over the (merged) shape."""
+    it = "unsigned int" if index32 else "long long"
+    n_out = len(out_dtypes)
+    red_dt = out_dtypes[0] if reduce_op else None
+    src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    if reduce_op:
+        src.append(emit_block_reduce(reduce_op, red_dt))
+        src.append(emit_finalize(reduce_op, red_dt))
+    params = [f"const {CTYPE[dt]}* a{i}" for i, dt in enumerate(prog.leaves)]
+    if reduce_op:
+        params.append(f"{CTYPE[red_dt]}* partial")
+    else:
+        params += [f"{CTYPE[dt]}* o{i}" for i, dt in enumerate(out_dtypes)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params.append("const long long n")
+    params += [f"const {it} d{k}" for k in range(ndim)]
+    for i in range(len(prog.leaves)):
+        params += [f"const long long sa{i}_{k}" for k in range(ndim)]
+    if not reduce_op:
+        for o in range(n_out):
+            params += [f"const long long so{o}_{k}" for k in range(ndim)]
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{"]
+    if reduce_op:
+        L.append(f"    {CTYPE[red_dt]} acc0 = {_identity(reduce_op, red_dt)};")
+    L.append(f"    const long long stride = (long long)gridDim.x * {BLOCK};")
+    L.append(f"    for (long long g = (long long)blockIdx.x * {BLOCK} + threadIdx.x; g < n; g += stride) {{")
+    L.append(f"        {it} rem = ({it})g;")
+    for k in reversed(range(ndim)):
+        if k == 0:
+            L.append(f"        const {it} c0 = rem;")
+        else:
+            L.append(f"        const {it} c{k} = rem % d{k}; rem /= d{k};")
+    for i in range(len(prog.leaves)):
+        off = " + ".join(f"(long long)c{k} * sa{i}_{k}" for k in range(ndim)) or "0"
+        L.append(f"        const {CTYPE[prog.leaves[i]]} x{i} = a{i}[{off}];")
+    decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+    call = ([f"x{i}" for i in range(len(prog.leaves))] + [f"s{i}" for i in range(len(prog.scalars))]
+            + [f"t{o}" for o in range(n_out)])
+    L.append(f"        {decl} dr_body({', '.join(call)});")
+    if reduce_op:
+        L.append(f"        acc0 = {_combine(reduce_op, 'acc0', 't0')};")
+    else:
+        for o in range(n_out):
+            off = " + ".join(f"(long long)c{k} * so{o}_{k}" for k in range(ndim)) or "0"
+            L.append(f"        o{o}[{off}] = t{o};")
+    L.append("    }")
+    if reduce_op:
+        L.append("    acc0 = dr_block_reduce(acc0);")
+        L.append("    if (threadIdx.x == 0) partial[blockIdx.x] = acc0;")
+    L.append("}")
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"
+
+
+# ---- 2-D stencil kernel with an LDS halo tile ------------------------------
+
+def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=True):
+    """2-D tiled kernel; operands that are shifted views of one buffer are staged
+    through an LDS halo tile.
+
+    leaf_kind  per leaf: ('g', dy, dx) member of the halo group, shifted by
+               (dy, dx) elements from the group's reference view;
+               ('d',) separate 2-D operand with unit column stride, read directly;
+               ('b',) single element broadcast
+    group      None, or (dtype code, dy_max, dx_min, dx_max): extent of the shifts
+               (dy in [0, dy_max], dx in [dx_min, dx_max])
+
+    The block stages the (tile_h + dy_max) x (tile_w + dx_max - dx_min) window of
+    the buffer in LDS with coalesced loads, then every thread computes
+    tile_h * tile_w / 256 outputs reading its shifted operands from LDS.
+    Consecutive tile numbers go to one XCD, so tiles that share halo rows meet
+    in the same L2."""
+    rs = "__restrict__ " if restrict else ""
+    n_out = len(out_dtypes)
+    per_thread = tile_w * tile_h // BLOCK
+    assert tile_w * tile_h % BLOCK == 0
+    src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    params = []
+    for i, dt in enumerate(prog.leaves):
+        if leaf_kind[i][0] != "g":
+            params.append(f"const {CTYPE[dt]}* {rs}a{i}")
+    if group is not None:
+        gdt, dy_max, dx_min, dx_max = group
+        LW = tile_w + dx_max - dx_min
+        LH = tile_h + dy_max
+        params.append(f"const {CTYPE[gdt]}* {rs}gp")
+    params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += ["const int H", "const int W"]
+    if group is not None:
+        params += ["const long long grs", "const long long glo", "const long long ghi"]
+    params.append("const int tiles_x")
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "d":
+            params.append(f"const long long rs{i}")
+    params += [f"const long long ors{o}" for o in range(n_out)]
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{"]
+    if group is not None:
+        L.append(f"    __shared__ {CTYPE[gdt]} tile[{LH * LW}];")
+    L += [  # contiguous band of tiles per XCD (blocks are dealt round-robin to XCDs)
+         "    const int nb = gridDim.x;",
+         f"    const int xcd = blockIdx.x % {N_XCD};",
+         f"    const int slot = blockIdx.x / {N_XCD};",
+         f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;",
+         "    const int ty = t / tiles_x;",
+         "    const int tx = t - ty * tiles_x;",
+         f"    const int r0 = ty * {tile_h};",
+         f"    const int c0 = tx * {tile_w};"]
+    if group is not None:
+        L += [f"    for (int idx = threadIdx.x; idx < {LH * LW}; idx += {BLOCK}) {{",
+              f"        const int lr = idx / {LW};",
+              f"        const int lc = idx - lr * {LW};",
+              f"        const long long lin = (long long)(r0 + lr) * grs + (c0 + lc + ({dx_min}));",
+              "        if (lin >= glo && lin < ghi) tile[idx] = gp[lin];",
+              "    }",
+              "    __syncthreads();"]
+    L += ["#pragma unroll",
+          f"    for (int k = 0; k < {per_thread}; ++k) {{",
+          f"        const int e = threadIdx.x + k * {BLOCK};",
+          f"        const int lr = e / {tile_w};",
+          f"        const int lc = e - lr * {tile_w};",
+          "        const int i = r0 + lr;",
+          "        const int j = c0 + lc;",
+          "        if (i < H && j < W) {"]
+    args = []
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "g":
+            _, dy, dx = k
+            args.append(f"tile[(lr + {dy}) * {LW} + lc + ({dx - dx_min})]")
+        elif k[0] == "d":
+            args.append(f"a{i}[(long long)i * rs{i} + j]")
+        else:
+            args.append(f"a{i}[0]")
+    decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+    call = args + [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
+    L.append(f"            {decl} dr_body({', '.join(call)});")
+    for o in range(n_out):
+        L.append(f"            o{o}[(long long)i * ors{o} + j] = t{o};")
+    L += ["        }", "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"

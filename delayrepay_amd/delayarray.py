@@ -1,0 +1,785 @@
+"""Lazy NumPy look-alike: arithmetic builds a hash-consed expression DAG.
+
+Public names and protocol behaviour follow the reference's front end
+(delayrepay/delayarray.py): `DelayArray` intercepts NumPy ufuncs through
+`__array_ufunc__` (:46-61) and builds nodes instead of computing; a value is
+produced only when one is asked for (`get`, `run`, `repr`, indexing; :35-44,
+:101-128), by handing the whole DAG to the backend's `run` (:43).
+
+Deliberate differences from the reference, each needed for NumPy-exact results
+or bounded memory:
+  * the hash-cons table is keyed on (class, function, child identities, exact
+    scalar type and value) and holds nodes weakly; the reference keys on
+    `hash(args)` (:224-231), under which `Scalar(-1)`/`Scalar(-2)` and `2`/`2.0`
+    collide, and keeps every leaf alive for ever;
+  * NumPy >= 2 names the division ufunc `divide`; both spellings are accepted
+    (the reference's table knows only `true_divide`, :162-168);
+  * shapes follow NumPy broadcasting and stay lazy (the reference computes
+    unequal shapes eagerly, :47-55);
+  * dtypes follow NumPy promotion with weak Python scalars instead of being
+    copied between siblings (:462-467);
+  * an evaluated node is reused as a leaf by later expressions, and a cached
+    result is dropped when a leaf it was computed from has been written since;
+  * `sum` builds a `ReduceEx` (a stub in the reference, :272-283) that the HIP
+    backend fuses with the element-wise body;
+  * `dst[key] = lazy_expression` is handed to the backend as one fused write;
+  * `evaluate(a, b, ...)` computes several roots in one kernel.
+"""
+import numbers
+import weakref
+
+import numpy as np
+import numpy.lib.mixins
+
+from . import backend as be
+
+_backend = be.backend
+
+
+def cast(func):
+    """Decorator: wrap a backend array returned by `func` as a lazy leaf
+    (cf. delayarray.py:13-22)."""
+
+    def wrapper(*args, **kwargs):
+        res = func(*args, **kwargs)
+        if isinstance(res, DelayArray):
+            return res
+        return NPArray(res)
+
+    wrapper.__name__ = getattr(func, "__name__", "wrapped")
+    wrapper.__doc__ = getattr(func, "__doc__", None)
+    return wrapper
+
+
+def _unwrap(obj):
+    """Backend array (or plain object) behind a lazy array."""
+    if isinstance(obj, DelayArray):
+        return obj._force()
+    return obj
+
+
+class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
+    """Base of every node; also the user-visible array type."""
+
+    count = 0  # global creation serial (delayarray.py:27-32)
+
+    def __init__(self, *args, **kwargs):
+        self._count = DelayArray.count
+        DelayArray.count += 1
+
+    # ---- forcing ---------------------------------------------------------
+
+    def _force(self):
+        """Evaluate (once) and return the backend array."""
+        arr = self.__dict__.get("array")
+        if arr is not None:
+            deps = self.__dict__.get("_deps")
+            if deps is None or all(buf.version == ver for buf, ver in deps):
+                return arr
+            del self.array  # a leaf was written to since: recompute
+        self.array = _backend.run(self)
+        return self.array
+
+    def __array__(self, dtype=None, copy=None):
+        """Host `numpy.ndarray` holding the value (NumPy's conversion protocol)."""
+        host = self.get()
+        if dtype is not None and host.dtype != dtype:
+            host = host.astype(dtype)
+        return host
+
+    def get(self):
+        """Evaluate and copy to the host (delayarray.py:101-106)."""
+        arr = self._force()
+        getter = getattr(arr, "get", None)
+        return getter() if getter is not None else arr
+
+    def run(self):
+        """Evaluate on the device without copying back (delayarray.py:108-109)."""
+        self._force()
+
+    def __repr__(self):
+        return str(self.get())
+
+    def __float__(self):
+        return float(self.get())
+
+    def __int__(self):
+        return int(self.get())
+
+    def __bool__(self):
+        return bool(self.get())
+
+    # ---- NumPy protocols -------------------------------------------------
+
+    def __array_ufunc__(self, ufunc, method, *inputs, **kwargs):
+        if method == "reduce" and ufunc.__name__ in ("add", "maximum", "minimum"):
+            return _reduce(ufunc, inputs[0], **kwargs)
+        if method != "__call__":
+            return NotImplemented
+        if kwargs:
+            out = kwargs.get("out")
+            if isinstance(out, tuple) and len(out) == 1 and out[0] is inputs[0]:
+                # `x += y`: like the reference, build a new node and let Python rebind x
+                kwargs = {k: v for k, v in kwargs.items() if k != "out"}
+            bad = [k for k, v in kwargs.items() if v is not None]
+            if bad:
+                raise NotImplementedError(f"ufunc keyword(s) {bad} are not supported on lazy arrays")
+        if ufunc.__name__ == "matmul":
+            return self._dot(inputs, {})
+        args = [arg_to_numpy_ex(arg) for arg in inputs]
+        return create_ex(ufunc, args)
+
+    def __array_function__(self, func, types, args, kwargs):
+        if func.__name__ == "dot":
+            return self._dot(args, kwargs)
+        handler = HANDLED_FUNCTIONS.get(func)
+        if handler is None:
+            return NotImplemented
+        return handler(*args, **kwargs)
+
+    def __matmul__(self, other):
+        return self._dot([self, other], {})
+
+    def _dot(self, args, kwargs):
+        left, right = (arg_to_numpy_ex(a) for a in args[:2])
+        if len(left.shape) == 1 and len(right.shape) == 1:
+            # vector . vector: fused multiply + reduction
+            return _reduce(np.add, left * right)
+        return cast(_backend.fallback.dot)(left._force(), right._force())
+
+    def dot(self, other, out=None):
+        return self._dot([self, other], {})
+
+    def __gt__(self, other):
+        return np.greater(self, other)
+
+    def __lt__(self, other):
+        return np.less(self, other)
+
+    # ---- shape-like ------------------------------------------------------
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    @property
+    def size(self):
+        n = 1
+        for d in self.shape:
+            n *= d
+        return n
+
+    def __len__(self):
+        if not self.shape:
+            raise TypeError("len() of unsized object")
+        return self.shape[0]
+
+    @property
+    def T(self):
+        if len(self.shape) < 2:
+            return self
+        return np.transpose(self)
+
+    def reshape(self, *args, **kwargs):
+        return NPArray(self._force().reshape(*args, **kwargs))
+
+    def astype(self, dtype, **kwargs):
+        """Lazy cast, fused into whatever consumes it."""
+        dtype = np.dtype(dtype)
+        if dtype == self.dtype:
+            return self
+        return CastEx(dtype, self)
+
+    # ---- indexing --------------------------------------------------------
+
+    def __getitem__(self, key):
+        """Force, then wrap the backend *view* as a new leaf (delayarray.py:123-128)."""
+        key = _unwrap(key)
+        return NPArray(self._force()[key])
+
+    def __setitem__(self, key, item):
+        """Write into the materialised array.  A lazy right-hand side is handed
+        to the backend as one fused kernel writing straight into the destination
+        (the reference evaluates it to a temporary first, delayarray.py:114-121)."""
+        arr = self._force()
+        key = _unwrap(key)
+        if isinstance(item, DelayArray) and "array" not in item.__dict__:
+            _backend.run_into(item, arr[key])
+        else:
+            arr[key] = _unwrap(item)
+
+    # ---- reductions and friends -----------------------------------------
+
+    def sum(self, *args, **kwargs):
+        return np.sum(self, *args, **kwargs)
+
+    def max(self, *args, **kwargs):
+        return np.max(self, *args, **kwargs)
+
+    def min(self, *args, **kwargs):
+        return np.min(self, *args, **kwargs)
+
+    def mean(self, *args, **kwargs):
+        return np.mean(self, *args, **kwargs)
+
+    def var(self, *args, **kwargs):
+        return np.var(self, *args, **kwargs)
+
+    def repeat(self, *args, **kwargs):
+        return repeat(self, *args, **kwargs)
+
+    # ---- code-generation helpers ----------------------------------------
+
+    @property
+    def name(self):
+        return f"arr{self._count}"
+
+    @property
+    def inputs(self):
+        return {self.name: self}
+
+
+# ufunc name -> C infix operator (delayarray.py:162-168, plus NumPy 2's `divide`)
+OPS = {
+    "matmul": "@",
+    "add": "+",
+    "multiply": "*",
+    "subtract": "-",
+    "true_divide": "/",
+    "divide": "/",
+}
+
+# ufunc name -> C function spelling (delayarray.py:171-186, widened)
+FUNCS = {
+    "power": "pow",
+    "arctan2": "atan2",
+    "absolute": "abs",
+    "sin": "sin",
+    "cos": "cos",
+    "tan": "tan",
+    "sqrt": "sqrt",
+    "log": "log",
+    "negative": "-",
+    "exp": "exp",
+    "tanh": "tanh",
+    "sinh": "sinh",
+    "cosh": "cosh",
+    "arcsin": "asin",
+    "arccos": "acos",
+    "arctan": "atan",
+    "exp2": "exp2",
+    "expm1": "expm1",
+    "log2": "log2",
+    "log10": "log10",
+    "log1p": "log1p",
+    "cbrt": "cbrt",
+    "erf": "erf",
+    "erfc": "erfc",
+    "floor": "floor",
+    "ceil": "ceil",
+    "trunc": "trunc",
+    "rint": "rint",
+    "reciprocal": "1/",
+    "positive": "+",
+    "maximum": "max",
+    "minimum": "min",
+    "fmax": "fmax",
+    "fmin": "fmin",
+    "hypot": "hypot",
+    "copysign": "copysign",
+    "fmod": "fmod",
+    "greater": ">",
+    "less": "<",
+    "greater_equal": ">=",
+    "less_equal": "<=",
+    "equal": "==",
+    "not_equal": "!=",
+}
+
+ufunc_lookup = {
+    "matmul": _backend.np.matmul,
+    "add": _backend.np.add,
+    "multiply": _backend.np.multiply,
+    "subtract": _backend.np.subtract,
+    "true_divide": _backend.np.true_divide,
+    "divide": _backend.np.true_divide,
+}
+
+
+def calc_shape(left, right, op=None):
+    """Result shape of a binary node: NumPy broadcasting (a scalar is `()`)."""
+    if left == right:
+        return left
+    return tuple(np.broadcast_shapes(left, right))
+
+
+_RESOLVE_CACHE = {}
+
+
+def _descr(node):
+    """What NumPy's type resolution needs to know about an operand."""
+    if isinstance(node, Scalar):
+        val = node.val
+        if isinstance(val, np.generic):
+            return ("np", val.dtype.str)
+        if isinstance(val, bool):
+            return ("py", "b")
+        if isinstance(val, int):
+            return ("py", "i")
+        if isinstance(val, float):
+            return ("py", "f")
+        return ("py", "c")
+    return ("a", node.dtype.str)
+
+
+_PY_PROBE = {"b": True, "i": 1, "f": 1.0, "c": 1j}
+
+
+def result_dtype(func, descrs):
+    """dtype NumPy gives `func` on operands described by `descrs` (weak Python
+    scalars included); decided by NumPy itself on empty arrays."""
+    key = (func.__name__, descrs)
+    try:
+        return _RESOLVE_CACHE[key]
+    except KeyError:
+        pass
+    probes = []
+    for kind, code in descrs:
+        if kind == "a":
+            probes.append(np.empty(0, dtype=code))
+        elif kind == "np":
+            probes.append(np.dtype(code).type(1))
+        else:
+            probes.append(_PY_PROBE[code])
+    if all(kind != "a" for kind, _ in descrs):
+        probes[0] = np.empty(0, dtype=np.asarray(probes[0]).dtype)
+    with np.errstate(all="ignore"):
+        dt = func(*probes).dtype
+    _RESOLVE_CACHE[key] = dt
+    return dt
+
+
+def calc_type(func, children):
+    return result_dtype(func, tuple(_descr(c) for c in children))
+
+
+class Memoiser(type):
+    """Metaclass that hash-conses node construction: building the same node
+    twice yields the same object, so expressions form a DAG
+    (cf. delayarray.py:216-231; tests/test.py:145-162)."""
+
+    _cache = weakref.WeakValueDictionary()
+
+    def __call__(cls, *args):
+        key = cls._memo_key(*args)
+        node = Memoiser._cache.get(key)
+        if node is None:
+            node = super().__call__(*args)
+            node._key = key
+            Memoiser._cache[key] = node
+        return node
+
+
+def reset():
+    """Forget every hash-consed node (delayarray.py:234-236)."""
+    Memoiser._cache.clear()
+
+
+class NumpyEx(DelayArray, metaclass=Memoiser):
+    """Interior or leaf node of the expression DAG."""
+
+    children = ()
+
+    def __init__(self, children=()):
+        super().__init__()
+        self.children = list(children)
+
+    @classmethod
+    def _memo_key(cls, *args):
+        return (cls.__name__,) + tuple(
+            a.__name__ if isinstance(a, np.ufunc) else
+            id(a) if isinstance(a, DelayArray) else a
+            for a in args)
+
+    def __hash__(self):
+        return id(self)
+
+    @property
+    def inputs(self):
+        """Ordered, de-duplicated leaves (name -> node): kernel operand order."""
+        found = {}
+        stack = [self]
+        seen = set()
+        order = []
+        while stack:
+            node = stack.pop()
+            if id(node) in seen:
+                continue
+            seen.add(id(node))
+            if isinstance(node, NPArray) or "array" in node.__dict__:
+                order.append(node)
+            else:
+                stack.extend(reversed(node.children))
+        for node in order:
+            found[node.name] = node
+        return found
+
+
+class Funcable:
+    def to_op(self):
+        return OPS[self.func.__name__]
+
+
+class ReduceEx(NumpyEx, Funcable):
+    """Full reduction of an expression with a binary ufunc (`add`, `maximum`,
+    `minimum`); evaluated as the tail of the fused element-wise kernel."""
+
+    def __init__(self, func, arg):
+        super().__init__(children=[arg])
+        self.func = func
+        self.shape = ()
+        self.dtype = arg.dtype
+
+    @property
+    def name(self):
+        return f"redex{self._count}"
+
+
+class UnaryFuncEx(NumpyEx, Funcable):
+    def __init__(self, func, arg):
+        super().__init__(children=[arg])
+        self.func = func
+        self.shape = arg.shape
+        self.dtype = calc_type(func, [arg])
+
+    def to_op(self):
+        return FUNCS[self.func.__name__]
+
+    @property
+    def name(self):
+        return f"unfunc{self._count}"
+
+
+class CastEx(NumpyEx):
+    """`astype` on a lazy expression: a conversion fused into the kernel."""
+
+    def __init__(self, dtype, arg):
+        super().__init__(children=[arg])
+        self.shape = arg.shape
+        self.dtype = np.dtype(dtype)
+
+    @classmethod
+    def _memo_key(cls, dtype, arg):
+        return (cls.__name__, np.dtype(dtype).str, id(arg))
+
+    @property
+    def name(self):
+        return f"cast{self._count}"
+
+
+class BinaryFuncEx(NumpyEx):
+    def __init__(self, func, left, right):
+        super().__init__(children=[left, right])
+        self.func = func
+        self.shape = calc_shape(left.shape, right.shape, func)
+        self.dtype = calc_type(func, [left, right])
+
+    def to_op(self):
+        return FUNCS[self.func.__name__]
+
+    @property
+    def name(self):
+        return f"binfun{self._count}"
+
+
+class BinaryNumpyEx(NumpyEx, Funcable):
+    """`+ - * /` node."""
+
+    def __init__(self, func, left, right):
+        super().__init__(children=[left, right])
+        self.func = func
+        self.shape = calc_shape(left.shape, right.shape, func)
+        self.dtype = calc_type(func, [left, right])
+
+    @property
+    def name(self):
+        return f"binex{self._count}"
+
+
+def pow_ex(func, left, right):
+    """`x ** k` with a Python-int k >= 2 becomes k-1 left-associated multiplies
+    (delayarray.py:316-324); k <= 1 returns x itself, as the reference does."""
+    exponent = right.val if isinstance(right, Scalar) else None
+    if not isinstance(exponent, int) or isinstance(exponent, bool):
+        return BinaryFuncEx(func, left, right)
+    ex = left
+    for _ in range(exponent - 1):
+        ex = BinaryNumpyEx(np.multiply, ex, left)
+    return ex
+
+
+def create_ex(func, args):
+    """Node factory with the reference's rewrites (delayarray.py:327-336)."""
+    name = func.__name__
+    if name in OPS:
+        return BinaryNumpyEx(func, *args)
+    if name == "square":
+        return BinaryNumpyEx(np.multiply, args[0], args[0])
+    if len(args) == 1:
+        return UnaryFuncEx(func, *args)
+    if name == "power":
+        return pow_ex(func, *args)
+    return BinaryFuncEx(func, *args)
+
+
+class NPArray(NumpyEx):
+    """Leaf: a backend array."""
+
+    def __init__(self, array):
+        super().__init__()
+        if not _backend.is_ndarray(array):
+            array = _backend.fallback.asarray(array)
+        self.array = array
+        self.shape = tuple(array.shape)
+        self.dtype = np.dtype(array.dtype)
+
+    @classmethod
+    def _memo_key(cls, array):
+        return ("NPArray", id(array))
+
+    def _force(self):
+        return self.array
+
+    def astype(self, dtype, **kwargs):
+        """Convert the leaf in place and return the same wrapper
+        (delayarray.py:401-408; tests/test.py:59-62)."""
+        dtype = np.dtype(dtype)
+        if dtype == self.dtype:
+            return self
+        converted = self.array.astype(dtype, **kwargs)
+        Memoiser._cache.pop(self._key, None)
+        self.array = converted
+        self.dtype = dtype
+        self._key = ("NPArray", id(converted))
+        Memoiser._cache[self._key] = self
+        return self
+
+    @property
+    def name(self):
+        return f"arr{self._count}"
+
+    @property
+    def inputs(self):
+        return {self.name: self}
+
+
+class Scalar(NumpyEx):
+    """A number.  Python numbers are weak (they take the dtype of the array
+    they meet); NumPy scalars keep theirs."""
+
+    def __init__(self, val):
+        super().__init__()
+        self.val = val
+        self.shape = ()
+
+    @classmethod
+    def _memo_key(cls, val):
+        return ("Scalar", type(val).__name__, repr(val))
+
+    @property
+    def dtype(self):
+        return np.asarray(self.val).dtype
+
+    def _force(self):
+        return self.val
+
+    @property
+    def name(self):
+        return str(self.val)
+
+    @property
+    def inputs(self):
+        return {}
+
+
+def arg_to_numpy_ex(arg):
+    """Operand -> node (delayarray.py:470-479)."""
+    if isinstance(arg, DelayArray):
+        return arg
+    if isinstance(arg, (numbers.Number, np.generic)):
+        return Scalar(arg)
+    if _backend.is_ndarray(arg) or isinstance(arg, np.ndarray):
+        if arg.ndim == 0 and isinstance(arg, np.ndarray):
+            return Scalar(arg[()])
+        return NPArray(arg)
+    raise NotImplementedError(f"cannot use a {type(arg).__name__} in a lazy expression")
+
+
+def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **unused):
+    """Full reduction -> 0-d backend array (what the reference's `sum` returns
+    on its GPU backend, delayarray.py:516-518); axis reductions are eager
+    backend calls on the materialised operand."""
+    arr = arg_to_numpy_ex(arr)
+    if out is not None or dtype is not None:
+        raise NotImplementedError("reductions with out= or dtype= are not supported")
+    if isinstance(axis, tuple) and sorted(a % max(arr.ndim, 1) for a in axis) == list(range(arr.ndim)):
+        axis = None
+    if arr.ndim <= 1 and axis in (0, -1):
+        axis = None
+    if axis is None and not keepdims and arr.size > 0:
+        return ReduceEx(func, arr)._force()
+    eager = {"add": "sum", "maximum": "max", "minimum": "min"}[func.__name__]
+    return getattr(_backend.fallback, eager)(arr._force(), axis=axis, keepdims=keepdims)
+
+
+def evaluate(*arrays):
+    """Evaluate several lazy arrays together, in one fused kernel when their
+    shapes agree, sharing common sub-expressions.  Returns the same objects."""
+    todo = [a for a in arrays if isinstance(a, DelayArray) and "array" not in a.__dict__]
+    if todo:
+        results = _backend.run_multi(todo)
+        for node, res in zip(todo, results):
+            node.array = res
+    return arrays
+
+
+def synchronize():
+    """Wait until the device has finished everything queued so far."""
+    _backend.synchronize()
+
+
+HANDLED_FUNCTIONS = {}
+
+
+def implements(np_function):
+    """Register an `__array_function__` implementation (delayarray.py:485-490)."""
+
+    def decorator(func):
+        HANDLED_FUNCTIONS[np_function] = func
+        return func
+
+    return decorator
+
+
+def _eager(name):
+    def call(arr, *args, **kwargs):
+        return getattr(_backend.fallback, name)(_unwrap(arr), *args, **kwargs)
+
+    call.__name__ = name
+    return call
+
+
+@implements(np.sum)
+def sum(arr, axis=None, **kwargs):
+    return _reduce(np.add, arr, axis=axis, **kwargs)
+
+
+@implements(np.max)
+def max(arr, axis=None, **kwargs):
+    return _reduce(np.maximum, arr, axis=axis, **kwargs)
+
+
+@implements(np.min)
+def min(arr, axis=None, **kwargs):
+    return _reduce(np.minimum, arr, axis=axis, **kwargs)
+
+
+@implements(np.mean)
+def mean(arr, axis=None, **kwargs):
+    arr = arg_to_numpy_ex(arr)
+    if axis is None and not kwargs:
+        return NPArray(_reduce(np.add, arr)) / arr.size
+    return _backend.fallback.mean(arr._force(), axis=axis, **kwargs)
+
+
+@implements(np.average)
+def average(arr, axis=None, weights=None, **kwargs):
+    if weights is None:
+        return mean(arr, axis=axis, **kwargs)
+    return _backend.fallback.average(_unwrap(arr), axis=axis, weights=_unwrap(weights), **kwargs)
+
+
+@implements(np.var)
+def var(arr, axis=None, ddof=0, **kwargs):
+    """Two-pass variance: mean, then the fused sum of squared deviations."""
+    arr = arg_to_numpy_ex(arr)
+    if axis is None and not kwargs:
+        centre = NPArray(_reduce(np.add, arr)) / arr.size
+        dev = arr - centre
+        return NPArray(_reduce(np.add, dev * dev)) / (arr.size - ddof)
+    return _backend.fallback.var(arr._force(), axis=axis, ddof=ddof, **kwargs)
+
+
+transpose = implements(np.transpose)(cast(_eager("transpose")))
+roll = implements(np.roll)(cast(_eager("roll")))
+repeat = implements(np.repeat)(cast(_eager("repeat")))
+cumsum = implements(np.cumsum)(cast(_eager("cumsum")))
+tile = implements(np.tile)(cast(_eager("tile")))
+diagflat = implements(np.diagflat)(cast(_eager("diagflat")))
+diag = implements(np.diag)(cast(_eager("diag")))
+
+
+# ufuncs re-exported under their NumPy names (delayarray.py:571-587)
+add = np.add
+multiply = np.multiply
+subtract = np.subtract
+divide = np.divide
+true_divide = np.true_divide
+dot = np.dot
+cos = np.cos
+sin = np.sin
+tan = np.tan
+tanh = np.tanh
+sinh = np.sinh
+cosh = np.cosh
+arcsin = np.arcsin
+arccos = np.arccos
+arctan = np.arctan
+arctan2 = np.arctan2
+exp = np.exp
+exp2 = np.exp2
+expm1 = np.expm1
+log = np.log
+log2 = np.log2
+log10 = np.log10
+log1p = np.log1p
+power = np.power
+sqrt = np.sqrt
+cbrt = np.cbrt
+square = np.square
+abs = np.abs
+absolute = np.absolute
+negative = np.negative
+maximum = np.maximum
+minimum = np.minimum
+greater = np.greater
+less = np.less
+floor = np.floor
+ceil = np.ceil
+hypot = np.hypot
+newaxis = None
+
+try:  # `erf` is a SciPy ufunc; the name is what the code generator keys on
+    from scipy.special import erf, erfc  # noqa: F401
+except ImportError:  # pragma: no cover
+    pass
+
+# dtypes
+double = np.double
+float64 = np.float64
+float32 = np.float32
+int32 = np.int32
+int64 = np.int64
+uint32 = np.uint32
+
+# creation routines: evaluated by the backend, wrapped as leaves
+# (delayarray.py:596-604, 620-625, 634-636, 641-643)
+for _name in ("empty", "empty_like", "eye", "identity", "ones", "ones_like", "zeros",
+              "zeros_like", "full", "full_like", "array", "asarray", "asanyarray",
+              "ascontiguousarray", "copy", "arange", "linspace", "logspace", "tri", "tril",
+              "triu", "asmatrix", "frombuffer", "fromfile", "fromfunction", "fromiter",
+              "fromstring", "loadtxt", "geomspace", "vander"):
+    _fn = getattr(_backend.fallback, _name, None)
+    if _fn is not None:
+        globals()[_name] = cast(_fn)
+del _name, _fn

@@ -1,0 +1,881 @@
+"""HIP fusion backend for MI355X (gfx950): the backend module the lazy front end
+binds to when `DELAY_CPU` is not set.
+
+Exports the duck-typed backend protocol of the reference's GPU backend
+(delayrepay/cuda.py:21-26,91-96): `np`, `fallback`, `is_ndarray(arr)`,
+`run(ex)`; plus `run_multi`, `run_into`, `synchronize` for the front end's
+multi-root, fused-assignment and timing entry points.
+
+`run` does what cuda.py:91-96 does with CuPy, without CuPy:
+  trace    one memoised walk of the DAG into a straight-line `Program`;
+  lower    choose a kernel shape from the operands' layouts, build the cache key
+           (structure + dtypes + layout classes + tunables) and, on a miss, emit
+           HIP C++ (`codegen`) and compile it with hiprtc through libdrhip
+           (in-memory cache, then an on-disk cache of code objects);
+  launch   pack the argument block and launch on the library stream; the output
+           comes from libdrhip's pooled allocator.
+Nothing is computed on the host, and there is no fall-back to NumPy: a missing
+library or GPU raises.
+"""
+import hashlib
+import os
+import struct
+import sys
+
+import numpy
+
+from . import codegen as cg
+from . import hiprt
+from .devarray import Buffer, ndarray, placeholder  # noqa: F401
+from .codegen import Program, dtype_code, code_dtype
+
+hiprt.lib()  # fail at import when libdrhip.so has not been built
+
+COMPILE_OPTS = [
+    "-O3",
+    "-ffp-contract=off",                      # a*b+c stays two roundings, like NumPy
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",  # no v_pk_*_f32
+]
+
+# Tunables; part of every cache key.  DELAYREPAY_TUNE="unroll=2,bpc=16" overrides.
+TUNE = {
+    "unroll": 4,      # vectors in flight per thread in flat kernels
+    "bpc": 8,         # resident blocks per CU that bound the grid of grid-stride kernels
+    "ntl": 1,         # non-temporal loads
+    "nts": 1,         # non-temporal stores
+    "tw": 128,        # stencil tile width (elements)
+    "th": 16,         # stencil tile height (rows)
+    "lds": 1,         # stage shifted views through LDS (0: read them directly)
+}
+for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
+    _k, _v = _kv.split("=")
+    TUNE[_k.strip()] = int(_v)
+
+_FUSED = "DELAY_UNFUSED" not in os.environ
+STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0}
+
+_SCALAR_FMT = {"f4": "f", "f8": "d", "i4": "i", "i8": "q", "u4": "I", "u1": "B", "b1": "B"}
+_COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal")
+
+
+def set_fused(flag):
+    """False: evaluate one kernel per DAG node with materialised temporaries (the
+    un-fused baseline the fused kernels are measured against)."""
+    global _FUSED
+    _FUSED = bool(flag)
+
+
+def is_ndarray(arr):
+    return isinstance(arr, ndarray)
+
+
+def synchronize():
+    hiprt.sync()
+
+
+# ---------------------------------------------------------------------------
+# tracing: DAG -> Program
+# ---------------------------------------------------------------------------
+
+class Tracer:
+    """Collects leaves, scalar parameters and SSA operations of one or more roots."""
+
+    def __init__(self, evaluated=None):
+        self.leaves = []
+        self.leaf_codes = []
+        self._leaf_index = {}
+        self.scalars = []
+        self.scalar_codes = []
+        self._scalar_index = {}
+        self.ops = []
+        self._memo = {}
+        self._evaluated = evaluated if evaluated is not None else {}
+
+    def leaf(self, arr):
+        code = dtype_code(arr.dtype)
+        key = (id(arr.buf), arr.offset, arr.shape, arr._strides, code)
+        idx = self._leaf_index.get(key)
+        if idx is None:
+            idx = len(self.leaves)
+            self._leaf_index[key] = idx
+            self.leaves.append(arr)
+            self.leaf_codes.append(code)
+        return ("l", idx), code
+
+    def scalar(self, value, code, ident=None):
+        key = (ident if ident is not None else ("v", repr(value)), code)
+        idx = self._scalar_index.get(key)
+        if idx is None:
+            idx = len(self.scalars)
+            self._scalar_index[key] = idx
+            with numpy.errstate(all="ignore"):
+                self.scalars.append(code_dtype(code).type(value))
+            self.scalar_codes.append(code)
+        return ("s", idx), code
+
+    def op(self, name, compute, result, refs):
+        self.ops.append((name, compute, result, tuple(refs)))
+        return ("v", len(self.ops) - 1), result
+
+    def visit(self, node):
+        from .delayarray import Scalar, CastEx, ReduceEx, NPArray, result_dtype, _descr
+        nid = id(node)
+        hit = self._memo.get(nid)
+        if hit is not None:
+            return hit
+        arr = self._evaluated.get(nid)
+        if arr is None:
+            arr = node.__dict__.get("array")
+            if arr is not None and not isinstance(node, NPArray):
+                deps = node.__dict__.get("_deps")
+                if deps is not None and any(buf.version != ver for buf, ver in deps):
+                    arr = None  # stale: recompute inside this kernel
+        if arr is not None:
+            res = self.leaf(arr)
+        elif isinstance(node, Scalar):
+            res = self.scalar(node.val, dtype_code(numpy.asarray(node.val).dtype), id(node))
+        elif isinstance(node, CastEx):
+            ref, code = self.visit(node.children[0])
+            target = dtype_code(node.dtype)
+            res = self.op("cast", target, target, [ref]) if code != target else (ref, code)
+        elif isinstance(node, ReduceEx):
+            res = self.leaf(node._force())
+        else:
+            func = node.func
+            name = func.__name__
+            if name not in cg.SUPPORTED_UFUNCS:
+                raise NotImplementedError(f"ufunc {name!r} cannot be fused by the HIP backend")
+            traced, descrs = [], []
+            for child in node.children:
+                if type(child) is Scalar:
+                    traced.append(None)
+                    descrs.append(_descr(child))
+                else:
+                    ref = self.visit(child)
+                    traced.append(ref)
+                    descrs.append(("a", code_dtype(ref[1]).str))
+            descrs = tuple(descrs)
+            result = dtype_code(result_dtype(func, descrs))
+            compute = result
+            if name in _COMPARES:
+                compute = dtype_code(result_dtype(numpy.add, descrs))
+            refs = []
+            for child, tr in zip(node.children, traced):
+                if tr is None:
+                    refs.append(self.scalar(child.val, compute, id(child))[0])
+                else:
+                    refs.append(tr[0])
+            res = self.op(name, compute, result, refs)
+        self._memo[nid] = res
+        return res
+
+    def program(self, roots):
+        return Program(self.leaf_codes, self.scalar_codes, self.ops, roots)
+
+    def deps(self):
+        seen = {}
+        for arr in self.leaves:
+            seen[id(arr.buf)] = arr.buf
+        return tuple((buf, buf.version) for buf in seen.values())
+
+
+# ---------------------------------------------------------------------------
+# layout analysis
+# ---------------------------------------------------------------------------
+
+def _broadcast_strides(arr, shape):
+    """Element strides of `arr` viewed at `shape` (NumPy broadcasting)."""
+    nd = len(shape)
+    pad = nd - len(arr.shape)
+    if pad < 0:
+        raise ValueError(f"operand of shape {arr.shape} does not broadcast to {shape}")
+    out = [0] * nd
+    for k in range(len(arr.shape)):
+        d = arr.shape[k]
+        if d == shape[pad + k]:
+            out[pad + k] = arr._strides[k] if d != 1 else 0
+        elif d == 1:
+            out[pad + k] = 0
+        else:
+            raise ValueError(f"operand of shape {arr.shape} does not broadcast to {shape}")
+    return out
+
+
+def _merge_dims(shape, stride_sets):
+    """Drop unit dims and merge neighbours that every operand walks contiguously."""
+    dims = [(d, [s[k] for s in stride_sets]) for k, d in enumerate(shape) if d != 1]
+    if not dims:
+        return [], [[] for _ in stride_sets]
+    merged = [dims[0]]
+    for d, strides in dims[1:]:
+        pd, ps = merged[-1]
+        if all(p == s * d for p, s in zip(ps, strides)):
+            merged[-1] = (pd * d, strides)
+        else:
+            merged.append((d, strides))
+    mshape = [d for d, _ in merged]
+    msets = [[st[i] for _, st in merged] for i in range(len(stride_sets))]
+    return mshape, msets
+
+
+class Lowered:
+    """A kernel choice for one evaluation: cache key, source builder, launch recipe."""
+
+    __slots__ = ("key", "kind", "emit", "fmt", "values", "grid", "fin_count", "lds")
+
+
+# ---------------------------------------------------------------------------
+# kernel cache
+# ---------------------------------------------------------------------------
+
+class Kernel:
+    __slots__ = ("func", "finalize", "packer", "source")
+
+
+_KERNELS = {}
+
+
+def _cache_dir():
+    d = os.environ.get("DELAYREPAY_CACHE_DIR")
+    if d is None:
+        d = os.path.join(os.path.expanduser("~"), ".cache", "delayrepay_amd")
+    return d
+
+
+def _load_or_compile(source):
+    """Module handle for `source`: on-disk code-object cache, else hiprtc."""
+    hiprt.init()
+    use_disk = "DELAYREPAY_NO_DISK_CACHE" not in os.environ
+    path = None
+    if use_disk:
+        arch = hiprt.device_info()["arch"]
+        digest = hashlib.sha256("\0".join([source, arch] + COMPILE_OPTS).encode()).hexdigest()
+        path = os.path.join(_cache_dir(), digest + ".co")
+        if os.path.exists(path):
+            try:
+                with open(path, "rb") as fh:
+                    module = hiprt.load_code(fh.read())
+                STATS["disk_hits"] += 1
+                return module
+            except (OSError, hiprt.DrhipError):
+                pass
+    module, code = hiprt.compile_module(source, "dr_kernel.hip", COMPILE_OPTS)
+    STATS["compiles"] += 1
+    if path is not None:
+        try:
+            os.makedirs(os.path.dirname(path), exist_ok=True)
+            tmp = f"{path}.{os.getpid()}.tmp"
+            with open(tmp, "wb") as fh:
+                fh.write(code)
+            os.replace(tmp, path)
+        except OSError:
+            pass
+    return module
+
+
+def _kernel_for(low, with_finalize):
+    kern = _KERNELS.get(low.key)
+    if kern is not None:
+        STATS["mem_hits"] += 1
+        return kern
+    source = low.emit()
+    module = _load_or_compile(source)
+    kern = Kernel()
+    kern.source = source
+    kern.func = hiprt.get_function(module, "dr_kernel")
+    kern.finalize = hiprt.get_function(module, "dr_finalize") if with_finalize else None
+    kern.packer = struct.Struct(low.fmt)
+    _KERNELS[low.key] = kern
+    return kern
+
+
+# ---------------------------------------------------------------------------
+# lowering
+# ---------------------------------------------------------------------------
+
+_CUS = None
+
+
+def _grid_cap():
+    """Blocks that fill the device `bpc` deep (256 CUs assumed until a device is open)."""
+    global _CUS
+    if _CUS is None:
+        if not hiprt._initialised:
+            return 256 * TUNE["bpc"]
+        _CUS = hiprt.device_info()["compute_units"]
+    return _CUS * TUNE["bpc"]
+
+
+def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, reduce_op,
+           in_place=False):
+    """Pick the kernel shape.  `out_ptrs`/`out_strides` describe the destinations
+    (element strides at `out_shape`); for a reduction they are empty and the
+    partial-sums pointer is appended at launch."""
+    n = 1
+    for d in out_shape:
+        n *= d
+    leaf_strides = [_broadcast_strides(a, out_shape) for a in leaves]
+    mshape, msets = _merge_dims(out_shape, leaf_strides + list(out_strides))
+    m_leaf, m_out = msets[:len(leaves)], msets[len(leaves):]
+    ndim = len(mshape)
+    low = Lowered()
+    low.lds = 0
+    low.fin_count = 0
+    scal_fmt = "".join(_SCALAR_FMT[c] for c in prog.scalars)
+    scal_vals = list(scalars)
+    tune = tuple(sorted(TUNE.items()))
+
+    flat = ndim <= 1 and all(s == [1] or s == [0] or s == [] for s in m_leaf) \
+        and all(s == [1] or s == [] for s in m_out)
+    if flat:
+        leaf_class = tuple("b" if (s == [0] and n > 1) else "c" for s in m_leaf)
+        ptrs = [a.ptr for a in leaves]
+        widths_ok = all(cg.ITEMSIZE[c] in (4, 8) for c, k in zip(prog.leaves, leaf_class) if k == "c")
+        align_ok = all(p % 16 == 0 for p, k in zip(ptrs, leaf_class) if k == "c")
+        if not reduce_op:
+            widths_ok = widths_ok and all(cg.ITEMSIZE[c] in (4, 8) for c in out_codes)
+            align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
+        vec = widths_ok and align_ok and n >= 64
+        unroll = TUNE["unroll"]
+        low.kind = "flat"
+        low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place, tune)
+        holder = {}
+
+        def emit():
+            src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, bool(TUNE["ntl"]),
+                                  bool(TUNE["nts"]), restrict=not in_place, reduce_op=reduce_op)
+            return src
+        low.emit = emit
+        if vec:
+            widths = [cg.ITEMSIZE[c] for c, k in zip(prog.leaves, leaf_class) if k == "c"]
+            if not reduce_op:
+                widths += [cg.ITEMSIZE[c] for c in out_codes]
+            E = 16 // min(widths) if widths else 4
+        else:
+            E = 1
+        work = max(1, n // E)
+        blocks = -(-work // (cg.BLOCK * unroll))
+        low.grid = max(1, min(blocks, _grid_cap()))
+        n_out_ptr = 1 if reduce_op else len(out_ptrs)
+        low.fmt = "@" + "P" * (len(ptrs) + n_out_ptr) + scal_fmt + "q"
+        low.values = (ptrs, scal_vals, [n])
+        if reduce_op:
+            low.fin_count = low.grid
+        return low
+
+    tiled = (not reduce_op and ndim == 2 and all(s[1] == 1 for s in m_out)
+             and all(s[1] == 1 or s == [0, 0] for s in m_leaf))
+    if tiled:
+        H, W = mshape
+        tw, th = TUNE["tw"], TUNE["th"]
+        # halo group: >= 2 leaves that are shifted views of one buffer
+        groups = {}
+        for i, (a, s) in enumerate(zip(leaves, m_leaf)):
+            if s[1] == 1 and s[0] > 0:
+                groups.setdefault((id(a.buf), s[0], prog.leaves[i]), []).append(i)
+        best = max(groups.values(), key=len) if groups else []
+        kinds = [None] * len(leaves)
+        group = None
+        if len(best) >= 2 and TUNE["lds"]:
+            rs = m_leaf[best[0]][0]
+            ref_off = min(leaves[i].offset for i in best)
+            shifts = {}
+            for i in best:
+                d = leaves[i].offset - ref_off
+                dy, dx = divmod(d, rs)
+                if dx > rs // 2:
+                    dy, dx = dy + 1, dx - rs
+                shifts[i] = (dy, dx)
+            dy_max = max(dy for dy, _ in shifts.values())
+            dx_min = min(dx for _, dx in shifts.values())
+            dx_max = max(dx for _, dx in shifts.values())
+            itemsize = cg.ITEMSIZE[prog.leaves[best[0]]]
+            lds_bytes = (th + dy_max) * (tw + dx_max - dx_min) * itemsize
+            if dy_max <= 16 and dx_max - dx_min <= 32 and lds_bytes <= 48 * 1024:
+                group = (prog.leaves[best[0]], dy_max, dx_min, dx_max)
+                for i in best:
+                    kinds[i] = ("g",) + shifts[i]
+                g_buf = leaves[best[0]].buf
+                g_ptr = g_buf.ptr + ref_off * itemsize
+                g_args = [rs, -ref_off, g_buf.nbytes // itemsize - ref_off]
+        for i, s in enumerate(m_leaf):
+            if kinds[i] is None:
+                kinds[i] = ("b",) if s == [0, 0] else ("d",)
+        kinds = tuple(kinds)
+        low.kind = "tile2d"
+        low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune)
+
+        def emit():
+            return cg.emit_stencil(prog, kinds, group, out_codes, tw, th, restrict=not in_place)
+        low.emit = emit
+        tiles_x = -(-W // tw)
+        tiles_y = -(-H // th)
+        low.grid = tiles_x * tiles_y
+        ptrs = [a.ptr for a, k in zip(leaves, kinds) if k[0] != "g"]
+        fmt = "@" + "P" * len(ptrs)
+        tail_vals = []
+        if group is not None:
+            fmt += "P"
+            ptrs.append(g_ptr)
+        fmt += "P" * len(out_ptrs) + scal_fmt + "ii"
+        tail_vals += [H, W]
+        if group is not None:
+            fmt += "qqq"
+            tail_vals += g_args
+        fmt += "i"
+        tail_vals.append(tiles_x)
+        for k, s in zip(kinds, m_leaf):
+            if k[0] == "d":
+                fmt += "q"
+                tail_vals.append(s[0])
+        for s in m_out:
+            fmt += "q"
+            tail_vals.append(s[0])
+        low.fmt = fmt
+        low.values = (ptrs, scal_vals, tail_vals)
+        return low
+
+    # general strided kernel
+    if ndim == 0:
+        mshape, m_leaf, m_out, ndim = [1], [[0] for _ in m_leaf], [[0] for _ in m_out], 1
+    index32 = n < 2 ** 31
+    low.kind = "nd"
+    low.key = ("nd", prog.key(), ndim, tuple(out_codes), index32, reduce_op, tune)
+
+    def emit():
+        return cg.emit_nd(prog, ndim, out_codes, index32, reduce_op)
+    low.emit = emit
+    blocks = -(-n // cg.BLOCK)
+    low.grid = max(1, min(blocks, _grid_cap()))
+    n_out_ptr = 1 if reduce_op else len(out_ptrs)
+    fmt = "@" + "P" * (len(leaves) + n_out_ptr) + scal_fmt + "q" + ("I" if index32 else "q") * ndim
+    tail = [n] + list(mshape)
+    for s in m_leaf:
+        fmt += "q" * ndim
+        tail += s
+    if not reduce_op:
+        for s in m_out:
+            fmt += "q" * ndim
+            tail += s
+    low.fmt = fmt
+    low.values = ([a.ptr for a in leaves], scal_vals, tail)
+    if reduce_op:
+        low.fin_count = low.grid
+    return low
+
+
+def _launch(low, out_ptrs, reduce_out=None, reduce_code=None):
+    """Compile if needed and launch.  For a reduction, `reduce_out` is the device
+    address of the 0-d result."""
+    ptrs, scal_vals, tail = low.values
+    for p in ptrs:
+        if not p:
+            raise RuntimeError("an operand has no device memory (placeholder array)")
+    kern = _kernel_for(low, reduce_out is not None)
+    if reduce_out is not None:
+        itemsize = cg.ITEMSIZE[reduce_code]
+        partial = hiprt.malloc(low.fin_count * itemsize)
+        args = kern.packer.pack(*ptrs, partial, *scal_vals, *tail)
+        hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
+        fin = struct.pack("@PPi", partial, reduce_out, low.fin_count)
+        hiprt.launch(kern.finalize, 1, cg.BLOCK, 0, fin, len(fin))
+        hiprt.free(partial)  # stream-ordered: safe to recycle once queued
+        STATS["launches"] += 2
+    else:
+        # tile2d puts the halo pointer after the direct operands; flat/nd have none
+        args = _pack(kern, low, ptrs, out_ptrs, scal_vals, tail)
+        hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
+        STATS["launches"] += 1
+
+
+def _pack(kern, low, ptrs, out_ptrs, scal_vals, tail):
+    return kern.packer.pack(*ptrs, *out_ptrs, *scal_vals, *tail)
+
+
+# ---------------------------------------------------------------------------
+# evaluation entry points
+# ---------------------------------------------------------------------------
+
+def _execute(tracer, roots, dsts=None, reduce_op=None, launch=True):
+    """Run traced `roots` (list of (ref, code)).  Returns output arrays (or the
+    `Lowered` object when `launch` is False)."""
+    prog = tracer.program(roots)
+    leaves = tracer.leaves
+    if reduce_op:
+        shape = numpy.broadcast_shapes(*[a.shape for a in leaves]) if leaves else ()
+        code = roots[0][1]
+        acc = "i8" if (reduce_op == "add" and code in ("i4", "u4", "u1", "b1")) else code
+        low = _lower(prog, leaves, tracer.scalars, tuple(shape), [acc], [], [], reduce_op)
+        if not launch:
+            return low
+        out = ndarray((), code_dtype(acc))
+        _launch(low, [], out.ptr, acc)
+        return [out]
+    if dsts is None:
+        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
+        make = ndarray if launch else placeholder
+        outs = [make(shape, code_dtype(code)) for _, code in roots]
+        in_place = False
+    else:
+        shape = dsts[0].shape
+        outs = dsts
+        in_place = any(a.buf is d.buf for a in leaves for d in dsts)
+    n = 1
+    for d in shape:
+        n *= d
+    if n == 0:
+        return outs
+    out_codes = [dtype_code(o.dtype) for o in outs]
+    out_ptrs = [o.ptr for o in outs]
+    out_strides = [_broadcast_strides(o, shape) for o in outs]
+    low = _lower(prog, leaves, tracer.scalars, shape, out_codes, out_ptrs, out_strides, None,
+                 in_place)
+    if not launch:
+        return low
+    _launch(low, out_ptrs)
+    return outs
+
+
+def _trace_root(tracer, node):
+    from .delayarray import ReduceEx
+    if isinstance(node, ReduceEx) and "array" not in node.__dict__:
+        raise TypeError("a reduction must be the root of its own evaluation")
+    return tracer.visit(node)
+
+
+def _run_unfused(ex, evaluated):
+    """One kernel per interior node, children first."""
+    from .delayarray import NPArray, Scalar, ReduceEx
+    nid = id(ex)
+    if nid in evaluated:
+        return evaluated[nid]
+    if isinstance(ex, NPArray):
+        return ex.array
+    for child in ex.children:
+        if not isinstance(child, (Scalar, NPArray)):
+            _run_unfused(child, evaluated)
+    tracer = Tracer(evaluated)
+    if isinstance(ex, ReduceEx):
+        root = tracer.visit(ex.children[0])
+        out = _execute(tracer, [root], reduce_op=ex.func.__name__)[0]
+    else:
+        root = tracer.visit(ex)
+        out = _execute(tracer, [root])[0]
+    evaluated[nid] = out
+    return out
+
+
+def run(ex):
+    """Evaluate one DAG root; returns a new device array owned by the caller
+    (cf. cuda.py:91-96)."""
+    from .delayarray import ReduceEx
+    if not _FUSED:
+        evaluated = {}
+        out = _run_unfused(ex, evaluated)
+        return out
+    tracer = Tracer()
+    if isinstance(ex, ReduceEx):
+        root = tracer.visit(ex.children[0])
+        out = _execute(tracer, [root], reduce_op=ex.func.__name__)[0]
+    else:
+        root = _trace_root(tracer, ex)
+        out = _execute(tracer, [root])[0]
+    ex.__dict__["_deps"] = tracer.deps()
+    return out
+
+
+def run_multi(exs):
+    """Evaluate several roots; roots of equal shape share one kernel (and their
+    common sub-expressions)."""
+    if not _FUSED:
+        return [run(ex) for ex in exs]
+    by_shape = {}
+    for i, ex in enumerate(exs):
+        by_shape.setdefault(tuple(ex.shape), []).append(i)
+    results = [None] * len(exs)
+    for shape, idxs in by_shape.items():
+        tracer = Tracer()
+        roots = [_trace_root(tracer, exs[i]) for i in idxs]
+        outs = _execute(tracer, roots)
+        deps = tracer.deps()
+        for i, out in zip(idxs, outs):
+            if out.shape != shape:   # every leaf of this root was a broadcast scalar
+                out = materialise(out, shape=shape)
+            results[i] = out
+            exs[i].__dict__["_deps"] = deps
+    return results
+
+
+def _extent(arr):
+    """[lo, hi) element range of the buffer that `arr` can touch."""
+    lo = hi = arr.offset
+    for d, s in zip(arr.shape, arr._strides):
+        if d == 0:
+            return (arr.offset, arr.offset)
+        if s >= 0:
+            hi += (d - 1) * s
+        else:
+            lo += (d - 1) * s
+    return lo, hi + 1
+
+
+def _same_view(a, b):
+    return (a.offset == b.offset and a.shape == b.shape and a._strides == b._strides
+            and a.dtype == b.dtype)
+
+
+def _write(tracer, root, dst):
+    """Launch traced `root` into the existing view `dst`, guarding against reading
+    what the kernel overwrites."""
+    shape = dst.shape
+    for a in tracer.leaves:
+        _broadcast_strides(a, shape)  # raises when the value does not fit the destination
+    hazard = False
+    d_lo, d_hi = _extent(dst)
+    for a in tracer.leaves:
+        if a.buf is dst.buf and not _same_view(a, dst):
+            a_lo, a_hi = _extent(a)
+            it = dst.dtype.itemsize
+            if a_lo * a.dtype.itemsize < d_hi * it and d_lo * it < a_hi * a.dtype.itemsize:
+                hazard = True
+    buf = dst.buf
+    if not hazard:
+        _execute(tracer, [root], dsts=[dst])
+        buf.touch()
+        return
+    # Ping-pong: write into the shadow allocation, which mirrors the buffer
+    # everywhere outside `region`, then swap the two device pointers.  Every view
+    # of the buffer (they share the Buffer object) sees the update at once.
+    region = (dst.offset, dst.shape, dst._strides, dst.dtype.str)
+    if buf.shadow is None:
+        buf.shadow = hiprt.malloc(max(buf.nbytes, 1))
+        buf.shadow_region = None
+    if buf.shadow_region != region:
+        hiprt.memcpy_d2d(buf.shadow, buf.ptr, buf.nbytes)
+    target = ndarray(dst.shape, dst.dtype, Buffer(buf.nbytes, ptr=buf.shadow), dst.offset,
+                     dst._strides)
+    try:
+        _execute(tracer, [root], dsts=[target])
+    finally:
+        target.buf.ptr = None  # borrowed pointer: must not be freed with the helper
+    buf.ptr, buf.shadow = buf.shadow, buf.ptr
+    buf.shadow_region = region
+    buf.version += 1
+
+
+def run_into(ex, dst):
+    """`dst[...] = ex` as one fused kernel writing the destination view directly."""
+    if not _FUSED:
+        assign(dst, run(ex))
+        return
+    tracer = Tracer()
+    root = _trace_root(tracer, ex)
+    _write(tracer, root, dst)
+
+
+def assign(dst, value):
+    """`dst[...] = value` for a number, a host array or a device array."""
+    from .delayarray import DelayArray
+    if isinstance(value, DelayArray):
+        if "array" in value.__dict__:
+            value = value._force()
+        else:
+            return run_into(value, dst)
+    tracer = Tracer()
+    if isinstance(value, ndarray):
+        root = tracer.leaf(value)
+    elif isinstance(value, (int, float, bool, numpy.generic)):
+        root = tracer.scalar(value, dtype_code(dst.dtype))
+    else:
+        host = numpy.asarray(value)
+        if host.ndim == 0:
+            root = tracer.scalar(host[()], dtype_code(dst.dtype))
+        else:
+            root = tracer.leaf(ndarray.from_host(host))
+    _write(tracer, root, dst)
+
+
+def materialise(arr, dtype=None, shape=None):
+    """Contiguous copy of a device array, optionally converted / broadcast."""
+    tracer = Tracer()
+    root = tracer.leaf(arr)
+    if dtype is not None and numpy.dtype(dtype) != arr.dtype:
+        code = dtype_code(dtype)
+        root = tracer.op("cast", code, code, [root[0]])
+    if shape is not None and tuple(shape) != arr.shape:
+        out = ndarray(shape, code_dtype(root[1]))
+        _execute(tracer, [root], dsts=[out])
+        return out
+    return _execute(tracer, [root])[0]
+
+
+def lower_only(exs, dst=None):
+    """Trace and lower without touching the device: returns (Lowered, source).
+    Works with placeholder arrays on a machine that has no GPU."""
+    from .delayarray import ReduceEx
+    if not isinstance(exs, (list, tuple)):
+        exs = [exs]
+    tracer = Tracer()
+    if isinstance(exs[0], ReduceEx):
+        root = tracer.visit(exs[0].children[0])
+        low = _execute(tracer, [root], reduce_op=exs[0].func.__name__, launch=False)
+    else:
+        roots = [tracer.visit(ex) for ex in exs]
+        low = _execute(tracer, roots, dsts=None if dst is None else [dst], launch=False)
+    return low, low.emit()
+
+
+def compile_source(source):
+    """hiprtc-compile generated source without loading it (no GPU needed)."""
+    return hiprt.compile_only(source, "dr_kernel.hip", COMPILE_OPTS)
+
+
+# ---------------------------------------------------------------------------
+# `np` and `fallback` namespaces of the backend protocol
+# ---------------------------------------------------------------------------
+
+def _upload(fn):
+    def wrapper(*args, **kwargs):
+        args = [a.get() if isinstance(a, ndarray) else a for a in args]
+        return ndarray.from_host(fn(*args, **kwargs))
+    wrapper.__name__ = fn.__name__
+    return wrapper
+
+
+def _filled(value_of):
+    def make(shape, *args, dtype=None, **kwargs):
+        value, default = value_of(args)
+        if dtype is None:
+            dtype = default
+        if isinstance(shape, (int, numpy.integer)):
+            shape = (int(shape),)
+        out = ndarray(tuple(shape), dtype)
+        if value is not None and out.size:
+            assign(out, value)
+        return out
+    return make
+
+
+def _like(maker):
+    def make(proto, *args, dtype=None, **kwargs):
+        proto = proto._force() if hasattr(proto, "_force") else proto
+        return maker(proto.shape, *args, dtype=dtype or proto.dtype)
+    return make
+
+
+class _Random:
+    """Host NumPy generators, uploaded (input generation; cf. delayrepay/random.py)."""
+
+    def __getattr__(self, name):
+        fn = getattr(numpy.random, name)
+        if name in ("seed", "get_state", "set_state"):
+            return fn
+        return _upload(fn)
+
+
+class _Fallback:
+    """Eager routines on device arrays (the reference uses `cupy` here, cuda.py:22).
+    Reductions and copies run as generated kernels; creation routines build on the
+    host and upload; what has no device implementation raises."""
+
+    newaxis = None
+    pi = numpy.pi
+
+    empty = staticmethod(_filled(lambda a: (None, numpy.float64)))
+    zeros = staticmethod(_filled(lambda a: (0, numpy.float64)))
+    ones = staticmethod(_filled(lambda a: (1, numpy.float64)))
+    full = staticmethod(_filled(lambda a: (a[0], numpy.asarray(a[0]).dtype)))
+    empty_like = staticmethod(_like(empty.__func__))
+    zeros_like = staticmethod(_like(zeros.__func__))
+    ones_like = staticmethod(_like(ones.__func__))
+    full_like = staticmethod(_like(full.__func__))
+
+    @staticmethod
+    def asarray(obj, dtype=None, **kwargs):
+        if hasattr(obj, "_force"):
+            obj = obj._force()
+        if isinstance(obj, ndarray):
+            return obj if dtype is None or numpy.dtype(dtype) == obj.dtype else obj.astype(dtype)
+        return ndarray.from_host(numpy.asarray(obj, dtype=dtype))
+
+    array = asarray
+    asanyarray = asarray
+
+    @staticmethod
+    def ascontiguousarray(obj, dtype=None):
+        arr = _Fallback.asarray(obj, dtype)
+        return arr if arr.is_contiguous else arr.copy()
+
+    @staticmethod
+    def copy(obj):
+        return _Fallback.asarray(obj).copy()
+
+    @staticmethod
+    def transpose(arr, axes=None):
+        return arr.transpose(axes) if axes is not None else arr.transpose()
+
+    @staticmethod
+    def _reduce(arr, name, axis, keepdims):
+        from .delayarray import NPArray, ReduceEx
+        if axis is not None or keepdims:
+            raise NotImplementedError("axis reductions are not implemented on the device yet")
+        return run(ReduceEx(getattr(numpy, name), NPArray(arr)))
+
+    @staticmethod
+    def sum(arr, axis=None, keepdims=False):
+        return _Fallback._reduce(arr, "add", axis, keepdims)
+
+    @staticmethod
+    def max(arr, axis=None, keepdims=False):
+        return _Fallback._reduce(arr, "maximum", axis, keepdims)
+
+    @staticmethod
+    def min(arr, axis=None, keepdims=False):
+        return _Fallback._reduce(arr, "minimum", axis, keepdims)
+
+    @staticmethod
+    def roll(arr, shift, axis=None):
+        if axis is None:
+            flat = arr.reshape(arr.size)
+            return _Fallback.roll(flat, shift, 0).reshape(arr.shape)
+        n = arr.shape[axis]
+        out = ndarray(arr.shape, arr.dtype)
+        if n == 0:
+            return out
+        shift %= n
+        head = [slice(None)] * arr.ndim
+        tail = [slice(None)] * arr.ndim
+        head[axis], tail[axis] = slice(shift, None), slice(0, n - shift)
+        assign(out[tuple(head)], arr[tuple(tail)])
+        if shift:
+            head[axis], tail[axis] = slice(0, shift), slice(n - shift, None)
+            assign(out[tuple(head)], arr[tuple(tail)])
+        return out
+
+    def __getattr__(self, name):
+        fn = getattr(numpy, name, None)
+        if name in ("eye", "identity", "arange", "linspace", "logspace", "geomspace", "tri",
+                    "frombuffer", "fromfile", "fromfunction", "fromiter", "fromstring",
+                    "loadtxt", "vander"):
+            return _upload(fn)
+        raise AttributeError(f"{name} has no device implementation in the HIP backend")
+
+
+class _Np:
+    """The slice of the array namespace the front end reads from `backend.np`
+    (delayarray.py:188-194, __init__.py:17, random.py:6-13)."""
+
+    pi = numpy.pi
+    random = _Random()
+    add = numpy.add
+    subtract = numpy.subtract
+    multiply = numpy.multiply
+    true_divide = numpy.true_divide
+    divide = numpy.divide
+    matmul = numpy.matmul
+
+
+np = _Np()
+fallback = _Fallback()
+
+sys.modules[__name__].np = np

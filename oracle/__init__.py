@@ -1,0 +1,3 @@
+"""CPU restatement of the reference's evaluation path.  TEST INFRASTRUCTURE ONLY:
+imported by tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg;
+never by the delayrepay_amd package."""
