@@ -22,6 +22,10 @@ extern "C" void drhip_k_launch_fill64(void* dst, uint64_t v, size_t n, hipStream
 extern "C" void drhip_k_launch_copy(void* dst, const void* src, size_t nvec,
                                     unsigned grid, hipStream_t s);
 
+extern "C" void drhip_k_launch_matmul(int is_double, const void* A, const void* B, void* C, long M,
+                                      long N, long K, long lda, long ldb, long ldc,
+                                      hipStream_t s);
+
 namespace {
 
 thread_local std::string t_err;
@@ -235,6 +239,20 @@ int drhip_copy_kernel(void* dst, const void* src, size_t nbytes, unsigned grid) 
     if (nbytes == 0) return 0;
     if (grid == 0) grid = (unsigned)g_prop.multiProcessorCount * 8u;
     drhip_k_launch_copy(dst, src, nbytes / 16, grid, g_stream);
+    HIP_TRY(hipGetLastError());
+    g_cnt.n_launches++;
+    return 0;
+}
+
+int drhip_matmul(int is_double, const void* a, const void* b, void* c, int64_t m, int64_t n,
+                 int64_t k, int64_t lda, int64_t ldb, int64_t ldc) {
+    NEED_INIT();
+    if (!a || !b || !c) return fail(DRHIP_EINVAL, "drhip_matmul", "null operand");
+    if (m < 0 || n < 0 || k < 0 || lda < k || ldb < n || ldc < n)
+        return fail(DRHIP_EINVAL, "drhip_matmul", "bad dimensions");
+    if (m == 0 || n == 0) return 0;
+    if ((m + 63) / 64 > 65535) return fail(DRHIP_EINVAL, "drhip_matmul", "too many rows");
+    drhip_k_launch_matmul(is_double, a, b, c, m, n, k, lda, ldb, ldc, g_stream);
     HIP_TRY(hipGetLastError());
     g_cnt.n_launches++;
     return 0;

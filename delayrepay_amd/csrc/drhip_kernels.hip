@@ -39,6 +39,55 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(u32x4* __restrict__ dst,
     }
 }
 
+// C[M,N] = A[M,K] * B[K,N], row-major with leading dimensions.  64x64 output tile
+// per 256-thread block, 4x4 outputs per thread, K staged through LDS 16 deep.
+// Serves the eager `dot` of the array namespace; it is not on the fused path.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void matmul_kernel(const T* __restrict__ A,
+                                                        const T* __restrict__ B,
+                                                        T* __restrict__ C, long M, long N, long K,
+                                                        long lda, long ldb, long ldc) {
+    constexpr int TM = 64, TN = 64, TK = 16;
+    __shared__ T As[TK][TM + 1];
+    __shared__ T Bs[TK][TN + 1];
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const long row0 = (long)blockIdx.y * TM, col0 = (long)blockIdx.x * TN;
+    T acc[4][4] = {};
+    for (long k0 = 0; k0 < K; k0 += TK) {
+        for (int i = threadIdx.x; i < TM * TK; i += kBlock) {
+            const int r = i / TK, k = i % TK;
+            const long gr = row0 + r, gk = k0 + k;
+            As[k][r] = (gr < M && gk < K) ? A[gr * lda + gk] : T(0);
+        }
+        for (int i = threadIdx.x; i < TK * TN; i += kBlock) {
+            const int k = i / TN, c = i % TN;
+            const long gk = k0 + k, gc = col0 + c;
+            Bs[k][c] = (gk < K && gc < N) ? B[gk * ldb + gc] : T(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < TK; ++k) {
+            T a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Bs[k][tx + 16 * j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const long r = row0 + ty * 4 + i, c = col0 + tx + 16 * j;
+            if (r < M && c < N) C[r * ldc + c] = acc[i][j];
+        }
+}
+
 unsigned fill_grid(size_t n) {
     size_t b = (n + kBlock - 1) / kBlock;
     const size_t cap = 256u * 16u;
@@ -61,4 +110,16 @@ extern "C" void drhip_k_launch_copy(void* dst, const void* src, size_t nvec, uns
                                     hipStream_t s) {
     hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(kBlock), 0, s, (u32x4*)dst,
                        (const u32x4*)src, nvec);
+}
+
+extern "C" void drhip_k_launch_matmul(int is_double, const void* A, const void* B, void* C, long M,
+                                      long N, long K, long lda, long ldb, long ldc,
+                                      hipStream_t s) {
+    dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+    if (is_double)
+        hipLaunchKernelGGL(matmul_kernel<double>, grid, dim3(kBlock), 0, s, (const double*)A,
+                           (const double*)B, (double*)C, M, N, K, lda, ldb, ldc);
+    else
+        hipLaunchKernelGGL(matmul_kernel<float>, grid, dim3(kBlock), 0, s, (const float*)A,
+                           (const float*)B, (float*)C, M, N, K, lda, ldb, ldc);
 }

@@ -39,10 +39,13 @@ COMPILE_OPTS = [
 
 # Tunables; part of every cache key.  DELAYREPAY_TUNE="unroll=2,bpc=16" overrides.
 TUNE = {
-    "unroll": 4,      # vectors in flight per thread in flat kernels
-    "bpc": 8,         # resident blocks per CU that bound the grid of grid-stride kernels
-    "ntl": 1,         # non-temporal loads
-    "nts": 1,         # non-temporal stores
+    "unroll": 1,      # 16-byte vectors per thread and chunk in flat element-wise kernels
+    "red_unroll": 4,  # the same for flat kernels with a reduction tail
+    "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
+    "bpc": 8,         # resident blocks per CU that bound the grid of `nd` kernels
+    "ntl": 1,         # non-temporal loads  } for working sets beyond `cache_mib`;
+    "nts": 1,         # non-temporal stores } smaller ones stay cacheable
+    "cache_mib": 200,  # working sets up to this size are left to the 256 MB Infinity Cache
     "tw": 128,        # stencil tile width (elements)
     "th": 16,         # stencil tile height (rows)
     "lds": 1,         # stage shifted views through LDS (0: read them directly)
@@ -336,14 +339,20 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
             widths_ok = widths_ok and all(cg.ITEMSIZE[c] in (4, 8) for c in out_codes)
             align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
         vec = widths_ok and align_ok and n >= 64
-        unroll = TUNE["unroll"]
+        unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
+        footprint = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
+        if not reduce_op:
+            footprint += sum(n * cg.ITEMSIZE[c] for c in out_codes)
+        streaming = footprint > TUNE["cache_mib"] << 20
+        ntl = bool(TUNE["ntl"]) and streaming
+        nts = bool(TUNE["nts"]) and streaming
         low.kind = "flat"
-        low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place, tune)
-        holder = {}
+        low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
+                   unroll, ntl, nts)
 
         def emit():
-            src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, bool(TUNE["ntl"]),
-                                  bool(TUNE["nts"]), restrict=not in_place, reduce_op=reduce_op)
+            src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
+                                  restrict=not in_place, reduce_op=reduce_op)
             return src
         low.emit = emit
         if vec:
@@ -353,9 +362,8 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
             E = 16 // min(widths) if widths else 4
         else:
             E = 1
-        work = max(1, n // E)
-        blocks = -(-work // (cg.BLOCK * unroll))
-        low.grid = max(1, min(blocks, _grid_cap()))
+        chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
+        low.grid = min(chunks, TUNE["red_blocks"] if reduce_op else (1 << 24) - 1)
         n_out_ptr = 1 if reduce_op else len(out_ptrs)
         low.fmt = "@" + "P" * (len(ptrs) + n_out_ptr) + scal_fmt + "q"
         low.values = (ptrs, scal_vals, [n])
@@ -709,6 +717,11 @@ def materialise(arr, dtype=None, shape=None):
     return _execute(tracer, [root])[0]
 
 
+def run_reduce_product(a, b):
+    from .delayarray import NPArray, ReduceEx
+    return run(ReduceEx(numpy.add, NPArray(a) * NPArray(b)))
+
+
 def lower_only(exs, dst=None):
     """Trace and lower without touching the device: returns (Lowered, source).
     Works with placeholder arrays on a machine that has no GPU."""
@@ -832,6 +845,33 @@ class _Fallback:
     @staticmethod
     def min(arr, axis=None, keepdims=False):
         return _Fallback._reduce(arr, "minimum", axis, keepdims)
+
+    @staticmethod
+    def dot(a, b):
+        """Matrix products on the device (vector.vector is fused by the front end)."""
+        a, b = _Fallback.asarray(a), _Fallback.asarray(b)
+        dt = numpy.result_type(a.dtype, b.dtype)
+        if dt.kind != "f":
+            dt = numpy.dtype(numpy.float64)
+        a = _Fallback.ascontiguousarray(a, dt)
+        b = _Fallback.ascontiguousarray(b, dt)
+        if a.ndim == 1 and b.ndim == 1:
+            return run_reduce_product(a, b)
+        a2 = a.reshape(1, -1) if a.ndim == 1 else a
+        b2 = b.reshape(-1, 1) if b.ndim == 1 else b
+        if a2.ndim != 2 or b2.ndim != 2 or a2.shape[1] != b2.shape[0]:
+            raise ValueError(f"shapes {a.shape} and {b.shape} not aligned")
+        m, k = a2.shape
+        n = b2.shape[1]
+        out = ndarray((m, n), dt)
+        hiprt.matmul(dt.itemsize == 8, a2.ptr, b2.ptr, out.ptr, m, n, k, k, n, n)
+        if a.ndim == 1:
+            return out.reshape(n)
+        if b.ndim == 1:
+            return out.reshape(m)
+        return out
+
+    matmul = dot
 
     @staticmethod
     def roll(arr, shift, axis=None):

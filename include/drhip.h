@@ -99,6 +99,12 @@ int drhip_fill64(void* dst_dev, uint64_t pattern, size_t nwords);
 int drhip_copy_kernel(void* dst_dev, const void* src_dev, size_t nbytes,
                       unsigned grid_blocks);
 
+/* Row-major C[m,n] = A[m,k] * B[k,n] in float (is_double = 0) or double, leading
+ * dimensions in elements.  Replaces `_backend.fallback.dot` = cupy.dot -> cuBLAS
+ * (delayarray.py:85) for matrix operands; eager, not part of the fused path. */
+int drhip_matmul(int is_double, const void* a, const void* b, void* c, int64_t m, int64_t n,
+                 int64_t k, int64_t lda, int64_t ldb, int64_t ldc);
+
 /* ---- run-time compilation ----------------------------------------------
  * Replaces cupy.ElementwiseKernel(...) construction (cuda.py:35-43), i.e.
  * NVRTC + module load.  `src` is HIP C++ text holding one or more

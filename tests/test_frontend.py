@@ -1,0 +1,300 @@
+"""Host logic of the lazy front end and of the code generator; no GPU needed.
+
+Leaves are placeholder device arrays (geometry and dtype, no memory), so DAG
+construction, tracing, lowering, source generation and hiprtc compilation are all
+exercised here; nothing is launched.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import delayrepay_amd as dr
+from delayrepay_amd import codegen as cg
+from delayrepay_amd import hip, hiprt
+from delayrepay_amd.delayarray import (BinaryFuncEx, BinaryNumpyEx, CastEx, NPArray, ReduceEx,
+                                       Scalar, UnaryFuncEx, Memoiser)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def leaf(shape, dtype=np.float32, **kw):
+    return NPArray(hip.placeholder(shape, dtype, **kw))
+
+
+# ---- C ABI ---------------------------------------------------------------------
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "drhip.h")).read()
+    declared = set(re.findall(r"\b(drhip_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 25
+    lib = ctypes.CDLL(hiprt.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in drhip.h but not exported"
+    assert declared == set(hiprt._SIGNATURES), "ctypes binding and header disagree"
+
+
+def test_uninitialised_library_reports_errors_without_a_gpu():
+    lib = hiprt.lib()
+    p = ctypes.c_void_p()
+    if not hiprt._initialised:
+        assert lib.drhip_malloc(ctypes.byref(p), 1024) == 20001       # DRHIP_ENOTINIT
+        assert b"drhip_init" in lib.drhip_last_error()
+    assert lib.drhip_compile(None, b"x", None, 0, None) == 20002      # DRHIP_EINVAL
+
+
+def test_compile_error_carries_the_hiprtc_log():
+    with pytest.raises(hiprt.DrhipError) as err:
+        hiprt.compile_only('extern "C" __global__ void k() { this is not C++; }', "bad.hip", [])
+    assert err.value.code > 10000
+    assert "error" in err.value.log
+
+
+# ---- laziness and hash-consing (reference tests/test.py:145-162) -------------------
+
+def test_memoise_leaf_and_expression_identity():
+    arr = hip.placeholder((3,), np.float64)
+    assert NPArray(arr) is NPArray(arr)
+    a = leaf((3,))
+    b = leaf((3,))
+    assert a is not b
+    assert np.sin(a) is np.sin(a)
+    assert (a + b) is (a + b)
+    assert (a + b) is not (b + a)
+
+
+def test_scalar_keys_do_not_collide():
+    assert Scalar(-1) is not Scalar(-2)          # hash((-1,)) == hash((-2,)) in CPython
+    assert Scalar(2) is not Scalar(2.0)
+    assert Scalar(0.0) is not Scalar(-0.0)
+    assert Scalar(2) is Scalar(2)
+    a = leaf((4,))
+    assert isinstance(a ** 2.0, BinaryFuncEx)    # float exponent stays pow()
+    assert isinstance(a ** 2, BinaryNumpyEx)
+
+
+def test_hash_cons_table_holds_nodes_weakly():
+    import gc
+    a = leaf((8,))
+    before = len(Memoiser._cache)
+    tmp = [a * float(i) for i in range(50)]
+    assert len(Memoiser._cache) >= before + 50
+    del tmp
+    gc.collect()
+    assert len(Memoiser._cache) <= before + 2
+
+
+def test_nothing_is_computed_while_building():
+    a, b = leaf((1 << 20,)), leaf((1 << 20,))
+    before = dict(hip.STATS)
+    z = np.sqrt(a * 2.0 + b) / 3
+    assert "array" not in z.__dict__
+    assert hip.STATS == before
+    assert z.shape == (1 << 20,) and z.dtype == np.float32
+
+
+def test_rewrites_follow_the_reference():
+    a = leaf((16,))
+    sq = np.square(a)                            # delayarray.py:330-331
+    assert isinstance(sq, BinaryNumpyEx) and sq.func is np.multiply
+    assert sq.children[0] is a and sq.children[1] is a
+    cube = a ** 3                                # delayarray.py:316-324: (a*a)*a
+    assert cube.func is np.multiply and cube.children[1] is a
+    assert cube.children[0].children[0] is a and cube.children[0].children[1] is a
+    assert (a ** 1) is a
+    assert isinstance(np.cos(a), UnaryFuncEx)
+    assert isinstance(np.arctan2(a, a), BinaryFuncEx)
+    assert isinstance(a / 2, BinaryNumpyEx)      # NumPy 2 calls the ufunc `divide`
+    assert isinstance((a + 1).astype(np.float64), CastEx)   # lazy nodes cast lazily
+    assert (a + 1).astype(np.float32) is (a + 1)
+    assert a.astype(np.float32) is a                         # delayarray.py:401-408
+
+
+def test_dtype_and_shape_inference_is_numpys():
+    f32, f64, i64 = leaf((4, 5)), leaf((4, 5), np.float64), leaf((4, 5), np.int64)
+    assert (f32 * 0.3).dtype == np.float32                 # weak Python scalar
+    assert (f32 * np.float64(0.3)).dtype == np.float64     # NumPy scalars are not weak
+    assert (f32 + f64).dtype == np.float64
+    assert (i64 * 2).dtype == np.int64
+    assert (i64 * 2.0).dtype == np.float64
+    assert (i64 / i64).dtype == np.float64
+    assert np.sqrt(i64).dtype == np.float64
+    assert (f32 > 0).dtype == np.bool_
+    row = leaf((1, 5))
+    col = leaf((4, 1))
+    assert (row + col).shape == (4, 5)
+    with pytest.raises(ValueError):
+        leaf((3,)) + leaf((4,))
+
+
+def test_unsupported_operands_raise():
+    a = leaf((4,))
+    with pytest.raises(NotImplementedError):
+        a + "text"
+    with pytest.raises(NotImplementedError):
+        np.add(a, 1, where=np.array([True] * 4))
+
+
+def test_inplace_operator_rebinds_like_the_reference():
+    a = leaf((4,))
+    b = a
+    b += 1
+    assert b is not a and isinstance(b, BinaryNumpyEx)
+
+
+# ---- tracing ---------------------------------------------------------------------
+
+def trace(ex):
+    t = hip.Tracer()
+    root = t.visit(ex)
+    return t, t.program([root])
+
+
+def test_shared_subexpression_is_traced_once():
+    a, b = leaf((64,), np.float64), leaf((64,), np.float64)
+    d = a - b
+    t, prog = trace(d * d * b)                   # the sum-of-squares body
+    assert [op[0] for op in prog.ops] == ["subtract", "multiply", "multiply"]
+    assert prog.ops[1][3] == (("v", 0), ("v", 0))
+    assert len(t.leaves) == 2
+
+
+def test_program_is_structural():
+    """Two instances of the same expression over different arrays and scalar values
+    give the same cache key (the reference's names embed a global counter and
+    always differ, delayarray.py:150-152)."""
+    def build(c0, c1):
+        x, y = leaf((128,)), leaf((128,))
+        return hip.lower_only(c0 * x + y * c1)[0].key
+    assert build(2.0, 3.0) == build(-7.5, 0.25)
+    x = leaf((128,))
+    assert hip.lower_only(2.0 * x)[0].key != hip.lower_only(2.0 * leaf((128,), np.float64))[0].key
+
+
+def test_scalars_become_typed_parameters():
+    x = leaf((256,))
+    t, prog = trace(0.3 * x + 1)
+    assert prog.scalars == ("f4", "f4")
+    assert t.scalars[0] == np.float32(0.3) and isinstance(t.scalars[0], np.float32)
+    src = hip.lower_only(0.3 * x + 1)[1]
+    assert "0.3" not in src                      # never an inlined (double) literal
+
+
+def test_same_geometry_views_are_one_leaf():
+    base = hip.placeholder((16, 16), np.float32)
+    v1, v2 = NPArray(base[1:-1, 1:-1]), NPArray(base[1:-1, 1:-1])
+    assert v1 is not v2
+    t, _ = trace(v1 + v2)
+    assert len(t.leaves) == 1
+
+
+# ---- lowering: which kernel shape, which key -------------------------------------------
+
+def test_contiguous_is_flat_and_vectorised():
+    x, y = leaf((1 << 16,)), leaf((1 << 16,))
+    low, src = hip.lower_only(2.0 * x + y)
+    assert low.kind == "flat"
+    assert "f4x4" in src and "__builtin_nontemporal" not in src      # small: stays cacheable
+    big = hip.lower_only(2.0 * leaf((1 << 26,)) + leaf((1 << 26,)))[1]
+    assert "__builtin_nontemporal_load" in big and "__builtin_nontemporal_store" in big
+    # 2-D contiguous operands collapse to the same flat kernel
+    assert hip.lower_only(2.0 * leaf((256, 256)) + leaf((256, 256)))[0].key == low.key
+
+
+def test_misaligned_view_uses_scalar_flat_kernel():
+    base = hip.placeholder((1 << 12,), np.float32)
+    low, src = hip.lower_only(NPArray(base[1:]) * 2.0)
+    assert low.kind == "flat" and "f4x4* " not in src.split("dr_kernel")[1]
+
+
+def test_broadcast_scalar_leaf_and_mixed_dtypes():
+    x = leaf((1 << 12,), np.float32)
+    s = leaf((), np.float64)
+    low, src = hip.lower_only(x * s)
+    assert low.kind == "flat" and "a1[0]" in src
+    assert "(double)l0" in src
+    hip.compile_source(src)
+
+
+def test_strided_and_broadcast_operands_use_nd():
+    a, b = leaf((64, 1, 32), np.float64), leaf((1, 48, 32), np.float32)
+    low, src = hip.lower_only(a * b + 1)
+    assert low.kind == "nd"
+    hip.compile_source(src)
+    m = hip.placeholder((100, 200), np.float32)
+    assert hip.lower_only(NPArray(m.T) * 2.0)[0].kind == "nd"
+
+
+def test_shifted_views_lower_to_lds_stencil():
+    n = 512
+    u = NPArray(hip.placeholder((n, n), np.float32))
+    rhs = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+    low, src = hip.lower_only(rhs)
+    assert low.kind == "tile2d"
+    assert "__shared__ float tile[" in src and "__syncthreads" in src
+    kinds = low.key[2]
+    assert sorted(k[1:] for k in kinds) == [(0, 0), (1, -1), (1, 1), (2, 0)]
+    hip.compile_source(src)
+    # association of the sum is the user's: ((up + down) + left) + right, then 0.25 *
+    body = src.split("dr_body")[1]
+    assert re.search(r"v0 = l0 \+ l1;\s+const float v1 = v0 \+ l2;\s+const float v2 = v1 \+ l3;"
+                     r"\s+const float v3 = s0 \* v2;", body)
+
+
+def test_reduction_lowers_to_fused_tail_with_finalize():
+    x, y, w = (leaf((1 << 20,), np.float64) for _ in range(3))
+    low, src = hip.lower_only(ReduceEx(np.add, (x - y) ** 2 * w))
+    assert low.kind == "flat" and low.fin_count == low.grid
+    assert "__shfl_down" in src and "dr_finalize" in src and "atomic" not in src
+    hip.compile_source(src)
+    assert ReduceEx(np.add, leaf((8,), np.int32)).dtype == np.int32
+    low, src = hip.lower_only(ReduceEx(np.add, leaf((1 << 12,), np.int32)))
+    assert "long long* __restrict__ partial" in src          # integer sums accumulate in int64
+
+
+def test_two_roots_share_one_kernel():
+    S, K, T = (leaf((1 << 16,), np.float64) for _ in range(3))
+    from oracle import numpy_oracle as orc    # expression text only; nothing is evaluated
+    call, put = orc.black_scholes_expr(dr, S, K, T, 0.02, 0.30)
+    low, src = hip.lower_only([call, put])
+    assert low.kind == "flat"
+    assert src.count("erf(") == 2 and src.count("exp(") == 1 and src.count("log(") == 1
+    assert src.count("sqrt(") == 1
+    assert "double& r0, double& r1" in src
+    hip.compile_source(src)
+
+
+@pytest.mark.parametrize("name", sorted(cg.SUPPORTED_UFUNCS - {"square"}))
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_every_supported_ufunc_generates_compilable_source(name, dtype):
+    fn = getattr(np, name, None)
+    if fn is None:
+        import scipy.special
+        fn = getattr(scipy.special, name)
+    a, b = leaf((1 << 10,), dtype), leaf((1 << 10,), dtype)
+    ex = fn(a) if fn.nin == 1 else fn(a, b)
+    low, src = hip.lower_only(ex)
+    hip.compile_source(src)
+    expect = ("f" if dtype == np.float32 else "")
+    if name in cg._FLOAT_FUNCS1:
+        assert f"{cg._FLOAT_FUNCS1[name]}{expect}(" in src
+
+
+def test_flags_keep_mul_add_separate_and_unpacked():
+    assert "-ffp-contract=off" in hip.COMPILE_OPTS
+    joined = " ".join(hip.COMPILE_OPTS)
+    assert "-target-feature -Xclang -packed-fp32-ops" in joined
+
+
+def test_unfusable_ufunc_is_rejected_clearly():
+    a = leaf((16,))
+    with pytest.raises(NotImplementedError, match="cannot be fused"):
+        hip.lower_only(np.logaddexp(a, a))
+
+
+def test_launching_on_placeholders_is_refused():
+    a = leaf((16,))
+    with pytest.raises(Exception):
+        (a + 1).get()

@@ -1,0 +1,405 @@
+"""Parity of the HIP fusion backend with the oracle, through libdrhip's C ABI.
+
+Bars (written out where they are applied):
+  + - * / and sqrt expressions          bit-exact
+  transcendental functions               <= 2 ulp in float32; <= 1e-13 relative in float64
+  Black-Scholes call/put                 |gpu - oracle| <= 2 ulp(float32) resp. 1e-13 (float64)
+                                         of max(S, K): the price is a difference of terms
+                                         of that size, so ulps of the (possibly tiny) result
+                                         would only measure cancellation, in NumPy as well
+  sum / max / min                        rtol 1e-13 (float64), 1e-6 (float32); max/min exact
+"""
+import numpy as np
+import pytest
+
+import delayrepay_amd as dr
+from delayrepay_amd import hip
+from oracle import numpy_oracle as orc
+from oracle.numpy_oracle import OracleArray
+from tests.helpers import bits_equal, golden, ulp_distance
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 2, 3, 4, 5, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4099, 100003, (1 << 20) + 1]
+
+
+# ---- C1 SAXPY ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("n", SIZES)
+def test_saxpy_bit_exact(n):
+    inp = orc.make_inputs("saxpy", n)
+    z = inp["a"] * dr.array(inp["x"]) + dr.array(inp["y"])
+    assert bits_equal(z.get(), orc.saxpy(inp["a"], inp["x"], inp["y"]))
+
+
+def test_saxpy_golden():
+    g = golden("configs_small.npz")
+    z = 2.0 * dr.array(g["saxpy_x"]) + dr.array(g["saxpy_y"])
+    assert bits_equal(z.get(), g["saxpy_z"])
+
+
+def test_saxpy_full_size():
+    inp = orc.make_inputs("saxpy")          # n = 2^24
+    z = inp["a"] * dr.array(inp["x"]) + dr.array(inp["y"])
+    assert bits_equal(z.get(), orc.saxpy(inp["a"], inp["x"], inp["y"]))
+
+
+@pytest.mark.parametrize("lo,hi", [(1, None), (0, -1), (3, -5), (2, 2 + 4096)])
+def test_saxpy_on_misaligned_contiguous_views(lo, hi):
+    inp = orc.make_inputs("saxpy", 10000)
+    x, y = dr.array(inp["x"]), dr.array(inp["y"])
+    z = 2.0 * x[lo:hi] + y[lo:hi]
+    assert bits_equal(z.get(), orc.saxpy(2.0, inp["x"][lo:hi], inp["y"][lo:hi]))
+
+
+def test_denormals_infinities_and_nans_pass_through():
+    tiny = np.finfo(np.float32).tiny
+    x = np.array([tiny / 4, -tiny / 2, tiny, 0.0, -0.0, np.inf, -np.inf, np.nan, 1e38, 3e38] * 13,
+                 np.float32)
+    y = x[::-1].copy()
+    with np.errstate(all="ignore"):
+        for fn in (lambda a, b: a * 0.5 + b, lambda a, b: a / b, lambda a, b: (a - b) * a,
+                   lambda a, b: a * a * a):
+            got = fn(dr.array(x), dr.array(y)).get()
+            assert bits_equal(got, fn(OracleArray(x), OracleArray(y)).get())
+
+
+# ---- C2 Horner --------------------------------------------------------------------------
+
+def horner_expr(c, x):
+    acc = c[8] * x + c[7]
+    for i in range(6, -1, -1):
+        acc = acc * x + c[i]
+    return acc
+
+
+@pytest.mark.parametrize("n", [1, 1000, 4097, (1 << 20) + 3])
+def test_horner_bit_exact(n):
+    inp = orc.make_inputs("horner", n)
+    y = horner_expr(inp["c"], dr.array(inp["x"]))
+    assert bits_equal(y.get(), orc.horner(inp["c"], inp["x"]))
+
+
+def test_horner_golden_and_kernel_reuse():
+    g = golden("configs_small.npz")
+    c = [float(v) for v in g["horner_c"]]
+    y = horner_expr(c, dr.array(g["horner_x"]))
+    assert bits_equal(y.get(), g["horner_y"])
+    compiles = hip.STATS["compiles"] + hip.STATS["disk_hits"]
+    other = [v * 0.5 - 0.1 for v in c]                     # new coefficients, same structure
+    y2 = horner_expr(other, dr.array(g["horner_x"]))
+    assert bits_equal(y2.get(), orc.horner(other, g["horner_x"]))
+    assert hip.STATS["compiles"] + hip.STATS["disk_hits"] == compiles
+
+
+def test_horner_full_size():
+    inp = orc.make_inputs("horner")         # n = 2^26
+    y = horner_expr(inp["c"], dr.array(inp["x"]))
+    assert bits_equal(y.get(), orc.horner(inp["c"], inp["x"]))
+
+
+# ---- C3 Black-Scholes -------------------------------------------------------------------
+
+def bs_check(cfg, n):
+    inp = orc.make_inputs(cfg, n)
+    S, K, T = (dr.array(inp[k]) for k in "SKT")
+    call, put = orc.black_scholes_expr(dr, S, K, T, inp["r"], inp["sigma"])
+    launches = hip.STATS["launches"]
+    dr.evaluate(call, put)
+    assert hip.STATS["launches"] == launches + 1           # both roots from ONE kernel
+    ocall, oput = orc.black_scholes(inp["S"], inp["K"], inp["T"], inp["r"], inp["sigma"])
+    scale = np.maximum(inp["S"], inp["K"])
+    dt = inp["S"].dtype
+    tol = 2 * np.finfo(np.float32).eps if dt == np.float32 else 1e-13
+    for got, ref in ((call.get(), ocall), (put.get(), oput)):
+        assert got.dtype == dt
+        err = np.abs(got.astype(np.float64) - ref.astype(np.float64)) / scale
+        assert err.max() <= tol, (cfg, err.max(), int(err.argmax()))
+    return call.get(), put.get(), inp
+
+
+@pytest.mark.parametrize("cfg", ["bs64", "bs32"])
+@pytest.mark.parametrize("n", [1, 1000, 65537])
+def test_black_scholes_within_tolerance(cfg, n):
+    bs_check(cfg, n)
+
+
+@pytest.mark.parametrize("cfg", ["bs64", "bs32"])
+def test_black_scholes_full_size_and_put_call_parity(cfg):
+    call, put, inp = bs_check(cfg, 1 << 25)
+    parity = inp["S"].astype(np.float64) - inp["K"] * np.exp(-inp["r"] * inp["T"].astype(np.float64))
+    scale = np.maximum(inp["S"], inp["K"])
+    tol = 8 * np.finfo(inp["S"].dtype).eps
+    assert np.max(np.abs((call.astype(np.float64) - put) - parity) / scale) <= tol
+
+
+@pytest.mark.parametrize("cfg", ["bs64", "bs32"])
+def test_black_scholes_golden(cfg):
+    g = golden("configs_small.npz")
+    S, K, T = (dr.array(g[f"{cfg}_{k}"]) for k in "SKT")
+    call, put = dr.evaluate(*orc.black_scholes_expr(dr, S, K, T, 0.02, 0.30))
+    scale = np.maximum(g[f"{cfg}_S"], g[f"{cfg}_K"])
+    tol = 2 * np.finfo(np.float32).eps if cfg == "bs32" else 1e-13
+    assert np.max(np.abs(call.get() - g[f"{cfg}_call"]) / scale) <= tol
+    assert np.max(np.abs(put.get() - g[f"{cfg}_put"]) / scale) <= tol
+
+
+EXACT = ("negative", "absolute", "sqrt", "floor", "ceil", "trunc", "rint", "reciprocal",
+         "add", "subtract", "multiply", "divide", "maximum", "minimum", "fmax", "fmin",
+         "copysign", "fmod")
+
+
+@pytest.mark.parametrize("tag", ["f32", "f64"])
+def test_every_function_on_the_special_value_table(tag):
+    """Per-function accuracy against the golden table (NumPy/SciPy values)."""
+    from tests.golden.make_golden import UNARY, BINARY
+    g = golden("special_values.npz")
+    x, y = dr.array(g[f"{tag}_x"]), dr.array(g[f"{tag}_y"])
+    worst = {}
+    for name, fn in list(UNARY.items()) + list(BINARY.items()):
+        got = (fn(x) if name in UNARY else fn(x, y)).get()
+        ref = g[f"{tag}_{name}"]
+        assert got.dtype == ref.dtype, name
+        assert np.array_equal(np.isnan(got), np.isnan(ref)), name
+        if name in EXACT:
+            assert bits_equal(got, ref), name
+            continue
+        finite = np.isfinite(ref)
+        assert np.array_equal(got[~finite & ~np.isnan(ref)], ref[~finite & ~np.isnan(ref)]), name
+        if tag == "f32":
+            d = ulp_distance(got[finite], ref[finite])
+            worst[name] = d.max() if d.size else 0
+            assert worst[name] <= 2, (name, worst[name])          # <= 2 ulp in float32
+        else:
+            denom = np.maximum(np.abs(ref[finite]), np.finfo(np.float64).tiny)
+            rel = np.abs(got[finite] - ref[finite]) / denom
+            worst[name] = rel.max() if rel.size else 0
+            assert worst[name] <= 1e-13, (name, worst[name])      # <= 1e-13 relative in float64
+    print(tag, "worst:", {k: float(v) for k, v in sorted(worst.items(), key=lambda kv: -kv[1])[:6]})
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_transcendentals_on_dense_random_arguments(dtype):
+    from scipy.special import erf
+    rs = np.random.RandomState(11)
+    n = 1 << 18
+    cases = {
+        "exp": (np.exp, rs.uniform(-20, 20, n)), "log": (np.log, rs.uniform(1e-6, 1e6, n)),
+        "erf": (erf, rs.uniform(-6, 6, n)), "sin": (np.sin, rs.uniform(-100, 100, n)),
+        "cos": (np.cos, rs.uniform(-100, 100, n)), "tanh": (np.tanh, rs.uniform(-10, 10, n)),
+        "sqrt": (np.sqrt, rs.uniform(0, 1e6, n)), "arctan": (np.arctan, rs.uniform(-50, 50, n)),
+    }
+    for name, (fn, arg) in cases.items():
+        arg = arg.astype(dtype)
+        got, ref = fn(dr.array(arg)).get(), fn(arg)
+        if dtype == np.float32:
+            assert ulp_distance(got, ref).max() <= (0 if name == "sqrt" else 2), name
+        else:
+            assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-300)) <= 1e-13, name
+
+
+# ---- C4 Jacobi and other shifted-slice stencils --------------------------------------------
+
+def jacobi_sweeps(u, sweeps):
+    for _ in range(sweeps):
+        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+    return u
+
+
+@pytest.mark.parametrize("shape", [(3, 3), (4, 7), (8, 8), (17, 130), (18, 131), (130, 257),
+                                   (129, 1000), (514, 514), (1000, 37)])
+@pytest.mark.parametrize("sweeps", [1, 10])
+def test_jacobi_bit_exact(shape, sweeps):
+    rs = np.random.RandomState(7)
+    u0 = np.zeros(shape, np.float32)
+    u0[1:-1, 1:-1] = rs.uniform(0, 1, (shape[0] - 2, shape[1] - 2))
+    u = jacobi_sweeps(dr.array(u0), sweeps)
+    assert bits_equal(u.get(), orc.jacobi(u0, sweeps))
+
+
+def test_jacobi_golden():
+    g = golden("configs_small.npz")
+    u = dr.array(g["jacobi_u0"])
+    assert bits_equal(jacobi_sweeps(u, 1).get(), g["jacobi_u1"])
+    assert bits_equal(jacobi_sweeps(u, 9).get(), g["jacobi_u10"])
+
+
+def test_jacobi_full_size():
+    inp = orc.make_inputs("jacobi")          # 8192 x 8192, 10 sweeps
+    u = jacobi_sweeps(dr.array(inp["u"]), inp["sweeps"])
+    got = u.get()
+    assert bits_equal(got, orc.jacobi(inp["u"], inp["sweeps"]))
+    assert not got[0].any() and not got[-1].any() and not got[:, 0].any() and not got[:, -1].any()
+
+
+def test_jacobi_uses_the_lds_kernel_once_compiled():
+    u = dr.array(np.zeros((64, 64), np.float32))
+    jacobi_sweeps(u, 1)
+    compiles = hip.STATS["compiles"] + hip.STATS["disk_hits"]
+    launches = hip.STATS["launches"]
+    jacobi_sweeps(u, 5)                       # new view objects every sweep, same structure
+    assert hip.STATS["compiles"] + hip.STATS["disk_hits"] == compiles
+    assert hip.STATS["launches"] == launches + 5      # one kernel per sweep, no copy-back
+
+
+def test_stencil_result_into_fresh_array_and_all_views_see_updates():
+    rs = np.random.RandomState(2)
+    a0 = rs.uniform(-1, 1, (70, 90)).astype(np.float32)
+    a = dr.array(a0)
+    inner = a[1:-1, 1:-1]                     # a view taken BEFORE the update
+    lap = a[:-2, 1:-1] + a[2:, 1:-1] + a[1:-1, :-2] + a[1:-1, 2:] - 4.0 * a[1:-1, 1:-1]
+    oa = OracleArray(a0.copy())
+    olap = oa[:-2, 1:-1] + oa[2:, 1:-1] + oa[1:-1, :-2] + oa[1:-1, 2:] - 4.0 * oa[1:-1, 1:-1]
+    assert bits_equal(lap.get(), olap.get())  # fresh (70-2, 90-2) output
+    a[1:-1, 1:-1] = 0.5 * (a[:-2, 1:-1] + a[2:, 1:-1])
+    oa[1:-1, 1:-1] = 0.5 * (oa[:-2, 1:-1] + oa[2:, 1:-1])
+    assert bits_equal(a.get(), oa.get())
+    assert bits_equal(inner.get(), oa.get()[1:-1, 1:-1])      # old view follows the buffer
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_wide_and_asymmetric_stencils(dtype):
+    rs = np.random.RandomState(4)
+    a0 = rs.uniform(-1, 1, (61, 203)).astype(dtype)
+
+    def nine_point(a):
+        return (a[:-2, :-2] + a[:-2, 1:-1] + a[:-2, 2:] + a[1:-1, :-2] + a[1:-1, 1:-1]
+                + a[1:-1, 2:] + a[2:, :-2] + a[2:, 1:-1] + a[2:, 2:]) / 9
+
+    def skewed(a):
+        return a[3:, 5:] * 2.0 - a[:-3, :-5] + a[1:-2, 2:-3]
+
+    for fn in (nine_point, skewed):
+        assert bits_equal(fn(dr.array(a0)).get(), fn(OracleArray(a0)).get()), fn.__name__
+
+
+def test_boundary_change_between_sweeps_is_seen():
+    """The ping-pong copy is refreshed when something else writes the buffer."""
+    u0 = np.zeros((20, 24), np.float32)
+    u0[1:-1, 1:-1] = np.random.RandomState(3).uniform(0, 1, (18, 22))
+    u, ou = dr.array(u0), OracleArray(u0.copy())
+    for step in range(4):
+        for arr in (u, ou):
+            arr[1:-1, 1:-1] = 0.25 * (arr[:-2, 1:-1] + arr[2:, 1:-1] + arr[1:-1, :-2] + arr[1:-1, 2:])
+            arr[0, :] = float(step + 1)       # heat the top edge
+    assert bits_equal(u.get(), ou.get())
+
+
+def test_in_place_elementwise_update_of_a_view():
+    a0 = np.random.RandomState(5).uniform(-1, 1, (33, 65)).astype(np.float32)
+    a, oa = dr.array(a0), OracleArray(a0.copy())
+    for arr in (a, oa):
+        arr[1:-1, 1:-1] = 2.0 * arr[1:-1, 1:-1] + 1.0
+        arr[5] = arr[6] * 3.0                 # rows: distinct memory, direct write
+        arr[:, 0] = 9
+    assert bits_equal(a.get(), oa.get())
+
+
+def test_overlapping_1d_shift_assignment():
+    a0 = np.arange(1000, dtype=np.float64)
+    a, oa = dr.array(a0), OracleArray(a0.copy())
+    for arr in (a, oa):
+        arr[1:] = arr[:-1] + arr[1:]          # reads what it overwrites: needs the temporary
+    assert bits_equal(a.get(), oa.get())
+
+
+# ---- C5 fused element-wise + reduction ------------------------------------------------------
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 1000, 4097, (1 << 20) + 3])
+def test_sumsq_within_rtol(n):
+    inp = orc.make_inputs("sumsq", n)
+    x, y, w = (dr.array(inp[k]) for k in "xyw")
+    launches = hip.STATS["launches"]
+    s = dr.sum((x - y) ** 2 * w)
+    assert hip.STATS["launches"] == launches + 2           # fused body+partials, finalize
+    ref = orc.sumsq(inp["x"], inp["y"], inp["w"])
+    assert abs(float(s) - ref) <= 1e-13 * abs(ref)         # documented rtol for the reduction
+
+
+def test_sumsq_golden():
+    g = golden("configs_small.npz")
+    s = dr.sum((dr.array(g["sumsq_x"]) - dr.array(g["sumsq_y"])) ** 2 * dr.array(g["sumsq_w"]))
+    assert abs(float(s) - float(g["sumsq_s"])) <= 1e-13 * float(g["sumsq_s"])
+
+
+def test_sumsq_full_size_and_sum_of_partial_sums():
+    inp = orc.make_inputs("sumsq")           # n = 2^27
+    x, y, w = (dr.array(inp[k]) for k in "xyw")
+    s = float(dr.sum((x - y) ** 2 * w))
+    ref = float(orc.sumsq(inp["x"], inp["y"], inp["w"]))
+    assert abs(s - ref) <= 1e-13 * abs(ref)
+    n = x.shape[0]
+    parts = [float(dr.sum((x[a:a + n // 8] - y[a:a + n // 8]) ** 2 * w[a:a + n // 8]))
+             for a in range(0, n, n // 8)]
+    assert abs(sum(parts) - s) <= 1e-13 * abs(s)
+    assert s == float(dr.sum((x - y) ** 2 * w))            # deterministic: no atomics
+
+
+def test_other_reductions_and_dtypes():
+    rs = np.random.RandomState(9)
+    a64 = rs.standard_normal(70001)
+    a32 = a64.astype(np.float32)
+    ai = rs.randint(-1000, 1000, 70001)
+    assert float(dr.max(dr.array(a64))) == a64.max()
+    assert float(dr.min(dr.array(a64) * 2.0)) == (a64 * 2.0).min()
+    assert float(dr.max(dr.array(a32))) == a32.max()
+    assert int(dr.sum(dr.array(ai))) == int(ai.sum())
+    assert int(dr.sum(dr.array(ai.astype(np.int32)))) == int(ai.sum())
+    s32 = dr.sum(dr.array(a32) * dr.array(a32))
+    assert s32.dtype == np.float32
+    assert abs(float(s32) - float(np.sum(a32 * a32))) <= 1e-6 * float(np.sum(a32 * a32))
+    nan = a64.copy()
+    nan[1234] = np.nan
+    assert np.isnan(float(dr.max(dr.array(nan))))           # NaN propagates, like numpy.max
+    m = dr.mean(dr.array(a64))
+    assert abs(float(m) - a64.mean()) <= 1e-13 * abs(a64.mean()) + 1e-16
+    v = dr.var(dr.array(a64))
+    assert abs(float(v) - a64.var()) <= 1e-12 * a64.var()
+    d = dr.array(a64).dot(dr.array(a64))
+    assert abs(float(d) - a64.dot(a64)) <= 1e-13 * a64.dot(a64)
+    strided = dr.array(rs.standard_normal((300, 70)))
+    sub = strided[::3, 5:60:2]
+    assert abs(float(dr.sum(sub * 2.0)) - float(np.sum(sub.get() * 2.0))) <= 1e-12 * 1e4
+
+
+# ---- fused == un-fused; broadcasting; mixed dtypes -------------------------------------------
+
+def test_unfused_mode_gives_identical_bits():
+    inp = orc.make_inputs("horner", 50000)
+    x = dr.array(inp["x"])
+    fused = horner_expr(inp["c"], x).get()
+    hip.set_fused(False)
+    try:
+        launches = hip.STATS["launches"]
+        y = horner_expr([c + 0.0 for c in inp["c"]], dr.array(inp["x"]))
+        unfused = y.get()
+        assert hip.STATS["launches"] == launches + 16       # one kernel per DAG node
+    finally:
+        hip.set_fused(True)
+    assert bits_equal(fused, unfused)
+
+
+def test_broadcasting_and_mixed_dtypes_follow_numpy():
+    rs = np.random.RandomState(6)
+    a = rs.standard_normal((17, 1, 33))
+    b = rs.standard_normal((1, 29, 33)).astype(np.float32)
+    c = rs.randint(-5, 5, (29, 1))
+    got = (dr.array(a) * dr.array(b) + dr.array(c) / 3).get()
+    ref = (OracleArray(a) * OracleArray(b) + OracleArray(c) / 3).get()
+    assert bits_equal(got, ref)
+    row = rs.standard_normal(40).astype(np.float32)
+    mat = rs.standard_normal((25, 40)).astype(np.float32)
+    assert bits_equal((dr.array(mat) - dr.array(row)).get(), mat - row)
+    assert bits_equal((dr.array(mat).T * 2.0).get(), mat.T * np.float32(2.0))
+    cmp = (dr.array(mat) > 0.25).get()
+    assert cmp.dtype == np.bool_ and np.array_equal(cmp, mat > 0.25)
+
+
+def test_astype_is_fused_and_exact():
+    x64 = np.random.RandomState(8).standard_normal(5000)
+    x = dr.array(x64)
+    got = ((x * 1.5).astype(np.float32) + 1).get()
+    ref = (x64 * 1.5).astype(np.float32) + np.float32(1)
+    assert bits_equal(got, ref)
+    i = dr.full((64,), 7).astype(np.float32)               # reference tests/test.py:74
+    assert i.dtype == np.float32 and bits_equal(i.get(), np.full((64,), 7).astype(np.float32))

@@ -1,0 +1,120 @@
+"""Device runtime (libdrhip through ctypes) and the device array class."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from delayrepay_amd import hip, hiprt
+from delayrepay_amd.devarray import ndarray
+
+pytestmark = pytest.mark.gpu
+
+
+def test_device_is_gfx950():
+    info = hiprt.device_info()
+    assert info["arch"].startswith("gfx950")
+    assert info["wavefront_size"] == 64 and info["compute_units"] >= 200
+
+
+def test_pool_recycles_blocks():
+    hiprt.init()
+    before = hiprt.pool_stats()
+    p = hiprt.malloc(3 << 20)
+    hiprt.free(p)
+    q = hiprt.malloc((3 << 20) + 5)       # same 2 MiB-granular class
+    assert q == p
+    hiprt.free(q)
+    after = hiprt.pool_stats()
+    assert after["n_pool_hits"] >= before["n_pool_hits"] + 1
+    assert after["bytes_in_use"] == before["bytes_in_use"]
+    assert hiprt.lib().drhip_free(ctypes.c_void_p(12345)) == 20002   # foreign pointer rejected
+
+
+def test_copies_fill_and_copy_kernel_roundtrip():
+    host = np.random.RandomState(0).standard_normal(1 << 16).astype(np.float32)
+    a = ndarray.from_host(host)
+    b = ndarray(a.shape, a.dtype)
+    hiprt.copy_kernel(b.ptr, a.ptr, a.nbytes)
+    assert np.array_equal(b.get(), host)
+    hiprt.memcpy_d2d(b.ptr, a.ptr, a.nbytes // 2)
+    hiprt.fill32(b.ptr, 0x3F800000, 100)
+    got = b.get()
+    assert np.all(got[:100] == 1.0) and np.array_equal(got[100:], host[100:])
+    c = ndarray((1000,), np.float64)
+    hiprt.fill64(c.ptr, np.float64(-2.5).view(np.uint64).item(), 1000)
+    assert np.all(c.get() == -2.5)
+    with pytest.raises(hiprt.DrhipError):
+        hiprt.copy_kernel(b.ptr + 4, a.ptr, 64)       # misaligned
+
+
+def test_events_time_the_library_stream():
+    a = ndarray((1 << 24,), np.float32)
+    b = ndarray((1 << 24,), np.float32)
+    e0, e1 = hiprt.Event(), hiprt.Event()
+    e0.record()
+    for _ in range(5):
+        hiprt.copy_kernel(b.ptr, a.ptr, a.nbytes)
+    e1.record()
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1)
+    assert 0.01 < ms < 100
+
+
+def test_compile_cache_levels(tmp_path, monkeypatch):
+    monkeypatch.setenv("DELAYREPAY_CACHE_DIR", str(tmp_path))
+    src = ('extern "C" __global__ void dr_kernel(float* o, long long n) '
+           '{ if (threadIdx.x == 0) o[0] = 42.0f + (float)n; }\n')
+    before = dict(hip.STATS)
+    hip._load_or_compile(src)
+    assert hip.STATS["compiles"] == before["compiles"] + 1
+    assert len(list(tmp_path.glob("*.co"))) == 1
+    mod = hip._load_or_compile(src)                    # second time: code object from disk
+    assert hip.STATS["disk_hits"] == before["disk_hits"] + 1
+    fn = hiprt.get_function(mod, "dr_kernel")
+    out = ndarray((1,), np.float32)
+    import struct
+    args = struct.pack("@Pq", out.ptr, 8)
+    hiprt.launch(fn, 1, 64, 0, args, len(args))
+    assert out.get()[0] == 50.0
+    with pytest.raises(hiprt.DrhipError):
+        hiprt.launch(fn, 0, 64, 0, args, len(args))    # bad geometry is refused on the host
+
+
+def test_views_follow_numpy_basic_indexing():
+    host = np.arange(7 * 9 * 5, dtype=np.float64).reshape(7, 9, 5)
+    dev = ndarray.from_host(host)
+    keys = [np.s_[1:-1], np.s_[:, 2], np.s_[..., ::2], np.s_[::-1, 1:8:3, 4], np.s_[3],
+            np.s_[None, 2, :, None, 1], np.s_[-1, -1, -1], np.s_[5:2], np.s_[1:6:2, ::-2, 1:]]
+    for key in keys:
+        assert np.array_equal(dev[key].get(), host[key]), key
+        assert dev[key].shape == host[key].shape
+        assert dev[key].strides == host[key].strides or host[key].size <= 1
+    with pytest.raises(IndexError):
+        dev[7]
+    with pytest.raises(IndexError):
+        dev[0, 0, 0, 0]
+    with pytest.raises(NotImplementedError):
+        dev[[1, 2]]
+
+
+def test_setitem_fill_copy_astype_reshape():
+    host = np.zeros((6, 8), np.float32)
+    dev = ndarray.from_host(host)
+    dev[1:-1, ::2] = 3
+    host[1:-1, ::2] = 3
+    dev[0] = np.arange(8, dtype=np.float32)
+    host[0] = np.arange(8, dtype=np.float32)
+    dev[:, 7] = dev[:, 0]
+    host[:, 7] = host[:, 0]
+    dev[5, 1:4] = np.array([1.5, 2.5, 3.5])           # float64 source, converted on assignment
+    host[5, 1:4] = np.array([1.5, 2.5, 3.5])
+    assert np.array_equal(dev.get(), host)
+    assert np.array_equal(dev.T.copy().get(), host.T)
+    assert dev.T.copy().is_contiguous
+    assert np.array_equal(dev.astype(np.float64).get(), host.astype(np.float64))
+    assert np.array_equal(dev.astype(np.int32).get(), host.astype(np.int32))
+    assert np.array_equal(dev.reshape(8, 6).get(), host.reshape(8, 6))
+    assert np.array_equal(dev[:, ::2].reshape(-1).get(), host[:, ::2].reshape(-1))
+    assert float(dev[0, 3]) == 3.0 and dev[0, 3].item() == 3.0
+    empty = ndarray((0, 4), np.float32)
+    assert empty.get().shape == (0, 4)
