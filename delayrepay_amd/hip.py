@@ -472,6 +472,47 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
     return low
 
 
+class Replay:
+    """Kernel launches recorded by `record()`: calling the object issues them again
+    with the same arguments (same inputs, same outputs), without tracing, lowering
+    or allocating.  Used to time kernels back to back and to re-run a fixed
+    pipeline; it keeps the recorded outputs and scratch buffers alive."""
+
+    def __init__(self):
+        self.launches = []      # (function, grid, lds bytes, packed arguments)
+        self.keep = []
+        self._scratch = []
+
+    def __call__(self):
+        for func, grid, lds, args in self.launches:
+            hiprt.launch(func, grid, cg.BLOCK, lds, args, len(args))
+
+    def __del__(self):
+        for ptr in self._scratch:
+            hiprt.free(ptr)
+        self._scratch = []
+
+
+_RECORDING = None
+
+
+class record:
+    """Context manager: `with hip.record() as plan: ...` runs the body normally
+    and returns its kernel launches as a `Replay`."""
+
+    def __enter__(self):
+        global _RECORDING
+        if _RECORDING is not None:
+            raise RuntimeError("hip.record() does not nest")
+        _RECORDING = Replay()
+        return _RECORDING
+
+    def __exit__(self, *exc):
+        global _RECORDING
+        _RECORDING = None
+        return False
+
+
 def _launch(low, out_ptrs, reduce_out=None, reduce_code=None):
     """Compile if needed and launch.  For a reduction, `reduce_out` is the device
     address of the 0-d result."""
@@ -487,17 +528,18 @@ def _launch(low, out_ptrs, reduce_out=None, reduce_code=None):
         hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
         fin = struct.pack("@PPi", partial, reduce_out, low.fin_count)
         hiprt.launch(kern.finalize, 1, cg.BLOCK, 0, fin, len(fin))
-        hiprt.free(partial)  # stream-ordered: safe to recycle once queued
+        if _RECORDING is not None:
+            _RECORDING.launches += [(kern.func, low.grid, 0, args), (kern.finalize, 1, 0, fin)]
+            _RECORDING._scratch.append(partial)
+        else:
+            hiprt.free(partial)  # stream-ordered: safe to recycle once queued
         STATS["launches"] += 2
     else:
-        # tile2d puts the halo pointer after the direct operands; flat/nd have none
-        args = _pack(kern, low, ptrs, out_ptrs, scal_vals, tail)
+        args = kern.packer.pack(*ptrs, *out_ptrs, *scal_vals, *tail)
         hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
+        if _RECORDING is not None:
+            _RECORDING.launches.append((kern.func, low.grid, 0, args))
         STATS["launches"] += 1
-
-
-def _pack(kern, low, ptrs, out_ptrs, scal_vals, tail):
-    return kern.packer.pack(*ptrs, *out_ptrs, *scal_vals, *tail)
 
 
 # ---------------------------------------------------------------------------
@@ -518,6 +560,8 @@ def _execute(tracer, roots, dsts=None, reduce_op=None, launch=True):
             return low
         out = ndarray((), code_dtype(acc))
         _launch(low, [], out.ptr, acc)
+        if _RECORDING is not None:
+            _RECORDING.keep += [out] + list(leaves)
         return [out]
     if dsts is None:
         shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
@@ -541,6 +585,8 @@ def _execute(tracer, roots, dsts=None, reduce_op=None, launch=True):
     if not launch:
         return low
     _launch(low, out_ptrs)
+    if _RECORDING is not None:
+        _RECORDING.keep += list(outs) + list(leaves)
     return outs
 
 

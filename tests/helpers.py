@@ -34,9 +34,20 @@ def ulp_distance(a, b):
 
 
 def bits_equal(a, b):
+    """Same dtype, shape and bit patterns.  NaNs must sit at the same positions, but
+    their sign and payload are not compared: IEEE 754 leaves both unspecified for
+    invalid operations (x86 SSE returns the negative quiet NaN, gfx950 the positive)."""
     a = np.asarray(a)
     b = np.asarray(b)
-    return a.dtype == b.dtype and a.shape == b.shape and a.tobytes() == b.tobytes()
+    if a.dtype != b.dtype or a.shape != b.shape:
+        return False
+    if a.dtype.kind == "f":
+        na, nb = np.isnan(a), np.isnan(b)
+        if na.any() or nb.any():
+            if not np.array_equal(na, nb):
+                return False
+            a, b = np.where(na, 0, a), np.where(nb, 0, b)
+    return a.tobytes() == b.tobytes()
 
 
 _C_ORACLE = None

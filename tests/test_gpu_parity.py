@@ -3,10 +3,16 @@
 Bars (written out where they are applied):
   + - * / and sqrt expressions          bit-exact
   transcendental functions               <= 2 ulp in float32; <= 1e-13 relative in float64
-  Black-Scholes call/put                 |gpu - oracle| <= 2 ulp(float32) resp. 1e-13 (float64)
-                                         of max(S, K): the price is a difference of terms
-                                         of that size, so ulps of the (possibly tiny) result
-                                         would only measure cancellation, in NumPy as well
+  Black-Scholes call/put                 |gpu - oracle| <= 4 eps(float32) resp. 1e-13 (float64)
+                                         times max(S, K).  The price is a difference of
+                                         terms of that size, so ulps of the (possibly tiny)
+                                         result would only measure cancellation, in NumPy as
+                                         well; and the 27-node expression chains five
+                                         functions that each may differ by 2 ulp, so the
+                                         compound bound is wider than the per-function one
+                                         (measured: 2.4 eps at n = 2^25).  The float32 result
+                                         must also be as close to the float64 value as
+                                         NumPy's own float32 result is.
   sum / max / min                        rtol 1e-13 (float64), 1e-6 (float32); max/min exact
 """
 import numpy as np
@@ -110,11 +116,18 @@ def bs_check(cfg, n):
     ocall, oput = orc.black_scholes(inp["S"], inp["K"], inp["T"], inp["r"], inp["sigma"])
     scale = np.maximum(inp["S"], inp["K"])
     dt = inp["S"].dtype
-    tol = 2 * np.finfo(np.float32).eps if dt == np.float32 else 1e-13
+    tol = 4 * np.finfo(np.float32).eps if dt == np.float32 else 1e-13
     for got, ref in ((call.get(), ocall), (put.get(), oput)):
         assert got.dtype == dt
         err = np.abs(got.astype(np.float64) - ref.astype(np.float64)) / scale
         assert err.max() <= tol, (cfg, err.max(), int(err.argmax()))
+    if dt == np.float32:     # accuracy against the float64 evaluation of the same inputs
+        t_call, t_put = orc.black_scholes(*(inp[k].astype(np.float64) for k in "SKT"),
+                                          inp["r"], inp["sigma"])
+        for got, ref, truth in ((call.get(), ocall, t_call), (put.get(), oput, t_put)):
+            e_gpu = np.max(np.abs(got - truth) / scale)
+            e_np = np.max(np.abs(ref - truth) / scale)
+            assert e_gpu <= 1.5 * e_np + np.finfo(np.float32).eps, (e_gpu, e_np)
     return call.get(), put.get(), inp
 
 
@@ -139,7 +152,7 @@ def test_black_scholes_golden(cfg):
     S, K, T = (dr.array(g[f"{cfg}_{k}"]) for k in "SKT")
     call, put = dr.evaluate(*orc.black_scholes_expr(dr, S, K, T, 0.02, 0.30))
     scale = np.maximum(g[f"{cfg}_S"], g[f"{cfg}_K"])
-    tol = 2 * np.finfo(np.float32).eps if cfg == "bs32" else 1e-13
+    tol = 4 * np.finfo(np.float32).eps if cfg == "bs32" else 1e-13
     assert np.max(np.abs(call.get() - g[f"{cfg}_call"]) / scale) <= tol
     assert np.max(np.abs(put.get() - g[f"{cfg}_put"]) / scale) <= tol
 
