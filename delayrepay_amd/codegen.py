@@ -567,3 +567,115 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
     L += ["        }", "    }", "}"]
     src.append("\n".join(L))
     return "\n".join(src) + "\n"
+
+
+def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_per_thread,
+                     phase_group, phase_out, restrict=True, nt_load=False, nt_store=False):
+    """Vectorised form of `emit_stencil` for the common aligned case: the halo
+    group's row stride and every output's row stride are multiples of the 16-byte
+    vector width, and group and outputs have the same element size.
+
+    phase_group  (address of the group's reference element / itemsize) % VW
+    phase_out    (address of output element [0, 0] / itemsize) % VW
+    With these two phases fixed at compile time, tile origins are chosen so that
+    every global load into LDS and every global store is a naturally aligned
+    16-byte access; only the first/last column group of a row and loads at the
+    very ends of the buffer fall back to element accesses.
+
+    A block owns TW = groups_per_row * VW output columns by TH = (256 /
+    groups_per_row) * rows_per_thread rows.  Each thread computes VW adjacent
+    outputs per row for `rows_per_thread` consecutive rows, so shifted reads of
+    the same LDS words by neighbouring rows are shared in registers."""
+    gdt, dy_max, dx_min, dx_max = group
+    rs = "__restrict__ " if restrict else ""
+    vt, VW = VEC16[gdt]
+    n_out = len(out_dtypes)
+    GPR = groups_per_row
+    slots = BLOCK // GPR
+    TW = GPR * VW
+    TH = slots * rows_per_thread
+    ph = (phase_group - phase_out + dx_min) % VW
+    LW = -(-(TW + dx_max - dx_min + ph) // VW) * VW
+    LWV = LW // VW
+    LH = TH + dy_max
+    src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    params = []
+    for i, dt in enumerate(prog.leaves):
+        if leaf_kind[i][0] != "g":
+            params.append(f"const {CTYPE[dt]}* {rs}a{i}")
+    params.append(f"const {CTYPE[gdt]}* {rs}gp")
+    params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += ["const int H", "const int W", "const long long grs", "const long long glo",
+               "const long long ghi", "const int tiles_x"]
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "d":
+            params.append(f"const long long rs{i}")
+    params += [f"const long long ors{o}" for o in range(n_out)]
+    ct = CTYPE[gdt]
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{",
+         f"    __shared__ {vt} tile[{LH * LWV}];",
+         "    const int nb = gridDim.x;",
+         f"    const int xcd = blockIdx.x % {N_XCD};",
+         f"    const int slot = blockIdx.x / {N_XCD};",
+         f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;",
+         "    const int ty = t / tiles_x;",
+         "    const int tx = t - ty * tiles_x;",
+         f"    const int r0 = ty * {TH};",
+         f"    const int j0 = tx * {TW} - {phase_out};      // first output column of the tile",
+         f"    const int cs = j0 + ({dx_min}) - {ph};       // buffer column held in LDS column 0",
+         f"    for (int idx = threadIdx.x; idx < {LH * LWV}; idx += {BLOCK}) {{",
+         f"        const int lr = idx / {LWV};",
+         f"        const int lv = idx - lr * {LWV};",
+         f"        const long long lin = (long long)(r0 + lr) * grs + cs + lv * {VW};",
+         f"        {vt} val;",
+         f"        if (lin >= glo && lin + {VW} <= ghi) {{",
+         f"            val = {_ld(nt_load, f'(const {vt}*)(gp + lin)')};",
+         "        } else {",
+         "#pragma unroll",
+         f"            for (int e = 0; e < {VW}; ++e)",
+         f"                val[e] = (lin + e >= glo && lin + e < ghi) ? gp[lin + e] : ({ct})0;",
+         "        }",
+         "        tile[idx] = val;",
+         "    }",
+         "    __syncthreads();",
+         f"    const {ct}* ts = (const {ct}*)tile;",
+         f"    const int g = threadIdx.x % {GPR};",
+         f"    const int rw = threadIdx.x / {GPR};",
+         f"    const int jf = j0 + g * {VW};                // first of this thread's {VW} columns",
+         "#pragma unroll",
+         f"    for (int k = 0; k < {rows_per_thread}; ++k) {{",
+         f"        const int lr = rw * {rows_per_thread} + k;",
+         "        const int i = r0 + lr;",
+         "        if (i >= H) break;"]
+    for o, dt in enumerate(out_dtypes):
+        L.append(f"        {VEC16[dt][0]} R{o};")
+    for e in range(VW):
+        args = []
+        for i, k in enumerate(leaf_kind):
+            if k[0] == "g":
+                _, dy, dx = k
+                args.append(f"ts[(lr + {dy}) * {LW} + g * {VW} + {e + dx - dx_min + ph}]")
+            elif k[0] == "d":
+                args.append(f"((jf + {e} >= 0 && jf + {e} < W) ? a{i}[(long long)i * rs{i} + jf + {e}] "
+                            f": ({CTYPE[prog.leaves[i]]})0)")
+            else:
+                args.append(f"a{i}[0]")
+        decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+        call = args + [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
+        sets = " ".join(f"R{o}[{e}] = t{o};" for o in range(n_out))
+        L.append(f"        {{ {decl} dr_body({', '.join(call)}); {sets} }}")
+    L.append(f"        if (jf >= 0 && jf + {VW} <= W) {{")
+    for o, dt in enumerate(out_dtypes):
+        L.append("            " + _st(nt_store, f"R{o}",
+                                        f"({VEC16[dt][0]}*)(o{o} + (long long)i * ors{o} + jf)"))
+    L.append("        } else {")
+    L.append("#pragma unroll")
+    L.append(f"            for (int e = 0; e < {VW}; ++e)")
+    L.append("                if (jf + e >= 0 && jf + e < W) {")
+    for o in range(n_out):
+        L.append(f"                    o{o}[(long long)i * ors{o} + jf + e] = R{o}[e];")
+    L += ["                }", "        }", "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n", TW, TH, LH * LW * ITEMSIZE[gdt]

@@ -150,6 +150,41 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
     def dot(self, other, out=None):
         return self._dot([self, other], {})
 
+    # The arithmetic operators build nodes directly; going through
+    # NDArrayOperatorsMixin -> ufunc -> __array_ufunc__ gives the same node but
+    # costs several times more host time per operation.
+    def __add__(self, other):
+        return _binary(np.add, self, other)
+
+    def __radd__(self, other):
+        return _binary(np.add, other, self)
+
+    def __sub__(self, other):
+        return _binary(np.subtract, self, other)
+
+    def __rsub__(self, other):
+        return _binary(np.subtract, other, self)
+
+    def __mul__(self, other):
+        return _binary(np.multiply, self, other)
+
+    def __rmul__(self, other):
+        return _binary(np.multiply, other, self)
+
+    def __truediv__(self, other):
+        return _binary(np.true_divide, self, other)
+
+    def __rtruediv__(self, other):
+        return _binary(np.true_divide, other, self)
+
+    def __pow__(self, other):
+        return create_ex(np.power, [self, arg_to_numpy_ex(other)])
+
+    def __neg__(self):
+        return UnaryFuncEx(np.negative, self)
+
+    __iadd__, __isub__, __imul__, __itruediv__ = __add__, __sub__, __mul__, __truediv__
+
     def __gt__(self, other):
         return np.greater(self, other)
 
@@ -308,28 +343,42 @@ ufunc_lookup = {
 
 def calc_shape(left, right, op=None):
     """Result shape of a binary node: NumPy broadcasting (a scalar is `()`)."""
-    if left == right:
+    if left == right or not right:
         return left
+    if not left:
+        return right
     return tuple(np.broadcast_shapes(left, right))
 
 
 _RESOLVE_CACHE = {}
 
 
+_PY_DESCR = {bool: ("py", "b"), int: ("py", "i"), float: ("py", "f"), complex: ("py", "c")}
+_ARRAY_DESCR = {}
+
+
 def _descr(node):
     """What NumPy's type resolution needs to know about an operand."""
-    if isinstance(node, Scalar):
-        val = node.val
-        if isinstance(val, np.generic):
-            return ("np", val.dtype.str)
-        if isinstance(val, bool):
-            return ("py", "b")
-        if isinstance(val, int):
-            return ("py", "i")
-        if isinstance(val, float):
-            return ("py", "f")
-        return ("py", "c")
-    return ("a", node.dtype.str)
+    if type(node) is Scalar:
+        return node._descr
+    dt = node.dtype
+    try:
+        return _ARRAY_DESCR[dt]
+    except KeyError:
+        return _ARRAY_DESCR.setdefault(dt, ("a", dt.str))
+
+
+def _scalar_descr(val):
+    d = _PY_DESCR.get(type(val))
+    if d is not None:
+        return d
+    if isinstance(val, np.generic):
+        return ("np", val.dtype.str)
+    if isinstance(val, numbers.Integral):
+        return ("py", "i")
+    if isinstance(val, numbers.Real):
+        return ("py", "f")
+    return ("py", "c")
 
 
 _PY_PROBE = {"b": True, "i": 1, "f": 1.0, "c": 1j}
@@ -338,7 +387,7 @@ _PY_PROBE = {"b": True, "i": 1, "f": 1.0, "c": 1j}
 def result_dtype(func, descrs):
     """dtype NumPy gives `func` on operands described by `descrs` (weak Python
     scalars included); decided by NumPy itself on empty arrays."""
-    key = (func.__name__, descrs)
+    key = (func, descrs)
     try:
         return _RESOLVE_CACHE[key]
     except KeyError:
@@ -360,7 +409,39 @@ def result_dtype(func, descrs):
 
 
 def calc_type(func, children):
+    if len(children) == 2:
+        return result_dtype(func, (_descr(children[0]), _descr(children[1])))
     return result_dtype(func, tuple(_descr(c) for c in children))
+
+
+class _WeakTable:
+    """key -> node, holding nodes weakly (a lean WeakValueDictionary: node
+    construction is on the host's hot path)."""
+
+    def __init__(self):
+        self.data = data = {}
+
+        def gone(ref):
+            if data.get(ref.key) is ref:
+                del data[ref.key]
+        self._gone = gone
+
+    def get(self, key):
+        ref = self.data.get(key)
+        return ref() if ref is not None else None
+
+    def __setitem__(self, key, node):
+        self.data[key] = weakref.KeyedRef(node, self._gone, key)
+
+    def pop(self, key, default=None):
+        ref = self.data.pop(key, None)
+        return ref() if ref is not None else default
+
+    def __len__(self):
+        return len(self.data)
+
+    def clear(self):
+        self.data.clear()
 
 
 class Memoiser(type):
@@ -368,15 +449,16 @@ class Memoiser(type):
     twice yields the same object, so expressions form a DAG
     (cf. delayarray.py:216-231; tests/test.py:145-162)."""
 
-    _cache = weakref.WeakValueDictionary()
+    _cache = _WeakTable()
 
-    def __call__(cls, *args):
+    def __call__(cls, *args, _table=_cache, _get=_cache.data.get, _ref=weakref.KeyedRef):
         key = cls._memo_key(*args)
-        node = Memoiser._cache.get(key)
+        ref = _get(key)
+        node = ref() if ref is not None else None
         if node is None:
-            node = super().__call__(*args)
+            node = type.__call__(cls, *args)
             node._key = key
-            Memoiser._cache[key] = node
+            _table.data[key] = _ref(node, _table._gone, key)
         return node
 
 
@@ -395,11 +477,12 @@ class NumpyEx(DelayArray, metaclass=Memoiser):
         self.children = list(children)
 
     @classmethod
-    def _memo_key(cls, *args):
-        return (cls.__name__,) + tuple(
-            a.__name__ if isinstance(a, np.ufunc) else
-            id(a) if isinstance(a, DelayArray) else a
-            for a in args)
+    def _memo_key(cls, func, *children):
+        # children are kept alive by the node, so their ids stay unique while the
+        # table entry exists
+        if len(children) == 2:
+            return (cls, func, id(children[0]), id(children[1]))
+        return (cls, func) + tuple(id(c) for c in children)
 
     def __hash__(self):
         return id(self)
@@ -470,7 +553,7 @@ class CastEx(NumpyEx):
 
     @classmethod
     def _memo_key(cls, dtype, arg):
-        return (cls.__name__, np.dtype(dtype).str, id(arg))
+        return (cls, np.dtype(dtype).str, id(arg))
 
     @property
     def name(self):
@@ -545,7 +628,7 @@ class NPArray(NumpyEx):
 
     @classmethod
     def _memo_key(cls, array):
-        return ("NPArray", id(array))
+        return (cls, id(array))
 
     def _force(self):
         return self.array
@@ -560,7 +643,7 @@ class NPArray(NumpyEx):
         Memoiser._cache.pop(self._key, None)
         self.array = converted
         self.dtype = dtype
-        self._key = ("NPArray", id(converted))
+        self._key = (NPArray, id(converted))
         Memoiser._cache[self._key] = self
         return self
 
@@ -581,10 +664,12 @@ class Scalar(NumpyEx):
         super().__init__()
         self.val = val
         self.shape = ()
+        self._descr = _scalar_descr(val)
 
     @classmethod
     def _memo_key(cls, val):
-        return ("Scalar", type(val).__name__, repr(val))
+        # 2 and 2.0 differ by type; 0.0 and -0.0 (equal, same type) by their text
+        return (cls, type(val), val if val else repr(val))
 
     @property
     def dtype(self):
@@ -602,10 +687,20 @@ class Scalar(NumpyEx):
         return {}
 
 
+def _binary(func, left, right):
+    if not isinstance(left, DelayArray):
+        left = arg_to_numpy_ex(left)
+    if not isinstance(right, DelayArray):
+        right = arg_to_numpy_ex(right)
+    return BinaryNumpyEx(func, left, right)
+
+
 def arg_to_numpy_ex(arg):
     """Operand -> node (delayarray.py:470-479)."""
     if isinstance(arg, DelayArray):
         return arg
+    if type(arg) in _PY_DESCR:
+        return Scalar(arg)
     if isinstance(arg, (numbers.Number, np.generic)):
         return Scalar(arg)
     if _backend.is_ndarray(arg) or isinstance(arg, np.ndarray):

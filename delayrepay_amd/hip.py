@@ -49,6 +49,11 @@ TUNE = {
     "tw": 128,        # stencil tile width (elements)
     "th": 16,         # stencil tile height (rows)
     "lds": 1,         # stage shifted views through LDS (0: read them directly)
+    "svec": 1,        # aligned stencils: 16-byte loads into LDS and 16-byte stores
+    "gpr": 64,        # vectorised stencil: 16-byte column groups per tile row
+    "rpt": 2,         # vectorised stencil: consecutive rows per thread
+    "sntl": 0,        # vectorised stencil: non-temporal loads / stores
+    "snts": 1,
 }
 for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
     _k, _v = _kv.split("=")
@@ -80,6 +85,33 @@ def synchronize():
 # tracing: DAG -> Program
 # ---------------------------------------------------------------------------
 
+def _scalar_value(value, code):
+    """Python number to hand to struct.pack for a parameter of dtype `code`."""
+    if code == "f8" or code == "f4":
+        # native-mode struct packing of 'f' is a C cast: round to nearest, overflow to
+        # infinity, which is what numpy.float32(value) gives
+        return float(value)
+    with numpy.errstate(all="ignore"):
+        return code_dtype(code).type(value).item()
+
+
+_FE = None          # the front-end module, bound on first use (it imports this one)
+_CODES = {}
+
+
+def _bind_frontend():
+    global _FE
+    from . import delayarray
+    _FE = delayarray
+
+
+def _code_of(dtype):
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        return _CODES.setdefault(dtype, dtype_code(dtype))
+
+
 class Tracer:
     """Collects leaves, scalar parameters and SSA operations of one or more roots."""
 
@@ -95,7 +127,7 @@ class Tracer:
         self._evaluated = evaluated if evaluated is not None else {}
 
     def leaf(self, arr):
-        code = dtype_code(arr.dtype)
+        code = _code_of(arr.dtype)
         key = (id(arr.buf), arr.offset, arr.shape, arr._strides, code)
         idx = self._leaf_index.get(key)
         if idx is None:
@@ -106,13 +138,15 @@ class Tracer:
         return ("l", idx), code
 
     def scalar(self, value, code, ident=None):
+        """Scalar kernel parameter of dtype `code`; the value is converted at pack
+        time (struct packs Python numbers to float/double exactly as NumPy casts
+        a weak scalar)."""
         key = (ident if ident is not None else ("v", repr(value)), code)
         idx = self._scalar_index.get(key)
         if idx is None:
             idx = len(self.scalars)
             self._scalar_index[key] = idx
-            with numpy.errstate(all="ignore"):
-                self.scalars.append(code_dtype(code).type(value))
+            self.scalars.append(_scalar_value(value, code))
             self.scalar_codes.append(code)
         return ("s", idx), code
 
@@ -121,55 +155,52 @@ class Tracer:
         return ("v", len(self.ops) - 1), result
 
     def visit(self, node):
-        from .delayarray import Scalar, CastEx, ReduceEx, NPArray, result_dtype, _descr
+        memo = self._memo
         nid = id(node)
-        hit = self._memo.get(nid)
+        hit = memo.get(nid)
         if hit is not None:
             return hit
-        arr = self._evaluated.get(nid)
+        if _FE is None:
+            _bind_frontend()
+        kind = type(node)
+        arr = self._evaluated.get(nid) if self._evaluated else None
         if arr is None:
             arr = node.__dict__.get("array")
-            if arr is not None and not isinstance(node, NPArray):
+            if arr is not None and kind is not _FE.NPArray:
                 deps = node.__dict__.get("_deps")
                 if deps is not None and any(buf.version != ver for buf, ver in deps):
                     arr = None  # stale: recompute inside this kernel
         if arr is not None:
             res = self.leaf(arr)
-        elif isinstance(node, Scalar):
-            res = self.scalar(node.val, dtype_code(numpy.asarray(node.val).dtype), id(node))
-        elif isinstance(node, CastEx):
+        elif kind is _FE.BinaryNumpyEx or kind is _FE.BinaryFuncEx or kind is _FE.UnaryFuncEx:
+            func = node.func
+            name = func.__name__
+            result = _code_of(node.dtype)
+            compute = result
+            if name in _COMPARES:
+                compute = dtype_code(_FE.result_dtype(
+                    numpy.add, tuple(_FE._descr(c) for c in node.children)))
+            elif name not in cg.SUPPORTED_UFUNCS:
+                raise NotImplementedError(f"ufunc {name!r} cannot be fused by the HIP backend")
+            refs = []
+            for child in node.children:
+                if type(child) is _FE.Scalar:
+                    refs.append(self.scalar(child.val, compute, id(child))[0])
+                else:
+                    refs.append(self.visit(child)[0])
+            self.ops.append((name, compute, result, tuple(refs)))
+            res = (("v", len(self.ops) - 1), result)
+        elif kind is _FE.Scalar:
+            res = self.scalar(node.val, dtype_code(numpy.asarray(node.val).dtype), nid)
+        elif kind is _FE.CastEx:
             ref, code = self.visit(node.children[0])
             target = dtype_code(node.dtype)
             res = self.op("cast", target, target, [ref]) if code != target else (ref, code)
-        elif isinstance(node, ReduceEx):
+        elif kind is _FE.ReduceEx:
             res = self.leaf(node._force())
         else:
-            func = node.func
-            name = func.__name__
-            if name not in cg.SUPPORTED_UFUNCS:
-                raise NotImplementedError(f"ufunc {name!r} cannot be fused by the HIP backend")
-            traced, descrs = [], []
-            for child in node.children:
-                if type(child) is Scalar:
-                    traced.append(None)
-                    descrs.append(_descr(child))
-                else:
-                    ref = self.visit(child)
-                    traced.append(ref)
-                    descrs.append(("a", code_dtype(ref[1]).str))
-            descrs = tuple(descrs)
-            result = dtype_code(result_dtype(func, descrs))
-            compute = result
-            if name in _COMPARES:
-                compute = dtype_code(result_dtype(numpy.add, descrs))
-            refs = []
-            for child, tr in zip(node.children, traced):
-                if tr is None:
-                    refs.append(self.scalar(child.val, compute, id(child))[0])
-                else:
-                    refs.append(tr[0])
-            res = self.op(name, compute, result, refs)
-        self._memo[nid] = res
+            raise NotImplementedError(f"{kind.__name__} nodes cannot be evaluated by the HIP backend")
+        memo[nid] = res
         return res
 
     def program(self, roots):
@@ -411,10 +442,32 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
                 kinds[i] = ("b",) if s == [0, 0] else ("d",)
         kinds = tuple(kinds)
         low.kind = "tile2d"
-        low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune)
+        vec_ok = False
+        if group is not None and TUNE["svec"]:
+            gsize = cg.ITEMSIZE[group[0]]
+            vw = 16 // gsize
+            vec_ok = (gsize in (4, 8) and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
+                      and g_args[0] % vw == 0 and all(s[0] % vw == 0 for s in m_out)
+                      and len({(p // gsize) % vw for p in out_ptrs}) == 1)
+        if vec_ok:
+            ph_g = (g_ptr // gsize) % vw
+            ph_o = (out_ptrs[0] // gsize) % vw
+            gpr, rpt = TUNE["gpr"], TUNE["rpt"]
+            sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
+            low.key = ("tile2dv", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o,
+                       gpr, rpt, sntl, snts)
+            tw, th = gpr * vw, (cg.BLOCK // gpr) * rpt
 
-        def emit():
-            return cg.emit_stencil(prog, kinds, group, out_codes, tw, th, restrict=not in_place)
+            def emit():
+                return cg.emit_stencil_vec(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o,
+                                           restrict=not in_place, nt_load=sntl, nt_store=snts)[0]
+            W = W + ph_o          # tiles start `ph_o` columns left of the view
+        else:
+            low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune)
+
+            def emit():
+                return cg.emit_stencil(prog, kinds, group, out_codes, tw, th,
+                                       restrict=not in_place)
         low.emit = emit
         tiles_x = -(-W // tw)
         tiles_y = -(-H // th)
@@ -426,7 +479,7 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
             fmt += "P"
             ptrs.append(g_ptr)
         fmt += "P" * len(out_ptrs) + scal_fmt + "ii"
-        tail_vals += [H, W]
+        tail_vals += [mshape[0], mshape[1]]
         if group is not None:
             fmt += "qqq"
             tail_vals += g_args

@@ -177,7 +177,11 @@ def test_scalars_become_typed_parameters():
     x = leaf((256,))
     t, prog = trace(0.3 * x + 1)
     assert prog.scalars == ("f4", "f4")
-    assert t.scalars[0] == np.float32(0.3) and isinstance(t.scalars[0], np.float32)
+    import struct
+    assert struct.pack("f", t.scalars[0]) == np.float32(0.3).tobytes()    # rounded as NumPy does
+    big = struct.pack("@f", hip._scalar_value(1e60, "f4"))    # overflow -> inf, like np.float32(1e60)
+    assert np.frombuffer(big, np.float32)[0] == np.inf
+    assert hip._scalar_value(3, "i8") == 3 and hip._scalar_value(2, "f8") == 2.0
     src = hip.lower_only(0.3 * x + 1)[1]
     assert "0.3" not in src                      # never an inlined (double) literal
 
@@ -233,10 +237,17 @@ def test_shifted_views_lower_to_lds_stencil():
     rhs = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
     low, src = hip.lower_only(rhs)
     assert low.kind == "tile2d"
-    assert "__shared__ float tile[" in src and "__syncthreads" in src
-    kinds = low.key[2]
+    assert "__shared__ float tile[" in src and "__syncthreads" in src      # fresh output: rows
+    kinds = low.key[2]                                                    # of 510 are unaligned
     assert sorted(k[1:] for k in kinds) == [(0, 0), (1, -1), (1, 1), (2, 0)]
     hip.compile_source(src)
+    # written back into the grid's interior, rows stay 16-byte periodic: vector variant
+    dst = hip.placeholder((n - 2, n - 2), np.float32, strides=(n, 1), offset=n + 1)
+    low, vsrc = hip.lower_only(rhs, dst=dst)
+    assert low.key[0] == "tile2dv" and "__shared__ f4x4 tile[" in vsrc
+    assert "*(f4x4*)(o0 +" in vsrc and "*(const f4x4*)(gp + lin)" in vsrc
+    hip.compile_source(vsrc)
+    src = vsrc
     # association of the sum is the user's: ((up + down) + left) + right, then 0.25 *
     body = src.split("dr_body")[1]
     assert re.search(r"v0 = l0 \+ l1;\s+const float v1 = v0 \+ l2;\s+const float v2 = v1 \+ l3;"
