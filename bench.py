@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all",
                     help="horner (headline) | saxpy | bs32 | bs64 | jacobi | sumsq | all")
+    ap.add_argument("--settle", type=float, default=0.25,
+                    help="seconds of untimed load before each timed region (clock ramp-up)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-unfused", action="store_true", help="skip the un-fused leg")
     return ap.parse_args()
@@ -130,6 +132,13 @@ def main():
         for _ in range(W):
             keep = step()
         hiprt.sync()
+        # The GPU raises its clocks only under sustained load (an ALU-heavy kernel
+        # measures ~25% slower during the first 30 ms): keep it busy before timing.
+        t_warm = time.perf_counter()
+        while time.perf_counter() - t_warm < args.settle:
+            for _ in range(10):
+                keep = step()
+            hiprt.sync()
         # whole-step throughput: K steps, wall clock between two synchronisations
         t0 = time.perf_counter()
         for _ in range(K):
@@ -145,9 +154,11 @@ def main():
                 keep = step()
         steps_per_replay = 2 if wl.get("pair") else 1
         reps = max(1, K // steps_per_replay)
-        for _ in range(2):
-            plan()
-        hiprt.sync()
+        t_warm = time.perf_counter()
+        while time.perf_counter() - t_warm < args.settle / 2:
+            for _ in range(10):
+                plan()
+            hiprt.sync()
         e0, e1 = hiprt.Event(), hiprt.Event()
         e0.record()
         for _ in range(reps):

@@ -18,6 +18,7 @@ or bounded memory:
     unequal shapes eagerly, :47-55);
   * dtypes follow NumPy promotion with weak Python scalars instead of being
     copied between siblings (:462-467);
+  * `astype` on a leaf returns a new leaf instead of converting in place (:401-408);
   * an evaluated node is reused as a leaf by later expressions, and a cached
     result is dropped when a leaf it was computed from has been written since;
   * `sum` builds a `ReduceEx` (a stub in the reference, :272-283) that the HIP
@@ -463,8 +464,11 @@ class Memoiser(type):
 
 
 def reset():
-    """Forget every hash-consed node (delayarray.py:234-236)."""
+    """Forget every hash-consed node (delayarray.py:234-236) and every cached plan."""
     Memoiser._cache.clear()
+    forget = getattr(_backend, "forget", None)
+    if forget is not None:
+        forget()
 
 
 class NumpyEx(DelayArray, metaclass=Memoiser):
@@ -628,24 +632,26 @@ class NPArray(NumpyEx):
 
     @classmethod
     def _memo_key(cls, array):
+        # Device views with the same buffer and geometry are the same leaf, so the
+        # slices an iterative loop re-creates every pass (`u[1:-1, 2:]`) map to the
+        # same node, and the expression built on them to the same DAG.
+        buf = getattr(array, "buf", None)
+        if buf is not None:
+            return (cls, id(buf), array.offset, array.shape, array._strides, array.dtype.str)
         return (cls, id(array))
 
     def _force(self):
         return self.array
 
     def astype(self, dtype, **kwargs):
-        """Convert the leaf in place and return the same wrapper
-        (delayarray.py:401-408; tests/test.py:59-62)."""
+        """Converted copy as a new leaf.  (The reference converts the leaf in place
+        and returns the same wrapper, delayarray.py:401-408, which silently changes
+        every expression already built on it; `arr = arr.astype(t)`, the form its
+        tests use at tests/test.py:59-62,74-77, behaves the same either way.)"""
         dtype = np.dtype(dtype)
         if dtype == self.dtype:
             return self
-        converted = self.array.astype(dtype, **kwargs)
-        Memoiser._cache.pop(self._key, None)
-        self.array = converted
-        self.dtype = dtype
-        self._key = (NPArray, id(converted))
-        Memoiser._cache[self._key] = self
-        return self
+        return NPArray(self.array.astype(dtype, **kwargs))
 
     @property
     def name(self):

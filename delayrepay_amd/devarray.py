@@ -46,12 +46,14 @@ class Buffer:
         self.version += 1
         self.shadow_region = None
 
-    def __del__(self):
+    def __del__(self, _free=hiprt.free):
+        # `_free` is bound at definition time: module globals may already be gone
+        # when buffers are finalised at interpreter exit
         if self.ptr:
-            hiprt.free(self.ptr)
+            _free(self.ptr)
             self.ptr = None
         if self.shadow:
-            hiprt.free(self.shadow)
+            _free(self.shadow)
             self.shadow = None
 
 

@@ -17,6 +17,7 @@ multi-root, fused-assignment and timing entry points.
 Nothing is computed on the host, and there is no fall-back to NumPy: a missing
 library or GPU raises.
 """
+import collections
 import hashlib
 import os
 import struct
@@ -42,6 +43,7 @@ TUNE = {
     "unroll": 1,      # 16-byte vectors per thread and chunk in flat element-wise kernels
     "red_unroll": 4,  # the same for flat kernels with a reduction tail
     "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
+    "flat_cap": 0,    # most blocks of a flat element-wise kernel (0: one chunk per block)
     "bpc": 8,         # resident blocks per CU that bound the grid of `nd` kernels
     "ntl": 1,         # non-temporal loads  } for working sets beyond `cache_mib`;
     "nts": 1,         # non-temporal stores } smaller ones stay cacheable
@@ -60,7 +62,7 @@ for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
     TUNE[_k.strip()] = int(_v)
 
 _FUSED = "DELAY_UNFUSED" not in os.environ
-STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0}
+STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0}
 
 _SCALAR_FMT = {"f4": "f", "f8": "d", "i4": "i", "i8": "q", "u4": "I", "u1": "B", "b1": "B"}
 _COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal")
@@ -69,8 +71,19 @@ _COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equ
 def set_fused(flag):
     """False: evaluate one kernel per DAG node with materialised temporaries (the
     un-fused baseline the fused kernels are measured against)."""
-    global _FUSED
+    global _FUSED, _STAMP
     _FUSED = bool(flag)
+    _STAMP += 1
+
+
+def set_tune(**kwargs):
+    """Change tunables at run time (they are part of every cache key)."""
+    global _STAMP
+    for k, v in kwargs.items():
+        if k not in TUNE:
+            raise KeyError(k)
+        TUNE[k] = int(v)
+    _STAMP += 1
 
 
 def is_ndarray(arr):
@@ -125,6 +138,7 @@ class Tracer:
         self.ops = []
         self._memo = {}
         self._evaluated = evaluated if evaluated is not None else {}
+        self.leaf_nodes = []      # (node, its array, the deps it was computed from or None)
 
     def leaf(self, arr):
         code = _code_of(arr.dtype)
@@ -172,6 +186,7 @@ class Tracer:
                     arr = None  # stale: recompute inside this kernel
         if arr is not None:
             res = self.leaf(arr)
+            self.leaf_nodes.append((node, arr, node.__dict__.get("_deps")))
         elif kind is _FE.BinaryNumpyEx or kind is _FE.BinaryFuncEx or kind is _FE.UnaryFuncEx:
             func = node.func
             name = func.__name__
@@ -255,7 +270,7 @@ def _merge_dims(shape, stride_sets):
 class Lowered:
     """A kernel choice for one evaluation: cache key, source builder, launch recipe."""
 
-    __slots__ = ("key", "kind", "emit", "fmt", "values", "grid", "fin_count", "lds")
+    __slots__ = ("key", "kind", "emit", "fmt", "srcs", "scal", "tail", "grid", "fin_count", "lds")
 
 
 # ---------------------------------------------------------------------------
@@ -394,10 +409,12 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
         else:
             E = 1
         chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
-        low.grid = min(chunks, TUNE["red_blocks"] if reduce_op else (1 << 24) - 1)
+        cap = TUNE["red_blocks"] if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
+        low.grid = min(chunks, cap)
         n_out_ptr = 1 if reduce_op else len(out_ptrs)
         low.fmt = "@" + "P" * (len(ptrs) + n_out_ptr) + scal_fmt + "q"
-        low.values = (ptrs, scal_vals, [n])
+        low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+        low.scal, low.tail = scal_vals, [n]
         if reduce_op:
             low.fin_count = low.grid
         return low
@@ -436,6 +453,7 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
                     kinds[i] = ("g",) + shifts[i]
                 g_buf = leaves[best[0]].buf
                 g_ptr = g_buf.ptr + ref_off * itemsize
+                g_src = (g_buf, ref_off * itemsize)
                 g_args = [rs, -ref_off, g_buf.nbytes // itemsize - ref_off]
         for i, s in enumerate(m_leaf):
             if kinds[i] is None:
@@ -472,12 +490,12 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
         tiles_x = -(-W // tw)
         tiles_y = -(-H // th)
         low.grid = tiles_x * tiles_y
-        ptrs = [a.ptr for a, k in zip(leaves, kinds) if k[0] != "g"]
-        fmt = "@" + "P" * len(ptrs)
+        srcs = [(a.buf, a.offset * a.dtype.itemsize) for a, k in zip(leaves, kinds) if k[0] != "g"]
+        fmt = "@" + "P" * len(srcs)
         tail_vals = []
         if group is not None:
             fmt += "P"
-            ptrs.append(g_ptr)
+            srcs.append(g_src)
         fmt += "P" * len(out_ptrs) + scal_fmt + "ii"
         tail_vals += [mshape[0], mshape[1]]
         if group is not None:
@@ -493,7 +511,7 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
             fmt += "q"
             tail_vals.append(s[0])
         low.fmt = fmt
-        low.values = (ptrs, scal_vals, tail_vals)
+        low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
         return low
 
     # general strided kernel
@@ -519,7 +537,8 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
             fmt += "q" * ndim
             tail += s
     low.fmt = fmt
-    low.values = ([a.ptr for a in leaves], scal_vals, tail)
+    low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+    low.scal, low.tail = scal_vals, tail
     if reduce_op:
         low.fin_count = low.grid
     return low
@@ -566,18 +585,57 @@ class record:
         return False
 
 
-def _launch(low, out_ptrs, reduce_out=None, reduce_code=None):
-    """Compile if needed and launch.  For a reduction, `reduce_out` is the device
-    address of the 0-d result."""
-    ptrs, scal_vals, tail = low.values
-    for p in ptrs:
-        if not p:
-            raise RuntimeError("an operand has no device memory (placeholder array)")
-    kern = _kernel_for(low, reduce_out is not None)
+_STAMP = 0            # bumped whenever tunables or the fusion mode change
+_RECENT = collections.deque(maxlen=int(os.environ.get("DELAYREPAY_KEEP", "16")))
+
+
+def forget():
+    """Drop the recently evaluated roots kept alive for plan reuse."""
+    _RECENT.clear()
+
+
+class Plan:
+    """Everything needed to launch an evaluated expression again: the lowered
+    kernel choice, the leaves it reads, the shape and dtypes it produces.
+
+    A plan is cached on the root node, and the last few evaluated roots are kept
+    alive, so re-building the same expression over the same arrays (the body of an
+    iterative loop) finds its nodes in the hash-cons table and its plan here: no
+    tracing, no layout analysis, no cache-key hashing, only an argument pack and a
+    launch.  `valid()` re-checks what could have changed underneath."""
+
+    __slots__ = ("low", "kern", "checks", "stamp", "shape", "out_dtypes", "acc", "leaves",
+                 "hazard", "region", "empty")
+
+    def valid(self):
+        if self.stamp != _STAMP:
+            return False
+        for node, arr, deps in self.checks:
+            if node.__dict__.get("array") is not arr:
+                return False
+            if deps is not None:
+                for buf, ver in deps:
+                    if buf.version != ver:
+                        return False
+        return True
+
+    def deps(self):
+        seen = {}
+        for arr in self.leaves:
+            seen[id(arr.buf)] = arr.buf
+        return tuple((buf, buf.version) for buf in seen.values())
+
+
+def _fire(plan, out_ptrs, reduce_out=None):
+    """Compile on first use, pack the argument block, launch."""
+    low = plan.low
+    kern = plan.kern
+    if kern is None:
+        kern = plan.kern = _kernel_for(low, reduce_out is not None)
+    ptrs = [buf.ptr + off for buf, off in low.srcs]
     if reduce_out is not None:
-        itemsize = cg.ITEMSIZE[reduce_code]
-        partial = hiprt.malloc(low.fin_count * itemsize)
-        args = kern.packer.pack(*ptrs, partial, *scal_vals, *tail)
+        partial = hiprt.malloc(low.fin_count * cg.ITEMSIZE[plan.acc])
+        args = kern.packer.pack(*ptrs, partial, *low.scal, *low.tail)
         hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
         fin = struct.pack("@PPi", partial, reduce_out, low.fin_count)
         hiprt.launch(kern.finalize, 1, cg.BLOCK, 0, fin, len(fin))
@@ -588,7 +646,7 @@ def _launch(low, out_ptrs, reduce_out=None, reduce_code=None):
             hiprt.free(partial)  # stream-ordered: safe to recycle once queued
         STATS["launches"] += 2
     else:
-        args = kern.packer.pack(*ptrs, *out_ptrs, *scal_vals, *tail)
+        args = kern.packer.pack(*ptrs, *out_ptrs, *low.scal, *low.tail)
         hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
         if _RECORDING is not None:
             _RECORDING.launches.append((kern.func, low.grid, 0, args))
@@ -599,53 +657,82 @@ def _launch(low, out_ptrs, reduce_out=None, reduce_code=None):
 # evaluation entry points
 # ---------------------------------------------------------------------------
 
-def _execute(tracer, roots, dsts=None, reduce_op=None, launch=True):
-    """Run traced `roots` (list of (ref, code)).  Returns output arrays (or the
-    `Lowered` object when `launch` is False)."""
+def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False):
+    """Lower traced `roots` (list of (ref, code)) into a Plan.  `dst`: existing
+    destination view (single root); `dry`: placeholders instead of device memory."""
     prog = tracer.program(roots)
     leaves = tracer.leaves
+    plan = Plan()
+    plan.kern = None
+    plan.stamp = _STAMP
+    plan.checks = tracer.leaf_nodes
+    plan.leaves = list(leaves)
+    plan.hazard = False
+    plan.region = None
+    plan.acc = None
+    plan.empty = False
     if reduce_op:
-        shape = numpy.broadcast_shapes(*[a.shape for a in leaves]) if leaves else ()
-        code = roots[0][1]
-        acc = "i8" if (reduce_op == "add" and code in ("i4", "u4", "u1", "b1")) else code
-        low = _lower(prog, leaves, tracer.scalars, tuple(shape), [acc], [], [], reduce_op)
-        if not launch:
-            return low
-        out = ndarray((), code_dtype(acc))
-        _launch(low, [], out.ptr, acc)
-        if _RECORDING is not None:
-            _RECORDING.keep += [out] + list(leaves)
-        return [out]
-    if dsts is None:
         shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
-        make = ndarray if launch else placeholder
-        outs = [make(shape, code_dtype(code)) for _, code in roots]
+        code = roots[0][1]
+        plan.acc = "i8" if (reduce_op == "add" and code in ("i4", "u4", "u1", "b1")) else code
+        plan.shape = ()
+        plan.out_dtypes = [code_dtype(plan.acc)]
+        plan.low = _lower(prog, leaves, tracer.scalars, shape, [plan.acc], [], [], reduce_op)
+        return plan
+    if dst is None:
+        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
+        plan.out_dtypes = [code_dtype(code) for _, code in roots]
+        out_codes = [code for _, code in roots]
+        out_ptrs = [0] * len(roots)          # pool blocks are 256-byte aligned
+        out_strides = [list(_contiguous(shape))] * len(roots)
         in_place = False
     else:
-        shape = dsts[0].shape
-        outs = dsts
-        in_place = any(a.buf is d.buf for a in leaves for d in dsts)
+        shape = dst.shape
+        plan.out_dtypes = [dst.dtype]
+        out_codes = [dtype_code(dst.dtype)]
+        out_ptrs = [dst.offset * dst.dtype.itemsize]   # alignment relative to the buffer start
+        out_strides = [_broadcast_strides(dst, shape)]
+        in_place = any(a.buf is dst.buf for a in leaves)
+    plan.shape = shape
     n = 1
     for d in shape:
         n *= d
     if n == 0:
-        return outs
-    out_codes = [dtype_code(o.dtype) for o in outs]
-    out_ptrs = [o.ptr for o in outs]
-    out_strides = [_broadcast_strides(o, shape) for o in outs]
-    low = _lower(prog, leaves, tracer.scalars, shape, out_codes, out_ptrs, out_strides, None,
-                 in_place)
-    if not launch:
-        return low
-    _launch(low, out_ptrs)
+        plan.empty = True
+        plan.low = None
+        return plan
+    plan.low = _lower(prog, leaves, tracer.scalars, shape, out_codes, out_ptrs, out_strides, None,
+                      in_place)
+    return plan
+
+
+def _contiguous(shape):
+    strides, acc = [], 1
+    for d in reversed(shape):
+        strides.append(acc if d != 1 else 0)
+        acc *= d
+    return tuple(reversed(strides))
+
+
+def _launch_fresh(plan):
+    """Allocate outputs for `plan` and launch it; returns the output arrays."""
+    if plan.acc is not None:
+        out = ndarray((), plan.out_dtypes[0])
+        _fire(plan, [], out.ptr)
+        outs = [out]
+    else:
+        outs = [ndarray(plan.shape, dt) for dt in plan.out_dtypes]
+        if not plan.empty:
+            _fire(plan, [o.ptr for o in outs])
     if _RECORDING is not None:
-        _RECORDING.keep += list(outs) + list(leaves)
+        _RECORDING.keep += outs + plan.leaves
     return outs
 
 
 def _trace_root(tracer, node):
-    from .delayarray import ReduceEx
-    if isinstance(node, ReduceEx) and "array" not in node.__dict__:
+    if _FE is None:
+        _bind_frontend()
+    if type(node) is _FE.ReduceEx and "array" not in node.__dict__:
         raise TypeError("a reduction must be the root of its own evaluation")
     return tracer.visit(node)
 
@@ -664,10 +751,10 @@ def _run_unfused(ex, evaluated):
     tracer = Tracer(evaluated)
     if isinstance(ex, ReduceEx):
         root = tracer.visit(ex.children[0])
-        out = _execute(tracer, [root], reduce_op=ex.func.__name__)[0]
+        out = _launch_fresh(_make_plan(tracer, [root], reduce_op=ex.func.__name__))[0]
     else:
         root = tracer.visit(ex)
-        out = _execute(tracer, [root])[0]
+        out = _launch_fresh(_make_plan(tracer, [root]))[0]
     evaluated[nid] = out
     return out
 
@@ -675,19 +762,26 @@ def _run_unfused(ex, evaluated):
 def run(ex):
     """Evaluate one DAG root; returns a new device array owned by the caller
     (cf. cuda.py:91-96)."""
-    from .delayarray import ReduceEx
     if not _FUSED:
-        evaluated = {}
-        out = _run_unfused(ex, evaluated)
-        return out
-    tracer = Tracer()
-    if isinstance(ex, ReduceEx):
-        root = tracer.visit(ex.children[0])
-        out = _execute(tracer, [root], reduce_op=ex.func.__name__)[0]
+        return _run_unfused(ex, {})
+    d = ex.__dict__
+    plan = d.get("_plan")
+    if plan is None or not plan.valid():
+        if _FE is None:
+            _bind_frontend()
+        tracer = Tracer()
+        if type(ex) is _FE.ReduceEx:
+            root = tracer.visit(ex.children[0])
+            plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__)
+        else:
+            root = _trace_root(tracer, ex)
+            plan = _make_plan(tracer, [root])
+        d["_plan"] = plan
+        _RECENT.append(ex)
     else:
-        root = _trace_root(tracer, ex)
-        out = _execute(tracer, [root])[0]
-    ex.__dict__["_deps"] = tracer.deps()
+        STATS["plan_hits"] += 1
+    out = _launch_fresh(plan)[0]
+    d["_deps"] = plan.deps()
     return out
 
 
@@ -701,10 +795,20 @@ def run_multi(exs):
         by_shape.setdefault(tuple(ex.shape), []).append(i)
     results = [None] * len(exs)
     for shape, idxs in by_shape.items():
-        tracer = Tracer()
-        roots = [_trace_root(tracer, exs[i]) for i in idxs]
-        outs = _execute(tracer, roots)
-        deps = tracer.deps()
+        first = exs[idxs[0]].__dict__
+        key = tuple(id(exs[i]) for i in idxs)
+        cached = first.get("_multi")
+        if cached is not None and cached[0] == key and cached[1].valid():
+            plan = cached[1]
+            STATS["plan_hits"] += 1
+        else:
+            tracer = Tracer()
+            roots = [_trace_root(tracer, exs[i]) for i in idxs]
+            plan = _make_plan(tracer, roots)
+            first["_multi"] = (key, plan, [exs[i] for i in idxs])
+            _RECENT.append(exs[idxs[0]])
+        outs = _launch_fresh(plan)
+        deps = plan.deps()
         for i, out in zip(idxs, outs):
             if out.shape != shape:   # every leaf of this root was a broadcast scalar
                 out = materialise(out, shape=shape)
@@ -731,9 +835,9 @@ def _same_view(a, b):
             and a.dtype == b.dtype)
 
 
-def _write(tracer, root, dst):
-    """Launch traced `root` into the existing view `dst`, guarding against reading
-    what the kernel overwrites."""
+def _plan_write(tracer, root, dst):
+    """Plan for launching traced `root` into the existing view `dst`; decides
+    whether the kernel would read what it overwrites."""
     shape = dst.shape
     for a in tracer.leaves:
         _broadcast_strides(a, shape)  # raises when the value does not fit the destination
@@ -745,29 +849,56 @@ def _write(tracer, root, dst):
             it = dst.dtype.itemsize
             if a_lo * a.dtype.itemsize < d_hi * it and d_lo * it < a_hi * a.dtype.itemsize:
                 hazard = True
+    if hazard:
+        # the kernel will write a different allocation: lower it as not-in-place
+        stand_in = ndarray(dst.shape, dst.dtype, _Elsewhere(dst.buf.nbytes), dst.offset,
+                           dst._strides)
+        plan = _make_plan(tracer, [root], dst=stand_in)
+    else:
+        plan = _make_plan(tracer, [root], dst=dst)
+    plan.hazard = hazard
+    plan.region = (dst.offset, dst.shape, dst._strides, dst.dtype.str)
+    return plan
+
+
+class _Elsewhere(Buffer):
+    """Stands for "an allocation other than the source buffer, same layout" while
+    lowering a ping-pong write; owns no memory."""
+
+    __slots__ = ()
+
+    def __init__(self, nbytes):
+        self.nbytes = nbytes
+        self.ptr = 0
+        self.version = 0
+        self.shadow = None
+        self.shadow_region = None
+
+
+def _write(plan, dst):
+    """Launch `plan` into `dst`."""
     buf = dst.buf
-    if not hazard:
-        _execute(tracer, [root], dsts=[dst])
-        buf.touch()
+    if plan.empty:
         return
-    # Ping-pong: write into the shadow allocation, which mirrors the buffer
-    # everywhere outside `region`, then swap the two device pointers.  Every view
-    # of the buffer (they share the Buffer object) sees the update at once.
-    region = (dst.offset, dst.shape, dst._strides, dst.dtype.str)
-    if buf.shadow is None:
-        buf.shadow = hiprt.malloc(max(buf.nbytes, 1))
-        buf.shadow_region = None
-    if buf.shadow_region != region:
-        hiprt.memcpy_d2d(buf.shadow, buf.ptr, buf.nbytes)
-    target = ndarray(dst.shape, dst.dtype, Buffer(buf.nbytes, ptr=buf.shadow), dst.offset,
-                     dst._strides)
-    try:
-        _execute(tracer, [root], dsts=[target])
-    finally:
-        target.buf.ptr = None  # borrowed pointer: must not be freed with the helper
-    buf.ptr, buf.shadow = buf.shadow, buf.ptr
-    buf.shadow_region = region
-    buf.version += 1
+    off = dst.offset * dst.dtype.itemsize
+    if not plan.hazard:
+        _fire(plan, [buf.ptr + off])
+        buf.touch()
+    else:
+        # Ping-pong: write into the shadow allocation, which mirrors the buffer
+        # everywhere outside `region`, then swap the two device pointers.  Every view
+        # of the buffer (they share the Buffer object) sees the update at once.
+        if buf.shadow is None:
+            buf.shadow = hiprt.malloc(max(buf.nbytes, 1))
+            buf.shadow_region = None
+        if buf.shadow_region != plan.region:
+            hiprt.memcpy_d2d(buf.shadow, buf.ptr, buf.nbytes)
+        _fire(plan, [buf.shadow + off])
+        buf.ptr, buf.shadow = buf.shadow, buf.ptr
+        buf.shadow_region = plan.region
+        buf.version += 1
+    if _RECORDING is not None:
+        _RECORDING.keep += [dst] + plan.leaves
 
 
 def run_into(ex, dst):
@@ -775,9 +906,19 @@ def run_into(ex, dst):
     if not _FUSED:
         assign(dst, run(ex))
         return
-    tracer = Tracer()
-    root = _trace_root(tracer, ex)
-    _write(tracer, root, dst)
+    d = ex.__dict__
+    key = (id(dst.buf), dst.offset, dst.shape, dst._strides, dst.dtype.str)
+    cached = d.get("_into")
+    if cached is not None and cached[0] == key and cached[1].valid():
+        plan = cached[1]
+        STATS["plan_hits"] += 1
+    else:
+        tracer = Tracer()
+        root = _trace_root(tracer, ex)
+        plan = _plan_write(tracer, root, dst)
+        d["_into"] = (key, plan, dst.buf)     # holding the buffer keeps its id unique
+        _RECENT.append(ex)
+    _write(plan, dst)
 
 
 def assign(dst, value):
@@ -799,7 +940,7 @@ def assign(dst, value):
             root = tracer.scalar(host[()], dtype_code(dst.dtype))
         else:
             root = tracer.leaf(ndarray.from_host(host))
-    _write(tracer, root, dst)
+    _write(_plan_write(tracer, root, dst), dst)
 
 
 def materialise(arr, dtype=None, shape=None):
@@ -811,9 +952,9 @@ def materialise(arr, dtype=None, shape=None):
         root = tracer.op("cast", code, code, [root[0]])
     if shape is not None and tuple(shape) != arr.shape:
         out = ndarray(shape, code_dtype(root[1]))
-        _execute(tracer, [root], dsts=[out])
+        _write(_plan_write(tracer, root, out), out)
         return out
-    return _execute(tracer, [root])[0]
+    return _launch_fresh(_make_plan(tracer, [root]))[0]
 
 
 def run_reduce_product(a, b):
@@ -830,10 +971,11 @@ def lower_only(exs, dst=None):
     tracer = Tracer()
     if isinstance(exs[0], ReduceEx):
         root = tracer.visit(exs[0].children[0])
-        low = _execute(tracer, [root], reduce_op=exs[0].func.__name__, launch=False)
+        low = _make_plan(tracer, [root], reduce_op=exs[0].func.__name__).low
+    elif dst is not None:
+        low = _plan_write(tracer, tracer.visit(exs[0]), dst).low
     else:
-        roots = [tracer.visit(ex) for ex in exs]
-        low = _execute(tracer, roots, dsts=None if dst is None else [dst], launch=False)
+        low = _make_plan(tracer, [tracer.visit(ex) for ex in exs]).low
     return low, low.emit()
 
 

@@ -149,8 +149,9 @@ def malloc(nbytes):
 
 def free(ptr):
     # called from finalisers: never raise during interpreter shutdown
-    if _lib is not None and ptr:
-        _lib.drhip_free(ptr)
+    lib_ = _lib
+    if lib_ is not None and ptr:
+        lib_.drhip_free(ptr)
 
 
 def pool_stats():

@@ -416,3 +416,36 @@ def test_astype_is_fused_and_exact():
     assert bits_equal(got, ref)
     i = dr.full((64,), 7).astype(np.float32)               # reference tests/test.py:74
     assert i.dtype == np.float32 and bits_equal(i.get(), np.full((64,), 7).astype(np.float32))
+
+
+# ---- plan reuse -------------------------------------------------------------------------------
+
+def test_repeated_expression_reuses_its_plan_and_stays_correct():
+    inp = orc.make_inputs("saxpy", 5000)
+    x, y = dr.array(inp["x"]), dr.array(inp["y"])
+    first = hip.run(2.0 * x + y)
+    hits = hip.STATS["plan_hits"]
+    again = hip.run(2.0 * x + y)              # same nodes from the hash-cons table
+    assert hip.STATS["plan_hits"] == hits + 1
+    assert bits_equal(first.get(), again.get()) and first.ptr != again.ptr
+    x[:] = x * 3.0                            # leaves change: same plan, new values
+    ref = orc.saxpy(2.0, inp["x"] * np.float32(3.0), inp["y"])
+    assert bits_equal((2.0 * x + y).get(), ref)
+    x64 = x.astype(np.float64)                # a new leaf; expressions on x are untouched
+    assert x.dtype == np.float32 and bits_equal((2.0 * x + y).get(), ref)
+    assert bits_equal((2.0 * x64 + y).get(),
+                      2.0 * (inp["x"] * np.float32(3.0)).astype(np.float64) + inp["y"])
+
+
+def test_sweeps_reuse_one_plan():
+    u0 = np.zeros((40, 72), np.float32)
+    u0[1:-1, 1:-1] = np.random.RandomState(1).uniform(0, 1, (38, 70))
+    u = dr.array(u0)
+    jacobi_sweeps(u, 2)
+    hits = hip.STATS["plan_hits"]
+    jacobi_sweeps(u, 6)
+    assert hip.STATS["plan_hits"] == hits + 6
+    assert bits_equal(u.get(), orc.jacobi(u0, 8))
+    dr.reset()
+    jacobi_sweeps(u, 1)
+    assert bits_equal(u.get(), orc.jacobi(u0, 9))
