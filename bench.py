@@ -34,6 +34,22 @@ HBM_PEAK_GBPS = 8000.0
 METRIC = "fused-kernel effective HBM GB/s (% of MI355X peak); Gelem/s vs unfused"
 
 
+def measured_traffic(name):
+    """HBM bytes per launch of a workload's kernel as measured with rocprofv3
+    counters (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel); the figures
+    live in profiles/hbm_traffic.txt as `<workload> <bytes>` lines."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    try:
+        with open(path) as fh:
+            for ln in fh:
+                parts = ln.split()
+                if len(parts) >= 2 and parts[0] == name:
+                    return int(float(parts[1]))
+    except OSError:
+        pass
+    return None
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -44,6 +60,7 @@ def parse():
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before each timed region (clock ramp-up)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-copy", action="store_true", help="skip the plain-copy ceiling leg")
     ap.add_argument("--no-unfused", action="store_true", help="skip the un-fused leg")
     return ap.parse_args()
 
@@ -223,6 +240,28 @@ def main():
         print(f"[bench] {name}: {results[name]}", file=sys.stderr, flush=True)
         hiprt.pool_trim()
 
+    # the plain streaming copy (1 GiB in, 1 GiB out): measured ceiling of the memory
+    # system for a read+write stream, and the known-size kernel against which the
+    # profiler's FETCH_SIZE / WRITE_SIZE counters are calibrated
+    copy = None
+    if not args.no_copy:
+        nb = 1 << 30
+        a, b = hip.ndarray((nb // 4,), np.float32), hip.ndarray((nb // 4,), np.float32)
+        hiprt.fill32(a.ptr, 0x3F800000, nb // 4)
+        for _ in range(3):
+            hiprt.copy_kernel(b.ptr, a.ptr, nb)
+        hiprt.sync()
+        e0, e1 = hiprt.Event(), hiprt.Event()
+        e0.record()
+        for _ in range(10):
+            hiprt.copy_kernel(b.ptr, a.ptr, nb)
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_ms(e1) / 10
+        copy = {"bytes_read": nb, "bytes_written": nb, "us": round(ms * 1e3, 1),
+                "GBps": round(2 * nb / ms / 1e6, 1), "frac": round(2 * nb / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        del a, b
+
     head = results.get("horner") or results[names[0]]
     head_name = "horner" if "horner" in results else names[0]
     line = {
@@ -247,6 +286,12 @@ def main():
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"]},
         "configs": results,
     }
+    if copy is not None:
+        line["copy_kernel"] = copy
+    traffic = measured_traffic(head_name)
+    if traffic is not None:
+        line["roofline"]["traffic"] = traffic
+        line["roofline"]["traffic_source"] = "profiles/hbm_traffic.txt (rocprofv3 --pmc, calibrated)"
     if "cpu" in head:
         line["cpu_baseline"] = {
             "value": head["cpu"]["GBps"], "unit": "GB/s", "cores": 1, "kind": "port",

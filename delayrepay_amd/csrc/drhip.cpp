@@ -237,7 +237,11 @@ int drhip_copy_kernel(void* dst, const void* src, size_t nbytes, unsigned grid) 
     if (nbytes % 16 || (uintptr_t)dst % 16 || (uintptr_t)src % 16)
         return fail(DRHIP_EINVAL, "drhip_copy_kernel", "size and pointers must be multiples of 16");
     if (nbytes == 0) return 0;
-    if (grid == 0) grid = (unsigned)g_prop.multiProcessorCount * 8u;
+    if (grid == 0) {  // one run of 256 vectors per block
+        size_t runs = nbytes / 16 / 256;
+        if (runs == 0) runs = 1;
+        grid = (unsigned)(runs < (size_t(1) << 23) ? runs : (size_t(1) << 23));
+    }
     drhip_k_launch_copy(dst, src, nbytes / 16, grid, g_stream);
     HIP_TRY(hipGetLastError());
     g_cnt.n_launches++;

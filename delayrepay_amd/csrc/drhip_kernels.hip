@@ -17,23 +17,20 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(W* __restrict__ dst, W v, 
     for (; i < n; i += stride) dst[i] = v;
 }
 
-// 128-bit loads and stores, grid-stride, four independent vectors in flight
-// per thread and iteration.
+// 128-bit non-temporal loads and stores.  A block copies runs of 256 consecutive
+// vectors and advances by gridDim.x runs; launched with one run per block, which is
+// the fastest read+write pattern measured on MI355X (the DRAM access stream stays
+// nearly sequential).
 __global__ __launch_bounds__(kBlock) void copy_kernel(u32x4* __restrict__ dst,
                                                       const u32x4* __restrict__ src, size_t nvec) {
-    const size_t stride = (size_t)gridDim.x * kBlock;
-    size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    for (; i + 3 * stride < nvec; i += 4 * stride) {
+    const size_t nrun = nvec / kBlock;
+    for (size_t r = blockIdx.x; r < nrun; r += gridDim.x) {
+        const size_t i = r * kBlock + threadIdx.x;
         u32x4 a = __builtin_nontemporal_load(src + i);
-        u32x4 b = __builtin_nontemporal_load(src + i + stride);
-        u32x4 c = __builtin_nontemporal_load(src + i + 2 * stride);
-        u32x4 d = __builtin_nontemporal_load(src + i + 3 * stride);
         __builtin_nontemporal_store(a, dst + i);
-        __builtin_nontemporal_store(b, dst + i + stride);
-        __builtin_nontemporal_store(c, dst + i + 2 * stride);
-        __builtin_nontemporal_store(d, dst + i + 3 * stride);
     }
-    for (; i < nvec; i += stride) {
+    for (size_t i = nrun * kBlock + (size_t)blockIdx.x * kBlock + threadIdx.x; i < nvec;
+         i += (size_t)gridDim.x * kBlock) {
         u32x4 a = __builtin_nontemporal_load(src + i);
         __builtin_nontemporal_store(a, dst + i);
     }

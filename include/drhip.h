@@ -93,9 +93,10 @@ int drhip_memcpy_d2d(void* dst_dev, const void* src_dev, size_t nbytes);
  * (no memset node, so the call is safe to record into a HIP graph). */
 int drhip_fill32(void* dst_dev, uint32_t pattern, size_t nwords);
 int drhip_fill64(void* dst_dev, uint64_t pattern, size_t nwords);
-/* Plain streaming copy kernel (128-bit loads and stores, grid-stride); used
- * as the measured ceiling of the memory system next to generated kernels and
- * to calibrate profiler byte counters.  nbytes must be a multiple of 16. */
+/* Plain streaming copy kernel (128-bit non-temporal loads and stores); used as
+ * the measured ceiling of the memory system next to generated kernels and to
+ * calibrate profiler byte counters.  nbytes must be a multiple of 16;
+ * grid_blocks = 0 picks one run of 256 vectors per block. */
 int drhip_copy_kernel(void* dst_dev, const void* src_dev, size_t nbytes,
                       unsigned grid_blocks);
 
