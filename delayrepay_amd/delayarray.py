@@ -727,7 +727,7 @@ def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **unused
         axis = None
     if arr.ndim <= 1 and axis in (0, -1):
         axis = None
-    if axis is None and not keepdims and arr.size > 0:
+    if axis is None and not keepdims:
         return ReduceEx(func, arr)._force()
     eager = {"add": "sum", "maximum": "max", "minimum": "min"}[func.__name__]
     return getattr(_backend.fallback, eager)(arr._force(), axis=axis, keepdims=keepdims)

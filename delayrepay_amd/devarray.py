@@ -140,7 +140,9 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
 
     @classmethod
     def from_host(cls, host):
-        host = np.ascontiguousarray(host)
+        host = np.asarray(host)
+        if not host.flags.c_contiguous:       # (ascontiguousarray would make 0-d into 1-d)
+            host = np.ascontiguousarray(host)
         if host.dtype.name not in SUPPORTED_DTYPES:
             if host.dtype.kind in "iu":
                 host = host.astype(np.int64)

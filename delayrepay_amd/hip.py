@@ -677,6 +677,13 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False):
         plan.acc = "i8" if (reduce_op == "add" and code in ("i4", "u4", "u1", "b1")) else code
         plan.shape = ()
         plan.out_dtypes = [code_dtype(plan.acc)]
+        if 0 in shape:
+            if reduce_op != "add":
+                raise ValueError(f"zero-size array to reduction operation {reduce_op} "
+                                 "which has no identity")
+            plan.empty = True
+            plan.low = None
+            return plan
         plan.low = _lower(prog, leaves, tracer.scalars, shape, [plan.acc], [], [], reduce_op)
         return plan
     if dst is None:
@@ -718,7 +725,10 @@ def _launch_fresh(plan):
     """Allocate outputs for `plan` and launch it; returns the output arrays."""
     if plan.acc is not None:
         out = ndarray((), plan.out_dtypes[0])
-        _fire(plan, [], out.ptr)
+        if plan.empty:       # sum over nothing
+            (hiprt.fill64 if out.itemsize == 8 else hiprt.fill32)(out.ptr, 0, 1)
+        else:
+            _fire(plan, [], out.ptr)
         outs = [out]
     else:
         outs = [ndarray(plan.shape, dt) for dt in plan.out_dtypes]

@@ -449,3 +449,39 @@ def test_sweeps_reuse_one_plan():
     dr.reset()
     jacobi_sweeps(u, 1)
     assert bits_equal(u.get(), orc.jacobi(u0, 9))
+
+
+# ---- edges: empty, 0-d, more than 2^31 elements -------------------------------------------------
+
+def test_empty_and_zero_dimensional_arrays():
+    e = dr.array(np.zeros((0,), np.float32))
+    assert (e * 2.0 + 1).get().shape == (0,)
+    assert float(dr.sum(e)) == 0.0 and dr.sum(e).dtype == np.float32
+    with pytest.raises(ValueError):
+        dr.max(e)
+    e2 = dr.array(np.zeros((3, 0, 5)))
+    assert (e2 + e2).get().shape == (3, 0, 5)
+    e[:] = 1.0                                       # writes nothing, must not launch
+    s = dr.array(np.float64(3.0))                    # 0-d leaf
+    assert s.shape == () and float(s * 2 + 1) == 7.0
+    v = dr.array(np.arange(5.0))
+    assert np.array_equal((v * s).get(), np.arange(5.0) * 3.0)
+    one = dr.array(np.array([2.5], np.float32))
+    assert np.array_equal((one + one).get(), np.array([5.0], np.float32))
+
+
+def test_more_than_2_to_31_elements():
+    """64-bit indexing: n = 2^31 + 5 float32 (8 GiB per array)."""
+    n = (1 << 31) + 5
+    x = dr.zeros(n, dtype=np.float32)
+    x[:] = 1.5
+    x[n - 3:] = 2.5
+    z = 2.0 * x + 1.0
+    tail = z[n - 6:].get()
+    assert np.array_equal(tail, np.array([4, 4, 4, 6, 6, 6], np.float32))
+    assert float(z[1 << 31]) == 4.0 and float(z[0]) == 4.0
+    total = float(dr.sum(z.astype(np.float64)))
+    assert total == 4.0 * (n - 3) + 6.0 * 3
+    strided = z[::3]                                  # > 2^31 / 3 elements through the nd kernel
+    assert float(dr.max(strided * 1.0)) == 6.0 or float(dr.max(strided * 1.0)) == 4.0
+    assert float(dr.sum((strided * 0.0 + 1.0).astype(np.float64))) == float(len(range(0, n, 3)))
