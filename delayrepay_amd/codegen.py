@@ -679,3 +679,82 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
     L += ["                }", "        }", "    }", "}"]
     src.append("\n".join(L))
     return "\n".join(src) + "\n", TW, TH, LH * LW * ITEMSIZE[gdt]
+
+
+# ---- reduction along some axes ------------------------------------------------
+
+def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
+    """Reduce the (fused) expression over `rdim` merged dimensions, keeping `kdim`.
+
+    strategy 'col'  one thread per output, looping over the reduced extent:
+                    coalesced when the fastest-varying memory dimension is kept
+                    (e.g. sum over axis 0 of a row-major matrix);
+             'row'  one block per output, threads striding over the reduced extent,
+                    wave64 shuffle + LDS tree at the end: coalesced when the
+                    fastest-varying dimension is reduced (e.g. sum over the last axis).
+    Parameters: leaf pointers, output pointer, scalars, K, R, kept dims, reduced
+    dims, then per leaf its kept strides and its reduced strides (elements)."""
+    ct = CTYPE[acc_dt]
+    src = [PREAMBLE, emit_body(prog, [acc_dt])]
+    if strategy == "row":
+        src.append(emit_block_reduce(op, acc_dt))
+    params = [f"const {CTYPE[dt]}* a{i}" for i, dt in enumerate(prog.leaves)]
+    params.append(f"{ct}* out")
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += ["const long long K", "const long long R"]
+    params += [f"const long long dk{d}" for d in range(kdim)]
+    params += [f"const long long dr{d}" for d in range(rdim)]
+    for i in range(len(prog.leaves)):
+        params += [f"const long long sk{i}_{d}" for d in range(kdim)]
+        params += [f"const long long sr{i}_{d}" for d in range(rdim)]
+    nl = len(prog.leaves)
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{"]
+
+    def decompose(var, dims, prefix, n, out_prefix, indent):
+        """Lines turning linear index `var` into per-leaf offsets `out_prefix{i}`."""
+        pad = " " * indent
+        lines = [f"{pad}long long rem_{prefix} = {var};"]
+        for i in range(nl):
+            lines.append(f"{pad}long long {out_prefix}{i} = 0;")
+        for d in reversed(range(n)):
+            if d == 0:
+                lines.append(f"{pad}const long long c_{prefix}{d} = rem_{prefix};")
+            else:
+                lines.append(f"{pad}const long long c_{prefix}{d} = rem_{prefix} % {dims}{d}; "
+                             f"rem_{prefix} /= {dims}{d};")
+            for i in range(nl):
+                lines.append(f"{pad}{out_prefix}{i} += c_{prefix}{d} * s{prefix}{i}_{d};")
+        return lines
+
+    call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
+    if strategy == "col":
+        L.append(f"    const long long stride = (long long)gridDim.x * {BLOCK};")
+        L.append(f"    for (long long g = (long long)blockIdx.x * {BLOCK} + threadIdx.x; g < K; g += stride) {{")
+        L += decompose("g", "dk", "k", kdim, "bk", 8)
+        L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
+        L.append("        for (long long r = 0; r < R; ++r) {")
+        L += decompose("r", "dr", "r", rdim, "br", 12)
+        args = [f"a{i}[bk{i} + br{i}]" for i in range(nl)]
+        L.append(f"            {ct} t0; dr_body({', '.join(args + call_tail)});")
+        L.append(f"            acc = {_combine(op, 'acc', 't0')};")
+        L.append("        }")
+        L.append("        out[g] = acc;")
+        L.append("    }")
+    else:
+        L.append("    for (long long g = blockIdx.x; g < K; g += gridDim.x) {")
+        L += decompose("g", "dk", "k", kdim, "bk", 8)
+        L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
+        L.append(f"        for (long long r = threadIdx.x; r < R; r += {BLOCK}) {{")
+        L += decompose("r", "dr", "r", rdim, "br", 12)
+        args = [f"a{i}[bk{i} + br{i}]" for i in range(nl)]
+        L.append(f"            {ct} t0; dr_body({', '.join(args + call_tail)});")
+        L.append(f"            acc = {_combine(op, 'acc', 't0')};")
+        L.append("        }")
+        L.append("        acc = dr_block_reduce(acc);")
+        L.append("        if (threadIdx.x == 0) out[g] = acc;")
+        L.append("        __syncthreads();")
+        L.append("    }")
+    L.append("}")
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"

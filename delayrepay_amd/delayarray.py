@@ -518,14 +518,23 @@ class Funcable:
 
 
 class ReduceEx(NumpyEx, Funcable):
-    """Full reduction of an expression with a binary ufunc (`add`, `maximum`,
-    `minimum`); evaluated as the tail of the fused element-wise kernel."""
+    """Reduction of an expression with a binary ufunc (`add`, `maximum`, `minimum`),
+    over everything (`axis` None) or over a tuple of axes; evaluated as the tail of
+    the fused element-wise kernel."""
 
-    def __init__(self, func, arg):
+    def __init__(self, func, arg, axis=None):
         super().__init__(children=[arg])
         self.func = func
-        self.shape = ()
+        self.axis = axis
+        if axis is None:
+            self.shape = ()
+        else:
+            self.shape = tuple(d for k, d in enumerate(arg.shape) if k not in axis)
         self.dtype = arg.dtype
+
+    @classmethod
+    def _memo_key(cls, func, arg, axis=None):
+        return (cls, func, id(arg), axis)
 
     @property
     def name(self):
@@ -723,14 +732,28 @@ def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **unused
     arr = arg_to_numpy_ex(arr)
     if out is not None or dtype is not None:
         raise NotImplementedError("reductions with out= or dtype= are not supported")
-    if isinstance(axis, tuple) and sorted(a % max(arr.ndim, 1) for a in axis) == list(range(arr.ndim)):
-        axis = None
-    if arr.ndim <= 1 and axis in (0, -1):
-        axis = None
-    if axis is None and not keepdims:
-        return ReduceEx(func, arr)._force()
-    eager = {"add": "sum", "maximum": "max", "minimum": "min"}[func.__name__]
-    return getattr(_backend.fallback, eager)(arr._force(), axis=axis, keepdims=keepdims)
+    ndim = arr.ndim
+    if axis is not None:
+        axes = (axis,) if isinstance(axis, (int, np.integer)) else tuple(axis)
+        norm = []
+        for a in axes:
+            a = int(a)
+            if not -ndim <= a < ndim:
+                raise np.exceptions.AxisError(a, ndim)
+            norm.append(a % ndim)
+        if len(set(norm)) != len(norm):
+            raise ValueError("duplicate value in 'axis'")
+        axis = tuple(sorted(norm))
+        if len(axis) == ndim:
+            axis = None
+    if not hasattr(_backend, "run_multi"):      # NumPy backend: plain library call
+        eager = {"add": "sum", "maximum": "max", "minimum": "min"}[func.__name__]
+        return getattr(_backend.fallback, eager)(arr._force(), axis=axis, keepdims=keepdims)
+    res = ReduceEx(func, arr, axis)._force() if axis is not None else ReduceEx(func, arr)._force()
+    if keepdims:
+        full = tuple(1 if (axis is None or k in axis) else d for k, d in enumerate(arr.shape))
+        res = res.reshape(full)
+    return res if axis is None and not keepdims else NPArray(res)
 
 
 def evaluate(*arrays):
@@ -786,11 +809,16 @@ def min(arr, axis=None, **kwargs):
 
 
 @implements(np.mean)
-def mean(arr, axis=None, **kwargs):
+def mean(arr, axis=None, keepdims=False, **kwargs):
     arr = arg_to_numpy_ex(arr)
-    if axis is None and not kwargs:
-        return NPArray(_reduce(np.add, arr)) / arr.size
-    return _backend.fallback.mean(arr._force(), axis=axis, **kwargs)
+    if kwargs:
+        return _backend.fallback.mean(arr._force(), axis=axis, keepdims=keepdims, **kwargs)
+    total = _reduce(np.add, arr, axis=axis, keepdims=keepdims)
+    total = total if isinstance(total, DelayArray) else NPArray(total)
+    count = arr.size // total.size if total.size else 0
+    if arr.dtype.kind in "iub":
+        total = total.astype(np.float64)
+    return total / count
 
 
 @implements(np.average)
@@ -801,14 +829,18 @@ def average(arr, axis=None, weights=None, **kwargs):
 
 
 @implements(np.var)
-def var(arr, axis=None, ddof=0, **kwargs):
-    """Two-pass variance: mean, then the fused sum of squared deviations."""
+def var(arr, axis=None, ddof=0, keepdims=False, **kwargs):
+    """Two-pass variance: mean, then the fused mean of squared deviations."""
     arr = arg_to_numpy_ex(arr)
-    if axis is None and not kwargs:
-        centre = NPArray(_reduce(np.add, arr)) / arr.size
-        dev = arr - centre
-        return NPArray(_reduce(np.add, dev * dev)) / (arr.size - ddof)
-    return _backend.fallback.var(arr._force(), axis=axis, ddof=ddof, **kwargs)
+    if kwargs:
+        return _backend.fallback.var(arr._force(), axis=axis, ddof=ddof, keepdims=keepdims,
+                                     **kwargs)
+    centre = mean(arr, axis=axis, keepdims=True)
+    dev = arr - centre
+    total = _reduce(np.add, dev * dev, axis=axis, keepdims=keepdims)
+    total = total if isinstance(total, DelayArray) else NPArray(total)
+    count = arr.size // total.size if total.size else 0
+    return total / (count - ddof)
 
 
 transpose = implements(np.transpose)(cast(_eager("transpose")))

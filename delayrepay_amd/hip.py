@@ -544,6 +544,51 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
     return low
 
 
+def _lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op):
+    """Kernel choice for reducing over `axes` of the (broadcast) `shape`."""
+    kept = [d for d in range(len(shape)) if d not in axes]
+    full = [_broadcast_strides(a, shape) for a in leaves]
+    kshape = [shape[d] for d in kept]
+    rshape = [shape[d] for d in axes]
+    kmerged, ksets = _merge_dims(kshape, [[s[d] for d in kept] for s in full])
+    rmerged, rsets = _merge_dims(rshape, [[s[d] for d in axes] for s in full])
+    if not kmerged:
+        kmerged, ksets = [1], [[0] for _ in leaves]
+    if not rmerged:
+        rmerged, rsets = [1], [[0] for _ in leaves]
+    K = R = 1
+    for d in kmerged:
+        K *= d
+    for d in rmerged:
+        R *= d
+    # coalescing decides the strategy: which side holds the unit-stride dimension
+    inner_kept = any(s[-1] == 1 for s in ksets)
+    inner_red = any(s[-1] == 1 for s in rsets)
+    strategy = "col" if (inner_kept and not inner_red) or R < 64 else "row"
+    low = Lowered()
+    low.lds = 0
+    low.fin_count = 0
+    low.kind = "axis"
+    kdim, rdim = len(kmerged), len(rmerged)
+    low.key = ("axis", prog.key(), kdim, rdim, acc, reduce_op, strategy)
+
+    def emit():
+        return cg.emit_axis_reduce(prog, kdim, rdim, acc, reduce_op, strategy)
+    low.emit = emit
+    if strategy == "col":
+        low.grid = max(1, min(-(-K // cg.BLOCK), _grid_cap()))
+    else:
+        low.grid = max(1, min(K, _grid_cap() * 4))
+    low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+               + "qq" + "q" * (kdim + rdim) + "q" * ((kdim + rdim) * len(leaves)))
+    tail = [K, R] + list(kmerged) + list(rmerged)
+    for ks, rs in zip(ksets, rsets):
+        tail += list(ks) + list(rs)
+    low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+    low.scal, low.tail = list(scalars), tail
+    return low
+
+
 class Replay:
     """Kernel launches recorded by `record()`: calling the object issues them again
     with the same arguments (same inputs, same outputs), without tracing, lowering
@@ -605,7 +650,7 @@ class Plan:
     launch.  `valid()` re-checks what could have changed underneath."""
 
     __slots__ = ("low", "kern", "checks", "stamp", "shape", "out_dtypes", "acc", "leaves",
-                 "hazard", "region", "empty")
+                 "hazard", "region", "empty", "axes")
 
     def valid(self):
         if self.stamp != _STAMP:
@@ -657,7 +702,7 @@ def _fire(plan, out_ptrs, reduce_out=None):
 # evaluation entry points
 # ---------------------------------------------------------------------------
 
-def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False):
+def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False, axes=None):
     """Lower traced `roots` (list of (ref, code)) into a Plan.  `dst`: existing
     destination view (single root); `dry`: placeholders instead of device memory."""
     prog = tracer.program(roots)
@@ -671,12 +716,26 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False):
     plan.region = None
     plan.acc = None
     plan.empty = False
+    plan.axes = False
     if reduce_op:
         shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
         code = roots[0][1]
         plan.acc = "i8" if (reduce_op == "add" and code in ("i4", "u4", "u1", "b1")) else code
-        plan.shape = ()
         plan.out_dtypes = [code_dtype(plan.acc)]
+        if axes is not None:
+            plan.shape = tuple(d for k, d in enumerate(shape) if k not in axes)
+            plan.axes = True
+            if 0 in shape:
+                if reduce_op != "add" and 0 in [shape[k] for k in axes]:
+                    raise ValueError(f"zero-size array to reduction operation {reduce_op} "
+                                     "which has no identity")
+                plan.empty = True
+                plan.low = None
+                return plan
+            plan.low = _lower_axis_reduce(prog, leaves, tracer.scalars, shape, axes, plan.acc,
+                                          reduce_op)
+            return plan
+        plan.shape = ()
         if 0 in shape:
             if reduce_op != "add":
                 raise ValueError(f"zero-size array to reduction operation {reduce_op} "
@@ -723,7 +782,15 @@ def _contiguous(shape):
 
 def _launch_fresh(plan):
     """Allocate outputs for `plan` and launch it; returns the output arrays."""
-    if plan.acc is not None:
+    if plan.axes:
+        out = ndarray(plan.shape, plan.out_dtypes[0])
+        if plan.empty:
+            if out.size:
+                assign(out, 0)
+        else:
+            _fire(plan, [out.ptr])
+        outs = [out]
+    elif plan.acc is not None:
         out = ndarray((), plan.out_dtypes[0])
         if plan.empty:       # sum over nothing
             (hiprt.fill64 if out.itemsize == 8 else hiprt.fill32)(out.ptr, 0, 1)
@@ -761,7 +828,8 @@ def _run_unfused(ex, evaluated):
     tracer = Tracer(evaluated)
     if isinstance(ex, ReduceEx):
         root = tracer.visit(ex.children[0])
-        out = _launch_fresh(_make_plan(tracer, [root], reduce_op=ex.func.__name__))[0]
+        out = _launch_fresh(_make_plan(tracer, [root], reduce_op=ex.func.__name__,
+                                       axes=ex.axis))[0]
     else:
         root = tracer.visit(ex)
         out = _launch_fresh(_make_plan(tracer, [root]))[0]
@@ -782,7 +850,7 @@ def run(ex):
         tracer = Tracer()
         if type(ex) is _FE.ReduceEx:
             root = tracer.visit(ex.children[0])
-            plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__)
+            plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__, axes=ex.axis)
         else:
             root = _trace_root(tracer, ex)
             plan = _make_plan(tracer, [root])
@@ -981,7 +1049,7 @@ def lower_only(exs, dst=None):
     tracer = Tracer()
     if isinstance(exs[0], ReduceEx):
         root = tracer.visit(exs[0].children[0])
-        low = _make_plan(tracer, [root], reduce_op=exs[0].func.__name__).low
+        low = _make_plan(tracer, [root], reduce_op=exs[0].func.__name__, axes=exs[0].axis).low
     elif dst is not None:
         low = _plan_write(tracer, tracer.visit(exs[0]), dst).low
     else:
@@ -1080,10 +1148,8 @@ class _Fallback:
 
     @staticmethod
     def _reduce(arr, name, axis, keepdims):
-        from .delayarray import NPArray, ReduceEx
-        if axis is not None or keepdims:
-            raise NotImplementedError("axis reductions are not implemented on the device yet")
-        return run(ReduceEx(getattr(numpy, name), NPArray(arr)))
+        from .delayarray import NPArray, _reduce
+        return _reduce(getattr(numpy, name), NPArray(arr), axis=axis, keepdims=keepdims)
 
     @staticmethod
     def sum(arr, axis=None, keepdims=False):

@@ -485,3 +485,45 @@ def test_more_than_2_to_31_elements():
     strided = z[::3]                                  # > 2^31 / 3 elements through the nd kernel
     assert float(dr.max(strided * 1.0)) == 6.0 or float(dr.max(strided * 1.0)) == 4.0
     assert float(dr.sum((strided * 0.0 + 1.0).astype(np.float64))) == float(len(range(0, n, 3)))
+
+
+# ---- reductions along axes -------------------------------------------------------------------------
+
+@pytest.mark.parametrize("axis", [0, 1, 2, -1, (0, 1), (0, 2), (1, 2), (0, 1, 2)])
+def test_axis_reductions_match_numpy(axis):
+    rs = np.random.RandomState(12)
+    a = rs.standard_normal((37, 70, 129))
+    b = rs.standard_normal((70, 1)).astype(np.float32)
+    da, db = dr.array(a), dr.array(b)
+    got = dr.sum(da * db + 1.0, axis=axis)
+    ref = np.sum(a * b + 1.0, axis=axis)
+    got = np.asarray(got.get() if hasattr(got, "get") else got)
+    assert got.shape == ref.shape and got.dtype == ref.dtype
+    np.testing.assert_allclose(got, ref, rtol=1e-12, atol=1e-12)
+    mx = dr.max(da, axis=axis)
+    mx = np.asarray(mx.get() if hasattr(mx, "get") else mx)
+    assert np.array_equal(mx, np.max(a, axis=axis))
+    kd = dr.sum(da, axis=axis, keepdims=True)
+    assert kd.get().shape == np.sum(a, axis=axis, keepdims=True).shape
+
+
+def test_axis_mean_var_on_views_and_integers():
+    rs = np.random.RandomState(13)
+    a = rs.standard_normal((64, 300))
+    da = dr.array(a)
+    np.testing.assert_allclose(dr.mean(da, axis=0).get(), a.mean(axis=0), rtol=1e-12, atol=1e-15)
+    np.testing.assert_allclose(dr.mean(da, axis=1).get(), a.mean(axis=1), rtol=1e-12, atol=1e-15)
+    np.testing.assert_allclose(dr.var(da, axis=1).get(), a.var(axis=1), rtol=1e-11)
+    np.testing.assert_allclose(dr.var(da, axis=0, ddof=1).get(), a.var(axis=0, ddof=1), rtol=1e-11)
+    np.testing.assert_allclose(float(dr.var(da)), a.var(), rtol=1e-11)
+    t = da.T[5:200:3]                                   # strided, transposed view
+    np.testing.assert_allclose(dr.sum(t, axis=0).get(), a.T[5:200:3].sum(axis=0), rtol=1e-12)
+    np.testing.assert_allclose(dr.sum(t * 2.0, axis=1).get(), (a.T[5:200:3] * 2.0).sum(axis=1),
+                               rtol=1e-12)
+    i = rs.randint(-50, 50, (33, 17)).astype(np.int32)
+    s = dr.sum(dr.array(i), axis=0).get()
+    assert s.dtype == np.int64 and np.array_equal(s, i.sum(axis=0))
+    assert dr.mean(dr.array(i), axis=1).get().dtype == np.float64
+    np.testing.assert_allclose(dr.mean(dr.array(i), axis=1).get(), i.mean(axis=1), rtol=1e-14)
+    with pytest.raises(np.exceptions.AxisError):
+        dr.sum(da, axis=2)
