@@ -527,3 +527,31 @@ def test_axis_mean_var_on_views_and_integers():
     np.testing.assert_allclose(dr.mean(dr.array(i), axis=1).get(), i.mean(axis=1), rtol=1e-14)
     with pytest.raises(np.exceptions.AxisError):
         dr.sum(da, axis=2)
+
+
+# ---- every tunable code path gives the same bits ------------------------------------------------------
+
+TUNE_VARIANTS = [
+    {"unroll": 2}, {"unroll": 4, "flat_cap": 512}, {"red_unroll": 1, "red_blocks": 64},
+    {"ntl": 0, "nts": 0}, {"cache_mib": 0}, {"svec": 0}, {"lds": 0}, {"gpr": 32, "rpt": 4},
+    {"gpr": 128, "rpt": 1}, {"tw": 64, "th": 8, "svec": 0}, {"sntl": 1, "snts": 0},
+]
+
+
+@pytest.mark.parametrize("variant", TUNE_VARIANTS, ids=lambda v: ",".join(f"{k}={x}" for k, x in v.items()))
+def test_tunables_do_not_change_results(variant):
+    saved = dict(hip.TUNE)
+    hip.set_tune(**variant)
+    try:
+        inp = orc.make_inputs("horner", 70001)
+        assert bits_equal(horner_expr(inp["c"], dr.array(inp["x"])).get(),
+                          orc.horner(inp["c"], inp["x"]))
+        u0 = np.zeros((67, 301), np.float32)
+        u0[1:-1, 1:-1] = np.random.RandomState(7).uniform(0, 1, (65, 299))
+        assert bits_equal(jacobi_sweeps(dr.array(u0), 3).get(), orc.jacobi(u0, 3))
+        g = golden("configs_small.npz")
+        s = dr.sum((dr.array(g["sumsq_x"]) - dr.array(g["sumsq_y"])) ** 2 * dr.array(g["sumsq_w"]))
+        assert abs(float(s) - float(g["sumsq_s"])) <= 1e-13 * float(g["sumsq_s"])
+        bs_check("bs64", 5000)
+    finally:
+        hip.set_tune(**saved)
