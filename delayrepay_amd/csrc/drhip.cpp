@@ -33,6 +33,7 @@ thread_local std::string t_log;
 thread_local std::vector<char> t_code;
 
 bool g_init = false;
+bool g_capturing = false;
 int g_device = -1;
 hipStream_t g_stream = nullptr;
 hipDeviceProp_t g_prop;
@@ -129,6 +130,8 @@ int drhip_malloc(void** dptr, size_t nbytes) {
     g_pool.st.n_mallocs++;
     auto it = g_pool.free_lists.find(c);
     void* p = nullptr;
+    if (g_capturing && (it == g_pool.free_lists.end() || it->second.empty()))
+        return fail(DRHIP_EINVAL, "drhip_malloc", "would call hipMalloc while capturing a graph");
     if (it != g_pool.free_lists.end() && !it->second.empty()) {
         p = it->second.back();
         it->second.pop_back();
@@ -190,6 +193,7 @@ int drhip_pool_trim(void) {
 
 int drhip_memcpy_h2d(void* dst, const void* src, size_t n) {
     NEED_INIT();
+    if (g_capturing) return fail(DRHIP_EINVAL, "drhip_memcpy_h2d", "not allowed while capturing a graph");
     if (n == 0) return 0;
     HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, g_stream));
     // pageable source: the caller may reuse it as soon as we return
@@ -199,6 +203,7 @@ int drhip_memcpy_h2d(void* dst, const void* src, size_t n) {
 
 int drhip_memcpy_d2h(void* dst, const void* src, size_t n) {
     NEED_INIT();
+    if (g_capturing) return fail(DRHIP_EINVAL, "drhip_memcpy_d2h", "not allowed while capturing a graph");
     if (n == 0) return 0;
     HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, g_stream));
     HIP_TRY(hipStreamSynchronize(g_stream));
@@ -207,6 +212,7 @@ int drhip_memcpy_d2h(void* dst, const void* src, size_t n) {
 
 int drhip_memcpy_d2d(void* dst, const void* src, size_t n) {
     NEED_INIT();
+    if (g_capturing) return fail(DRHIP_EINVAL, "drhip_memcpy_d2d", "not allowed while capturing a graph");
     if (n == 0) return 0;
     HIP_TRY(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, g_stream));
     return 0;
@@ -363,10 +369,54 @@ int drhip_launch(void* func, unsigned grid_x, unsigned block_x, unsigned lds_byt
     return 0;
 }
 
+// ---- graphs ----------------------------------------------------------------
+
+int drhip_graph_begin(void) {
+    NEED_INIT();
+    if (g_capturing) return fail(DRHIP_EINVAL, "drhip_graph_begin", "a capture is already open");
+    HIP_TRY(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
+    g_capturing = true;
+    return 0;
+}
+
+int drhip_graph_end(void** graph_exec) {
+    NEED_INIT();
+    if (!g_capturing) return fail(DRHIP_EINVAL, "drhip_graph_end", "no capture is open");
+    g_capturing = false;
+    hipGraph_t graph = nullptr;
+    HIP_TRY(hipStreamEndCapture(g_stream, &graph));
+    if (!graph_exec) {
+        (void)hipGraphDestroy(graph);
+        return fail(DRHIP_EINVAL, "drhip_graph_end", "null out");
+    }
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail((int)e, "hipGraphInstantiate", hipGetErrorString(e));
+    *graph_exec = (void*)exec;
+    return 0;
+}
+
+int drhip_graph_launch(void* graph_exec) {
+    NEED_INIT();
+    if (!graph_exec) return fail(DRHIP_EINVAL, "drhip_graph_launch", "null graph");
+    HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, g_stream));
+    g_cnt.n_launches++;
+    return 0;
+}
+
+int drhip_graph_destroy(void* graph_exec) {
+    NEED_INIT();
+    if (!graph_exec) return 0;
+    HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    return 0;
+}
+
 // ---- sync / events ---------------------------------------------------------
 
 int drhip_sync(void) {
     NEED_INIT();
+    if (g_capturing) return fail(DRHIP_EINVAL, "drhip_sync", "not allowed while capturing a graph");
     HIP_TRY(hipStreamSynchronize(g_stream));
     return 0;
 }

@@ -599,10 +599,27 @@ class Replay:
         self.launches = []      # (function, grid, lds bytes, packed arguments)
         self.keep = []
         self._scratch = []
+        self._graph = None
 
     def __call__(self):
+        if self._graph is not None:
+            self._graph.launch()
+            return
         for func, grid, lds, args in self.launches:
             hiprt.launch(func, grid, cg.BLOCK, lds, args, len(args))
+
+    def as_graph(self):
+        """Capture the recorded launches into a HIP graph; later calls replay the
+        whole sequence with a single launch."""
+        if self._graph is None and self.launches:
+            hiprt.Graph.begin()
+            try:
+                for func, grid, lds, args in self.launches:
+                    hiprt.launch(func, grid, cg.BLOCK, lds, args, len(args))
+            finally:
+                graph = hiprt.Graph.end()
+            self._graph = graph
+        return self
 
     def __del__(self):
         for ptr in self._scratch:

@@ -82,6 +82,10 @@ _SIGNATURES = {
     "drhip_get_function": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]),
     "drhip_compile_log": (C.c_char_p, []),
     "drhip_launch": (C.c_int, [C.c_void_p, C.c_uint, C.c_uint, C.c_uint, C.c_void_p, C.c_size_t]),
+    "drhip_graph_begin": (C.c_int, []),
+    "drhip_graph_end": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "drhip_graph_launch": (C.c_int, [C.c_void_p]),
+    "drhip_graph_destroy": (C.c_int, [C.c_void_p]),
     "drhip_sync": (C.c_int, []),
     "drhip_event_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "drhip_event_destroy": (C.c_int, [C.c_void_p]),
@@ -244,6 +248,32 @@ def launch(func, grid, block, lds_bytes, argbuf, nbytes):
 
 def sync():
     _check(lib().drhip_sync())
+
+
+class Graph:
+    """Instantiated HIP graph of the launches issued inside `with Graph.capture()`."""
+
+    def __init__(self, handle):
+        self.h = handle
+
+    @staticmethod
+    def begin():
+        init()
+        _check(_lib.drhip_graph_begin())
+
+    @staticmethod
+    def end():
+        h = C.c_void_p()
+        _check(_lib.drhip_graph_end(C.byref(h)))
+        return Graph(h.value)
+
+    def launch(self):
+        _check(_lib.drhip_graph_launch(self.h))
+
+    def __del__(self):
+        if _lib is not None and self.h:
+            _lib.drhip_graph_destroy(self.h)
+            self.h = None
 
 
 class Event:

@@ -134,6 +134,18 @@ const char* drhip_compile_log(void);
 int drhip_launch(void* func, unsigned grid_x, unsigned block_x,
                  unsigned lds_bytes, const void* args, size_t args_bytes);
 
+/* ---- HIP graphs -----------------------------------------------------------
+ * Capture the launches issued between begin and end into a graph and replay
+ * them with one call: for launch-bound loops (small arrays, many sweeps).  The
+ * reference has no counterpart (it launches kernel by kernel, cuda.py:96).
+ * Between begin and end only drhip_launch, drhip_fill32/64 and
+ * drhip_copy_kernel may be called (no allocation, copy or synchronisation);
+ * captured kernels keep the device addresses they were recorded with. */
+int drhip_graph_begin(void);
+int drhip_graph_end(void** graph_exec);
+int drhip_graph_launch(void* graph_exec);
+int drhip_graph_destroy(void* graph_exec);
+
 /* ---- synchronisation and timing ---------------------------------------- */
 int drhip_sync(void);
 int drhip_event_create(void** ev);

@@ -118,3 +118,49 @@ def test_setitem_fill_copy_astype_reshape():
     assert float(dev[0, 3]) == 3.0 and dev[0, 3].item() == 3.0
     empty = ndarray((0, 4), np.float32)
     assert empty.get().shape == (0, 4)
+
+
+def test_recorded_launches_replay_as_a_hip_graph():
+    """A graph of recorded kernels must give the eager result on every replay, with
+    the program's own eager work and synchronisations in between."""
+    import delayrepay_amd as dr
+    from oracle import numpy_oracle as orc
+    rs = np.random.RandomState(21)
+    u0 = np.zeros((130, 258), np.float32)
+    u0[1:-1, 1:-1] = rs.uniform(0, 1, (128, 256))
+    x0 = rs.standard_normal(5000)
+    u = dr.array(u0)
+    x = dr.array(x0)
+
+    def sweep():
+        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+
+    sweep()
+    sweep()                                  # warm: shadow buffer exists, plan cached
+    with hip.record() as plan:
+        sweep()
+        sweep()                              # ping-pong pair: back in the same allocation
+        total = dr.sum(x * x)                # a reduction (two kernels) in the same graph
+    done = 4
+    assert len(plan.launches) == 4
+    expect_total = float(np.sum(x0 * x0))
+    assert abs(float(total) - expect_total) <= 1e-13 * expect_total
+    plan.as_graph()
+    for rep in range(4):
+        hiprt.fill64(total.ptr, 0, 1)        # eager work between replays
+        plan()
+        done += 2
+        hiprt.sync()
+        assert np.array_equal(u.get(), orc.jacobi(u0, done)), rep
+        assert abs(float(total) - expect_total) <= 1e-13 * expect_total
+        y = (x * 2.0).get()                  # unrelated eager kernel + copy
+        assert np.array_equal(y, x0 * 2.0)
+    # the library refuses what a capture cannot hold
+    hiprt.Graph.begin()
+    try:
+        with pytest.raises(hiprt.DrhipError):
+            hiprt.sync()
+        with pytest.raises(hiprt.DrhipError):
+            hiprt.memcpy_d2d(total.ptr, total.ptr, 8)
+    finally:
+        hiprt.Graph.end()
