@@ -26,6 +26,9 @@ extern "C" void drhip_k_launch_matmul(int is_double, const void* A, const void* 
                                       long N, long K, long lda, long ldb, long ldc,
                                       hipStream_t s);
 
+extern "C" int drhip_k_cumsum(int kind, void* temp, size_t* temp_bytes, const void* in, void* out,
+                              size_t n, hipStream_t s);
+
 namespace {
 
 thread_local std::string t_err;
@@ -264,6 +267,25 @@ int drhip_matmul(int is_double, const void* a, const void* b, void* c, int64_t m
     if ((m + 63) / 64 > 65535) return fail(DRHIP_EINVAL, "drhip_matmul", "too many rows");
     drhip_k_launch_matmul(is_double, a, b, c, m, n, k, lda, ldb, ldc, g_stream);
     HIP_TRY(hipGetLastError());
+    g_cnt.n_launches++;
+    return 0;
+}
+
+int drhip_cumsum(int kind, const void* in, void* out, size_t n) {
+    NEED_INIT();
+    if (kind < 0 || kind > 3) return fail(DRHIP_EINVAL, "drhip_cumsum", "kind must be 0..3");
+    if (n == 0) return 0;
+    if (!in || !out) return fail(DRHIP_EINVAL, "drhip_cumsum", "null operand");
+    if (n > (size_t)0x7fffffff) return fail(DRHIP_EINVAL, "drhip_cumsum", "more than 2^31-1 elements");
+    size_t bytes = 0;
+    int rc = drhip_k_cumsum(kind, nullptr, &bytes, in, out, n, g_stream);
+    if (rc) return fail(rc, "hipcub::DeviceScan (size query)", hipGetErrorString((hipError_t)rc));
+    void* temp = nullptr;
+    rc = drhip_malloc(&temp, bytes ? bytes : 1);
+    if (rc) return rc;
+    rc = drhip_k_cumsum(kind, temp, &bytes, in, out, n, g_stream);
+    drhip_free(temp);  // stream-ordered reuse
+    if (rc) return fail(rc, "hipcub::DeviceScan", hipGetErrorString((hipError_t)rc));
     g_cnt.n_launches++;
     return 0;
 }

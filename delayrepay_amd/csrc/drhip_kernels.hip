@@ -2,6 +2,7 @@
 // used as the measured ceiling of the memory system.  Generated expression
 // kernels are not here; they are emitted as source at run time.
 #include <hip/hip_runtime.h>
+#include <hipcub/hipcub.hpp>
 #include <stdint.h>
 
 namespace {
@@ -119,4 +120,23 @@ extern "C" void drhip_k_launch_matmul(int is_double, const void* A, const void* 
     else
         hipLaunchKernelGGL(matmul_kernel<float>, grid, dim3(kBlock), 0, s, (const float*)A,
                            (const float*)B, (float*)C, M, N, K, lda, ldb, ldc);
+}
+
+// Inclusive prefix sum of n elements (hipCUB device scan).  Two-phase protocol:
+// with temp == nullptr only *temp_bytes is set.
+template <typename T>
+static hipError_t scan_sum(void* temp, size_t* temp_bytes, const void* in, void* out, size_t n,
+                           hipStream_t s) {
+    return hipcub::DeviceScan::InclusiveSum(temp, *temp_bytes, (const T*)in, (T*)out, (int)n, s);
+}
+
+extern "C" int drhip_k_cumsum(int kind, void* temp, size_t* temp_bytes, const void* in, void* out,
+                              size_t n, hipStream_t s) {
+    switch (kind) {
+        case 0: return (int)scan_sum<float>(temp, temp_bytes, in, out, n, s);
+        case 1: return (int)scan_sum<double>(temp, temp_bytes, in, out, n, s);
+        case 2: return (int)scan_sum<int32_t>(temp, temp_bytes, in, out, n, s);
+        case 3: return (int)scan_sum<int64_t>(temp, temp_bytes, in, out, n, s);
+    }
+    return (int)hipErrorInvalidValue;
 }

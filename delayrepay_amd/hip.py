@@ -1207,6 +1207,125 @@ class _Fallback:
 
     matmul = dot
 
+    # -- routines the front end reaches through `fallback.<name>` (delayarray.py:511-568,615):
+    #    evaluated on the device through the lazy front end, returned as device arrays
+
+    @staticmethod
+    def _eager(fn, *args, **kwargs):
+        from . import delayarray as fe
+        wrapped = [fe.NPArray(a) if isinstance(a, ndarray) else a for a in args]
+        res = fn(*wrapped, **kwargs)
+        return res._force() if isinstance(res, fe.DelayArray) else res
+
+    @staticmethod
+    def mean(arr, axis=None, keepdims=False):
+        from . import delayarray as fe
+        return _Fallback._eager(fe.mean, arr, axis=axis, keepdims=keepdims)
+
+    @staticmethod
+    def var(arr, axis=None, ddof=0, keepdims=False):
+        from . import delayarray as fe
+        return _Fallback._eager(fe.var, arr, axis=axis, ddof=ddof, keepdims=keepdims)
+
+    @staticmethod
+    def average(arr, axis=None, weights=None):
+        from . import delayarray as fe
+        if weights is None:
+            return _Fallback.mean(arr, axis=axis)
+        a, w = fe.NPArray(_Fallback.asarray(arr)), fe.NPArray(_Fallback.asarray(weights))
+        num = fe._reduce(numpy.add, a * w, axis=axis)
+        den = fe._reduce(numpy.add, w if w.shape == a.shape else w + 0 * a, axis=axis)
+        num = num if isinstance(num, fe.DelayArray) else fe.NPArray(num)
+        den = den if isinstance(den, fe.DelayArray) else fe.NPArray(den)
+        return (num / den)._force()
+
+    @staticmethod
+    def maximum(a, b):
+        return _Fallback._eager(numpy.maximum, a, b)
+
+    @staticmethod
+    def minimum(a, b):
+        return _Fallback._eager(numpy.minimum, a, b)
+
+    @staticmethod
+    def greater(a, b):
+        return _Fallback._eager(numpy.greater, a, b)
+
+    @staticmethod
+    def less(a, b):
+        return _Fallback._eager(numpy.less, a, b)
+
+    @staticmethod
+    def repeat(arr, repeats, axis=None):
+        """Each element `repeats` times (an integer), as a broadcast view made dense."""
+        arr = _Fallback.asarray(arr)
+        if not isinstance(repeats, (int, numpy.integer)):
+            raise NotImplementedError("repeat with per-element counts is not implemented on the device")
+        if axis is None:
+            arr, axis = arr.reshape(arr.size), 0
+        axis %= max(arr.ndim, 1)
+        shape = arr.shape[:axis + 1] + (int(repeats),) + arr.shape[axis + 1:]
+        strides = arr._strides[:axis + 1] + (0,) + arr._strides[axis + 1:]
+        dense = materialise(ndarray(shape, arr.dtype, arr.buf, arr.offset, strides))
+        return dense.reshape(arr.shape[:axis] + (arr.shape[axis] * int(repeats),) + arr.shape[axis + 1:])
+
+    @staticmethod
+    def tile(arr, reps):
+        """The array repeated `reps` times along each axis."""
+        arr = _Fallback.asarray(arr)
+        reps = (reps,) if isinstance(reps, (int, numpy.integer)) else tuple(reps)
+        nd = max(arr.ndim, len(reps))
+        reps = (1,) * (nd - len(reps)) + tuple(int(r) for r in reps)
+        shape = (1,) * (nd - arr.ndim) + arr.shape
+        strides = (0,) * (nd - arr.ndim) + arr._strides
+        vshape, vstrides = [], []
+        for r, d, s in zip(reps, shape, strides):
+            vshape += [r, d]
+            vstrides += [0, s]
+        dense = materialise(ndarray(vshape, arr.dtype, arr.buf, arr.offset, vstrides))
+        return dense.reshape(tuple(r * d for r, d in zip(reps, shape)))
+
+    @staticmethod
+    def cumsum(arr, axis=None):
+        arr = _Fallback.asarray(arr)
+        if axis is not None and arr.ndim > 1:
+            raise NotImplementedError("cumsum along an axis of an N-d array is not implemented "
+                                      "on the device")
+        kinds = {"float32": 0, "float64": 1, "int32": 2, "int64": 3}
+        if arr.dtype.name not in kinds:
+            arr = arr.astype(numpy.int64 if arr.dtype.kind in "iub" else numpy.float64)
+        elif arr.dtype == numpy.int32:
+            arr = arr.astype(numpy.int64)           # NumPy accumulates small ints in int64
+        flat = arr.reshape(arr.size) if arr.is_contiguous else arr.copy().reshape(arr.size)
+        out = ndarray((arr.size,), flat.dtype)
+        hiprt.cumsum(kinds[flat.dtype.name], flat.ptr, out.ptr, arr.size)
+        return out
+
+    @staticmethod
+    def diag(arr, k=0):
+        arr = _Fallback.asarray(arr)
+        if arr.ndim == 2:
+            rows, cols = arr.shape
+            r0, c0 = (0, k) if k >= 0 else (-k, 0)
+            n = max(0, min(rows - r0, cols - c0))
+            view = ndarray((n,), arr.dtype, arr.buf,
+                           arr.offset + r0 * arr._strides[0] + c0 * arr._strides[1],
+                           (arr._strides[0] + arr._strides[1],))
+            return materialise(view)
+        if arr.ndim == 1:
+            n = arr.shape[0] + abs(k)
+            out = _Fallback.zeros((n, n), dtype=arr.dtype)
+            r0, c0 = (0, k) if k >= 0 else (-k, 0)
+            target = ndarray((arr.shape[0],), arr.dtype, out.buf, r0 * n + c0, (n + 1,))
+            assign(target, arr)
+            return out
+        raise ValueError("Input must be 1- or 2-d.")
+
+    @staticmethod
+    def diagflat(arr, k=0):
+        arr = _Fallback.asarray(arr)
+        return _Fallback.diag(arr.reshape(arr.size), k)
+
     @staticmethod
     def roll(arr, shift, axis=None):
         if axis is None:

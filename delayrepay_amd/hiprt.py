@@ -74,6 +74,7 @@ _SIGNATURES = {
     "drhip_fill64": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t]),
     "drhip_copy_kernel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint]),
     "drhip_matmul": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int64] * 6),
+    "drhip_cumsum": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]),
     "drhip_compile": (C.c_int, [C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_int,
                                 C.POINTER(C.c_void_p)]),
     "drhip_code_get": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]),
@@ -194,6 +195,10 @@ def copy_kernel(dst, src, nbytes, grid_blocks=0):
 
 def matmul(is_double, a, b, c, m, n, k, lda, ldb, ldc):
     _check(_lib.drhip_matmul(int(is_double), a, b, c, m, n, k, lda, ldb, ldc))
+
+
+def cumsum(kind, src, dst, n):
+    _check(_lib.drhip_cumsum(kind, src, dst, n))
 
 
 def _opts_array(opts):

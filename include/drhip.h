@@ -106,6 +106,11 @@ int drhip_copy_kernel(void* dst_dev, const void* src_dev, size_t nbytes,
 int drhip_matmul(int is_double, const void* a, const void* b, void* c, int64_t m, int64_t n,
                  int64_t k, int64_t lda, int64_t ldb, int64_t ldc);
 
+/* Inclusive prefix sum of n contiguous elements; kind 0 float, 1 double, 2 int32,
+ * 3 int64.  Replaces `_backend.fallback.cumsum` = cupy.cumsum (delayarray.py:558);
+ * eager, not part of the fused path. */
+int drhip_cumsum(int kind, const void* in_dev, void* out_dev, size_t n);
+
 /* ---- run-time compilation ----------------------------------------------
  * Replaces cupy.ElementwiseKernel(...) construction (cuda.py:35-43), i.e.
  * NVRTC + module load.  `src` is HIP C++ text holding one or more

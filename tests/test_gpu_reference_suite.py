@@ -189,3 +189,61 @@ class TestSurface:
         a = array(x)
         assert np.array_equal((a + x).get(), 2 * x)
         assert np.array_equal((x * a).get(), x * x)
+
+
+class TestEagerRoutines:
+    """Everything the front end reaches through `backend.fallback`
+    (delayarray.py:85,511-568,588,615) exists on the device backend."""
+
+    def setup_method(self):
+        rs = np.random.RandomState(30)
+        self.a0 = rs.standard_normal((12, 17))
+        self.a = array(self.a0)
+
+    def test_namespace_is_complete(self):
+        fb = dnp.backend.fallback
+        for name in ("dot var sum transpose roll max maximum average repeat cumsum greater less "
+                     "tile newaxis empty empty_like eye identity ones ones_like zeros zeros_like "
+                     "full full_like array asarray asanyarray ascontiguousarray copy arange "
+                     "linspace logspace tri").split():
+            assert hasattr(fb, name), name
+
+    def test_repeat_tile_cumsum_diag(self):
+        a0, a = self.a0, self.a
+        assert np.array_equal(np.repeat(a, 3).get(), np.repeat(a0, 3))
+        assert np.array_equal(np.repeat(a, 2, axis=0).get(), np.repeat(a0, 2, axis=0))
+        assert np.array_equal(np.repeat(a, 4, axis=1).get(), np.repeat(a0, 4, axis=1))
+        assert np.array_equal(a.repeat(2).get(), a0.repeat(2))
+        assert np.array_equal(np.tile(a, 3).get(), np.tile(a0, 3))
+        assert np.array_equal(np.tile(a, (2, 1, 3)).get(), np.tile(a0, (2, 1, 3)))
+        v0 = a0[3].copy()
+        npt.assert_allclose(np.cumsum(array(v0)).get(), np.cumsum(v0), rtol=1e-13)
+        npt.assert_allclose(np.cumsum(a).get(), np.cumsum(a0), rtol=1e-12, atol=1e-12)
+        i0 = np.arange(1, 5001, dtype=np.int32)
+        c = np.cumsum(array(i0)).get()
+        assert c.dtype == np.int64 and np.array_equal(c, np.cumsum(i0))
+        assert np.array_equal(np.diag(a).get(), np.diag(a0))
+        assert np.array_equal(np.diag(a, 2).get(), np.diag(a0, 2))
+        assert np.array_equal(np.diag(a, -3).get(), np.diag(a0, -3))
+        assert np.array_equal(np.diag(array(v0), 1).get(), np.diag(v0, 1))
+        assert np.array_equal(np.diagflat(array(a0[:2, :2].copy())).get(), np.diagflat(a0[:2, :2]))
+
+    def test_statistics_and_elementwise_fallbacks(self):
+        a0, a = self.a0, self.a
+        fb = dnp.backend.fallback
+        raw = a._force()
+        npt.assert_allclose(fb.var(raw).get(), a0.var(), rtol=1e-12)
+        npt.assert_allclose(fb.var(raw, axis=0).get(), a0.var(axis=0), rtol=1e-12)
+        npt.assert_allclose(fb.average(raw).get(), np.average(a0), rtol=1e-12)
+        w0 = np.random.RandomState(31).uniform(1, 2, a0.shape)
+        npt.assert_allclose(np.average(a, weights=array(w0)).get(), np.average(a0, weights=w0), rtol=1e-12)
+        npt.assert_allclose(np.average(a, axis=1, weights=array(w0)).get(),
+                            np.average(a0, axis=1, weights=w0), rtol=1e-12)
+        assert np.array_equal(fb.maximum(raw, 0.25).get(), np.maximum(a0, 0.25))
+        assert np.array_equal(fb.greater(raw, 0.0).get(), a0 > 0)
+        assert np.array_equal(fb.less(raw, raw.T.copy().T).get(), a0 < a0)
+        assert np.array_equal(fb.transpose(raw).get(), a0.T)
+        assert float(fb.max(raw)) == a0.max() and float(fb.sum(raw)) == pytest.approx(a0.sum(), rel=1e-13)
+        npt.assert_allclose(np.var(a), a0.var(), rtol=1e-12)
+        npt.assert_allclose(a.var(), a0.var(), rtol=1e-12)
+        npt.assert_allclose(float(a.sum()), a0.sum(), rtol=1e-13)
