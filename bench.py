@@ -171,6 +171,13 @@ def main():
             keep = step()
             if wl.get("pair"):
                 keep = step()
+        names_by_func = {}
+        for kern in hip._KERNELS.values():
+            nm = kern.source.split('extern "C" __global__')[-1].split("void ")[1].split("(")[0]
+            names_by_func[kern.func] = nm
+            if kern.finalize:
+                names_by_func[kern.finalize] = nm + "_fin"
+        kernel_names = sorted({names_by_func.get(f, "?") for f, _, _, _ in plan.launches})
         steps_per_replay = 2 if wl.get("pair") else 1
         reps = max(1, K // steps_per_replay)
         t_warm = time.perf_counter()
@@ -188,6 +195,7 @@ def main():
         del plan
         res = {
             "workload": wl["desc"], "dtype": wl["dtype"], "elements": wl["n"],
+            "kernel": kernel_names,
             "algorithmic_bytes": wl["nbytes"],
             "ms_per_step": round(ms_per_step, 5),
             "GBps": round(wl["nbytes"] / ms_per_step / 1e6, 1),
@@ -289,7 +297,7 @@ def main():
                    "device": info["name"] or info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": head["kernel_GBps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": head["roofline_frac"], "traffic": None,
-                     "kernel": "dr_kernel (generated, flat)", "kernel_us": head["kernel_us"],
+                     "kernel": head["kernel"][0], "kernel_us": head["kernel_us"],
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"]},
         "configs": results,
     }

@@ -322,17 +322,29 @@ def _load_or_compile(source):
     return module
 
 
+def _kernel_name(low):
+    """Symbol of the generated kernel: shape kind plus a digest of the cache key, so
+    that profilers list structurally different kernels separately."""
+    kind = low.kind + ("_reduce" if low.fin_count else "")
+    return f"dr_{kind}_{hashlib.sha1(repr(low.key).encode()).hexdigest()[:10]}"
+
+
+def _source(low):
+    name = _kernel_name(low)
+    return low.emit().replace("dr_finalize", name + "_fin").replace("dr_kernel", name), name
+
+
 def _kernel_for(low, with_finalize):
     kern = _KERNELS.get(low.key)
     if kern is not None:
         STATS["mem_hits"] += 1
         return kern
-    source = low.emit()
+    source, name = _source(low)
     module = _load_or_compile(source)
     kern = Kernel()
     kern.source = source
-    kern.func = hiprt.get_function(module, "dr_kernel")
-    kern.finalize = hiprt.get_function(module, "dr_finalize") if with_finalize else None
+    kern.func = hiprt.get_function(module, name)
+    kern.finalize = hiprt.get_function(module, name + "_fin") if with_finalize else None
     kern.packer = struct.Struct(low.fmt)
     _KERNELS[low.key] = kern
     return kern
@@ -1071,7 +1083,7 @@ def lower_only(exs, dst=None):
         low = _plan_write(tracer, tracer.visit(exs[0]), dst).low
     else:
         low = _make_plan(tracer, [tracer.visit(ex) for ex in exs]).low
-    return low, low.emit()
+    return low, _source(low)[0]
 
 
 def compile_source(source):

@@ -211,7 +211,8 @@ def test_contiguous_is_flat_and_vectorised():
 def test_misaligned_view_uses_scalar_flat_kernel():
     base = hip.placeholder((1 << 12,), np.float32)
     low, src = hip.lower_only(NPArray(base[1:]) * 2.0)
-    assert low.kind == "flat" and "f4x4* " not in src.split("dr_kernel")[1]
+    assert low.kind == "flat" and "f4x4*)" not in src.split('extern "C"')[1]
+    assert hip._kernel_name(low).startswith("dr_flat_") and hip._kernel_name(low) in src
 
 
 def test_broadcast_scalar_leaf_and_mixed_dtypes():
@@ -259,7 +260,8 @@ def test_reduction_lowers_to_fused_tail_with_finalize():
     x, y, w = (leaf((1 << 20,), np.float64) for _ in range(3))
     low, src = hip.lower_only(ReduceEx(np.add, (x - y) ** 2 * w))
     assert low.kind == "flat" and low.fin_count == low.grid
-    assert "__shfl_down" in src and "dr_finalize" in src and "atomic" not in src
+    assert "__shfl_down" in src and "_fin(" in src and "atomic" not in src
+    assert hip._kernel_name(low).startswith("dr_flat_reduce_")
     hip.compile_source(src)
     assert ReduceEx(np.add, leaf((8,), np.int32)).dtype == np.int32
     low, src = hip.lower_only(ReduceEx(np.add, leaf((1 << 12,), np.int32)))
