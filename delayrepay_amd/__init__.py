@@ -9,7 +9,7 @@ from . import backend as _be
 from .delayarray import *  # noqa: F401,F403
 from .delayarray import (DelayArray, NPArray, Scalar, NumpyEx, BinaryNumpyEx, BinaryFuncEx,  # noqa: F401
                          UnaryFuncEx, ReduceEx, CastEx, Memoiser, reset, evaluate, synchronize,
-                         sum, max, min, abs, mean, var, average)
+                         sum, max, min, abs, mean, var, average, where, clip, WhereEx)
 from . import random  # noqa: F401
 
 backend = _be.backend

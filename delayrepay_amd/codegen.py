@@ -88,9 +88,14 @@ _INFIX = {"add": "+", "subtract": "-", "multiply": "*", "divide": "/", "true_div
 _COMPARE = {"greater": ">", "less": "<", "greater_equal": ">=", "less_equal": "<=",
             "equal": "==", "not_equal": "!="}
 
+# results are bool; arithmetic happens in the operands' common type
+_PREDICATES = {"isnan", "isinf", "isfinite", "logical_not", "logical_and", "logical_or",
+               "logical_xor"}
+
 SUPPORTED_UFUNCS = (set(_FLOAT_FUNCS1) | set(_FLOAT_FUNCS2) | set(_INFIX) | set(_COMPARE)
+                    | _PREDICATES
                     | {"negative", "positive", "absolute", "fabs", "reciprocal", "maximum",
-                       "minimum", "square"})
+                       "minimum", "square", "sign"})
 
 
 def _fn(name, dt):
@@ -108,6 +113,26 @@ def op_expr(name, dt, args):
         return f"{args[0]} {_INFIX[name]} {args[1]}"
     if name in _COMPARE:
         return f"(unsigned char)({args[0]} {_COMPARE[name]} {args[1]})"
+    if name == "isnan":
+        return f"(unsigned char)({args[0]} != {args[0]})"
+    if name == "isinf":
+        return (f"(unsigned char)({_fn('fabs', dt)}({args[0]}) == __builtin_inf{'f' if dt == 'f4' else ''}())"
+                if is_float else "(unsigned char)0")
+    if name == "isfinite":
+        return (f"(unsigned char)({_fn('fabs', dt)}({args[0]}) < __builtin_inf{'f' if dt == 'f4' else ''}())"
+                if is_float else "(unsigned char)1")
+    if name == "logical_not":
+        return f"(unsigned char)({args[0]} == 0)"
+    if name == "logical_and":
+        return f"(unsigned char)(({args[0]} != 0) && ({args[1]} != 0))"
+    if name == "logical_or":
+        return f"(unsigned char)(({args[0]} != 0) || ({args[1]} != 0))"
+    if name == "logical_xor":
+        return f"(unsigned char)(({args[0]} != 0) != ({args[1]} != 0))"
+    if name == "sign":      # NaN stays NaN, as in NumPy
+        a = args[0]
+        body = f"({CTYPE[dt]})(({a} > 0) - ({a} < 0))"
+        return f"(({a} != {a}) ? {a} : {body})" if is_float else body
     if name == "negative":
         return f"-{args[0]}"
     if name == "positive":
@@ -185,6 +210,9 @@ def emit_body(prog, out_dtypes, fname="dr_body"):
         cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
         if name == "cast":
             expr = cargs[0]
+        elif name == "where":    # the condition keeps its own type
+            k, j = args[0]
+            expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
         else:
             expr = op_expr(name, cdt, cargs)
         lines.append(f"    const {CTYPE[rdt]} v{i} = {expr};")

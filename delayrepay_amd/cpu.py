@@ -30,6 +30,7 @@ class CpuVisitor(Visitor):
     visit_UnaryFuncEx = _apply
     visit_BinaryFuncEx = _apply
     visit_BinaryNumpyEx = _apply
+    visit_WhereEx = _apply
 
     def visit_CastEx(self, node):
         return self.visit(node.children[0]).astype(node.dtype)

@@ -602,6 +602,20 @@ class BinaryNumpyEx(NumpyEx, Funcable):
         return f"binex{self._count}"
 
 
+class WhereEx(NumpyEx):
+    """`where(cond, x, y)`: element-wise selection, fused like any other node."""
+
+    def __init__(self, func, cond, x, y):
+        super().__init__(children=[cond, x, y])
+        self.func = func
+        self.shape = calc_shape(calc_shape(cond.shape, x.shape), y.shape)
+        self.dtype = calc_type(np.add, [x, y])
+
+    @property
+    def name(self):
+        return f"where{self._count}"
+
+
 def pow_ex(func, left, right):
     """`x ** k` with a Python-int k >= 2 becomes k-1 left-associated multiplies
     (delayarray.py:316-324); k <= 1 returns x itself, as the reference does."""
@@ -808,6 +822,23 @@ def min(arr, axis=None, **kwargs):
     return _reduce(np.minimum, arr, axis=axis, **kwargs)
 
 
+@implements(np.where)
+def where(cond, x=None, y=None):
+    if x is None or y is None:
+        raise NotImplementedError("where(cond) without values (nonzero) is not supported")
+    return WhereEx(np.where, *(arg_to_numpy_ex(a) for a in (cond, x, y)))
+
+
+@implements(np.clip)
+def clip(arr, a_min=None, a_max=None, **kwargs):
+    out = arg_to_numpy_ex(arr)
+    if a_min is not None:
+        out = np.maximum(out, a_min)
+    if a_max is not None:
+        out = np.minimum(out, a_max)
+    return out
+
+
 @implements(np.mean)
 def mean(arr, axis=None, keepdims=False, **kwargs):
     arr = arg_to_numpy_ex(arr)
@@ -890,6 +921,13 @@ less = np.less
 floor = np.floor
 ceil = np.ceil
 hypot = np.hypot
+sign = np.sign
+isnan = np.isnan
+isinf = np.isinf
+isfinite = np.isfinite
+logical_and = np.logical_and
+logical_or = np.logical_or
+logical_not = np.logical_not
 newaxis = None
 
 try:  # `erf` is a SciPy ufunc; the name is what the code generator keys on

@@ -65,7 +65,8 @@ _FUSED = "DELAY_UNFUSED" not in os.environ
 STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0}
 
 _SCALAR_FMT = {"f4": "f", "f8": "d", "i4": "i", "i8": "q", "u4": "I", "u1": "B", "b1": "B"}
-_COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal")
+_COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal") \
+    + tuple(cg._PREDICATES)
 
 
 def set_fused(flag):
@@ -192,9 +193,12 @@ class Tracer:
             name = func.__name__
             result = _code_of(node.dtype)
             compute = result
-            if name in _COMPARES:
+            if name in _COMPARES:     # arithmetic in the operands' common type, bool out
+                descrs = tuple(_FE._descr(c) for c in node.children)
                 compute = dtype_code(_FE.result_dtype(
-                    numpy.add, tuple(_FE._descr(c) for c in node.children)))
+                    numpy.add if len(descrs) == 2 else numpy.positive, descrs))
+                if compute == "b1" and name not in cg._PREDICATES:
+                    compute = "u1"
             elif name not in cg.SUPPORTED_UFUNCS:
                 raise NotImplementedError(f"ufunc {name!r} cannot be fused by the HIP backend")
             refs = []
@@ -204,6 +208,17 @@ class Tracer:
                 else:
                     refs.append(self.visit(child)[0])
             self.ops.append((name, compute, result, tuple(refs)))
+            res = (("v", len(self.ops) - 1), result)
+        elif kind is _FE.WhereEx:
+            result = _code_of(node.dtype)
+            refs = []
+            for pos, child in enumerate(node.children):
+                if type(child) is _FE.Scalar:
+                    code = result if pos else dtype_code(numpy.asarray(child.val).dtype)
+                    refs.append(self.scalar(child.val, code, id(child))[0])
+                else:
+                    refs.append(self.visit(child)[0])
+            self.ops.append(("where", result, result, tuple(refs)))
             res = (("v", len(self.ops) - 1), result)
         elif kind is _FE.Scalar:
             res = self.scalar(node.val, dtype_code(numpy.asarray(node.val).dtype), nid)

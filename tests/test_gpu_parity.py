@@ -555,3 +555,30 @@ def test_tunables_do_not_change_results(variant):
         bs_check("bs64", 5000)
     finally:
         hip.set_tune(**saved)
+
+
+def test_where_clip_sign_and_predicates():
+    rs = np.random.RandomState(14)
+    a0 = rs.standard_normal(4099).astype(np.float32)
+    a0[::97] = np.nan
+    a0[5::131] = np.inf
+    a0[7::113] = -np.inf
+    a0[11::89] = 0.0
+    b0 = rs.standard_normal(4099).astype(np.float32)
+    a, b = dr.array(a0), dr.array(b0)
+    with np.errstate(all="ignore"):
+        assert bits_equal(np.where(a > b, a * 2.0, b).get(), np.where(a0 > b0, a0 * np.float32(2.0), b0))
+        assert bits_equal(np.where(a > 0, a, 0.0).get(), np.where(a0 > 0, a0, np.float32(0.0)))
+        assert bits_equal(np.where(np.isnan(a), b, a).get(), np.where(np.isnan(a0), b0, a0))
+        assert bits_equal(np.clip(a, -0.5, 0.75).get(), np.clip(a0, -0.5, 0.75))
+        assert bits_equal(np.sign(a).get(), np.sign(a0))
+        for fn in (np.isnan, np.isinf, np.isfinite, np.logical_not):
+            got = fn(a).get()
+            assert got.dtype == np.bool_ and np.array_equal(got, fn(a0)), fn.__name__
+        assert np.array_equal(np.logical_and(a > 0, b > 0).get(), np.logical_and(a0 > 0, b0 > 0))
+        assert np.array_equal(np.logical_or(a, b > 1).get(), np.logical_or(a0, b0 > 1))
+        cnt = dr.sum(a > b)
+        assert int(cnt) == int(np.sum(a0 > b0)) and cnt.dtype == np.int64
+    i0 = rs.randint(-3, 4, 1000)
+    assert np.array_equal(np.sign(dr.array(i0)).get(), np.sign(i0))
+    assert np.array_equal(np.where(dr.array(i0) > 0, dr.array(i0), -1).get(), np.where(i0 > 0, i0, -1))
