@@ -36,7 +36,7 @@ class CpuVisitor(Visitor):
         return self.visit(node.children[0]).astype(node.dtype)
 
     def visit_ReduceEx(self, node):
-        return node.func.reduce(self.visit(node.children[0]), axis=None)
+        return node.func.reduce(self.visit(node.children[0]), axis=node.axis)
 
 
 def run(ex):

@@ -760,9 +760,6 @@ def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **unused
         axis = tuple(sorted(norm))
         if len(axis) == ndim:
             axis = None
-    if not hasattr(_backend, "run_multi"):      # NumPy backend: plain library call
-        eager = {"add": "sum", "maximum": "max", "minimum": "min"}[func.__name__]
-        return getattr(_backend.fallback, eager)(arr._force(), axis=axis, keepdims=keepdims)
     res = ReduceEx(func, arr, axis)._force() if axis is not None else ReduceEx(func, arr)._force()
     if keepdims:
         full = tuple(1 if (axis is None or k in axis) else d for k, d in enumerate(arr.shape))
