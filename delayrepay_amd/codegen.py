@@ -598,7 +598,8 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
 
 
 def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_per_thread,
-                     phase_group, phase_out, restrict=True, nt_load=False, nt_store=False):
+                     phase_group, phase_out, restrict=True, nt_load=False, nt_store=False,
+                     xcd_bands=True):
     """Vectorised form of `emit_stencil` for the common aligned case: the halo
     group's row stride and every output's row stride are multiples of the 16-byte
     vector width, and group and outputs have the same element size.
@@ -647,7 +648,8 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
          "    const int nb = gridDim.x;",
          f"    const int xcd = blockIdx.x % {N_XCD};",
          f"    const int slot = blockIdx.x / {N_XCD};",
-         f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;",
+         (f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;" if xcd_bands
+          else "    const int t = blockIdx.x;"),
          "    const int ty = t / tiles_x;",
          "    const int tx = t - ty * tiles_x;",
          f"    const int r0 = ty * {TH};",

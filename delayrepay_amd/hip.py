@@ -54,6 +54,7 @@ TUNE = {
     "svec": 1,        # aligned stencils: 16-byte loads into LDS and 16-byte stores
     "gpr": 64,        # vectorised stencil: 16-byte column groups per tile row
     "rpt": 2,         # vectorised stencil: consecutive rows per thread
+    "xcd": 1,         # vectorised stencil: give each XCD a contiguous band of tiles
     "sntl": 0,        # vectorised stencil: non-temporal loads / stores
     "snts": 1,
 }
@@ -499,13 +500,15 @@ def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, r
             ph_o = (out_ptrs[0] // gsize) % vw
             gpr, rpt = TUNE["gpr"], TUNE["rpt"]
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
+            bands = bool(TUNE["xcd"])
             low.key = ("tile2dv", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o,
-                       gpr, rpt, sntl, snts)
+                       gpr, rpt, sntl, snts, bands)
             tw, th = gpr * vw, (cg.BLOCK // gpr) * rpt
 
             def emit():
                 return cg.emit_stencil_vec(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o,
-                                           restrict=not in_place, nt_load=sntl, nt_store=snts)[0]
+                                           restrict=not in_place, nt_load=sntl, nt_store=snts,
+                                           xcd_bands=bands)[0]
             W = W + ph_o          # tiles start `ph_o` columns left of the view
         else:
             low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune)
