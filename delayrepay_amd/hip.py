@@ -29,6 +29,8 @@ from . import codegen as cg
 from . import hiprt
 from .devarray import Buffer, ndarray, placeholder  # noqa: F401
 from .codegen import Program, dtype_code, code_dtype
+from .lowering import (TUNE, Lowered, broadcast_strides as _broadcast_strides, lower as _lower,
+                       lower_axis_reduce as _lower_axis_reduce)
 
 hiprt.lib()  # fail at import when libdrhip.so has not been built
 
@@ -38,34 +40,9 @@ COMPILE_OPTS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",  # no v_pk_*_f32
 ]
 
-# Tunables; part of every cache key.  DELAYREPAY_TUNE="unroll=2,bpc=16" overrides.
-TUNE = {
-    "unroll": 1,      # 16-byte vectors per thread and chunk in flat element-wise kernels
-    "red_unroll": 4,  # the same for flat kernels with a reduction tail
-    "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
-    "flat_cap": 0,    # most blocks of a flat element-wise kernel (0: one chunk per block)
-    "bpc": 8,         # resident blocks per CU that bound the grid of `nd` kernels
-    "ntl": 1,         # non-temporal loads  } for working sets beyond `cache_mib`;
-    "nts": 1,         # non-temporal stores } smaller ones stay cacheable
-    "cache_mib": 200,  # working sets up to this size are left to the 256 MB Infinity Cache
-    "tw": 128,        # stencil tile width (elements)
-    "th": 16,         # stencil tile height (rows)
-    "lds": 1,         # stage shifted views through LDS (0: read them directly)
-    "svec": 1,        # aligned stencils: 16-byte loads into LDS and 16-byte stores
-    "gpr": 64,        # vectorised stencil: 16-byte column groups per tile row
-    "rpt": 2,         # vectorised stencil: consecutive rows per thread
-    "xcd": 1,         # vectorised stencil: give each XCD a contiguous band of tiles
-    "sntl": 0,        # vectorised stencil: non-temporal loads / stores
-    "snts": 1,
-}
-for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
-    _k, _v = _kv.split("=")
-    TUNE[_k.strip()] = int(_v)
-
 _FUSED = "DELAY_UNFUSED" not in os.environ
 STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0}
 
-_SCALAR_FMT = {"f4": "f", "f8": "d", "i4": "i", "i8": "q", "u4": "I", "u1": "B", "b1": "B"}
 _COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal") \
     + tuple(cg._PREDICATES)
 
@@ -245,51 +222,6 @@ class Tracer:
 
 
 # ---------------------------------------------------------------------------
-# layout analysis
-# ---------------------------------------------------------------------------
-
-def _broadcast_strides(arr, shape):
-    """Element strides of `arr` viewed at `shape` (NumPy broadcasting)."""
-    nd = len(shape)
-    pad = nd - len(arr.shape)
-    if pad < 0:
-        raise ValueError(f"operand of shape {arr.shape} does not broadcast to {shape}")
-    out = [0] * nd
-    for k in range(len(arr.shape)):
-        d = arr.shape[k]
-        if d == shape[pad + k]:
-            out[pad + k] = arr._strides[k] if d != 1 else 0
-        elif d == 1:
-            out[pad + k] = 0
-        else:
-            raise ValueError(f"operand of shape {arr.shape} does not broadcast to {shape}")
-    return out
-
-
-def _merge_dims(shape, stride_sets):
-    """Drop unit dims and merge neighbours that every operand walks contiguously."""
-    dims = [(d, [s[k] for s in stride_sets]) for k, d in enumerate(shape) if d != 1]
-    if not dims:
-        return [], [[] for _ in stride_sets]
-    merged = [dims[0]]
-    for d, strides in dims[1:]:
-        pd, ps = merged[-1]
-        if all(p == s * d for p, s in zip(ps, strides)):
-            merged[-1] = (pd * d, strides)
-        else:
-            merged.append((d, strides))
-    mshape = [d for d, _ in merged]
-    msets = [[st[i] for _, st in merged] for i in range(len(stride_sets))]
-    return mshape, msets
-
-
-class Lowered:
-    """A kernel choice for one evaluation: cache key, source builder, launch recipe."""
-
-    __slots__ = ("key", "kind", "emit", "fmt", "srcs", "scal", "tail", "grid", "fin_count", "lds")
-
-
-# ---------------------------------------------------------------------------
 # kernel cache
 # ---------------------------------------------------------------------------
 
@@ -364,259 +296,6 @@ def _kernel_for(low, with_finalize):
     kern.packer = struct.Struct(low.fmt)
     _KERNELS[low.key] = kern
     return kern
-
-
-# ---------------------------------------------------------------------------
-# lowering
-# ---------------------------------------------------------------------------
-
-_CUS = None
-
-
-def _grid_cap():
-    """Blocks that fill the device `bpc` deep (256 CUs assumed until a device is open)."""
-    global _CUS
-    if _CUS is None:
-        if not hiprt._initialised:
-            return 256 * TUNE["bpc"]
-        _CUS = hiprt.device_info()["compute_units"]
-    return _CUS * TUNE["bpc"]
-
-
-def _lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, reduce_op,
-           in_place=False):
-    """Pick the kernel shape.  `out_ptrs`/`out_strides` describe the destinations
-    (element strides at `out_shape`); for a reduction they are empty and the
-    partial-sums pointer is appended at launch."""
-    n = 1
-    for d in out_shape:
-        n *= d
-    leaf_strides = [_broadcast_strides(a, out_shape) for a in leaves]
-    mshape, msets = _merge_dims(out_shape, leaf_strides + list(out_strides))
-    m_leaf, m_out = msets[:len(leaves)], msets[len(leaves):]
-    ndim = len(mshape)
-    low = Lowered()
-    low.lds = 0
-    low.fin_count = 0
-    scal_fmt = "".join(_SCALAR_FMT[c] for c in prog.scalars)
-    scal_vals = list(scalars)
-    tune = tuple(sorted(TUNE.items()))
-
-    flat = ndim <= 1 and all(s == [1] or s == [0] or s == [] for s in m_leaf) \
-        and all(s == [1] or s == [] for s in m_out)
-    if flat:
-        leaf_class = tuple("b" if (s == [0] and n > 1) else "c" for s in m_leaf)
-        ptrs = [a.ptr for a in leaves]
-        widths_ok = all(cg.ITEMSIZE[c] in (4, 8) for c, k in zip(prog.leaves, leaf_class) if k == "c")
-        align_ok = all(p % 16 == 0 for p, k in zip(ptrs, leaf_class) if k == "c")
-        if not reduce_op:
-            widths_ok = widths_ok and all(cg.ITEMSIZE[c] in (4, 8) for c in out_codes)
-            align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
-        vec = widths_ok and align_ok and n >= 64
-        unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
-        footprint = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
-        if not reduce_op:
-            footprint += sum(n * cg.ITEMSIZE[c] for c in out_codes)
-        streaming = footprint > TUNE["cache_mib"] << 20
-        ntl = bool(TUNE["ntl"]) and streaming
-        nts = bool(TUNE["nts"]) and streaming
-        low.kind = "flat"
-        low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
-                   unroll, ntl, nts)
-
-        def emit():
-            src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
-                                  restrict=not in_place, reduce_op=reduce_op)
-            return src
-        low.emit = emit
-        if vec:
-            widths = [cg.ITEMSIZE[c] for c, k in zip(prog.leaves, leaf_class) if k == "c"]
-            if not reduce_op:
-                widths += [cg.ITEMSIZE[c] for c in out_codes]
-            E = 16 // min(widths) if widths else 4
-        else:
-            E = 1
-        chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
-        cap = TUNE["red_blocks"] if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
-        low.grid = min(chunks, cap)
-        n_out_ptr = 1 if reduce_op else len(out_ptrs)
-        low.fmt = "@" + "P" * (len(ptrs) + n_out_ptr) + scal_fmt + "q"
-        low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
-        low.scal, low.tail = scal_vals, [n]
-        if reduce_op:
-            low.fin_count = low.grid
-        return low
-
-    tiled = (not reduce_op and ndim == 2 and all(s[1] == 1 for s in m_out)
-             and all(s[1] == 1 or s == [0, 0] for s in m_leaf))
-    if tiled:
-        H, W = mshape
-        tw, th = TUNE["tw"], TUNE["th"]
-        # halo group: >= 2 leaves that are shifted views of one buffer
-        groups = {}
-        for i, (a, s) in enumerate(zip(leaves, m_leaf)):
-            if s[1] == 1 and s[0] > 0:
-                groups.setdefault((id(a.buf), s[0], prog.leaves[i]), []).append(i)
-        best = max(groups.values(), key=len) if groups else []
-        kinds = [None] * len(leaves)
-        group = None
-        if len(best) >= 2 and TUNE["lds"]:
-            rs = m_leaf[best[0]][0]
-            ref_off = min(leaves[i].offset for i in best)
-            shifts = {}
-            for i in best:
-                d = leaves[i].offset - ref_off
-                dy, dx = divmod(d, rs)
-                if dx > rs // 2:
-                    dy, dx = dy + 1, dx - rs
-                shifts[i] = (dy, dx)
-            dy_max = max(dy for dy, _ in shifts.values())
-            dx_min = min(dx for _, dx in shifts.values())
-            dx_max = max(dx for _, dx in shifts.values())
-            itemsize = cg.ITEMSIZE[prog.leaves[best[0]]]
-            lds_bytes = (th + dy_max) * (tw + dx_max - dx_min) * itemsize
-            if dy_max <= 16 and dx_max - dx_min <= 32 and lds_bytes <= 48 * 1024:
-                group = (prog.leaves[best[0]], dy_max, dx_min, dx_max)
-                for i in best:
-                    kinds[i] = ("g",) + shifts[i]
-                g_buf = leaves[best[0]].buf
-                g_ptr = g_buf.ptr + ref_off * itemsize
-                g_src = (g_buf, ref_off * itemsize)
-                g_args = [rs, -ref_off, g_buf.nbytes // itemsize - ref_off]
-        for i, s in enumerate(m_leaf):
-            if kinds[i] is None:
-                kinds[i] = ("b",) if s == [0, 0] else ("d",)
-        kinds = tuple(kinds)
-        low.kind = "tile2d"
-        vec_ok = False
-        if group is not None and TUNE["svec"]:
-            gsize = cg.ITEMSIZE[group[0]]
-            vw = 16 // gsize
-            vec_ok = (gsize in (4, 8) and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
-                      and g_args[0] % vw == 0 and all(s[0] % vw == 0 for s in m_out)
-                      and len({(p // gsize) % vw for p in out_ptrs}) == 1)
-        if vec_ok:
-            ph_g = (g_ptr // gsize) % vw
-            ph_o = (out_ptrs[0] // gsize) % vw
-            gpr, rpt = TUNE["gpr"], TUNE["rpt"]
-            sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
-            bands = bool(TUNE["xcd"])
-            low.key = ("tile2dv", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o,
-                       gpr, rpt, sntl, snts, bands)
-            tw, th = gpr * vw, (cg.BLOCK // gpr) * rpt
-
-            def emit():
-                return cg.emit_stencil_vec(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o,
-                                           restrict=not in_place, nt_load=sntl, nt_store=snts,
-                                           xcd_bands=bands)[0]
-            W = W + ph_o          # tiles start `ph_o` columns left of the view
-        else:
-            low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune)
-
-            def emit():
-                return cg.emit_stencil(prog, kinds, group, out_codes, tw, th,
-                                       restrict=not in_place)
-        low.emit = emit
-        tiles_x = -(-W // tw)
-        tiles_y = -(-H // th)
-        low.grid = tiles_x * tiles_y
-        srcs = [(a.buf, a.offset * a.dtype.itemsize) for a, k in zip(leaves, kinds) if k[0] != "g"]
-        fmt = "@" + "P" * len(srcs)
-        tail_vals = []
-        if group is not None:
-            fmt += "P"
-            srcs.append(g_src)
-        fmt += "P" * len(out_ptrs) + scal_fmt + "ii"
-        tail_vals += [mshape[0], mshape[1]]
-        if group is not None:
-            fmt += "qqq"
-            tail_vals += g_args
-        fmt += "i"
-        tail_vals.append(tiles_x)
-        for k, s in zip(kinds, m_leaf):
-            if k[0] == "d":
-                fmt += "q"
-                tail_vals.append(s[0])
-        for s in m_out:
-            fmt += "q"
-            tail_vals.append(s[0])
-        low.fmt = fmt
-        low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
-        return low
-
-    # general strided kernel
-    if ndim == 0:
-        mshape, m_leaf, m_out, ndim = [1], [[0] for _ in m_leaf], [[0] for _ in m_out], 1
-    index32 = n < 2 ** 31
-    low.kind = "nd"
-    low.key = ("nd", prog.key(), ndim, tuple(out_codes), index32, reduce_op, tune)
-
-    def emit():
-        return cg.emit_nd(prog, ndim, out_codes, index32, reduce_op)
-    low.emit = emit
-    blocks = -(-n // cg.BLOCK)
-    low.grid = max(1, min(blocks, _grid_cap()))
-    n_out_ptr = 1 if reduce_op else len(out_ptrs)
-    fmt = "@" + "P" * (len(leaves) + n_out_ptr) + scal_fmt + "q" + ("I" if index32 else "q") * ndim
-    tail = [n] + list(mshape)
-    for s in m_leaf:
-        fmt += "q" * ndim
-        tail += s
-    if not reduce_op:
-        for s in m_out:
-            fmt += "q" * ndim
-            tail += s
-    low.fmt = fmt
-    low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
-    low.scal, low.tail = scal_vals, tail
-    if reduce_op:
-        low.fin_count = low.grid
-    return low
-
-
-def _lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op):
-    """Kernel choice for reducing over `axes` of the (broadcast) `shape`."""
-    kept = [d for d in range(len(shape)) if d not in axes]
-    full = [_broadcast_strides(a, shape) for a in leaves]
-    kshape = [shape[d] for d in kept]
-    rshape = [shape[d] for d in axes]
-    kmerged, ksets = _merge_dims(kshape, [[s[d] for d in kept] for s in full])
-    rmerged, rsets = _merge_dims(rshape, [[s[d] for d in axes] for s in full])
-    if not kmerged:
-        kmerged, ksets = [1], [[0] for _ in leaves]
-    if not rmerged:
-        rmerged, rsets = [1], [[0] for _ in leaves]
-    K = R = 1
-    for d in kmerged:
-        K *= d
-    for d in rmerged:
-        R *= d
-    # coalescing decides the strategy: which side holds the unit-stride dimension
-    inner_kept = any(s[-1] == 1 for s in ksets)
-    inner_red = any(s[-1] == 1 for s in rsets)
-    strategy = "col" if (inner_kept and not inner_red) or R < 64 else "row"
-    low = Lowered()
-    low.lds = 0
-    low.fin_count = 0
-    low.kind = "axis"
-    kdim, rdim = len(kmerged), len(rmerged)
-    low.key = ("axis", prog.key(), kdim, rdim, acc, reduce_op, strategy)
-
-    def emit():
-        return cg.emit_axis_reduce(prog, kdim, rdim, acc, reduce_op, strategy)
-    low.emit = emit
-    if strategy == "col":
-        low.grid = max(1, min(-(-K // cg.BLOCK), _grid_cap()))
-    else:
-        low.grid = max(1, min(K, _grid_cap() * 4))
-    low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
-               + "qq" + "q" * (kdim + rdim) + "q" * ((kdim + rdim) * len(leaves)))
-    tail = [K, R] + list(kmerged) + list(rmerged)
-    for ks, rs in zip(ksets, rsets):
-        tail += list(ks) + list(rs)
-    low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
-    low.scal, low.tail = list(scalars), tail
-    return low
 
 
 class Replay:
@@ -1109,296 +788,6 @@ def compile_source(source):
     return hiprt.compile_only(source, "dr_kernel.hip", COMPILE_OPTS)
 
 
-# ---------------------------------------------------------------------------
-# `np` and `fallback` namespaces of the backend protocol
-# ---------------------------------------------------------------------------
-
-def _upload(fn):
-    def wrapper(*args, **kwargs):
-        args = [a.get() if isinstance(a, ndarray) else a for a in args]
-        return ndarray.from_host(fn(*args, **kwargs))
-    wrapper.__name__ = fn.__name__
-    return wrapper
-
-
-def _filled(value_of):
-    def make(shape, *args, dtype=None, **kwargs):
-        value, default = value_of(args)
-        if dtype is None:
-            dtype = default
-        if isinstance(shape, (int, numpy.integer)):
-            shape = (int(shape),)
-        out = ndarray(tuple(shape), dtype)
-        if value is not None and out.size:
-            assign(out, value)
-        return out
-    return make
-
-
-def _like(maker):
-    def make(proto, *args, dtype=None, **kwargs):
-        proto = proto._force() if hasattr(proto, "_force") else proto
-        return maker(proto.shape, *args, dtype=dtype or proto.dtype)
-    return make
-
-
-class _Random:
-    """Host NumPy generators, uploaded (input generation; cf. delayrepay/random.py)."""
-
-    def __getattr__(self, name):
-        fn = getattr(numpy.random, name)
-        if name in ("seed", "get_state", "set_state"):
-            return fn
-        return _upload(fn)
-
-
-class _Fallback:
-    """Eager routines on device arrays (the reference uses `cupy` here, cuda.py:22).
-    Reductions and copies run as generated kernels; creation routines build on the
-    host and upload; what has no device implementation raises."""
-
-    newaxis = None
-    pi = numpy.pi
-
-    empty = staticmethod(_filled(lambda a: (None, numpy.float64)))
-    zeros = staticmethod(_filled(lambda a: (0, numpy.float64)))
-    ones = staticmethod(_filled(lambda a: (1, numpy.float64)))
-    full = staticmethod(_filled(lambda a: (a[0], numpy.asarray(a[0]).dtype)))
-    empty_like = staticmethod(_like(empty.__func__))
-    zeros_like = staticmethod(_like(zeros.__func__))
-    ones_like = staticmethod(_like(ones.__func__))
-    full_like = staticmethod(_like(full.__func__))
-
-    @staticmethod
-    def asarray(obj, dtype=None, **kwargs):
-        if hasattr(obj, "_force"):
-            obj = obj._force()
-        if isinstance(obj, ndarray):
-            return obj if dtype is None or numpy.dtype(dtype) == obj.dtype else obj.astype(dtype)
-        return ndarray.from_host(numpy.asarray(obj, dtype=dtype))
-
-    array = asarray
-    asanyarray = asarray
-
-    @staticmethod
-    def ascontiguousarray(obj, dtype=None):
-        arr = _Fallback.asarray(obj, dtype)
-        return arr if arr.is_contiguous else arr.copy()
-
-    @staticmethod
-    def copy(obj):
-        return _Fallback.asarray(obj).copy()
-
-    @staticmethod
-    def transpose(arr, axes=None):
-        return arr.transpose(axes) if axes is not None else arr.transpose()
-
-    @staticmethod
-    def _reduce(arr, name, axis, keepdims):
-        from .delayarray import NPArray, _reduce
-        return _reduce(getattr(numpy, name), NPArray(arr), axis=axis, keepdims=keepdims)
-
-    @staticmethod
-    def sum(arr, axis=None, keepdims=False):
-        return _Fallback._reduce(arr, "add", axis, keepdims)
-
-    @staticmethod
-    def max(arr, axis=None, keepdims=False):
-        return _Fallback._reduce(arr, "maximum", axis, keepdims)
-
-    @staticmethod
-    def min(arr, axis=None, keepdims=False):
-        return _Fallback._reduce(arr, "minimum", axis, keepdims)
-
-    @staticmethod
-    def dot(a, b):
-        """Matrix products on the device (vector.vector is fused by the front end)."""
-        a, b = _Fallback.asarray(a), _Fallback.asarray(b)
-        dt = numpy.result_type(a.dtype, b.dtype)
-        if dt.kind != "f":
-            dt = numpy.dtype(numpy.float64)
-        a = _Fallback.ascontiguousarray(a, dt)
-        b = _Fallback.ascontiguousarray(b, dt)
-        if a.ndim == 1 and b.ndim == 1:
-            return run_reduce_product(a, b)
-        a2 = a.reshape(1, -1) if a.ndim == 1 else a
-        b2 = b.reshape(-1, 1) if b.ndim == 1 else b
-        if a2.ndim != 2 or b2.ndim != 2 or a2.shape[1] != b2.shape[0]:
-            raise ValueError(f"shapes {a.shape} and {b.shape} not aligned")
-        m, k = a2.shape
-        n = b2.shape[1]
-        out = ndarray((m, n), dt)
-        hiprt.matmul(dt.itemsize == 8, a2.ptr, b2.ptr, out.ptr, m, n, k, k, n, n)
-        if a.ndim == 1:
-            return out.reshape(n)
-        if b.ndim == 1:
-            return out.reshape(m)
-        return out
-
-    matmul = dot
-
-    # -- routines the front end reaches through `fallback.<name>` (delayarray.py:511-568,615):
-    #    evaluated on the device through the lazy front end, returned as device arrays
-
-    @staticmethod
-    def _eager(fn, *args, **kwargs):
-        from . import delayarray as fe
-        wrapped = [fe.NPArray(a) if isinstance(a, ndarray) else a for a in args]
-        res = fn(*wrapped, **kwargs)
-        return res._force() if isinstance(res, fe.DelayArray) else res
-
-    @staticmethod
-    def mean(arr, axis=None, keepdims=False):
-        from . import delayarray as fe
-        return _Fallback._eager(fe.mean, arr, axis=axis, keepdims=keepdims)
-
-    @staticmethod
-    def var(arr, axis=None, ddof=0, keepdims=False):
-        from . import delayarray as fe
-        return _Fallback._eager(fe.var, arr, axis=axis, ddof=ddof, keepdims=keepdims)
-
-    @staticmethod
-    def average(arr, axis=None, weights=None):
-        from . import delayarray as fe
-        if weights is None:
-            return _Fallback.mean(arr, axis=axis)
-        a, w = fe.NPArray(_Fallback.asarray(arr)), fe.NPArray(_Fallback.asarray(weights))
-        num = fe._reduce(numpy.add, a * w, axis=axis)
-        den = fe._reduce(numpy.add, w if w.shape == a.shape else w + 0 * a, axis=axis)
-        num = num if isinstance(num, fe.DelayArray) else fe.NPArray(num)
-        den = den if isinstance(den, fe.DelayArray) else fe.NPArray(den)
-        return (num / den)._force()
-
-    @staticmethod
-    def maximum(a, b):
-        return _Fallback._eager(numpy.maximum, a, b)
-
-    @staticmethod
-    def minimum(a, b):
-        return _Fallback._eager(numpy.minimum, a, b)
-
-    @staticmethod
-    def greater(a, b):
-        return _Fallback._eager(numpy.greater, a, b)
-
-    @staticmethod
-    def less(a, b):
-        return _Fallback._eager(numpy.less, a, b)
-
-    @staticmethod
-    def repeat(arr, repeats, axis=None):
-        """Each element `repeats` times (an integer), as a broadcast view made dense."""
-        arr = _Fallback.asarray(arr)
-        if not isinstance(repeats, (int, numpy.integer)):
-            raise NotImplementedError("repeat with per-element counts is not implemented on the device")
-        if axis is None:
-            arr, axis = arr.reshape(arr.size), 0
-        axis %= max(arr.ndim, 1)
-        shape = arr.shape[:axis + 1] + (int(repeats),) + arr.shape[axis + 1:]
-        strides = arr._strides[:axis + 1] + (0,) + arr._strides[axis + 1:]
-        dense = materialise(ndarray(shape, arr.dtype, arr.buf, arr.offset, strides))
-        return dense.reshape(arr.shape[:axis] + (arr.shape[axis] * int(repeats),) + arr.shape[axis + 1:])
-
-    @staticmethod
-    def tile(arr, reps):
-        """The array repeated `reps` times along each axis."""
-        arr = _Fallback.asarray(arr)
-        reps = (reps,) if isinstance(reps, (int, numpy.integer)) else tuple(reps)
-        nd = max(arr.ndim, len(reps))
-        reps = (1,) * (nd - len(reps)) + tuple(int(r) for r in reps)
-        shape = (1,) * (nd - arr.ndim) + arr.shape
-        strides = (0,) * (nd - arr.ndim) + arr._strides
-        vshape, vstrides = [], []
-        for r, d, s in zip(reps, shape, strides):
-            vshape += [r, d]
-            vstrides += [0, s]
-        dense = materialise(ndarray(vshape, arr.dtype, arr.buf, arr.offset, vstrides))
-        return dense.reshape(tuple(r * d for r, d in zip(reps, shape)))
-
-    @staticmethod
-    def cumsum(arr, axis=None):
-        arr = _Fallback.asarray(arr)
-        if axis is not None and arr.ndim > 1:
-            raise NotImplementedError("cumsum along an axis of an N-d array is not implemented "
-                                      "on the device")
-        kinds = {"float32": 0, "float64": 1, "int32": 2, "int64": 3}
-        if arr.dtype.name not in kinds:
-            arr = arr.astype(numpy.int64 if arr.dtype.kind in "iub" else numpy.float64)
-        elif arr.dtype == numpy.int32:
-            arr = arr.astype(numpy.int64)           # NumPy accumulates small ints in int64
-        flat = arr.reshape(arr.size) if arr.is_contiguous else arr.copy().reshape(arr.size)
-        out = ndarray((arr.size,), flat.dtype)
-        hiprt.cumsum(kinds[flat.dtype.name], flat.ptr, out.ptr, arr.size)
-        return out
-
-    @staticmethod
-    def diag(arr, k=0):
-        arr = _Fallback.asarray(arr)
-        if arr.ndim == 2:
-            rows, cols = arr.shape
-            r0, c0 = (0, k) if k >= 0 else (-k, 0)
-            n = max(0, min(rows - r0, cols - c0))
-            view = ndarray((n,), arr.dtype, arr.buf,
-                           arr.offset + r0 * arr._strides[0] + c0 * arr._strides[1],
-                           (arr._strides[0] + arr._strides[1],))
-            return materialise(view)
-        if arr.ndim == 1:
-            n = arr.shape[0] + abs(k)
-            out = _Fallback.zeros((n, n), dtype=arr.dtype)
-            r0, c0 = (0, k) if k >= 0 else (-k, 0)
-            target = ndarray((arr.shape[0],), arr.dtype, out.buf, r0 * n + c0, (n + 1,))
-            assign(target, arr)
-            return out
-        raise ValueError("Input must be 1- or 2-d.")
-
-    @staticmethod
-    def diagflat(arr, k=0):
-        arr = _Fallback.asarray(arr)
-        return _Fallback.diag(arr.reshape(arr.size), k)
-
-    @staticmethod
-    def roll(arr, shift, axis=None):
-        if axis is None:
-            flat = arr.reshape(arr.size)
-            return _Fallback.roll(flat, shift, 0).reshape(arr.shape)
-        n = arr.shape[axis]
-        out = ndarray(arr.shape, arr.dtype)
-        if n == 0:
-            return out
-        shift %= n
-        head = [slice(None)] * arr.ndim
-        tail = [slice(None)] * arr.ndim
-        head[axis], tail[axis] = slice(shift, None), slice(0, n - shift)
-        assign(out[tuple(head)], arr[tuple(tail)])
-        if shift:
-            head[axis], tail[axis] = slice(0, shift), slice(n - shift, None)
-            assign(out[tuple(head)], arr[tuple(tail)])
-        return out
-
-    def __getattr__(self, name):
-        fn = getattr(numpy, name, None)
-        if name in ("eye", "identity", "arange", "linspace", "logspace", "geomspace", "tri",
-                    "frombuffer", "fromfile", "fromfunction", "fromiter", "fromstring",
-                    "loadtxt", "vander"):
-            return _upload(fn)
-        raise AttributeError(f"{name} has no device implementation in the HIP backend")
-
-
-class _Np:
-    """The slice of the array namespace the front end reads from `backend.np`
-    (delayarray.py:188-194, __init__.py:17, random.py:6-13)."""
-
-    pi = numpy.pi
-    random = _Random()
-    add = numpy.add
-    subtract = numpy.subtract
-    multiply = numpy.multiply
-    true_divide = numpy.true_divide
-    divide = numpy.divide
-    matmul = numpy.matmul
-
-
-np = _Np()
-fallback = _Fallback()
-
-sys.modules[__name__].np = np
+# the `np` and `fallback` namespaces of the backend protocol live in arrayns.py (it
+# imports this module, hence the late import)
+from .arrayns import fallback, np  # noqa: E402,F401

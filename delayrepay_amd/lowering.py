@@ -1,0 +1,336 @@
+"""Layout analysis and kernel choice of the HIP backend.
+
+Given a traced `Program` and the geometry of its operands, decide which kernel
+shape evaluates it (`flat`, `tile2d`/`tile2dv`, `nd`, `axis`), build the cache key
+(program + layout classes + dtypes + the tunables that shape the source), and
+prepare the launch recipe: grid, argument-block format, pointer sources and the
+constant tail of the argument block.  The reference has no counterpart: CuPy's
+ElementwiseKernel does its own (contiguous-or-generic) indexing (cuda.py:35-43).
+"""
+import os
+
+from . import codegen as cg
+from . import hiprt
+
+# Tunables; part of every cache key.  DELAYREPAY_TUNE="unroll=2,bpc=16" overrides.
+TUNE = {
+    "unroll": 1,      # 16-byte vectors per thread and chunk in flat element-wise kernels
+    "red_unroll": 4,  # the same for flat kernels with a reduction tail
+    "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
+    "flat_cap": 0,    # most blocks of a flat element-wise kernel (0: one chunk per block)
+    "bpc": 8,         # resident blocks per CU that bound the grid of `nd` kernels
+    "ntl": 1,         # non-temporal loads  } for working sets beyond `cache_mib`;
+    "nts": 1,         # non-temporal stores } smaller ones stay cacheable
+    "cache_mib": 200,  # working sets up to this size are left to the 256 MB Infinity Cache
+    "tw": 128,        # stencil tile width (elements)
+    "th": 16,         # stencil tile height (rows)
+    "lds": 1,         # stage shifted views through LDS (0: read them directly)
+    "svec": 1,        # aligned stencils: 16-byte loads into LDS and 16-byte stores
+    "gpr": 64,        # vectorised stencil: 16-byte column groups per tile row
+    "rpt": 2,         # vectorised stencil: consecutive rows per thread
+    "xcd": 1,         # vectorised stencil: give each XCD a contiguous band of tiles
+    "sntl": 0,        # vectorised stencil: non-temporal loads / stores
+    "snts": 1,
+}
+for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
+    _k, _v = _kv.split("=")
+    TUNE[_k.strip()] = int(_v)
+
+_SCALAR_FMT = {"f4": "f", "f8": "d", "i4": "i", "i8": "q", "u4": "I", "u1": "B", "b1": "B"}
+
+# ---------------------------------------------------------------------------
+# layout analysis
+# ---------------------------------------------------------------------------
+
+def broadcast_strides(arr, shape):
+    """Element strides of `arr` viewed at `shape` (NumPy broadcasting)."""
+    nd = len(shape)
+    pad = nd - len(arr.shape)
+    if pad < 0:
+        raise ValueError(f"operand of shape {arr.shape} does not broadcast to {shape}")
+    out = [0] * nd
+    for k in range(len(arr.shape)):
+        d = arr.shape[k]
+        if d == shape[pad + k]:
+            out[pad + k] = arr._strides[k] if d != 1 else 0
+        elif d == 1:
+            out[pad + k] = 0
+        else:
+            raise ValueError(f"operand of shape {arr.shape} does not broadcast to {shape}")
+    return out
+
+
+def merge_dims(shape, stride_sets):
+    """Drop unit dims and merge neighbours that every operand walks contiguously."""
+    dims = [(d, [s[k] for s in stride_sets]) for k, d in enumerate(shape) if d != 1]
+    if not dims:
+        return [], [[] for _ in stride_sets]
+    merged = [dims[0]]
+    for d, strides in dims[1:]:
+        pd, ps = merged[-1]
+        if all(p == s * d for p, s in zip(ps, strides)):
+            merged[-1] = (pd * d, strides)
+        else:
+            merged.append((d, strides))
+    mshape = [d for d, _ in merged]
+    msets = [[st[i] for _, st in merged] for i in range(len(stride_sets))]
+    return mshape, msets
+
+
+class Lowered:
+    """A kernel choice for one evaluation: cache key, source builder, launch recipe."""
+
+    __slots__ = ("key", "kind", "emit", "fmt", "srcs", "scal", "tail", "grid", "fin_count", "lds")
+
+
+# ---------------------------------------------------------------------------
+# lowering
+# ---------------------------------------------------------------------------
+
+_CUS = None
+
+
+def grid_cap():
+    """Blocks that fill the device `bpc` deep (256 CUs assumed until a device is open)."""
+    global _CUS
+    if _CUS is None:
+        if not hiprt._initialised:
+            return 256 * TUNE["bpc"]
+        _CUS = hiprt.device_info()["compute_units"]
+    return _CUS * TUNE["bpc"]
+
+
+def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, reduce_op,
+           in_place=False):
+    """Pick the kernel shape.  `out_ptrs`/`out_strides` describe the destinations
+    (element strides at `out_shape`); for a reduction they are empty and the
+    partial-sums pointer is appended at launch."""
+    n = 1
+    for d in out_shape:
+        n *= d
+    leaf_strides = [broadcast_strides(a, out_shape) for a in leaves]
+    mshape, msets = merge_dims(out_shape, leaf_strides + list(out_strides))
+    m_leaf, m_out = msets[:len(leaves)], msets[len(leaves):]
+    ndim = len(mshape)
+    low = Lowered()
+    low.lds = 0
+    low.fin_count = 0
+    scal_fmt = "".join(_SCALAR_FMT[c] for c in prog.scalars)
+    scal_vals = list(scalars)
+    tune = tuple(sorted(TUNE.items()))
+
+    flat = ndim <= 1 and all(s == [1] or s == [0] or s == [] for s in m_leaf) \
+        and all(s == [1] or s == [] for s in m_out)
+    if flat:
+        leaf_class = tuple("b" if (s == [0] and n > 1) else "c" for s in m_leaf)
+        ptrs = [a.ptr for a in leaves]
+        widths_ok = all(cg.ITEMSIZE[c] in (4, 8) for c, k in zip(prog.leaves, leaf_class) if k == "c")
+        align_ok = all(p % 16 == 0 for p, k in zip(ptrs, leaf_class) if k == "c")
+        if not reduce_op:
+            widths_ok = widths_ok and all(cg.ITEMSIZE[c] in (4, 8) for c in out_codes)
+            align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
+        vec = widths_ok and align_ok and n >= 64
+        unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
+        footprint = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
+        if not reduce_op:
+            footprint += sum(n * cg.ITEMSIZE[c] for c in out_codes)
+        streaming = footprint > TUNE["cache_mib"] << 20
+        ntl = bool(TUNE["ntl"]) and streaming
+        nts = bool(TUNE["nts"]) and streaming
+        low.kind = "flat"
+        low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
+                   unroll, ntl, nts)
+
+        def emit():
+            src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
+                                  restrict=not in_place, reduce_op=reduce_op)
+            return src
+        low.emit = emit
+        if vec:
+            widths = [cg.ITEMSIZE[c] for c, k in zip(prog.leaves, leaf_class) if k == "c"]
+            if not reduce_op:
+                widths += [cg.ITEMSIZE[c] for c in out_codes]
+            E = 16 // min(widths) if widths else 4
+        else:
+            E = 1
+        chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
+        cap = TUNE["red_blocks"] if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
+        low.grid = min(chunks, cap)
+        n_out_ptr = 1 if reduce_op else len(out_ptrs)
+        low.fmt = "@" + "P" * (len(ptrs) + n_out_ptr) + scal_fmt + "q"
+        low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+        low.scal, low.tail = scal_vals, [n]
+        if reduce_op:
+            low.fin_count = low.grid
+        return low
+
+    tiled = (not reduce_op and ndim == 2 and all(s[1] == 1 for s in m_out)
+             and all(s[1] == 1 or s == [0, 0] for s in m_leaf))
+    if tiled:
+        H, W = mshape
+        tw, th = TUNE["tw"], TUNE["th"]
+        # halo group: >= 2 leaves that are shifted views of one buffer
+        groups = {}
+        for i, (a, s) in enumerate(zip(leaves, m_leaf)):
+            if s[1] == 1 and s[0] > 0:
+                groups.setdefault((id(a.buf), s[0], prog.leaves[i]), []).append(i)
+        best = max(groups.values(), key=len) if groups else []
+        kinds = [None] * len(leaves)
+        group = None
+        if len(best) >= 2 and TUNE["lds"]:
+            rs = m_leaf[best[0]][0]
+            ref_off = min(leaves[i].offset for i in best)
+            shifts = {}
+            for i in best:
+                d = leaves[i].offset - ref_off
+                dy, dx = divmod(d, rs)
+                if dx > rs // 2:
+                    dy, dx = dy + 1, dx - rs
+                shifts[i] = (dy, dx)
+            dy_max = max(dy for dy, _ in shifts.values())
+            dx_min = min(dx for _, dx in shifts.values())
+            dx_max = max(dx for _, dx in shifts.values())
+            itemsize = cg.ITEMSIZE[prog.leaves[best[0]]]
+            lds_bytes = (th + dy_max) * (tw + dx_max - dx_min) * itemsize
+            if dy_max <= 16 and dx_max - dx_min <= 32 and lds_bytes <= 48 * 1024:
+                group = (prog.leaves[best[0]], dy_max, dx_min, dx_max)
+                for i in best:
+                    kinds[i] = ("g",) + shifts[i]
+                g_buf = leaves[best[0]].buf
+                g_ptr = g_buf.ptr + ref_off * itemsize
+                g_src = (g_buf, ref_off * itemsize)
+                g_args = [rs, -ref_off, g_buf.nbytes // itemsize - ref_off]
+        for i, s in enumerate(m_leaf):
+            if kinds[i] is None:
+                kinds[i] = ("b",) if s == [0, 0] else ("d",)
+        kinds = tuple(kinds)
+        low.kind = "tile2d"
+        vec_ok = False
+        if group is not None and TUNE["svec"]:
+            gsize = cg.ITEMSIZE[group[0]]
+            vw = 16 // gsize
+            vec_ok = (gsize in (4, 8) and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
+                      and g_args[0] % vw == 0 and all(s[0] % vw == 0 for s in m_out)
+                      and len({(p // gsize) % vw for p in out_ptrs}) == 1)
+        if vec_ok:
+            ph_g = (g_ptr // gsize) % vw
+            ph_o = (out_ptrs[0] // gsize) % vw
+            gpr, rpt = TUNE["gpr"], TUNE["rpt"]
+            sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
+            bands = bool(TUNE["xcd"])
+            low.key = ("tile2dv", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o,
+                       gpr, rpt, sntl, snts, bands)
+            tw, th = gpr * vw, (cg.BLOCK // gpr) * rpt
+
+            def emit():
+                return cg.emit_stencil_vec(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o,
+                                           restrict=not in_place, nt_load=sntl, nt_store=snts,
+                                           xcd_bands=bands)[0]
+            W = W + ph_o          # tiles start `ph_o` columns left of the view
+        else:
+            low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune)
+
+            def emit():
+                return cg.emit_stencil(prog, kinds, group, out_codes, tw, th,
+                                       restrict=not in_place)
+        low.emit = emit
+        tiles_x = -(-W // tw)
+        tiles_y = -(-H // th)
+        low.grid = tiles_x * tiles_y
+        srcs = [(a.buf, a.offset * a.dtype.itemsize) for a, k in zip(leaves, kinds) if k[0] != "g"]
+        fmt = "@" + "P" * len(srcs)
+        tail_vals = []
+        if group is not None:
+            fmt += "P"
+            srcs.append(g_src)
+        fmt += "P" * len(out_ptrs) + scal_fmt + "ii"
+        tail_vals += [mshape[0], mshape[1]]
+        if group is not None:
+            fmt += "qqq"
+            tail_vals += g_args
+        fmt += "i"
+        tail_vals.append(tiles_x)
+        for k, s in zip(kinds, m_leaf):
+            if k[0] == "d":
+                fmt += "q"
+                tail_vals.append(s[0])
+        for s in m_out:
+            fmt += "q"
+            tail_vals.append(s[0])
+        low.fmt = fmt
+        low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
+        return low
+
+    # general strided kernel
+    if ndim == 0:
+        mshape, m_leaf, m_out, ndim = [1], [[0] for _ in m_leaf], [[0] for _ in m_out], 1
+    index32 = n < 2 ** 31
+    low.kind = "nd"
+    low.key = ("nd", prog.key(), ndim, tuple(out_codes), index32, reduce_op, tune)
+
+    def emit():
+        return cg.emit_nd(prog, ndim, out_codes, index32, reduce_op)
+    low.emit = emit
+    blocks = -(-n // cg.BLOCK)
+    low.grid = max(1, min(blocks, grid_cap()))
+    n_out_ptr = 1 if reduce_op else len(out_ptrs)
+    fmt = "@" + "P" * (len(leaves) + n_out_ptr) + scal_fmt + "q" + ("I" if index32 else "q") * ndim
+    tail = [n] + list(mshape)
+    for s in m_leaf:
+        fmt += "q" * ndim
+        tail += s
+    if not reduce_op:
+        for s in m_out:
+            fmt += "q" * ndim
+            tail += s
+    low.fmt = fmt
+    low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+    low.scal, low.tail = scal_vals, tail
+    if reduce_op:
+        low.fin_count = low.grid
+    return low
+
+
+def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op):
+    """Kernel choice for reducing over `axes` of the (broadcast) `shape`."""
+    kept = [d for d in range(len(shape)) if d not in axes]
+    full = [broadcast_strides(a, shape) for a in leaves]
+    kshape = [shape[d] for d in kept]
+    rshape = [shape[d] for d in axes]
+    kmerged, ksets = merge_dims(kshape, [[s[d] for d in kept] for s in full])
+    rmerged, rsets = merge_dims(rshape, [[s[d] for d in axes] for s in full])
+    if not kmerged:
+        kmerged, ksets = [1], [[0] for _ in leaves]
+    if not rmerged:
+        rmerged, rsets = [1], [[0] for _ in leaves]
+    K = R = 1
+    for d in kmerged:
+        K *= d
+    for d in rmerged:
+        R *= d
+    # coalescing decides the strategy: which side holds the unit-stride dimension
+    inner_kept = any(s[-1] == 1 for s in ksets)
+    inner_red = any(s[-1] == 1 for s in rsets)
+    strategy = "col" if (inner_kept and not inner_red) or R < 64 else "row"
+    low = Lowered()
+    low.lds = 0
+    low.fin_count = 0
+    low.kind = "axis"
+    kdim, rdim = len(kmerged), len(rmerged)
+    low.key = ("axis", prog.key(), kdim, rdim, acc, reduce_op, strategy)
+
+    def emit():
+        return cg.emit_axis_reduce(prog, kdim, rdim, acc, reduce_op, strategy)
+    low.emit = emit
+    if strategy == "col":
+        low.grid = max(1, min(-(-K // cg.BLOCK), grid_cap()))
+    else:
+        low.grid = max(1, min(K, grid_cap() * 4))
+    low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+               + "qq" + "q" * (kdim + rdim) + "q" * ((kdim + rdim) * len(leaves)))
+    tail = [K, R] + list(kmerged) + list(rmerged)
+    for ks, rs in zip(ksets, rsets):
+        tail += list(ks) + list(rs)
+    low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+    low.scal, low.tail = list(scalars), tail
+    return low
