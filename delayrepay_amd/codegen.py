@@ -600,115 +600,133 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
 def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_per_thread,
                      phase_group, phase_out, restrict=True, nt_load=False, nt_store=False,
                      xcd_bands=True):
-    """Vectorised form of `emit_stencil` for the common aligned case: the halo
-    group's row stride and every output's row stride are multiples of the 16-byte
-    vector width, and group and outputs have the same element size.
+    """Vectorised 2-D tiled kernel for the aligned case: every output's row stride
+    is a multiple of the 16-byte vector width VW and all outputs start at the same
+    address phase (`phase_out` = address of output [0, 0] / itemsize, mod VW).
 
-    phase_group  (address of the group's reference element / itemsize) % VW
-    phase_out    (address of output element [0, 0] / itemsize) % VW
-    With these two phases fixed at compile time, tile origins are chosen so that
-    every global load into LDS and every global store is a naturally aligned
-    16-byte access; only the first/last column group of a row and loads at the
-    very ends of the buffer fall back to element accesses.
+    leaf_kind  per leaf: ('g', dy, dx) member of the halo group (staged through LDS);
+               ('dv',) 2-D operand whose rows have the outputs' phase and a stride
+               that is a multiple of VW: read with 16-byte loads;
+               ('d',) other 2-D operand with unit column stride: element loads;
+               ('b',) single element broadcast
+    group      None, or (dtype code, dy_max, dx_min, dx_max) with the group's row
+               stride a multiple of VW and `phase_group` its reference element's phase
 
-    A block owns TW = groups_per_row * VW output columns by TH = (256 /
-    groups_per_row) * rows_per_thread rows.  Each thread computes VW adjacent
-    outputs per row for `rows_per_thread` consecutive rows, so shifted reads of
-    the same LDS words by neighbouring rows are shared in registers."""
-    gdt, dy_max, dx_min, dx_max = group
+    Tiles start `phase_out` columns left of the view, so a thread's VW adjacent
+    outputs are one aligned 16-byte store; the first/last column group of a row takes
+    an element-wise path.  A block owns TW = groups_per_row * VW columns by
+    TH = (256 / groups_per_row) * rows_per_thread rows; a thread computes VW outputs
+    for `rows_per_thread` consecutive rows, so shifted LDS reads of neighbouring rows
+    are shared in registers."""
     rs = "__restrict__ " if restrict else ""
-    vt, VW = VEC16[gdt]
+    first = group[0] if group is not None else out_dtypes[0]
+    vt, VW = VEC16[first]
     n_out = len(out_dtypes)
     GPR = groups_per_row
     slots = BLOCK // GPR
     TW = GPR * VW
     TH = slots * rows_per_thread
-    ph = (phase_group - phase_out + dx_min) % VW
-    LW = -(-(TW + dx_max - dx_min + ph) // VW) * VW
-    LWV = LW // VW
-    LH = TH + dy_max
     src = [PREAMBLE, emit_body(prog, out_dtypes)]
     params = []
     for i, dt in enumerate(prog.leaves):
         if leaf_kind[i][0] != "g":
             params.append(f"const {CTYPE[dt]}* {rs}a{i}")
-    params.append(f"const {CTYPE[gdt]}* {rs}gp")
+    if group is not None:
+        gdt, dy_max, dx_min, dx_max = group
+        ph = (phase_group - phase_out + dx_min) % VW
+        LW = -(-(TW + dx_max - dx_min + ph) // VW) * VW
+        LWV = LW // VW
+        LH = TH + dy_max
+        ct = CTYPE[gdt]
+        params.append(f"const {ct}* {rs}gp")
     params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
-    params += ["const int H", "const int W", "const long long grs", "const long long glo",
-               "const long long ghi", "const int tiles_x"]
+    params += ["const int H", "const int W"]
+    if group is not None:
+        params += ["const long long grs", "const long long glo", "const long long ghi"]
+    params.append("const int tiles_x")
     for i, k in enumerate(leaf_kind):
-        if k[0] == "d":
+        if k[0] in ("d", "dv"):
             params.append(f"const long long rs{i}")
     params += [f"const long long ors{o}" for o in range(n_out)]
-    ct = CTYPE[gdt]
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
-         f"void dr_kernel({', '.join(params)})", "{",
-         f"    __shared__ {vt} tile[{LH * LWV}];",
-         "    const int nb = gridDim.x;",
-         f"    const int xcd = blockIdx.x % {N_XCD};",
-         f"    const int slot = blockIdx.x / {N_XCD};",
-         (f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;" if xcd_bands
-          else "    const int t = blockIdx.x;"),
-         "    const int ty = t / tiles_x;",
-         "    const int tx = t - ty * tiles_x;",
-         f"    const int r0 = ty * {TH};",
-         f"    const int j0 = tx * {TW} - {phase_out};      // first output column of the tile",
-         f"    const int cs = j0 + ({dx_min}) - {ph};       // buffer column held in LDS column 0",
-         f"    for (int idx = threadIdx.x; idx < {LH * LWV}; idx += {BLOCK}) {{",
-         f"        const int lr = idx / {LWV};",
-         f"        const int lv = idx - lr * {LWV};",
-         f"        const long long lin = (long long)(r0 + lr) * grs + cs + lv * {VW};",
-         f"        {vt} val;",
-         f"        if (lin >= glo && lin + {VW} <= ghi) {{",
-         f"            val = {_ld(nt_load, f'(const {vt}*)(gp + lin)')};",
-         "        } else {",
-         "#pragma unroll",
-         f"            for (int e = 0; e < {VW}; ++e)",
-         f"                val[e] = (lin + e >= glo && lin + e < ghi) ? gp[lin + e] : ({ct})0;",
-         "        }",
-         "        tile[idx] = val;",
-         "    }",
-         "    __syncthreads();",
-         f"    const {ct}* ts = (const {ct}*)tile;",
-         f"    const int g = threadIdx.x % {GPR};",
-         f"    const int rw = threadIdx.x / {GPR};",
-         f"    const int jf = j0 + g * {VW};                // first of this thread's {VW} columns",
-         "#pragma unroll",
-         f"    for (int k = 0; k < {rows_per_thread}; ++k) {{",
-         f"        const int lr = rw * {rows_per_thread} + k;",
-         "        const int i = r0 + lr;",
-         "        if (i >= H) break;"]
+         f"void dr_kernel({', '.join(params)})", "{"]
+    if group is not None:
+        L.append(f"    __shared__ {vt} tile[{LH * LWV}];")
+    L += ["    const int nb = gridDim.x;",
+          f"    const int xcd = blockIdx.x % {N_XCD};",
+          f"    const int slot = blockIdx.x / {N_XCD};",
+          (f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;" if xcd_bands
+           else "    const int t = blockIdx.x;"),
+          "    const int ty = t / tiles_x;",
+          "    const int tx = t - ty * tiles_x;",
+          f"    const int r0 = ty * {TH};",
+          f"    const int j0 = tx * {TW} - {phase_out};      // first output column of the tile"]
+    if group is not None:
+        L += [f"    const int cs = j0 + ({dx_min}) - {ph};       // buffer column held in LDS column 0",
+              f"    for (int idx = threadIdx.x; idx < {LH * LWV}; idx += {BLOCK}) {{",
+              f"        const int lr = idx / {LWV};",
+              f"        const int lv = idx - lr * {LWV};",
+              f"        const long long lin = (long long)(r0 + lr) * grs + cs + lv * {VW};",
+              f"        {vt} val;",
+              f"        if (lin >= glo && lin + {VW} <= ghi) {{",
+              f"            val = {_ld(nt_load, f'(const {vt}*)(gp + lin)')};",
+              "        } else {",
+              "#pragma unroll",
+              f"            for (int e = 0; e < {VW}; ++e)",
+              f"                val[e] = (lin + e >= glo && lin + e < ghi) ? gp[lin + e] : ({ct})0;",
+              "        }",
+              "        tile[idx] = val;",
+              "    }",
+              "    __syncthreads();",
+              f"    const {ct}* ts = (const {ct}*)tile;"]
+    L += [f"    const int g = threadIdx.x % {GPR};",
+          f"    const int rw = threadIdx.x / {GPR};",
+          f"    const int jf = j0 + g * {VW};                // first of this thread's {VW} columns",
+          f"    const bool inner = jf >= 0 && jf + {VW} <= W;",
+          "#pragma unroll",
+          f"    for (int k = 0; k < {rows_per_thread}; ++k) {{",
+          f"        const int lr = rw * {rows_per_thread} + k;",
+          "        const int i = r0 + lr;",
+          "        if (i >= H) break;"]
+
+    def operand(i, k, e, vector_path):
+        if k[0] == "g":
+            _, dy, dx = k
+            return f"ts[(lr + {dy}) * {LW} + g * {VW} + {e + dx - dx_min + ph}]"
+        if k[0] == "dv" and vector_path:
+            return f"D{i}[{e}]"
+        if k[0] in ("d", "dv"):
+            return f"a{i}[(long long)i * rs{i} + jf + {e}]"
+        return f"a{i}[0]"
+
+    decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+    tail_args = [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
+    L.append("        if (inner) {")
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "dv":
+            lvt = VEC16[prog.leaves[i]][0]
+            ptr = f"(const {lvt}*)(a{i} + (long long)i * rs{i} + jf)"
+            L.append(f"            const {lvt} D{i} = {_ld(nt_load, ptr)};")
     for o, dt in enumerate(out_dtypes):
-        L.append(f"        {VEC16[dt][0]} R{o};")
+        L.append(f"            {VEC16[dt][0]} R{o};")
     for e in range(VW):
-        args = []
-        for i, k in enumerate(leaf_kind):
-            if k[0] == "g":
-                _, dy, dx = k
-                args.append(f"ts[(lr + {dy}) * {LW} + g * {VW} + {e + dx - dx_min + ph}]")
-            elif k[0] == "d":
-                args.append(f"((jf + {e} >= 0 && jf + {e} < W) ? a{i}[(long long)i * rs{i} + jf + {e}] "
-                            f": ({CTYPE[prog.leaves[i]]})0)")
-            else:
-                args.append(f"a{i}[0]")
-        decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
-        call = args + [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
+        args = [operand(i, k, e, True) for i, k in enumerate(leaf_kind)]
         sets = " ".join(f"R{o}[{e}] = t{o};" for o in range(n_out))
-        L.append(f"        {{ {decl} dr_body({', '.join(call)}); {sets} }}")
-    L.append(f"        if (jf >= 0 && jf + {VW} <= W) {{")
+        L.append(f"            {{ {decl} dr_body({', '.join(args + tail_args)}); {sets} }}")
     for o, dt in enumerate(out_dtypes):
         L.append("            " + _st(nt_store, f"R{o}",
                                         f"({VEC16[dt][0]}*)(o{o} + (long long)i * ors{o} + jf)"))
     L.append("        } else {")
-    L.append("#pragma unroll")
-    L.append(f"            for (int e = 0; e < {VW}; ++e)")
-    L.append("                if (jf + e >= 0 && jf + e < W) {")
-    for o in range(n_out):
-        L.append(f"                    o{o}[(long long)i * ors{o} + jf + e] = R{o}[e];")
-    L += ["                }", "        }", "    }", "}"]
+    for e in range(VW):
+        args = [operand(i, k, e, False) for i, k in enumerate(leaf_kind)]
+        stores = " ".join(f"o{o}[(long long)i * ors{o} + jf + {e}] = t{o};" for o in range(n_out))
+        L.append(f"            if (jf + {e} >= 0 && jf + {e} < W) "
+                 f"{{ {decl} dr_body({', '.join(args + tail_args)}); {stores} }}")
+    L += ["        }", "    }", "}"]
     src.append("\n".join(L))
-    return "\n".join(src) + "\n", TW, TH, LH * LW * ITEMSIZE[gdt]
+    lds_bytes = LH * LW * ITEMSIZE[first] if group is not None else 0
+    return "\n".join(src) + "\n", TW, TH, lds_bytes
 
 
 # ---- reduction along some axes ------------------------------------------------
@@ -716,22 +734,25 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
 def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
     """Reduce the (fused) expression over `rdim` merged dimensions, keeping `kdim`.
 
-    strategy 'col'  one thread per output, looping over the reduced extent:
-                    coalesced when the fastest-varying memory dimension is kept
-                    (e.g. sum over axis 0 of a row-major matrix);
-             'row'  one block per output, threads striding over the reduced extent,
-                    wave64 shuffle + LDS tree at the end: coalesced when the
-                    fastest-varying dimension is reduced (e.g. sum over the last axis).
-    Parameters: leaf pointers, output pointer, scalars, K, R, kept dims, reduced
-    dims, then per leaf its kept strides and its reduced strides (elements)."""
+    The reduced extent R may be cut into S slices of RS elements; the kernel then
+    writes S partial results per output and a second launch reduces those.
+
+    strategy 'col'  a block owns 64 adjacent outputs (one per lane) and one slice;
+                    its 4 waves walk different reduced indices and meet through LDS.
+                    Coalesced when the fastest-varying memory dimension is kept
+                    (sum over axis 0 of a row-major matrix).  Partials: [slice][output].
+             'row'  a wave owns one (output, slice); its lanes stride over the
+                    reduced extent and meet with a shuffle tree.  Coalesced when the
+                    fastest-varying dimension is reduced (sum over the last axis).
+                    Partials: [output][slice].
+    Parameters: leaf pointers, output pointer, scalars, K, R, S, RS, kept dims,
+    reduced dims, then per leaf its kept strides and its reduced strides."""
     ct = CTYPE[acc_dt]
     src = [PREAMBLE, emit_body(prog, [acc_dt])]
-    if strategy == "row":
-        src.append(emit_block_reduce(op, acc_dt))
-    params = [f"const {CTYPE[dt]}* a{i}" for i, dt in enumerate(prog.leaves)]
-    params.append(f"{ct}* out")
+    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
+    params.append(f"{ct}* __restrict__ out")
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
-    params += ["const long long K", "const long long R"]
+    params += ["const long long K", "const long long R", "const long long S", "const long long RS"]
     params += [f"const long long dk{d}" for d in range(kdim)]
     params += [f"const long long dr{d}" for d in range(rdim)]
     for i in range(len(prog.leaves)):
@@ -758,33 +779,64 @@ def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
         return lines
 
     call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
+    args = [f"a{i}[bk{i} + br{i}]" for i in range(nl)]
+    ident = _identity(op, acc_dt)
     if strategy == "col":
-        L.append(f"    const long long stride = (long long)gridDim.x * {BLOCK};")
-        L.append(f"    for (long long g = (long long)blockIdx.x * {BLOCK} + threadIdx.x; g < K; g += stride) {{")
-        L += decompose("g", "dk", "k", kdim, "bk", 8)
-        L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
-        L.append("        for (long long r = 0; r < R; ++r) {")
-        L += decompose("r", "dr", "r", rdim, "br", 12)
-        args = [f"a{i}[bk{i} + br{i}]" for i in range(nl)]
-        L.append(f"            {ct} t0; dr_body({', '.join(args + call_tail)});")
-        L.append(f"            acc = {_combine(op, 'acc', 't0')};")
-        L.append("        }")
-        L.append("        out[g] = acc;")
-        L.append("    }")
+        waves = BLOCK // WAVE
+        L += [f"    __shared__ {ct} red[{waves}][{WAVE}];",
+              f"    const int tx = threadIdx.x & {WAVE - 1};",
+              "    const int ty = threadIdx.x >> 6;",
+              f"    const long long ktiles = (K + {WAVE - 1}) / {WAVE};",
+              "    for (long long b = blockIdx.x; b < ktiles * S; b += gridDim.x) {",
+              "        const long long sl = b / ktiles;",
+              f"        const long long g = (b - sl * ktiles) * {WAVE} + tx;",
+              f"        {ct} acc = {ident};",
+              "        if (g < K) {"]
+        L += decompose("g", "dk", "k", kdim, "bk", 12)
+        L += ["            const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;",
+              "#pragma unroll 4",
+              f"            for (long long r = sl * RS + ty; r < r_end; r += {waves}) {{"]
+        L += decompose("r", "dr", "r", rdim, "br", 16)
+        L += [f"                {ct} t0; dr_body({', '.join(args + call_tail)});",
+              f"                acc = {_combine(op, 'acc', 't0')};",
+              "            }",
+              "        }",
+              "        red[ty][tx] = acc;",
+              "        __syncthreads();",
+              "        if (ty == 0 && g < K) {",
+              "#pragma unroll",
+              f"            for (int w = 1; w < {waves}; ++w) acc = {_combine(op, 'acc', 'red[w][tx]')};",
+              "            out[sl * K + g] = acc;",
+              "        }",
+              "        __syncthreads();",
+              "    }"]
     else:
-        L.append("    for (long long g = blockIdx.x; g < K; g += gridDim.x) {")
+        shfl = "__shfl_down(acc, off, 64)"
+        if acc_dt in ("u1", "b1"):
+            shfl = f"({ct})__shfl_down((int)acc, off, 64)"
+        L += [f"    const int lane = threadIdx.x & {WAVE - 1};",
+              f"    const long long nwaves = (long long)gridDim.x * {BLOCK // WAVE};",
+              "#pragma unroll 2",
+              f"    for (long long o = (long long)blockIdx.x * {BLOCK // WAVE} + (threadIdx.x >> 6); "
+              "o < K * S; o += nwaves) {",
+              "        const long long g = o / S;",
+              "        const long long sl = o - g * S;"]
         L += decompose("g", "dk", "k", kdim, "bk", 8)
-        L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
-        L.append(f"        for (long long r = threadIdx.x; r < R; r += {BLOCK}) {{")
+        L += [f"        {ct} acc = {ident};",
+              "        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;",
+              "#pragma unroll 4",
+              f"        for (long long r = sl * RS + lane; r < r_end; r += {WAVE}) {{"]
         L += decompose("r", "dr", "r", rdim, "br", 12)
-        args = [f"a{i}[bk{i} + br{i}]" for i in range(nl)]
-        L.append(f"            {ct} t0; dr_body({', '.join(args + call_tail)});")
-        L.append(f"            acc = {_combine(op, 'acc', 't0')};")
-        L.append("        }")
-        L.append("        acc = dr_block_reduce(acc);")
-        L.append("        if (threadIdx.x == 0) out[g] = acc;")
-        L.append("        __syncthreads();")
-        L.append("    }")
+        L += [f"            {ct} t0; dr_body({', '.join(args + call_tail)});",
+              f"            acc = {_combine(op, 'acc', 't0')};",
+              "        }",
+              "#pragma unroll",
+              f"        for (int off = {WAVE // 2}; off > 0; off >>= 1) {{",
+              f"            const {ct} other = {shfl};",
+              f"            acc = {_combine(op, 'acc', 'other')};",
+              "        }",
+              "        if (lane == 0) out[o] = acc;",
+              "    }"]
     L.append("}")
     src.append("\n".join(L))
     return "\n".join(src) + "\n"

@@ -376,7 +376,7 @@ class Plan:
     launch.  `valid()` re-checks what could have changed underneath."""
 
     __slots__ = ("low", "kern", "checks", "stamp", "shape", "out_dtypes", "acc", "leaves",
-                 "hazard", "region", "empty", "axes")
+                 "hazard", "region", "empty", "axes", "second", "kern2", "scratch")
 
     def valid(self):
         if self.stamp != _STAMP:
@@ -404,6 +404,24 @@ def _fire(plan, out_ptrs, reduce_out=None):
     if kern is None:
         kern = plan.kern = _kernel_for(low, reduce_out is not None)
     ptrs = [buf.ptr + off for buf, off in low.srcs]
+    if plan.second is not None:
+        # two-pass axis reduction: partials into pooled scratch, then reduce those
+        low2 = plan.second
+        kern2 = plan.kern2
+        if kern2 is None:
+            kern2 = plan.kern2 = _kernel_for(low2, False)
+        scratch = hiprt.malloc(plan.scratch)
+        args = kern.packer.pack(*ptrs, scratch, *low.scal, *low.tail)
+        hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
+        args2 = kern2.packer.pack(scratch, *out_ptrs, *low2.tail)
+        hiprt.launch(kern2.func, low2.grid, cg.BLOCK, 0, args2, len(args2))
+        if _RECORDING is not None:
+            _RECORDING.launches += [(kern.func, low.grid, 0, args), (kern2.func, low2.grid, 0, args2)]
+            _RECORDING._scratch.append(scratch)
+        else:
+            hiprt.free(scratch)
+        STATS["launches"] += 2
+        return
     if reduce_out is not None:
         partial = hiprt.malloc(low.fin_count * cg.ITEMSIZE[plan.acc])
         args = kern.packer.pack(*ptrs, partial, *low.scal, *low.tail)
@@ -443,6 +461,9 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False, axes=None):
     plan.acc = None
     plan.empty = False
     plan.axes = False
+    plan.second = None
+    plan.kern2 = None
+    plan.scratch = 0
     if reduce_op:
         shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
         code = roots[0][1]
@@ -458,8 +479,18 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False, axes=None):
                 plan.empty = True
                 plan.low = None
                 return plan
-            plan.low = _lower_axis_reduce(prog, leaves, tracer.scalars, shape, axes, plan.acc,
-                                          reduce_op)
+            plan.low, S, K, strategy = _lower_axis_reduce(prog, leaves, tracer.scalars, shape,
+                                                          axes, plan.acc, reduce_op)
+            if S > 1:
+                # second pass over the S partials of every output: an identity program on
+                # a stand-in array with the partials' layout (pointer filled in at launch)
+                acc_dt = code_dtype(plan.acc)
+                pshape, paxis = ((S, K), (0,)) if strategy == "col" else ((K, S), (1,))
+                stand_in = ndarray(pshape, acc_dt, _Elsewhere(S * K * acc_dt.itemsize))
+                prog2 = Program([plan.acc], [], [], [(("l", 0), plan.acc)])
+                plan.second = _lower_axis_reduce(prog2, [stand_in], [], pshape, paxis, plan.acc,
+                                                 reduce_op, slices=1)[0]
+                plan.scratch = S * K * acc_dt.itemsize
             return plan
         plan.shape = ()
         if 0 in shape:

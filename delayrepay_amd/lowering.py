@@ -19,6 +19,10 @@ TUNE = {
     "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
     "flat_cap": 0,    # most blocks of a flat element-wise kernel (0: one chunk per block)
     "bpc": 8,         # resident blocks per CU that bound the grid of `nd` kernels
+    "ax_blocks": 4096,   # axis reductions: blocks ('col') / waves ('row') worth of work to
+    "ax_waves": 32768,   # aim for before the reduced extent is cut into slices
+    "ax_rows": 4,        # 'row' strategy: outputs per wave (grid-stride), to amortise set-up
+    "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ntl": 1,         # non-temporal loads  } for working sets beyond `cache_mib`;
     "nts": 1,         # non-temporal stores } smaller ones stay cacheable
     "cache_mib": 200,  # working sets up to this size are left to the 256 MB Infinity Cache
@@ -206,15 +210,22 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         kinds = tuple(kinds)
         low.kind = "tile2d"
         vec_ok = False
-        if group is not None and TUNE["svec"]:
-            gsize = cg.ITEMSIZE[group[0]]
-            vw = 16 // gsize
-            vec_ok = (gsize in (4, 8) and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
-                      and g_args[0] % vw == 0 and all(s[0] % vw == 0 for s in m_out)
-                      and len({(p // gsize) % vw for p in out_ptrs}) == 1)
+        if TUNE["svec"] and out_codes:
+            gsize = cg.ITEMSIZE[group[0]] if group is not None else cg.ITEMSIZE[out_codes[0]]
+            vw = 16 // gsize if gsize in (4, 8) else 0
+            vec_ok = (vw > 0 and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
+                      and all(s[0] % vw == 0 for s in m_out)
+                      and len({(p // gsize) % vw for p in out_ptrs}) == 1
+                      and (group is None or g_args[0] % vw == 0))
         if vec_ok:
-            ph_g = (g_ptr // gsize) % vw
             ph_o = (out_ptrs[0] // gsize) % vw
+            ph_g = (g_ptr // gsize) % vw if group is not None else 0
+            # direct operands whose rows share the outputs' alignment load as vectors
+            kinds = tuple(
+                ("dv",) if (k[0] == "d" and cg.ITEMSIZE[prog.leaves[i]] == gsize
+                            and m_leaf[i][0] % vw == 0
+                            and (leaves[i].ptr // gsize) % vw == ph_o) else k
+                for i, k in enumerate(kinds))
             gpr, rpt = TUNE["gpr"], TUNE["rpt"]
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
             bands = bool(TUNE["xcd"])
@@ -251,7 +262,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         fmt += "i"
         tail_vals.append(tiles_x)
         for k, s in zip(kinds, m_leaf):
-            if k[0] == "d":
+            if k[0] in ("d", "dv"):
                 fmt += "q"
                 tail_vals.append(s[0])
         for s in m_out:
@@ -291,8 +302,12 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     return low
 
 
-def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op):
-    """Kernel choice for reducing over `axes` of the (broadcast) `shape`."""
+def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices=None):
+    """Kernel choice for reducing over `axes` of the (broadcast) `shape`.
+
+    Returns (first pass, S): when S > 1 the first pass writes S partial results
+    per output ([slice][output] for 'col', [output][slice] for 'row') and the
+    caller runs a second reduction over them."""
     kept = [d for d in range(len(shape)) if d not in axes]
     full = [broadcast_strides(a, shape) for a in leaves]
     kshape = [shape[d] for d in kept]
@@ -311,11 +326,21 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op):
     # coalescing decides the strategy: which side holds the unit-stride dimension
     inner_kept = any(s[-1] == 1 for s in ksets)
     inner_red = any(s[-1] == 1 for s in rsets)
-    strategy = "col" if (inner_kept and not inner_red) or R < 64 else "row"
+    strategy = "col" if (inner_kept and not inner_red) else "row"
+    # enough independent pieces to fill the device: cut the reduced extent into slices
+    if slices is not None:
+        S = slices
+    elif strategy == "col":
+        ktiles = -(-K // cg.WAVE)
+        S = max(1, min(-(-TUNE["ax_blocks"] // ktiles), R // 32, TUNE["ax_slices"]))
+    else:
+        S = max(1, min(-(-TUNE["ax_waves"] // K), R // 256, TUNE["ax_slices"]))
+    RS = -(-R // S)
+    S = -(-R // RS)
     low = Lowered()
     low.lds = 0
     low.fin_count = 0
-    low.kind = "axis"
+    low.kind = "axis_" + strategy
     kdim, rdim = len(kmerged), len(rmerged)
     low.key = ("axis", prog.key(), kdim, rdim, acc, reduce_op, strategy)
 
@@ -323,14 +348,14 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op):
         return cg.emit_axis_reduce(prog, kdim, rdim, acc, reduce_op, strategy)
     low.emit = emit
     if strategy == "col":
-        low.grid = max(1, min(-(-K // cg.BLOCK), grid_cap()))
+        low.grid = max(1, min(-(-K // cg.WAVE) * S, 1 << 20))
     else:
-        low.grid = max(1, min(K, grid_cap() * 4))
+        low.grid = max(1, min(-(-(K * S) // (cg.BLOCK // cg.WAVE) // TUNE["ax_rows"]), 1 << 20))
     low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
-               + "qq" + "q" * (kdim + rdim) + "q" * ((kdim + rdim) * len(leaves)))
-    tail = [K, R] + list(kmerged) + list(rmerged)
+               + "qqqq" + "q" * (kdim + rdim) + "q" * ((kdim + rdim) * len(leaves)))
+    tail = [K, R, S, RS] + list(kmerged) + list(rmerged)
     for ks, rs in zip(ksets, rsets):
         tail += list(ks) + list(rs)
     low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
     low.scal, low.tail = list(scalars), tail
-    return low
+    return low, S, K, strategy
