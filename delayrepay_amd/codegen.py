@@ -840,3 +840,82 @@ def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
     L.append("}")
     src.append("\n".join(L))
     return "\n".join(src) + "\n"
+
+
+# ---- 2-D kernel with transposed operands ------------------------------------------
+
+T_TILE = 64      # square tile edge: both the transposed read and the write coalesce
+
+
+def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True):
+    """2-D tiled kernel for expressions in which some operand is walked along the
+    output's rows by its unit stride (a transposed view).
+
+    leaf_kind  per leaf: ('t',) unit stride along output dimension 0: its 64x64 tile
+               is read along its own contiguous direction into LDS and read back
+               transposed (rows padded by one word, so neither side has bank
+               conflicts); ('d',) unit stride along output dimension 1, read directly;
+               ('b',) single element broadcast
+    Parameters: leaf pointers, output pointers, scalars, H, W, tiles_x, then per 't'
+    leaf its stride along output columns, per 'd' leaf its row stride, per output its
+    row stride."""
+    rs = "__restrict__ " if restrict else ""
+    n_out = len(out_dtypes)
+    T = T_TILE
+    per_thread = T * T // BLOCK
+    src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    params = [f"const {CTYPE[dt]}* {rs}a{i}" for i, dt in enumerate(prog.leaves)]
+    params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += ["const int H", "const int W", "const int tiles_x"]
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "t":
+            params.append(f"const long long cs{i}")
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "d":
+            params.append(f"const long long rs{i}")
+    params += [f"const long long ors{o}" for o in range(n_out)]
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{"]
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "t":
+            L.append(f"    __shared__ {CTYPE[prog.leaves[i]]} tt{i}[{T * (T + 1)}];")
+    L += ["    const int ty = blockIdx.x / tiles_x;",
+          "    const int tx = blockIdx.x - ty * tiles_x;",
+          f"    const int r0 = ty * {T};",
+          f"    const int c0 = tx * {T};",
+          # transposed operands: consecutive threads walk output ROWS (their unit stride)
+          "#pragma unroll",
+          f"    for (int k = 0; k < {per_thread}; ++k) {{",
+          f"        const int e = threadIdx.x + k * {BLOCK};",
+          f"        const int lc = e / {T};",
+          f"        const int lr = e - lc * {T};",
+          "        if (r0 + lr < H && c0 + lc < W) {"]
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "t":
+            L.append(f"            tt{i}[lc * {T + 1} + lr] = a{i}[(long long)(c0 + lc) * cs{i} + (r0 + lr)];")
+    L += ["        }", "    }", "    __syncthreads();",
+          "#pragma unroll",
+          f"    for (int k = 0; k < {per_thread}; ++k) {{",
+          f"        const int e = threadIdx.x + k * {BLOCK};",
+          f"        const int lr = e / {T};",
+          f"        const int lc = e - lr * {T};",
+          "        const int i = r0 + lr;",
+          "        const int j = c0 + lc;",
+          "        if (i < H && j < W) {"]
+    args = []
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "t":
+            args.append(f"tt{i}[lc * {T + 1} + lr]")
+        elif k[0] == "d":
+            args.append(f"a{i}[(long long)i * rs{i} + j]")
+        else:
+            args.append(f"a{i}[0]")
+    decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+    call = args + [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
+    L.append(f"            {decl} dr_body({', '.join(call)});")
+    for o in range(n_out):
+        L.append(f"            o{o}[(long long)i * ors{o} + j] = t{o};")
+    L += ["        }", "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"

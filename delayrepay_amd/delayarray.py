@@ -219,6 +219,21 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
     def reshape(self, *args, **kwargs):
         return NPArray(self._force().reshape(*args, **kwargs))
 
+    def copy(self):
+        """Evaluated, contiguous copy as a new leaf."""
+        return NPArray(_backend.fallback.copy(self._force()))
+
+    def ravel(self):
+        return self.reshape(self.size)
+
+    def transpose(self, *axes):
+        """Permuted view of the evaluated array, as a new leaf."""
+        if len(axes) == 1 and not isinstance(axes[0], (int, np.integer)):
+            axes = tuple(axes[0]) if axes[0] is not None else ()
+        return np.transpose(self, axes or None)
+
+    flatten = ravel
+
     def astype(self, dtype, **kwargs):
         """Lazy cast, fused into whatever consumes it."""
         dtype = np.dtype(dtype)

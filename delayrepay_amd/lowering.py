@@ -272,6 +272,42 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
         return low
 
+    # operands walked along the output's rows by their unit stride (transposed views)
+    transposed = (not reduce_op and ndim == 2 and all(s[1] == 1 for s in m_out)
+                  and all(s[1] == 1 or s == [0, 0] or (s[0] == 1 and s[1] != 1) for s in m_leaf)
+                  and any(s[0] == 1 and s[1] != 1 for s in m_leaf))
+    if transposed:
+        kinds = tuple(("b",) if s == [0, 0] else ("d",) if s[1] == 1 else ("t",) for s in m_leaf)
+        lds_bytes = sum((cg.T_TILE + 1) * cg.T_TILE * cg.ITEMSIZE[c]
+                        for c, k in zip(prog.leaves, kinds) if k[0] == "t")
+        if lds_bytes <= 64 * 1024:
+            H, W = mshape
+            low.kind = "tile2dt"
+            low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place)
+
+            def emit():
+                return cg.emit_tile_transpose(prog, kinds, out_codes, restrict=not in_place)
+            low.emit = emit
+            tiles_x = -(-W // cg.T_TILE)
+            low.grid = tiles_x * -(-H // cg.T_TILE)
+            fmt = "@" + "P" * (len(leaves) + len(out_ptrs)) + scal_fmt + "iii"
+            tail_vals = [H, W, tiles_x]
+            for k, s in zip(kinds, m_leaf):
+                if k[0] == "t":
+                    fmt += "q"
+                    tail_vals.append(s[1])
+            for k, s in zip(kinds, m_leaf):
+                if k[0] == "d":
+                    fmt += "q"
+                    tail_vals.append(s[0])
+            for s in m_out:
+                fmt += "q"
+                tail_vals.append(s[0])
+            low.fmt = fmt
+            low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+            low.scal, low.tail = scal_vals, tail_vals
+            return low
+
     # general strided kernel
     if ndim == 0:
         mshape, m_leaf, m_out, ndim = [1], [[0] for _ in m_leaf], [[0] for _ in m_out], 1

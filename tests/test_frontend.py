@@ -230,7 +230,10 @@ def test_strided_and_broadcast_operands_use_nd():
     assert low.kind == "nd"
     hip.compile_source(src)
     m = hip.placeholder((100, 200), np.float32)
-    assert hip.lower_only(NPArray(m.T) * 2.0)[0].kind == "nd"
+    low, src = hip.lower_only(NPArray(m.T) * 2.0)           # transposed operand: through LDS
+    assert low.kind == "tile2dt" and "__shared__ float tt0[" in src
+    hip.compile_source(src)
+    assert hip.lower_only(NPArray(m[::2, ::3]) * 2.0)[0].kind == "nd"
 
 
 def test_shifted_views_lower_to_lds_stencil():

@@ -582,3 +582,19 @@ def test_where_clip_sign_and_predicates():
     i0 = rs.randint(-3, 4, 1000)
     assert np.array_equal(np.sign(dr.array(i0)).get(), np.sign(i0))
     assert np.array_equal(np.where(dr.array(i0) > 0, dr.array(i0), -1).get(), np.where(i0 > 0, i0, -1))
+
+
+def test_transposed_operands_go_through_lds_and_match():
+    rs = np.random.RandomState(15)
+    for shape in [(64, 64), (100, 200), (257, 63), (1, 300), (1000, 3)]:
+        a0 = rs.standard_normal(shape).astype(np.float32)
+        b0 = rs.standard_normal(shape[::-1])
+        a, b = dr.array(a0), dr.array(b0)
+        assert bits_equal((a.T * 2.0).get(), a0.T * np.float32(2.0))
+        assert bits_equal((a.T + b).get(), a0.T + b0)                   # mixed dtypes, one transposed
+        assert bits_equal((a.T * b.T.T + 1.0).get(), a0.T * b0 + 1.0)
+        assert bits_equal(a.T.copy().get(), np.ascontiguousarray(a0.T))
+    c0 = rs.standard_normal((40, 50, 60))
+    c = dr.array(c0)
+    assert bits_equal((c.transpose(2, 0, 1) * 1.5).get(), c0.transpose(2, 0, 1) * 1.5)   # general nd
+    assert bits_equal((c.transpose(1, 0, 2) + 1).get(), c0.transpose(1, 0, 2) + 1)
