@@ -56,7 +56,9 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all",
-                    help="horner (headline) | saxpy | bs32 | bs64 | jacobi | sumsq | all")
+                    help="horner (headline) | saxpy | bs32 | bs64 | jacobi | sumsq | all (these six); "
+                         "dot | axis0 | axis1 | rowbcast | transpose | next (these five: the "
+                         "operations either side of the five configurations)")
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before each timed region (clock ramp-up)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0,
@@ -92,7 +94,8 @@ def main():
 
     # ---- the workloads: (inputs on device, step function, bytes, elements, cpu function)
     def make(name):
-        inp = orc.make_inputs(name)
+        inp = orc.make_inputs(name) if name in ("saxpy", "horner", "bs32", "bs64", "jacobi",
+                                                "sumsq") else None
         if name == "saxpy":
             x, y = dr.array(inp["x"]), dr.array(inp["y"])
             n = inp["x"].size
@@ -134,6 +137,34 @@ def main():
                         step=lambda: hip.run(ReduceEx(np.add, (x - y) ** 2 * w)),
                         cpu=lambda: orc.sumsq(inp["x"][:m], inp["y"][:m], inp["w"][:m]),
                         cpu_frac=0.25)
+        # ---- operations either side of the five configurations (no CPU sample kept small)
+        rs = np.random.RandomState(0)
+        if name == "dot":
+            n = 1 << 27
+            hx, hy = rs.standard_normal(n), rs.standard_normal(n)
+            x, y = dr.array(hx), dr.array(hy)
+            return dict(dtype="f64", n=n, nbytes=16 * n, desc="dot(x, y) f64 n=2^27 (fused multiply-reduce)",
+                        step=lambda: hip.run(ReduceEx(np.add, x * y)),
+                        cpu=lambda: np.dot(hx[:n // 4], hy[:n // 4]), cpu_frac=0.25)
+        if name in ("axis0", "axis1", "rowbcast", "transpose"):
+            N = 16384
+            ha = rs.standard_normal((N, N)).astype(np.float32)
+            a = dr.array(ha)
+            if name in ("axis0", "axis1"):
+                ax = int(name[-1])
+                return dict(dtype="f32", n=N * N, nbytes=4 * N * N + 4 * N,
+                            desc=f"sum(a, axis={ax}) f32 16384x16384",
+                            step=lambda: hip.run(ReduceEx(np.add, a, (ax,))),
+                            cpu=lambda: ha[:N // 4].sum(axis=ax), cpu_frac=0.25)
+            if name == "rowbcast":
+                hr = rs.standard_normal(N).astype(np.float32)
+                r = dr.array(hr)
+                return dict(dtype="f32", n=N * N, nbytes=8 * N * N + 4 * N,
+                            desc="a + row (broadcast) f32 16384x16384",
+                            step=lambda: hip.run(a + r), cpu=lambda: ha[:N // 4] + hr, cpu_frac=0.25)
+            return dict(dtype="f32", n=N * N, nbytes=8 * N * N, desc="a.T * 2 f32 16384x16384",
+                        step=lambda: hip.run(a.T * 2.0),
+                        cpu=lambda: ha[:, :N // 4].T * np.float32(2.0), cpu_frac=0.25)
         raise KeyError(name)
 
     def measure(name):
@@ -247,8 +278,9 @@ def main():
         del keep, wl
         return res
 
-    names = ["horner", "saxpy", "bs32", "bs64", "jacobi", "sumsq"] if args.workload == "all" \
-        else [args.workload]
+    names = {"all": ["horner", "saxpy", "bs32", "bs64", "jacobi", "sumsq"],
+             "next": ["dot", "axis0", "axis1", "rowbcast", "transpose"]}.get(args.workload,
+                                                                             [args.workload])
     results = {}
     for name in names:
         results[name] = measure(name)
