@@ -1,0 +1,132 @@
+"""Seeded random expressions over random views, compared bit for bit with the
+NumPy oracle.  Every operation used is exact in IEEE arithmetic (+ - * / sqrt abs
+negate maximum minimum comparisons where casts), so any difference is a bug in
+tracing, lowering (flat / tile2d / tile2dv / tile2dt / nd / reductions) or code
+generation, not rounding.  Operand layouts: dense, offset slices, strided slices,
+transposes, row / column / scalar broadcasts; dtypes float32, float64, int32, int64."""
+import numpy as np
+import pytest
+
+import delayrepay_amd as dr
+from delayrepay_amd import hip
+from oracle.numpy_oracle import OracleArray
+from tests.helpers import bits_equal
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64, np.float32, np.float64, np.int32, np.int64]
+
+
+def make_host(rs, shape, dtype):
+    if np.dtype(dtype).kind == "i":
+        return rs.randint(-4, 5, shape).astype(dtype)
+    vals = rs.uniform(-2, 2, shape)
+    vals[rs.uniform(size=shape) < 0.03] = 0.0
+    return vals.astype(dtype)
+
+
+def random_leaf(rs, shape):
+    """(device lazy array, oracle array) of broadcast-compatible shape."""
+    dtype = DTYPES[rs.randint(len(DTYPES))]
+    kind = rs.randint(8)
+    if len(shape) == 1:
+        (n,) = shape
+        if kind in (0, 1, 2):
+            host, key = make_host(rs, (n,), dtype), np.s_[:]
+        elif kind in (3, 4):
+            off = rs.randint(1, 6)
+            host, key = make_host(rs, (n + off + 2,), dtype), np.s_[off:off + n]
+        elif kind == 5:
+            step = rs.randint(2, 4)
+            host, key = make_host(rs, (n * step,), dtype), np.s_[::step]
+        elif kind == 6:
+            host, key = make_host(rs, (1,), dtype), np.s_[:]
+        else:
+            host, key = make_host(rs, (n,), dtype), np.s_[::-1]
+        return dr.array(host)[key], OracleArray(host.copy())[key]
+    h, w = shape
+    if kind in (0, 1):
+        host, key, t = make_host(rs, (h, w), dtype), np.s_[:, :], False
+    elif kind == 2:
+        a, b = rs.randint(0, 3), rs.randint(0, 5)
+        host, key, t = make_host(rs, (h + a + 1, w + b + 2), dtype), np.s_[a:a + h, b:b + w], False
+    elif kind == 3:
+        host, key, t = make_host(rs, (h * 2, w * 3), dtype), np.s_[::2, ::3], False
+    elif kind == 4:
+        host, key, t = make_host(rs, (w, h), dtype), np.s_[:, :], True
+    elif kind == 5:
+        host, key, t = make_host(rs, (1, w), dtype), np.s_[:, :], False
+    elif kind == 6:
+        host, key, t = make_host(rs, (h, 1), dtype), np.s_[:, :], False
+    else:
+        host, key, t = make_host(rs, (w,), dtype), np.s_[:], False
+    d, o = dr.array(host)[key], OracleArray(host.copy())[key]
+    return (d.T, OracleArray(o.a.T)) if t else (d, o)
+
+
+UNARY = [np.negative, np.absolute, lambda x: np.sqrt(np.absolute(x)), lambda x: x * x,
+         lambda x: x.astype(np.float32), lambda x: x.astype(np.float64), lambda x: 0.5 * x,
+         lambda x: x + 1, lambda x: 3 - x, lambda x: x / 2.0]
+BINARY = [np.add, np.subtract, np.multiply, np.true_divide, np.maximum, np.minimum,
+          lambda a, b: np.where(a > b, a, b * 2), lambda a, b: np.where(a < 0, b, a),
+          lambda a, b: (a >= b).astype(np.float32) + a]
+
+
+def random_expr(rs, shape, depth):
+    if depth == 0 or rs.uniform() < 0.15:
+        return random_leaf(rs, shape)
+    if rs.uniform() < 0.35:
+        fn = UNARY[rs.randint(len(UNARY))]
+        d, o = random_expr(rs, shape, depth - 1)
+        return fn(d), fn(o)
+    fn = BINARY[rs.randint(len(BINARY))]
+    d1, o1 = random_expr(rs, shape, depth - 1)
+    d2, o2 = random_expr(rs, shape, depth - 1)
+    return fn(d1, d2), fn(o1, o2)
+
+
+def full_shape_leaf(rs, shape):
+    """A leaf that really has `shape` (so the expression's shape is not all-broadcast)."""
+    host = make_host(rs, shape, DTYPES[rs.randint(4)])
+    return dr.array(host), OracleArray(host.copy())
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_random_expression(seed):
+    rs = np.random.RandomState(1000 + seed)
+    if rs.uniform() < 0.4:
+        shape = (int(rs.choice([1, 5, 63, 64, 257, 1000, 4099])),)
+    else:
+        shape = (int(rs.choice([1, 3, 8, 33, 64, 130])), int(rs.choice([1, 4, 7, 64, 129, 260])))
+    with np.errstate(all="ignore"):
+        d, o = random_expr(rs, shape, depth=int(rs.randint(1, 5)))
+        anchor_d, anchor_o = full_shape_leaf(rs, shape)
+        d, o = d + anchor_d, o + anchor_o
+        mode = rs.randint(5)
+        if mode <= 1:
+            got, ref = d.get(), o.get()
+        elif mode == 2:                      # fused full reduction (exact for max/min)
+            got = np.asarray(dr.max(d).get())
+            ref = np.asarray(np.max(o.a))
+        elif mode == 3 and len(shape) == 2:  # axis reduction (max: order-independent)
+            axis = int(rs.randint(2))
+            got, ref = dr.max(d, axis=axis).get(), np.max(o.a, axis=axis)
+        else:                                # fused assignment into a view of a bigger array
+            pad = tuple(s + 3 for s in shape)
+            host = make_host(rs, pad, np.float64)
+            dst_d, dst_o = dr.array(host), host.copy()
+            key = tuple(slice(1, 1 + s) for s in shape)
+            dst_d[key] = d
+            dst_o[key] = o.a
+            got, ref = dst_d.get(), dst_o
+    assert bits_equal(got, np.asarray(ref)), (seed, shape, mode)
+
+
+def test_fuzz_reached_every_kernel_shape():
+    """Runs after the cases above: the kernel cache must hold every shape kind."""
+    kinds = {}
+    for key in hip._KERNELS:
+        kinds[key[0]] = kinds.get(key[0], 0) + 1
+    print("kernel kinds compiled:", kinds)
+    for kind in ("flat", "nd", "tile2d", "tile2dv", "tile2dt", "axis"):
+        assert kinds.get(kind, 0) > 0, kind
