@@ -214,12 +214,6 @@ class Tracer:
     def program(self, roots):
         return Program(self.leaf_codes, self.scalar_codes, self.ops, roots)
 
-    def deps(self):
-        seen = {}
-        for arr in self.leaves:
-            seen[id(arr.buf)] = arr.buf
-        return tuple((buf, buf.version) for buf in seen.values())
-
 
 # ---------------------------------------------------------------------------
 # kernel cache
@@ -446,9 +440,10 @@ def _fire(plan, out_ptrs, reduce_out=None):
 # evaluation entry points
 # ---------------------------------------------------------------------------
 
-def _make_plan(tracer, roots, dst=None, reduce_op=None, dry=False, axes=None):
+def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
     """Lower traced `roots` (list of (ref, code)) into a Plan.  `dst`: existing
-    destination view (single root); `dry`: placeholders instead of device memory."""
+    destination view (single root); `reduce_op`/`axes`: reduce the single root with
+    that ufunc over everything (axes None) or over those axes."""
     prog = tracer.program(roots)
     leaves = tracer.leaves
     plan = Plan()
