@@ -23,9 +23,10 @@ TUNE = {
     "ax_waves": 32768,   # aim for before the reduced extent is cut into slices
     "ax_rows": 4,        # 'row' strategy: outputs per wave (grid-stride), to amortise set-up
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
-    "ntl": 1,         # non-temporal loads  } for working sets beyond `cache_mib`;
-    "nts": 1,         # non-temporal stores } smaller ones stay cacheable
+    "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
+    "nts": 1,         # allow non-temporal stores }
     "cache_mib": 200,  # working sets up to this size are left to the 256 MB Infinity Cache
+    "ntl_mib": 320,   # inputs beyond this size are read with non-temporal loads
     "tw": 128,        # stencil tile width (elements)
     "th": 16,         # stencil tile height (rows)
     "lds": 1,         # stage shifted views through LDS (0: read them directly)
@@ -135,12 +136,16 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
         vec = widths_ok and align_ok and n >= 64
         unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
-        footprint = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
+        in_bytes = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
+        footprint = in_bytes
         if not reduce_op:
             footprint += sum(n * cg.ITEMSIZE[c] for c in out_codes)
-        streaming = footprint > TUNE["cache_mib"] << 20
-        ntl = bool(TUNE["ntl"]) and streaming
-        nts = bool(TUNE["nts"]) and streaming
+        # Cache policy, from measurement: a working set that fits the 256 MB Infinity
+        # Cache is left cacheable; beyond that outputs are written non-temporally (they
+        # are write-once streams) and inputs are read non-temporally only when they are
+        # too large to survive in the cache until a later kernel reads them again.
+        nts = bool(TUNE["nts"]) and footprint > TUNE["cache_mib"] << 20
+        ntl = bool(TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
         low.kind = "flat"
         low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
                    unroll, ntl, nts)
