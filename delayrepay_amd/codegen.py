@@ -509,16 +509,56 @@ def emit_nd(prog, ndim, out_dtypes, index32, reduce_op=None):
 
 # ---- 2-D stencil kernel with an LDS halo tile ------------------------------
 
-def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=True):
+def _row_bases(nouter, names, indent):
+    """Lines computing, for row index `i`, the element offset of that row in each
+    operand: `names` is a list of (variable, stride parameter prefix).  With one
+    outer dimension the offset is i * stride; with several, `i` is decomposed over
+    the outer extents od1.. (od0 is implied) and dotted with the operand's strides,
+    which is how N-d arrays and row/plane broadcasts are walked."""
+    pad = " " * indent
+    if nouter == 1:
+        return [f"{pad}const long long {var} = (long long)i * {sp}_0;" for var, sp in names]
+    lines = [f"{pad}long long rem_o = i;"]
+    lines += [f"{pad}long long {var} = 0;" for var, _ in names]
+    for d in reversed(range(nouter)):
+        if d == 0:
+            lines.append(f"{pad}const long long q0 = rem_o;")
+        else:
+            lines.append(f"{pad}const long long q{d} = rem_o % od{d}; rem_o /= od{d};")
+        lines += [f"{pad}{var} += q{d} * {sp}_{d};" for var, sp in names]
+    return lines
+
+
+def _outer_params(leaf_kind, n_out, nouter):
+    """Kernel parameters describing the outer dimensions: extents od1.., then the
+    outer strides of every directly read operand, then of every output."""
+    params = [f"const long long od{d}" for d in range(1, nouter)]
+    for i, k in enumerate(leaf_kind):
+        if k[0] in ("d", "dv", "r"):
+            params += [f"const long long os{i}_{d}" for d in range(nouter)]
+    for o in range(n_out):
+        params += [f"const long long oos{o}_{d}" for d in range(nouter)]
+    return params
+
+
+def _base_names(leaf_kind, n_out):
+    names = [(f"base{i}", f"os{i}") for i, k in enumerate(leaf_kind) if k[0] in ("d", "dv", "r")]
+    return names + [(f"obase{o}", f"oos{o}") for o in range(n_out)]
+
+
+def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=True, nouter=1):
     """2-D tiled kernel; operands that are shifted views of one buffer are staged
     through an LDS halo tile.
 
     leaf_kind  per leaf: ('g', dy, dx) member of the halo group, shifted by
                (dy, dx) elements from the group's reference view;
-               ('d',) separate 2-D operand with unit column stride, read directly;
+               ('d',) operand with unit stride along the last dimension, read directly;
+               ('r',) operand constant along the last dimension (column broadcast);
                ('b',) single element broadcast
     group      None, or (dtype code, dy_max, dx_min, dx_max): extent of the shifts
-               (dy in [0, dy_max], dx in [dx_min, dx_max])
+               (dy in [0, dy_max], dx in [dx_min, dx_max]); only with nouter == 1
+    nouter     number of merged dimensions in front of the last one: the kernel's
+               "rows" are their product (see `_row_bases`)
 
     The block stages the (tile_h + dy_max) x (tile_w + dx_max - dx_min) window of
     the buffer in LDS with coalesced loads, then every thread computes
@@ -545,10 +585,7 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
     if group is not None:
         params += ["const long long grs", "const long long glo", "const long long ghi"]
     params.append("const int tiles_x")
-    for i, k in enumerate(leaf_kind):
-        if k[0] == "d":
-            params.append(f"const long long rs{i}")
-    params += [f"const long long ors{o}" for o in range(n_out)]
+    params += _outer_params(leaf_kind, n_out, nouter)
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{"]
     if group is not None:
@@ -578,20 +615,23 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
           "        const int i = r0 + lr;",
           "        const int j = c0 + lc;",
           "        if (i < H && j < W) {"]
+    L += _row_bases(nouter, _base_names(leaf_kind, n_out), 12)
     args = []
     for i, k in enumerate(leaf_kind):
         if k[0] == "g":
             _, dy, dx = k
             args.append(f"tile[(lr + {dy}) * {LW} + lc + ({dx - dx_min})]")
         elif k[0] == "d":
-            args.append(f"a{i}[(long long)i * rs{i} + j]")
+            args.append(f"a{i}[base{i} + j]")
+        elif k[0] == "r":
+            args.append(f"a{i}[base{i}]")
         else:
             args.append(f"a{i}[0]")
     decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
     call = args + [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
     L.append(f"            {decl} dr_body({', '.join(call)});")
     for o in range(n_out):
-        L.append(f"            o{o}[(long long)i * ors{o} + j] = t{o};")
+        L.append(f"            o{o}[obase{o} + j] = t{o};")
     L += ["        }", "    }", "}"]
     src.append("\n".join(L))
     return "\n".join(src) + "\n"
@@ -599,7 +639,7 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
 
 def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_per_thread,
                      phase_group, phase_out, restrict=True, nt_load=False, nt_store=False,
-                     xcd_bands=True):
+                     xcd_bands=True, nouter=1):
     """Vectorised 2-D tiled kernel for the aligned case: every output's row stride
     is a multiple of the 16-byte vector width VW and all outputs start at the same
     address phase (`phase_out` = address of output [0, 0] / itemsize, mod VW).
@@ -607,7 +647,8 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
     leaf_kind  per leaf: ('g', dy, dx) member of the halo group (staged through LDS);
                ('dv',) 2-D operand whose rows have the outputs' phase and a stride
                that is a multiple of VW: read with 16-byte loads;
-               ('d',) other 2-D operand with unit column stride: element loads;
+               ('d',) other operand with unit stride along the last dimension: element
+               loads; ('r',) operand constant along the last dimension;
                ('b',) single element broadcast
     group      None, or (dtype code, dy_max, dx_min, dx_max) with the group's row
                stride a multiple of VW and `phase_group` its reference element's phase
@@ -645,10 +686,7 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
     if group is not None:
         params += ["const long long grs", "const long long glo", "const long long ghi"]
     params.append("const int tiles_x")
-    for i, k in enumerate(leaf_kind):
-        if k[0] in ("d", "dv"):
-            params.append(f"const long long rs{i}")
-    params += [f"const long long ors{o}" for o in range(n_out)]
+    params += _outer_params(leaf_kind, n_out, nouter)
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{"]
     if group is not None:
@@ -689,6 +727,7 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
           f"        const int lr = rw * {rows_per_thread} + k;",
           "        const int i = r0 + lr;",
           "        if (i >= H) break;"]
+    L += _row_bases(nouter, _base_names(leaf_kind, n_out), 8)
 
     def operand(i, k, e, vector_path):
         if k[0] == "g":
@@ -697,7 +736,9 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
         if k[0] == "dv" and vector_path:
             return f"D{i}[{e}]"
         if k[0] in ("d", "dv"):
-            return f"a{i}[(long long)i * rs{i} + jf + {e}]"
+            return f"a{i}[base{i} + jf + {e}]"
+        if k[0] == "r":
+            return f"a{i}[base{i}]"
         return f"a{i}[0]"
 
     decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
@@ -706,7 +747,7 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
     for i, k in enumerate(leaf_kind):
         if k[0] == "dv":
             lvt = VEC16[prog.leaves[i]][0]
-            ptr = f"(const {lvt}*)(a{i} + (long long)i * rs{i} + jf)"
+            ptr = f"(const {lvt}*)(a{i} + base{i} + jf)"
             L.append(f"            const {lvt} D{i} = {_ld(nt_load, ptr)};")
     for o, dt in enumerate(out_dtypes):
         L.append(f"            {VEC16[dt][0]} R{o};")
@@ -715,12 +756,11 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
         sets = " ".join(f"R{o}[{e}] = t{o};" for o in range(n_out))
         L.append(f"            {{ {decl} dr_body({', '.join(args + tail_args)}); {sets} }}")
     for o, dt in enumerate(out_dtypes):
-        L.append("            " + _st(nt_store, f"R{o}",
-                                        f"({VEC16[dt][0]}*)(o{o} + (long long)i * ors{o} + jf)"))
+        L.append("            " + _st(nt_store, f"R{o}", f"({VEC16[dt][0]}*)(o{o} + obase{o} + jf)"))
     L.append("        } else {")
     for e in range(VW):
         args = [operand(i, k, e, False) for i, k in enumerate(leaf_kind)]
-        stores = " ".join(f"o{o}[(long long)i * ors{o} + jf + {e}] = t{o};" for o in range(n_out))
+        stores = " ".join(f"o{o}[obase{o} + jf + {e}] = t{o};" for o in range(n_out))
         L.append(f"            if (jf + {e} >= 0 && jf + {e} < W) "
                  f"{{ {decl} dr_body({', '.join(args + tail_args)}); {stores} }}")
     L += ["        }", "    }", "}"]

@@ -173,19 +173,27 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             low.fin_count = low.grid
         return low
 
-    tiled = (not reduce_op and ndim == 2 and all(s[1] == 1 for s in m_out)
-             and all(s[1] == 1 or s == [0, 0] for s in m_leaf))
-    if tiled:
-        H, W = mshape
+    # Tiled family: the last merged dimension is walked with unit stride by every output
+    # and with stride 1 or 0 by every operand; the dimensions in front of it are the
+    # kernel's "rows" (decomposed per row when there are several).
+    nouter = ndim - 1
+    tiled = (not reduce_op and ndim >= 2 and all(s[-1] == 1 for s in m_out)
+             and all(s[-1] in (0, 1) for s in m_leaf))
+    rows = 1
+    for d in mshape[:-1]:
+        rows *= d
+    if tiled and rows < 2 ** 31 and mshape[-1] < 2 ** 31 - 4096:
+        H, W = rows, mshape[-1]
         tw, th = TUNE["tw"], TUNE["th"]
-        # halo group: >= 2 leaves that are shifted views of one buffer
-        groups = {}
-        for i, (a, s) in enumerate(zip(leaves, m_leaf)):
-            if s[1] == 1 and s[0] > 0:
-                groups.setdefault((id(a.buf), s[0], prog.leaves[i]), []).append(i)
-        best = max(groups.values(), key=len) if groups else []
         kinds = [None] * len(leaves)
         group = None
+        # halo group (2-D only): >= 2 leaves that are shifted views of one buffer
+        groups = {}
+        if ndim == 2:
+            for i, (a, s) in enumerate(zip(leaves, m_leaf)):
+                if s[1] == 1 and s[0] > 0:
+                    groups.setdefault((id(a.buf), s[0], prog.leaves[i]), []).append(i)
+        best = max(groups.values(), key=len) if groups else []
         if len(best) >= 2 and TUNE["lds"]:
             rs = m_leaf[best[0]][0]
             ref_off = min(leaves[i].offset for i in best)
@@ -211,7 +219,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                 g_args = [rs, -ref_off, g_buf.nbytes // itemsize - ref_off]
         for i, s in enumerate(m_leaf):
             if kinds[i] is None:
-                kinds[i] = ("b",) if s == [0, 0] else ("d",)
+                kinds[i] = ("b",) if not any(s) else ("d",) if s[-1] == 1 else ("r",)
         kinds = tuple(kinds)
         low.kind = "tile2d"
         vec_ok = False
@@ -219,7 +227,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             gsize = cg.ITEMSIZE[group[0]] if group is not None else cg.ITEMSIZE[out_codes[0]]
             vw = 16 // gsize if gsize in (4, 8) else 0
             vec_ok = (vw > 0 and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
-                      and all(s[0] % vw == 0 for s in m_out)
+                      and all(st % vw == 0 for s in m_out for st in s[:-1])
                       and len({(p // gsize) % vw for p in out_ptrs}) == 1
                       and (group is None or g_args[0] % vw == 0))
         if vec_ok:
@@ -228,54 +236,58 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             # direct operands whose rows share the outputs' alignment load as vectors
             kinds = tuple(
                 ("dv",) if (k[0] == "d" and cg.ITEMSIZE[prog.leaves[i]] == gsize
-                            and m_leaf[i][0] % vw == 0
+                            and all(st % vw == 0 for st in m_leaf[i][:-1])
                             and (leaves[i].ptr // gsize) % vw == ph_o) else k
                 for i, k in enumerate(kinds))
             gpr, rpt = TUNE["gpr"], TUNE["rpt"]
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
             bands = bool(TUNE["xcd"])
             low.key = ("tile2dv", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o,
-                       gpr, rpt, sntl, snts, bands)
+                       gpr, rpt, sntl, snts, bands, nouter)
             tw, th = gpr * vw, (cg.BLOCK // gpr) * rpt
 
             def emit():
                 return cg.emit_stencil_vec(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o,
                                            restrict=not in_place, nt_load=sntl, nt_store=snts,
-                                           xcd_bands=bands)[0]
-            W = W + ph_o          # tiles start `ph_o` columns left of the view
+                                           xcd_bands=bands, nouter=nouter)[0]
+            tiles_x = -(-(W + ph_o) // tw)     # tiles start `ph_o` columns left of the view
         else:
-            low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune)
+            low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune, nouter)
 
             def emit():
                 return cg.emit_stencil(prog, kinds, group, out_codes, tw, th,
-                                       restrict=not in_place)
+                                       restrict=not in_place, nouter=nouter)
+            tiles_x = -(-W // tw)
         low.emit = emit
-        tiles_x = -(-W // tw)
         tiles_y = -(-H // th)
-        low.grid = tiles_x * tiles_y
-        srcs = [(a.buf, a.offset * a.dtype.itemsize) for a, k in zip(leaves, kinds) if k[0] != "g"]
-        fmt = "@" + "P" * len(srcs)
-        tail_vals = []
-        if group is not None:
-            fmt += "P"
-            srcs.append(g_src)
-        fmt += "P" * len(out_ptrs) + scal_fmt + "ii"
-        tail_vals += [mshape[0], mshape[1]]
-        if group is not None:
-            fmt += "qqq"
-            tail_vals += g_args
-        fmt += "i"
-        tail_vals.append(tiles_x)
-        for k, s in zip(kinds, m_leaf):
-            if k[0] in ("d", "dv"):
-                fmt += "q"
-                tail_vals.append(s[0])
-        for s in m_out:
-            fmt += "q"
-            tail_vals.append(s[0])
-        low.fmt = fmt
-        low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
-        return low
+        if tiles_x * tiles_y < 2 ** 31:
+            low.grid = tiles_x * tiles_y
+            srcs = [(a.buf, a.offset * a.dtype.itemsize)
+                    for a, k in zip(leaves, kinds) if k[0] != "g"]
+            fmt = "@" + "P" * len(srcs)
+            tail_vals = []
+            if group is not None:
+                fmt += "P"
+                srcs.append(g_src)
+            fmt += "P" * len(out_ptrs) + scal_fmt + "ii"
+            tail_vals += [H, W]
+            if group is not None:
+                fmt += "qqq"
+                tail_vals += g_args
+            fmt += "i"
+            tail_vals.append(tiles_x)
+            fmt += "q" * (nouter - 1)
+            tail_vals += list(mshape[1:-1])
+            for k, s in zip(kinds, m_leaf):
+                if k[0] in ("d", "dv", "r"):
+                    fmt += "q" * nouter
+                    tail_vals += list(s[:-1])
+            for s in m_out:
+                fmt += "q" * nouter
+                tail_vals += list(s[:-1])
+            low.fmt = fmt
+            low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
+            return low
 
     # operands walked along the output's rows by their unit stride (transposed views)
     transposed = (not reduce_op and ndim == 2 and all(s[1] == 1 for s in m_out)

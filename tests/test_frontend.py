@@ -226,8 +226,12 @@ def test_broadcast_scalar_leaf_and_mixed_dtypes():
 
 def test_strided_and_broadcast_operands_use_nd():
     a, b = leaf((64, 1, 32), np.float64), leaf((1, 48, 32), np.float32)
-    low, src = hip.lower_only(a * b + 1)
-    assert low.kind == "nd"
+    low, src = hip.lower_only(a * b + 1)         # unit inner stride: tiled, rows = 64 * 48
+    assert low.kind == "tile2d" and "rem_o % od1" in src
+    hip.compile_source(src)
+    col = leaf((64, 1))
+    low, src = hip.lower_only(leaf((64, 32)) * col)          # column broadcast: one load per row
+    assert low.kind == "tile2d" and ("r",) in low.key[2]
     hip.compile_source(src)
     m = hip.placeholder((100, 200), np.float32)
     low, src = hip.lower_only(NPArray(m.T) * 2.0)           # transposed operand: through LDS
