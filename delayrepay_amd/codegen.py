@@ -29,6 +29,8 @@ Kernel shapes (all 256-thread blocks = 4 wave64, grid-stride):
 """
 import numpy as np
 
+from . import mathlib
+
 BLOCK = 256          # threads per block: 4 wave64
 WAVE = 64
 N_XCD = 8            # accelerator dies with private L2 on MI355X
@@ -170,16 +172,20 @@ class Program:
     roots    list of (ref, dtype code)
     """
 
-    __slots__ = ("leaves", "scalars", "ops", "roots")
+    __slots__ = ("leaves", "scalars", "ops", "roots", "own_math")
 
-    def __init__(self, leaves, scalars, ops, roots):
+    def __init__(self, leaves, scalars, ops, roots, own_math=True):
         self.leaves = tuple(leaves)
         self.scalars = tuple(scalars)
         self.ops = tuple(ops)
         self.roots = tuple(roots)
+        # float64 functions taken from `mathlib` instead of the device library
+        self.own_math = tuple(sorted({name for name, cdt, _, _ in self.ops
+                                      if cdt == "f8" and name in mathlib.FUNCTIONS})) \
+            if own_math else ()
 
     def key(self):
-        return (self.leaves, self.scalars, self.ops, self.roots)
+        return (self.leaves, self.scalars, self.ops, self.roots, self.own_math)
 
     def ref_dtype(self, ref):
         kind, i = ref
@@ -205,11 +211,14 @@ def emit_body(prog, out_dtypes, fname="dr_body"):
     params = [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
-    lines = [f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
+    lines = [mathlib.source(prog.own_math),
+             f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
     for i, (name, cdt, rdt, args) in enumerate(prog.ops):
         cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
         if name == "cast":
             expr = cargs[0]
+        elif cdt == "f8" and name in prog.own_math:
+            expr = f"{mathlib.FUNCTIONS[name][0]}({cargs[0]})"
         elif name == "where":    # the condition keeps its own type
             k, j = args[0]
             expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"

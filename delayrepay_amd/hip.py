@@ -212,7 +212,7 @@ class Tracer:
         return res
 
     def program(self, roots):
-        return Program(self.leaf_codes, self.scalar_codes, self.ops, roots)
+        return Program(self.leaf_codes, self.scalar_codes, self.ops, roots, TUNE["dmath"])
 
 
 # ---------------------------------------------------------------------------

@@ -36,6 +36,7 @@ TUNE = {
     "xcd": 1,         # vectorised stencil: give each XCD a contiguous band of tiles
     "sntl": 0,        # vectorised stencil: non-temporal loads / stores
     "snts": 1,
+    "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
 }
 for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
     _k, _v = _kv.split("=")

@@ -1,0 +1,147 @@
+"""Accuracy of the double-precision device math functions, on the CPU.
+
+`mathlib.source(..., HOST_MACROS)` is the same text the kernels include, with the
+reciprocal seed and the scalar-constant multiply-add spelled in plain C; it is built
+here with gcc and compared with 40-digit values (mpmath) and with libm / SciPy.
+The device build of the same text is checked against NumPy in the GPU tests."""
+import ctypes
+import subprocess
+
+import mpmath as mp
+import numpy as np
+import pytest
+import scipy.special
+
+from delayrepay_amd import hip, mathlib
+
+
+@pytest.fixture(scope="module")
+def host(tmp_path_factory):
+    d = tmp_path_factory.mktemp("mathlib")
+    src = mathlib.source(sorted(mathlib.FUNCTIONS), mathlib.HOST_MACROS)
+    for name, (fn, _) in mathlib.FUNCTIONS.items():
+        src += (f"void v_{name}(const double* x, double* y, long n)\n"
+                f"{{ for (long i = 0; i < n; i++) y[i] = {fn}(x[i]); }}\n")
+    (d / "m.c").write_text(src)
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
+                    str(d / "m.c"), "-lm"], check=True)
+    lib = ctypes.CDLL(str(d / "m.so"))
+
+    def call(name, x):
+        x = np.ascontiguousarray(x, dtype=np.float64)
+        y = np.empty_like(x)
+        getattr(lib, "v_" + name)(x.ctypes.data_as(ctypes.c_void_p),
+                                  y.ctypes.data_as(ctypes.c_void_p), ctypes.c_long(x.size))
+        return y
+    return call
+
+
+def ulp_error(got, x, exact):
+    """Largest |got - exact(x)| in units of the last place of the exact value."""
+    mp.mp.dps = 40
+    worst = 0.0
+    for g, v in zip(got, x):
+        e = exact(mp.mpf(float(v)))
+        if e == 0:
+            assert g == 0
+            continue
+        worst = max(worst, float(abs(mp.mpf(float(g)) - e) / mp.mpf(float(np.spacing(abs(float(e)))))))
+    return worst
+
+
+def test_log_accuracy_over_the_whole_range(host):
+    rs = np.random.RandomState(3)
+    x = np.concatenate([rs.uniform(1e-6, 1e6, 1 << 18), np.exp(rs.uniform(-744, 709, 1 << 18)),
+                        rs.uniform(0.5, 2, 1 << 18), 1 + rs.uniform(-1e-6, 1e-6, 1 << 16),
+                        [5e-324, 2.2250738585072014e-308, 1e-310, 1.0, np.nextafter(1, 2),
+                         np.nextafter(1, 0), 1.7976931348623157e308, 0.7071067811865475,
+                         0.7071067811865476, 1.4142135623730951]])
+    got = host("log", x)
+    ref = np.log(x)
+    assert np.max(np.abs(got - ref) / np.spacing(np.abs(ref))) <= 1.0      # libm itself: < 1 ulp
+    pick = np.r_[rs.choice(x.size - 10, 6000, replace=False), np.arange(x.size - 10, x.size)]
+    assert ulp_error(got[pick], x[pick], mp.log) <= 0.8
+
+
+def test_log_special_values(host):
+    got = host("log", [0.0, -0.0, -1.0, -np.inf, np.inf, np.nan, 1.0])
+    assert got[0] == -np.inf and got[1] == -np.inf
+    assert np.isnan(got[2]) and np.isnan(got[3]) and np.isnan(got[5])
+    assert got[4] == np.inf and got[6] == 0.0 and not np.signbit(got[6])
+
+
+def test_erf_accuracy(host):
+    rs = np.random.RandomState(4)
+    x = np.concatenate([rs.uniform(-6.5, 6.5, 1 << 19), rs.uniform(-1, 1, 1 << 18),
+                        rs.uniform(0.9, 1.1, 1 << 16), 10.0 ** rs.uniform(-300, 1, 1 << 16),
+                        [1.0, -1.0, np.nextafter(1, 0), np.nextafter(1, 2), 5.9, 6.0, 6.1,
+                         27.0, 1e300, 5e-324, 1e-310]])
+    got = host("erf", x)
+    ref = scipy.special.erf(x)
+    assert np.max(np.abs(got - ref) / np.spacing(np.abs(ref))) <= 3.5      # SciPy's is off by up to 2.6
+    assert np.all(np.abs(got) <= 1.0)
+    pick = np.r_[rs.choice(x.size - 11, 6000, replace=False), np.arange(x.size - 11, x.size)]
+    assert ulp_error(got[pick], x[pick], mp.erf) <= 1.0
+    # odd and monotone across the switch between the two branches
+    assert np.array_equal(host("erf", -x), -got)
+    near = np.sort(rs.uniform(1 - 1e-9, 1 + 1e-9, 4096))
+    assert np.all(np.diff(host("erf", near)) >= -np.spacing(1.0))
+
+
+def test_erf_special_values(host):
+    got = host("erf", [0.0, -0.0, np.inf, -np.inf, np.nan, 40.0, -40.0])
+    assert got[0] == 0 and not np.signbit(got[0]) and got[1] == 0 and np.signbit(got[1])
+    assert got[2] == 1 and got[3] == -1 and np.isnan(got[4]) and got[5] == 1 and got[6] == -1
+
+
+def test_exp_accuracy_and_limits(host):
+    rs = np.random.RandomState(5)
+    x = np.concatenate([rs.uniform(-20, 20, 1 << 18), rs.uniform(-745, 709.78, 1 << 18),
+                        rs.uniform(-1e-3, 1e-3, 1 << 16),
+                        [0.0, -0.0, 1.0, -1.0, 709.782712893384, 709.7827128933841, -708.3964185322641,
+                         -745.1332191019411, -745.1332191019412, -744.0, 1e-320, 0.5 * np.log(2)]])
+    got = host("exp", x)
+    with np.errstate(over="ignore"):
+        ref = np.exp(x)
+    assert np.array_equal(np.isinf(got), np.isinf(ref))
+    normal = (ref >= np.finfo(np.float64).tiny) & np.isfinite(ref)
+    assert np.max(np.abs(got[normal] - ref[normal]) / np.spacing(ref[normal])) <= 1.0
+    small = ref < np.finfo(np.float64).tiny
+    assert np.max(np.abs(got[small] - ref[small]) / 5e-324) <= 1.0              # denormal results: one step
+    pick = np.r_[rs.choice(x.size - 12, 6000, replace=False), np.arange(x.size - 12, x.size)]
+    pick = pick[normal[pick]]
+    assert ulp_error(got[pick], x[pick], mp.exp) <= 1.0
+    got = host("exp", [np.inf, -np.inf, np.nan, 710.0, 1e300, -746.0, -1e300, 0.0])
+    assert got[0] == np.inf and got[1] == 0 and np.isnan(got[2]) and got[3] == np.inf
+    assert got[4] == np.inf and got[5] == 0 and got[6] == 0 and got[7] == 1.0
+
+
+def test_device_source_compiles():
+    src = mathlib.source(["log", "erf", "exp"])
+    assert src.count("DR_FMA_K(") > 40 and src.count("dr_exp_reduced(double") == 1
+    kernel = ('extern "C" __global__ void k(const double* a, double* o)\n'
+              "{ int i = threadIdx.x; o[i] = dr_log_f8(a[i]) + dr_erf_f8(a[i]) + dr_exp_f8(a[i]); }\n")
+    assert len(hip.compile_source(src + kernel)) > 0
+
+
+def test_programs_name_the_functions_they_replace():
+    from delayrepay_amd.codegen import Program
+    ops = [("log", "f8", "f8", (("l", 0),)), ("erf", "f4", "f4", (("l", 1),))]
+    prog = Program(["f8", "f4"], [], ops, [(("v", 0), "f8")])
+    assert prog.own_math == ("log",)                 # float32 keeps the device library's erf
+    plain = Program(["f8", "f4"], [], ops, [(("v", 0), "f8")], own_math=False)
+    assert plain.own_math == () and plain.key() != prog.key()
+
+
+def test_coefficients_are_the_ones_the_fit_script_prints(capsys):
+    import re
+    from delayrepay_amd import mathlib_fit
+    mathlib_fit.main()
+    printed = set(re.findall(r"-?0x1\.[0-9a-f]+p[+-]\d+", capsys.readouterr().out))
+    used = set()
+    for _, pieces in mathlib.FUNCTIONS.values():
+        for piece in pieces:
+            used |= set(re.findall(r"-?0x1\.[0-9a-f]+p[+-]\d+", piece))
+    printed |= {"-" + h for h in printed}                       # -ln 2 (hi, lo)
+    assert used - printed == {"0x1.6a09e667f3bcdp-1"}            # sqrt(1/2)
+    assert float.fromhex("0x1.6a09e667f3bcdp-1") == np.sqrt(0.5)
