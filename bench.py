@@ -57,7 +57,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all",
                     help="horner (headline) | saxpy | bs32 | bs64 | jacobi | sumsq | all (these six); "
-                         "dot | axis0 | axis1 | rowbcast | transpose | next (these five: the "
+                         "dot | axis0 | axis1 | rowbcast | transpose | grid | next (these six: the "
                          "operations either side of the five configurations)")
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before each timed region (clock ramp-up)")
@@ -146,6 +146,16 @@ def main():
             return dict(dtype="f64", n=n, nbytes=16 * n, desc="dot(x, y) f64 n=2^27 (fused multiply-reduce)",
                         step=lambda: hip.run(ReduceEx(np.add, x * y)),
                         cpu=lambda: np.dot(hx[:n // 4], hy[:n // 4]), cpu_frac=0.25)
+        if name == "grid":
+            n = 1 << 26
+            c = orc.make_inputs("horner")["c"]
+            g = dr.linspace(-2.0, 2.0, n, dtype=np.float32)     # lazy: computed inside the kernel
+            m = n // 16
+            return dict(dtype="f32", n=n, nbytes=4 * n,
+                        desc="Horner degree-8 on linspace(-2, 2, n) f32 n=2^26 (grid generated in the kernel)",
+                        step=lambda: hip.run(horner_expr(c, g)),
+                        cpu=lambda: orc.horner(c, np.linspace(-2.0, 2.0, m, dtype=np.float32)),
+                        cpu_frac=1 / 16)
         if name in ("axis0", "axis1", "rowbcast", "transpose"):
             N = 16384
             ha = rs.standard_normal((N, N)).astype(np.float32)
@@ -279,7 +289,7 @@ def main():
         return res
 
     names = {"all": ["horner", "saxpy", "bs32", "bs64", "jacobi", "sumsq"],
-             "next": ["dot", "axis0", "axis1", "rowbcast", "transpose"]}.get(args.workload,
+             "next": ["dot", "axis0", "axis1", "rowbcast", "transpose", "grid"]}.get(args.workload,
                                                                              [args.workload])
     results = {}
     for name in names:

@@ -172,7 +172,7 @@ class Program:
     roots    list of (ref, dtype code)
     """
 
-    __slots__ = ("leaves", "scalars", "ops", "roots", "own_math")
+    __slots__ = ("leaves", "scalars", "ops", "roots", "own_math", "uses_index")
 
     def __init__(self, leaves, scalars, ops, roots, own_math=True):
         self.leaves = tuple(leaves)
@@ -183,6 +183,8 @@ class Program:
         self.own_math = tuple(sorted({name for name, cdt, _, _ in self.ops
                                       if cdt == "f8" and name in mathlib.FUNCTIONS})) \
             if own_math else ()
+        # 'iota' operations read the element index: only the flat kernel supplies it
+        self.uses_index = any(name == "iota" for name, _, _, _ in self.ops)
 
     def key(self):
         return (self.leaves, self.scalars, self.ops, self.roots, self.own_math)
@@ -208,7 +210,8 @@ def emit_body(prog, out_dtypes, fname="dr_body"):
     """Inline device function evaluating the whole program for one element.
 
     Parameters: leaf values, scalar values, then one reference per root."""
-    params = [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
+    params = ["const long long dr_i"] if prog.uses_index else []
+    params += [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
     lines = [mathlib.source(prog.own_math),
@@ -217,6 +220,8 @@ def emit_body(prog, out_dtypes, fname="dr_body"):
         cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
         if name == "cast":
             expr = cargs[0]
+        elif name == "iota":
+            expr = f"({CTYPE[cdt]})dr_i"
         elif cdt == "f8" and name in prog.own_math:
             expr = f"{mathlib.FUNCTIONS[name][0]}({cargs[0]})"
         elif name == "where":    # the condition keeps its own type
@@ -387,7 +392,8 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                     args.append(f"L{i}{tag}")
             outs = [f"t{o}" for o in range(n_out)]
             decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
-            call = f"dr_body({', '.join(args + scal + outs)});"
+            index = [f"({idx}) * {E} + {e}" if vec else f"({idx})"] if prog.uses_index else []
+            call = f"dr_body({', '.join(index + args + scal + outs)});"
             if reduce_op:
                 tail = f"acc{e} = {_combine(reduce_op, f'acc{e}', 't0')};"
             elif vec:
@@ -435,6 +441,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
         L.append(f"    const long long t = nvec * {E} + (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
         L.append("    if (t < n) {")
         args = [f"b{i}" if c == "b" else f"a{i}[t]" for i, c in enumerate(leaf_class)]
+        args = (["t"] if prog.uses_index else []) + args
         decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
         outs = [f"t{o}" for o in range(n_out)]
         L.append(f"        {decl} dr_body({', '.join(args + scal + outs)});")

@@ -11,6 +11,7 @@ from .visitor import Visitor
 
 np = numpy
 fallback = numpy
+GENERATED_LEAVES = True     # FullEx / IotaEx nodes are understood
 
 
 def is_ndarray(arr):
@@ -31,6 +32,14 @@ class CpuVisitor(Visitor):
     visit_BinaryFuncEx = _apply
     visit_BinaryNumpyEx = _apply
     visit_WhereEx = _apply
+
+    def visit_FullEx(self, node):
+        arr = node.__dict__.get("array")      # once forced it is an ordinary array
+        return arr if arr is not None else numpy.full(node.shape, node.val, dtype=node.dtype)
+
+    def visit_IotaEx(self, node):
+        arr = node.__dict__.get("array")
+        return arr if arr is not None else numpy.arange(node.shape[0]).astype(node.dtype)
 
     def visit_CastEx(self, node):
         return self.visit(node.children[0]).astype(node.dtype)

@@ -26,6 +26,7 @@ or bounded memory:
   * `dst[key] = lazy_expression` is handed to the backend as one fused write;
   * `evaluate(a, b, ...)` computes several roots in one kernel.
 """
+import math
 import numbers
 import weakref
 
@@ -731,6 +732,68 @@ class Scalar(NumpyEx):
         return {}
 
 
+class _Generated(NumpyEx):
+    """Base of leaves that are computed from the element index instead of read from
+    memory.  Every call makes a new node (never hash-consed): like any new array it
+    may be written to later, and two arrays must not share such a write."""
+
+    _serial = 0
+
+    @classmethod
+    def _memo_key(cls, *args):
+        _Generated._serial += 1
+        return (cls, _Generated._serial)
+
+    @property
+    def version(self):
+        """Results computed from this node while it was still lazy list it among their
+        dependencies, like a buffer, with version 0; once it has become an array it
+        may be written to, and those results are computed afresh."""
+        return 1 if "array" in self.__dict__ else 0
+
+    def _force(self):
+        arr = self.__dict__.get("array")
+        if arr is None:
+            arr = self.array = _backend.run(self)
+            self.__dict__.pop("_deps", None)     # from now on an array in its own right
+        return arr
+
+    @property
+    def inputs(self):
+        return {}
+
+
+class FullEx(_Generated):
+    """`full(shape, value)` (and `zeros`, `ones`) that has not been written to: inside
+    an expression it is a scalar kernel parameter and costs no memory traffic;
+    asked for on its own, or indexed, or assigned to, it becomes an ordinary array
+    (delayarray.py:596-604 allocate and fill at once)."""
+
+    def __init__(self, shape, val, dtype):
+        super().__init__()
+        self.shape = tuple(shape)
+        self.dtype = np.dtype(dtype)
+        self.val = self.dtype.type(val)
+
+    @property
+    def name(self):
+        return f"full{self._count}"
+
+
+class IotaEx(_Generated):
+    """0, 1, 2, ... n-1 in `dtype`: the index sequence `arange` and `linspace` are
+    built on.  Costs no memory traffic inside a 1-d expression of the same length."""
+
+    def __init__(self, n, dtype):
+        super().__init__()
+        self.shape = (int(n),)
+        self.dtype = np.dtype(dtype)
+
+    @property
+    def name(self):
+        return f"iota{self._count}"
+
+
 def _binary(func, left, right):
     if not isinstance(left, DelayArray):
         left = arg_to_numpy_ex(left)
@@ -966,3 +1029,131 @@ for _name in ("empty", "empty_like", "eye", "identity", "ones", "ones_like", "ze
     if _fn is not None:
         globals()[_name] = cast(_fn)
 del _name, _fn
+
+# Generated leaves: constant and index-valued arrays stay lazy when the backend can
+# compute them inside a kernel.  Arrays shorter than this are made at once, as before.
+GENERATE_FROM = 4096
+_eager_create = {k: globals()[k] for k in ("zeros", "ones", "full", "zeros_like", "ones_like",
+                                           "full_like", "arange", "linspace") if k in globals()}
+_GENERATES = bool(getattr(_backend, "GENERATED_LEAVES", False))
+
+
+def _shape_of(shape):
+    if isinstance(shape, (int, np.integer)):
+        return (int(shape),)
+    return tuple(int(d) for d in shape)
+
+
+def _lazy_full(shape, val, dtype):
+    """FullEx when that is worth it and the value fits the dtype; else None."""
+    if not _GENERATES:
+        return None
+    try:
+        shape = _shape_of(shape)
+        dtype = np.dtype(dtype)
+    except TypeError:
+        return None
+    size = 1
+    for d in shape:
+        size *= d
+    if size < GENERATE_FROM or dtype.kind not in "fiub" or dtype.itemsize > 8 \
+            or dtype == np.float16 or not isinstance(val, (numbers.Real, np.bool_)):
+        return None
+    return FullEx(shape, val, dtype)
+
+
+def zeros(shape, dtype=float, **kwargs):
+    node = None if kwargs.get("like") is not None else _lazy_full(shape, 0, dtype)
+    return node if node is not None else _eager_create["zeros"](shape, dtype=dtype, **kwargs)
+
+
+def ones(shape, dtype=float, **kwargs):
+    node = None if kwargs.get("like") is not None else _lazy_full(shape, 1, dtype)
+    return node if node is not None else _eager_create["ones"](shape, dtype=dtype, **kwargs)
+
+
+def full(shape, fill_value, dtype=None, **kwargs):
+    node = None
+    if kwargs.get("like") is None and isinstance(fill_value, (numbers.Real, np.bool_)):
+        node = _lazy_full(shape, fill_value, np.asarray(fill_value).dtype if dtype is None else dtype)
+    return node if node is not None else _eager_create["full"](shape, fill_value, dtype=dtype, **kwargs)
+
+
+def _like(name, val):
+    def create(a, *args, dtype=None, shape=None, **kwargs):
+        if name == "full_like":
+            (fill,), args = args[:1], args[1:]
+        else:
+            fill = val
+        if not args and hasattr(a, "shape") and hasattr(a, "dtype"):
+            node = _lazy_full(a.shape if shape is None else shape, fill,
+                              a.dtype if dtype is None else dtype)
+            if node is not None:
+                return node
+        extra = (fill,) if name == "full_like" else ()
+        return _eager_create[name](_unwrap(a), *extra, *args, dtype=dtype, shape=shape, **kwargs)
+
+    create.__name__ = name
+    return create
+
+
+zeros_like = _like("zeros_like", 0)
+ones_like = _like("ones_like", 1)
+full_like = _like("full_like", None)
+
+
+def arange(*args, **kwargs):
+    """NumPy's `arange`; long ranges of Python numbers stay lazy.  NumPy fills element
+    0 with `start`, element 1 with `start + step` (both computed in Python and then
+    converted), and element i >= 2 with `start + i*delta` in the array's own type,
+    where `delta` is the difference of the first two; so does this."""
+    lazy = _GENERATES and 1 <= len(args) <= 3 and set(kwargs) <= {"dtype"} \
+        and all(type(a) in (int, float) for a in args)
+    if lazy:
+        start, stop, step = (0, args[0], 1) if len(args) == 1 else (tuple(args) + (1,))[:3]
+        dtype = kwargs.get("dtype")
+        dtype = np.dtype(dtype) if dtype is not None else np.result_type(*args)
+        lazy = step != 0 and dtype in (np.float32, np.float64, np.int32, np.int64) \
+            and all(np.isfinite(a) for a in (start, stop, step))
+    if lazy:
+        n = math.ceil((stop - start) / step)
+        lazy = n >= GENERATE_FROM
+    if lazy and dtype.kind == "i":
+        info = np.iinfo(dtype)
+        lazy = all(type(a) is int for a in (start, stop, step)) \
+            and all(info.min <= v <= info.max for v in (start, start + (n - 1) * step))
+    if not lazy:
+        return _eager_create["arange"](*args, **kwargs)
+    first, second = dtype.type(start), dtype.type(start + step)
+    idx = IotaEx(n, dtype)
+    if dtype.kind == "i":
+        return first + idx * dtype.type(step)
+    with np.errstate(all="ignore"):
+        delta = dtype.type(second - first)
+    return where(idx == dtype.type(1), second, first + idx * delta)
+
+
+def linspace(start, stop, num=50, endpoint=True, retstep=False, dtype=None, axis=0, **kwargs):
+    """NumPy's `linspace`; long ones between Python numbers stay lazy: element i is
+    `i*step + start` in float64 with `step = (stop - start)/div`, the last one is
+    `stop` itself, then everything is converted to `dtype`."""
+    lazy = _GENERATES and not retstep and axis == 0 and not kwargs \
+        and type(start) in (int, float) and type(stop) in (int, float) \
+        and isinstance(num, (int, np.integer)) and num >= GENERATE_FROM \
+        and np.isfinite(start) and np.isfinite(stop) \
+        and (dtype is None or np.dtype(dtype) in (np.float32, np.float64))
+    if lazy:
+        div = num - 1 if endpoint else num
+        delta = np.float64(stop) - np.float64(start)
+        step = delta / div
+        lazy = step != 0 and np.isfinite(step)
+    if not lazy:
+        return _eager_create["linspace"](start, stop, num=num, endpoint=endpoint, retstep=retstep,
+                                         dtype=dtype, axis=axis, **kwargs)
+    idx = IotaEx(num, np.float64)
+    y = idx * step + np.float64(start)
+    if endpoint:
+        y = where(idx == np.float64(num - 1), np.float64(stop), y)
+    if dtype is not None and np.dtype(dtype) != np.float64:
+        y = y.astype(dtype)
+    return y

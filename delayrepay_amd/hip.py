@@ -65,6 +65,9 @@ def set_tune(**kwargs):
     _STAMP += 1
 
 
+GENERATED_LEAVES = True     # FullEx / IotaEx nodes are computed inside kernels
+
+
 def is_ndarray(arr):
     return isinstance(arr, ndarray)
 
@@ -118,6 +121,8 @@ class Tracer:
         self._memo = {}
         self._evaluated = evaluated if evaluated is not None else {}
         self.leaf_nodes = []      # (node, its array, the deps it was computed from or None)
+        self.gen_shapes = []      # shapes of generated leaves (they take part in broadcasting)
+        self.iotas = []           # index-valued generated leaves
 
     def leaf(self, arr):
         code = _code_of(arr.dtype)
@@ -206,10 +211,31 @@ class Tracer:
             res = self.op("cast", target, target, [ref]) if code != target else (ref, code)
         elif kind is _FE.ReduceEx:
             res = self.leaf(node._force())
+        elif kind is _FE.FullEx:      # a constant array is a scalar parameter
+            res = self.scalar(node.val, _code_of(node.dtype), nid)
+            self.gen_shapes.append(node.shape)
+            self.leaf_nodes.append((node, None, None))   # the plan holds while it stays unwritten
+        elif kind is _FE.IotaEx:      # the element index, converted
+            code = _code_of(node.dtype)
+            res = self.op("iota", code, code, [])
+            self.gen_shapes.append(node.shape)
+            self.iotas.append((res[0][1], node))
+            self.leaf_nodes.append((node, None, None))
         else:
             raise NotImplementedError(f"{kind.__name__} nodes cannot be evaluated by the HIP backend")
         memo[nid] = res
         return res
+
+    def materialise_indices(self):
+        """Turn every index-valued leaf into an array that is read like any other
+        (for kernels that do not walk a 1-d array of exactly that length)."""
+        for k, node in self.iotas:
+            arr = node._force()
+            ref, code = self.leaf(arr)
+            self.ops[k] = ("positive", code, code, (ref,))
+            self.leaf_nodes = [entry for entry in self.leaf_nodes if entry[0] is not node]
+            self.leaf_nodes.append((node, arr, node.__dict__.get("_deps")))
+        self.iotas = []
 
     def program(self, roots):
         return Program(self.leaf_codes, self.scalar_codes, self.ops, roots, TUNE["dmath"])
@@ -388,7 +414,8 @@ class Plan:
         seen = {}
         for arr in self.leaves:
             seen[id(arr.buf)] = arr.buf
-        return tuple((buf, buf.version) for buf in seen.values())
+        lazy = tuple((node, 0) for node, arr, _ in self.checks if arr is None)   # generated leaves
+        return tuple((buf, buf.version) for buf in seen.values()) + lazy
 
 
 def _fire(plan, out_ptrs, reduce_out=None):
@@ -444,6 +471,13 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
     """Lower traced `roots` (list of (ref, code)) into a Plan.  `dst`: existing
     destination view (single root); `reduce_op`/`axes`: reduce the single root with
     that ufunc over everything (axes None) or over those axes."""
+    if tracer.iotas:
+        # the element index is at hand only in the flat kernel, over a 1-d array
+        shape = dst.shape if dst is not None else tuple(numpy.broadcast_shapes(
+            *[a.shape for a in tracer.leaves], *tracer.gen_shapes))
+        if axes is not None or len(shape) != 1 or (dst is not None and dst._strides != (1,)) \
+                or any(node.shape != shape for _, node in tracer.iotas):
+            tracer.materialise_indices()
     prog = tracer.program(roots)
     leaves = tracer.leaves
     plan = Plan()
@@ -460,7 +494,7 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
     plan.kern2 = None
     plan.scratch = 0
     if reduce_op:
-        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
+        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves], *tracer.gen_shapes))
         code = roots[0][1]
         plan.acc = "i8" if (reduce_op == "add" and code in ("i4", "u4", "u1", "b1")) else code
         plan.out_dtypes = [code_dtype(plan.acc)]
@@ -496,9 +530,12 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
             plan.low = None
             return plan
         plan.low = _lower(prog, leaves, tracer.scalars, shape, [plan.acc], [], [], reduce_op)
+        if tracer.iotas and plan.low.kind != "flat":
+            tracer.materialise_indices()
+            return _make_plan(tracer, roots, None, reduce_op)
         return plan
     if dst is None:
-        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves])) if leaves else ()
+        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves], *tracer.gen_shapes))
         plan.out_dtypes = [code_dtype(code) for _, code in roots]
         out_codes = [code for _, code in roots]
         out_ptrs = [0] * len(roots)          # pool blocks are 256-byte aligned
@@ -521,6 +558,9 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
         return plan
     plan.low = _lower(prog, leaves, tracer.scalars, shape, out_codes, out_ptrs, out_strides, None,
                       in_place)
+    if tracer.iotas and plan.low.kind != "flat":
+        tracer.materialise_indices()
+        return _make_plan(tracer, roots, dst)
     return plan
 
 

@@ -53,6 +53,41 @@ SCRIPT = textwrap.dedent("""
     assert np.array_equal(p.get(), np.arange(12.0).reshape(3, 4) + 1)
     assert np.array_equal(np.where(a > 5, a, 0.0).get(), np.where(np.arange(12.0).reshape(3, 4) > 5,
                                                                    np.arange(12.0).reshape(3, 4), 0.0))
+
+    # generated leaves: long constant / index arrays stay lazy and give NumPy's exact bits
+    from delayrepay.delayarray import FullEx, WhereEx, BinaryNumpyEx
+    same = lambda got, ref: (got.dtype == ref.dtype and got.shape == ref.shape
+                             and got.tobytes() == ref.tobytes())
+    for args in [(10000,), (3, 20000), (0.0, 1000.0, 0.1), (1.5, 9000.25, 0.7), (5000, 0, -1),
+                 (10.0, -700.0, -0.07), (0.1, 1e4, 0.3)]:
+        for kw in ({}, {"dtype": np.float32}, {"dtype": np.float64}, {"dtype": np.int64}):
+            if kw.get("dtype") == np.int64 and any(isinstance(v, float) for v in args):
+                continue
+            lazy = dnp.arange(*args, **kw)
+            assert type(lazy) in (WhereEx, BinaryNumpyEx), (args, kw)
+            assert same(lazy.get(), np.arange(*args, **kw)), (args, kw)
+    for lo, hi, n, ep in [(0, 1, 10000, True), (-2.0, 2.0, 65537, True), (0.1, 1e6, 5000, False),
+                          (3, -3, 4096, True)]:
+        for dt in (None, np.float32, np.float64):
+            lazy = dnp.linspace(lo, hi, n, endpoint=ep, dtype=dt)
+            assert not isinstance(lazy, NPArray)
+            assert same(lazy.get(), np.linspace(lo, hi, n, endpoint=ep, dtype=dt)), (lo, hi, n, ep, dt)
+    assert isinstance(dnp.arange(10), NPArray) and isinstance(dnp.linspace(0, 1, 50), NPArray)
+    assert isinstance(dnp.arange(np.float32(0), 9000), NPArray)          # NumPy scalars: eager
+    assert same(dnp.linspace(0, 1, 5000, retstep=False, dtype=np.int64).get(),
+                np.linspace(0, 1, 5000, dtype=np.int64))
+    z = dnp.zeros((100, 100))
+    assert type(z) is FullEx and z.shape == (100, 100) and z.dtype == np.float64
+    assert dnp.zeros((100, 100)) is not z                                 # never shared
+    y = z + 1.5
+    assert same(y.get(), np.full((100, 100), 1.5))
+    z[1:3, 1:3] = 7.0                                                     # becomes a real array
+    expect = np.zeros((100, 100)); expect[1:3, 1:3] = 7.0
+    assert same(z.get(), expect) and same((z + 1).get(), expect + 1)
+    assert same(dnp.ones_like(y).get(), np.ones((100, 100)))
+    assert same(dnp.full((5000,), 3, dtype=np.int32).get(), np.full(5000, 3, np.int32))
+    assert same(dnp.full_like(y, 2.5, dtype=np.float32).get(), np.full((100, 100), 2.5, np.float32))
+    assert isinstance(dnp.zeros(8), NPArray) and isinstance(dnp.full((3,), "a"), NPArray)
     print("cpu-backend-ok")
 """)
 

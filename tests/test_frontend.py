@@ -14,8 +14,8 @@ import pytest
 import delayrepay_amd as dr
 from delayrepay_amd import codegen as cg
 from delayrepay_amd import hip, hiprt, mathlib
-from delayrepay_amd.delayarray import (BinaryFuncEx, BinaryNumpyEx, CastEx, NPArray, ReduceEx,
-                                       Scalar, UnaryFuncEx, Memoiser)
+from delayrepay_amd.delayarray import (BinaryFuncEx, BinaryNumpyEx, CastEx, FullEx, IotaEx, NPArray,
+                                       ReduceEx, Scalar, UnaryFuncEx, Memoiser)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -322,3 +322,35 @@ def test_launching_on_placeholders_is_refused():
     a = leaf((16,))
     with pytest.raises(Exception):
         (a + 1).get()
+
+
+def test_generated_leaves_cost_no_operand():
+    """`zeros/ones/full` are scalar parameters, `arange/linspace` are computed from the
+    element index: neither adds a pointer to the kernel."""
+    n = 1 << 20
+    x = leaf((n,), np.float32)
+    grid = dr.linspace(-2.0, 2.0, n, dtype=np.float32)
+    low, src = hip.lower_only(grid * x + dr.ones(n, dtype=np.float32))
+    assert low.kind == "flat" and len(low.srcs) == 1
+    assert "const long long dr_i" in src and "(double)dr_i" in src
+    assert src.count("const float* __restrict__ a") == 1
+    hip.compile_source(src)
+    low, src = hip.lower_only(dr.arange(n))                      # no operand at all
+    assert low.kind == "flat" and len(low.srcs) == 0 and "(long long)dr_i" in src
+    hip.compile_source(src)
+    low, src = hip.lower_only(dr.zeros((1 << 10, 1 << 10), dtype=np.float32))
+    assert low.kind == "flat" and len(low.srcs) == 0 and "dr_i" not in src
+    hip.compile_source(src)
+    # element-wise use next to a 2-d array: still no operand for the constant
+    m = leaf((1 << 10, 1 << 10), np.float32)
+    low, src = hip.lower_only(dr.zeros((1 << 10, 1 << 10), dtype=np.float32) + m * 2)
+    assert low.kind == "flat" and len(low.srcs) == 1
+
+
+def test_generated_leaves_are_never_shared_and_small_ones_are_eager():
+    a, b = dr.zeros(1 << 16), dr.zeros(1 << 16)
+    assert type(a) is FullEx and a is not b and (a + 1) is not (b + 1)
+    assert type(dr.arange(1 << 16).children[1].children[0]) is IotaEx
+    assert dr.arange(0, 1 << 16, 2).shape == (1 << 15,) and dr.arange(0.0, 10.0, 0.001).dtype == np.float64
+    assert dr.linspace(0, 1, 1 << 16).shape == (1 << 16,)
+    assert dr.linspace(0, 1, 1 << 16, dtype=np.float32).dtype == np.float32

@@ -598,3 +598,89 @@ def test_transposed_operands_go_through_lds_and_match():
     c = dr.array(c0)
     assert bits_equal((c.transpose(2, 0, 1) * 1.5).get(), c0.transpose(2, 0, 1) * 1.5)   # general nd
     assert bits_equal((c.transpose(1, 0, 2) + 1).get(), c0.transpose(1, 0, 2) + 1)
+
+
+# ---- generated leaves: constant and index-valued arrays computed inside the kernel ------------
+
+def _same(got, ref):
+    return got.dtype == ref.dtype and got.shape == ref.shape and got.tobytes() == ref.tobytes()
+
+
+@pytest.mark.parametrize("args", [(100000,), (3, 200001), (0.0, 1000.0, 0.01), (1.5, 90000.25, 0.7),
+                                  (50000, 0, -1), (10.0, -7000.0, -0.07), (0.1, 1e5, 0.3)])
+def test_arange_is_numpys_to_the_bit(args):
+    for kw in ({}, {"dtype": np.float32}, {"dtype": np.float64}, {"dtype": np.int64},
+               {"dtype": np.int32}):
+        if kw.get("dtype") in (np.int64, np.int32) and any(isinstance(v, float) for v in args):
+            continue
+        lazy = dr.arange(*args, **kw)
+        assert not isinstance(lazy, dr.NPArray)
+        assert _same(lazy.get(), np.arange(*args, **kw)), (args, kw)
+
+
+def test_linspace_is_numpys_to_the_bit():
+    for lo, hi, n, ep in [(0, 1, 10000, True), (-2.0, 2.0, (1 << 20) + 1, True),
+                          (0.1, 1e6, 5001, False), (3, -3, 4096, True)]:
+        for dt in (None, np.float32, np.float64):
+            lazy = dr.linspace(lo, hi, n, endpoint=ep, dtype=dt)
+            assert not isinstance(lazy, dr.NPArray)
+            assert _same(lazy.get(), np.linspace(lo, hi, n, endpoint=ep, dtype=dt)), (lo, hi, n, ep, dt)
+
+
+def test_generated_leaves_inside_expressions_and_other_kernel_shapes():
+    n = (1 << 18) + 3
+    x = np.random.RandomState(5).uniform(-1, 1, n).astype(np.float32)
+    before = hip.STATS["launches"]
+    got = (dr.linspace(-2.0, 2.0, n, dtype=np.float32) * dr.array(x) + dr.ones(n, dtype=np.float32)).get()
+    assert hip.STATS["launches"] - before == 1                    # one kernel, the grid is never stored
+    assert _same(got, np.linspace(-2.0, 2.0, n, dtype=np.float32) * x + np.ones(n, np.float32))
+    # fused with a reduction
+    s = dr.sum(dr.arange(n) * dr.array(x.astype(np.float64)))
+    ref = np.sum(np.arange(n) * x.astype(np.float64))
+    assert abs(float(s) - ref) <= 1e-12 * np.sum(np.abs(np.arange(n) * x.astype(np.float64)))
+    # index broadcast along rows of a matrix: the index array is materialised, result unchanged
+    m = np.random.RandomState(6).uniform(-1, 1, (7, 8192))
+    assert _same((dr.array(m) + dr.arange(8192)).get(), m + np.arange(8192))
+    assert _same((dr.array(m) * dr.linspace(0, 1, 8192)).get(), m * np.linspace(0, 1, 8192))
+    # written into a strided destination, and into a contiguous one
+    dst = dr.array(np.zeros((8192, 2)))
+    dst[:, 1] = dr.arange(0.0, 8192.0, 1.0) * 2
+    ref = np.zeros((8192, 2)); ref[:, 1] = np.arange(0.0, 8192.0, 1.0) * 2
+    assert _same(dst.get(), ref)
+    row = dr.array(np.zeros(8192))
+    row[:] = dr.arange(8192) + 0.5
+    assert _same(row.get(), np.arange(8192) + 0.5)
+    # axis reduction over an expression with a generated operand
+    assert np.allclose(dr.sum(dr.array(m) * dr.arange(8192), axis=1).get(),
+                       (m * np.arange(8192)).sum(axis=1), rtol=1e-13)
+
+
+def test_constant_arrays_stay_lazy_until_written():
+    z = dr.zeros((300, 400), dtype=np.float32)
+    assert "array" not in z.__dict__
+    a = np.random.RandomState(7).uniform(0, 1, (300, 400)).astype(np.float32)
+    y = z + dr.array(a) * 2
+    assert _same(y.get(), np.zeros((300, 400), np.float32) + a * 2) and "array" not in z.__dict__
+    assert _same(z.get(), np.zeros((300, 400), np.float32))        # asked for: now an array
+    z[1:-1, 1:-1] = 3.0
+    ref = np.zeros((300, 400), np.float32); ref[1:-1, 1:-1] = 3.0
+    w = z + dr.array(a) * 2                                        # same structure as y, new values
+    assert _same(w.get(), ref + a * 2)
+    # a plan made while the constant was lazy is not reused after the write
+    c = dr.full((1 << 14,), 2.5)
+    expr = c * 2.0
+    assert _same(expr.get(), np.full(1 << 14, 5.0))
+    c[0] = 1.0
+    ref = np.full(1 << 14, 2.5); ref[0] = 1.0
+    assert _same((c * 2.0).get(), ref * 2.0)
+    for make, ref in [(lambda: dr.ones((5000,), dtype=np.int32), np.ones(5000, np.int32)),
+                      (lambda: dr.full((70, 70), 7, dtype=np.int64), np.full((70, 70), 7, np.int64)),
+                      (lambda: dr.zeros_like(dr.array(a)), np.zeros_like(a)),
+                      (lambda: dr.full_like(dr.array(a), 1.5, dtype=np.float64), np.full_like(a, 1.5, dtype=np.float64)),
+                      (lambda: dr.zeros(4096, dtype=bool), np.zeros(4096, bool))]:
+        assert _same(make().get(), ref)
+    # the Jacobi set-up of configuration C4 starts from zeros and writes the interior
+    u = dr.zeros((64, 64), dtype=np.float32)
+    u[1:-1, 1:-1] = dr.array(a[:62, :62])
+    ref = np.zeros((64, 64), np.float32); ref[1:-1, 1:-1] = a[:62, :62]
+    assert _same(u.get(), ref)
