@@ -93,6 +93,10 @@ class _Fallback:
         return arr.transpose(axes) if axes is not None else arr.transpose()
 
     @staticmethod
+    def broadcast_to(arr, shape):
+        return _Fallback.asarray(arr).broadcast_to(shape)
+
+    @staticmethod
     def _reduce(arr, name, axis, keepdims):
         from .delayarray import NPArray, _reduce
         return _reduce(getattr(numpy, name), NPArray(arr), axis=axis, keepdims=keepdims)

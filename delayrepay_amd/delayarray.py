@@ -228,7 +228,8 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         return self.reshape(self.size)
 
     def transpose(self, *axes):
-        """Permuted view of the evaluated array, as a new leaf."""
+        """Permuted view of the evaluated array, as a new leaf; of a small unevaluated
+        element-wise expression: the expression over permuted views of its leaves."""
         if len(axes) == 1 and not isinstance(axes[0], (int, np.integer)):
             axes = tuple(axes[0]) if axes[0] is not None else ()
         return np.transpose(self, axes or None)
@@ -245,8 +246,15 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
     # ---- indexing --------------------------------------------------------
 
     def __getitem__(self, key):
-        """Force, then wrap the backend *view* as a new leaf (delayarray.py:123-128)."""
+        """Force, then wrap the backend *view* as a new leaf (delayarray.py:123-128).
+        A basic slice of a small unevaluated element-wise expression is instead the
+        same expression over slices of its leaves: only the part asked for is ever
+        computed, and shifted slices of one expression fuse into one stencil."""
         key = _unwrap(key)
+        if "array" not in self.__dict__ and type(self) in _ELEMENTWISE and _basic_key(key):
+            res = _over_views(self, lambda arr: arr[key])
+            if res is not None:
+                return res
         return NPArray(self._force()[key])
 
     def __setitem__(self, key, item):
@@ -632,6 +640,9 @@ class WhereEx(NumpyEx):
         return f"where{self._count}"
 
 
+_ELEMENTWISE = (BinaryNumpyEx, BinaryFuncEx, UnaryFuncEx, WhereEx, CastEx)
+
+
 def pow_ex(func, left, right):
     """`x ** k` with a Python-int k >= 2 becomes k-1 left-associated multiplies
     (delayarray.py:316-324); k <= 1 returns x itself, as the reference does."""
@@ -794,6 +805,62 @@ class IotaEx(_Generated):
         return f"iota{self._count}"
 
 
+PUSH_VIEWS_UP_TO = 48     # interior nodes; larger expressions are evaluated once, then viewed
+
+
+def _basic_key(key):
+    if not isinstance(key, tuple):
+        key = (key,)
+    return all(k is None or k is Ellipsis or isinstance(k, (slice, int, np.integer)) for k in key)
+
+
+def _over_views(root, view):
+    """The unevaluated element-wise expression `root` rebuilt over `view(leaf)` of each
+    leaf, every leaf first broadcast to the root's shape (so one view function serves
+    all of them); None when the expression is too large or holds something that has
+    to be evaluated first."""
+    shape = tuple(root.shape)
+    fb = _backend.fallback
+    memo = {}
+    budget = [PUSH_VIEWS_UP_TO]
+    new_shape = tuple(view(np.broadcast_to(np.empty((), dtype=bool), shape)).shape)
+
+    def walk(node):
+        hit = memo.get(id(node))
+        if hit is not None:
+            return hit
+        kind = type(node)
+        arr = node.__dict__.get("array")
+        if kind is Scalar:
+            res = node
+        elif arr is not None and kind is not FullEx and kind is not IotaEx or kind is NPArray:
+            res = NPArray(view(fb.broadcast_to(node._force(), shape)))
+        elif kind is FullEx and arr is None:
+            res = FullEx(new_shape, node.val, node.dtype)
+        elif kind in _ELEMENTWISE:
+            budget[0] -= 1
+            if budget[0] < 0:
+                raise _TooLarge
+            kids = [walk(c) for c in node.children]
+            if kind is CastEx:
+                res = CastEx(node.dtype, kids[0])
+            else:
+                res = kind(node.func, *kids)
+        else:       # reductions, index arrays, written-to constants: evaluate, then view
+            res = NPArray(view(fb.broadcast_to(node._force(), shape)))
+        memo[id(node)] = res
+        return res
+
+    try:
+        return walk(root)
+    except _TooLarge:
+        return None
+
+
+class _TooLarge(Exception):
+    pass
+
+
 def _binary(func, left, right):
     if not isinstance(left, DelayArray):
         left = arg_to_numpy_ex(left)
@@ -949,8 +1016,50 @@ def var(arr, axis=None, ddof=0, keepdims=False, **kwargs):
     return total / (count - ddof)
 
 
-transpose = implements(np.transpose)(cast(_eager("transpose")))
-roll = implements(np.roll)(cast(_eager("roll")))
+_eager_transpose = cast(_eager("transpose"))
+_eager_roll = cast(_eager("roll"))
+
+
+@implements(np.transpose)
+def transpose(arr, axes=None):
+    """View of the evaluated array with permuted axes (delayarray.py:521-524); a small
+    unevaluated element-wise expression is rebuilt over permuted views of its leaves."""
+    if isinstance(arr, DelayArray) and "array" not in arr.__dict__ and type(arr) in _ELEMENTWISE:
+        res = _over_views(arr, lambda a: a.transpose(axes) if axes is not None else a.transpose())
+        if res is not None:
+            return res
+    return _eager_transpose(arr, axes) if axes is not None else _eager_transpose(arr)
+
+
+@implements(np.roll)
+def roll(arr, shift, axis=None):
+    """`numpy.roll` (delayarray.py:527-530).  Along one axis of an unevaluated
+    element-wise expression the two pieces are computed straight into their shifted
+    places: two fused kernels, no unshifted temporary."""
+    lazy = isinstance(arr, DelayArray) and "array" not in arr.__dict__ \
+        and type(arr) in _ELEMENTWISE and isinstance(shift, (int, np.integer)) \
+        and (isinstance(axis, (int, np.integer)) or (axis is None and arr.ndim == 1)) and arr.size
+    if not lazy:
+        return _eager_roll(arr, shift, axis)
+    axis = 0 if axis is None else int(axis)
+    if not -arr.ndim <= axis < arr.ndim:
+        raise np.exceptions.AxisError(axis, arr.ndim)
+    axis %= arr.ndim
+    n = arr.shape[axis]
+    shift = int(shift) % n
+    out = empty(arr.shape, dtype=arr.dtype)
+
+    def cut(lo, hi):
+        return tuple(slice(lo, hi) if k == axis else slice(None) for k in range(arr.ndim))
+    if shift == 0:
+        out[...] = arr
+    else:
+        head, tail = arr[cut(0, n - shift)], arr[cut(n - shift, n)]
+        if isinstance(head, NPArray):       # too large to rebuild: evaluated once, copied twice
+            return _eager_roll(arr, shift, axis)
+        out[cut(shift, n)] = head
+        out[cut(0, shift)] = tail
+    return out
 repeat = implements(np.repeat)(cast(_eager("repeat")))
 cumsum = implements(np.cumsum)(cast(_eager("cumsum")))
 tile = implements(np.tile)(cast(_eager("tile")))

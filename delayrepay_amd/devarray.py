@@ -242,6 +242,22 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
         dst = self[key]
         hip.assign(dst, value)
 
+    def broadcast_to(self, shape):
+        """View with NumPy's broadcasting applied: new and stretched axes get stride 0."""
+        shape = tuple(int(d) for d in shape)
+        lead = len(shape) - self.ndim
+        if lead < 0:
+            raise ValueError(f"cannot broadcast shape {self.shape} to {shape}")
+        strides = [0] * lead
+        for have, want, stride in zip(self.shape, shape[lead:], self._strides):
+            if have == want:
+                strides.append(stride)
+            elif have == 1:
+                strides.append(0)
+            else:
+                raise ValueError(f"cannot broadcast shape {self.shape} to {shape}")
+        return self._view(shape, strides, self.offset)
+
     def reshape(self, *shape, **kwargs):
         if len(shape) == 1 and not isinstance(shape[0], numbers.Integral):
             shape = tuple(shape[0])

@@ -88,6 +88,29 @@ SCRIPT = textwrap.dedent("""
     assert same(dnp.full((5000,), 3, dtype=np.int32).get(), np.full(5000, 3, np.int32))
     assert same(dnp.full_like(y, 2.5, dtype=np.float32).get(), np.full((100, 100), 2.5, np.float32))
     assert isinstance(dnp.zeros(8), NPArray) and isinstance(dnp.full((3,), "a"), NPArray)
+
+    # views of unevaluated expressions are the expression over views of its leaves
+    rs = np.random.RandomState(2)
+    ha, hb = rs.uniform(-1, 1, (50, 70)), rs.uniform(-1, 1, 70)
+    A, B = array(ha), array(hb)
+    e, ref = A * 2 + B, ha * 2 + hb
+    r = e[1:-1, ::2]
+    assert not isinstance(r, NPArray) and r.shape == (48, 35) and "array" not in e.__dict__
+    assert same(r.get(), ref[1:-1, ::2]) and same(e[3].get(), ref[3])
+    assert same(e[:, None, 5].get(), ref[:, None, 5]) and same(e[..., -1].get(), ref[..., -1])
+    assert same(e.T.get(), ref.T) and same(np.transpose(e, (1, 0))[2:4].get(), ref.T[2:4])
+    assert same(np.roll(e, 7, axis=1).get(), np.roll(ref, 7, axis=1))
+    assert same(np.roll(e, -3, axis=0).get(), np.roll(ref, -3, axis=0))
+    assert same(np.roll(A[0] + 1, 5).get(), np.roll(ha[0] + 1, 5)) and "array" not in e.__dict__
+    s1, r1 = A + 1, ha + 1
+    lap = s1[:-2, 1:-1] + s1[2:, 1:-1] + s1[1:-1, :-2] + s1[1:-1, 2:]
+    assert same(lap.get(), r1[:-2, 1:-1] + r1[2:, 1:-1] + r1[1:-1, :-2] + r1[1:-1, 2:])
+    assert "array" not in s1.__dict__
+    assert same((dnp.zeros((50, 70)) + A)[2:5].get(), ha[2:5])
+    big = A
+    for _ in range(60):
+        big = big + 1.0
+    assert isinstance(big[1:3], NPArray) and "array" in big.__dict__       # too large: evaluated once
     print("cpu-backend-ok")
 """)
 

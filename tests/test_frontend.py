@@ -354,3 +354,22 @@ def test_generated_leaves_are_never_shared_and_small_ones_are_eager():
     assert dr.arange(0, 1 << 16, 2).shape == (1 << 15,) and dr.arange(0.0, 10.0, 0.001).dtype == np.float64
     assert dr.linspace(0, 1, 1 << 16).shape == (1 << 16,)
     assert dr.linspace(0, 1, 1 << 16, dtype=np.float32).dtype == np.float32
+
+
+def test_views_of_lazy_expressions_are_pushed_to_the_leaves():
+    a, b = leaf((512, 1024)), leaf((1024,))
+    e = a * 2 + b
+    r = e[1:-1, 4:-4]
+    assert type(r) is BinaryNumpyEx and r.shape == (510, 1016) and "array" not in e.__dict__
+    low, src = hip.lower_only(r)
+    assert len(low.srcs) == 2 and low.kind.startswith("tile2d")
+    # shifted slices of one expression become one LDS stencil over the expression's leaf
+    s = a + 1.0
+    lap = s[:-2, 1:-1] + s[2:, 1:-1] + s[1:-1, :-2] + s[1:-1, 2:]
+    low, src = hip.lower_only(lap)
+    assert low.kind in ("tile2d", "tile2dv") and "__shared__" in src and len(low.srcs) == 1
+    hip.compile_source(src)
+    # transposes: the leaves are read through the LDS transpose tile
+    low, src = hip.lower_only((a * 2).T)
+    assert low.kind == "tile2dt"
+    assert e.T.shape == (1024, 512) and "array" not in e.__dict__

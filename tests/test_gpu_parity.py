@@ -684,3 +684,41 @@ def test_constant_arrays_stay_lazy_until_written():
     u[1:-1, 1:-1] = dr.array(a[:62, :62])
     ref = np.zeros((64, 64), np.float32); ref[1:-1, 1:-1] = a[:62, :62]
     assert _same(u.get(), ref)
+
+
+# ---- views of unevaluated expressions -----------------------------------------------------------
+
+def test_slices_transposes_and_rolls_of_lazy_expressions():
+    rs = np.random.RandomState(12)
+    ha, hb = rs.uniform(-1, 1, (300, 520)).astype(np.float32), rs.uniform(-1, 1, 520).astype(np.float32)
+    A, B = dr.array(ha), dr.array(hb)
+    e, ref = A * 2 + B, ha * 2 + hb
+    before = hip.STATS["launches"]
+    assert _same(e[1:-1, ::2].get(), ref[1:-1, ::2])
+    assert hip.STATS["launches"] - before == 1 and "array" not in e.__dict__
+    assert _same(e[3].get(), ref[3]) and _same(e[:, None, 5].get(), ref[:, None, 5])
+    assert _same(e[..., -1].get(), ref[..., -1]) and _same(e[10:20, 7].get(), ref[10:20, 7])
+    assert _same(e.T.get(), ref.T) and _same(np.transpose(e, (1, 0))[2:40].get(), ref.T[2:40])
+    assert _same(np.roll(e, 7, axis=1).get(), np.roll(ref, 7, axis=1))
+    assert _same(np.roll(e, -3, axis=0).get(), np.roll(ref, -3, axis=0))
+    assert _same(np.roll(e, 0, axis=0).get(), ref)
+    assert _same(np.roll(A[0] + 1, 5).get(), np.roll(ha[0] + 1, 5)) and "array" not in e.__dict__
+    # a stencil on an expression: one kernel, the expression is never stored
+    s, r = A * A + 1, ha * ha + 1
+    before = hip.STATS["launches"]
+    lap = s[:-2, 1:-1] + s[2:, 1:-1] + s[1:-1, :-2] + s[1:-1, 2:]
+    assert _same(lap.get(), r[:-2, 1:-1] + r[2:, 1:-1] + r[1:-1, :-2] + r[1:-1, 2:])
+    assert hip.STATS["launches"] - before == 1 and "array" not in s.__dict__
+    # three dimensions, a lazy constant, an index array, a comparison
+    hc = rs.uniform(-1, 1, (6, 40, 130))
+    C = dr.array(hc)
+    assert _same((C * 3 - 1)[1:5, ::3, 2:-2].get(), (hc * 3 - 1)[1:5, ::3, 2:-2])
+    assert _same(np.transpose(C + 1, (2, 0, 1)).get(), np.transpose(hc + 1, (2, 0, 1)))
+    assert _same((dr.zeros((300, 520), dtype=np.float32) + A)[2:5].get(), ha[2:5])
+    assert _same((dr.arange(8192) * 2.0)[100:200].get(), (np.arange(8192) * 2.0)[100:200])
+    assert _same(dr.where(A > 0, A, 0.0)[::7, 1::5].get(), np.where(ha > 0, ha, np.float32(0))[::7, 1::5])
+    # too large to rebuild: evaluated once, then viewed
+    big, rbig = A, ha
+    for _ in range(60):
+        big, rbig = big + 1.0, rbig + np.float32(1.0)
+    assert _same(big[1:3].get(), rbig[1:3]) and "array" in big.__dict__
