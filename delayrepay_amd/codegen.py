@@ -903,7 +903,8 @@ def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
 T_TILE = 64      # square tile edge: both the transposed read and the write coalesce
 
 
-def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True):
+def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_load=False,
+                        nt_store=False):
     """2-D tiled kernel for expressions in which some operand is walked along the
     output's rows by its unit stride (a transposed view).
 
@@ -912,6 +913,10 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True):
                transposed (rows padded by one word, so neither side has bank
                conflicts); ('d',) unit stride along output dimension 1, read directly;
                ('b',) single element broadcast
+    vec        0, or the number of elements in 16 bytes when every array has that
+               element size, 16-byte aligned rows and row strides: tiles that lie
+               wholly inside the output then move 16 bytes per lane on both sides
+               (the transposition itself happens in LDS, one word at a time)
     Parameters: leaf pointers, output pointers, scalars, H, W, tiles_x, then per 't'
     leaf its stride along output columns, per 'd' leaf its row stride, per output its
     row stride."""
@@ -936,11 +941,63 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True):
     for i, k in enumerate(leaf_kind):
         if k[0] == "t":
             L.append(f"    __shared__ {CTYPE[prog.leaves[i]]} tt{i}[{T * (T + 1)}];")
-    L += ["    const int ty = blockIdx.x / tiles_x;",
-          "    const int tx = blockIdx.x - ty * tiles_x;",
+    # Diagonal order: blocks that run at the same time differ in both tile coordinates.
+    # With row-major order they would share r0, and the transposed operand's tiles
+    # (rows a power-of-two pitch apart) would all fall into the same few memory channels.
+    L += ["    const int band = blockIdx.x / tiles_x;",
+          "    const int tx = blockIdx.x - band * tiles_x;",
+          f"    const int ty = (band + tx) % ((H + {T - 1}) / {T});",
           f"    const int r0 = ty * {T};",
-          f"    const int c0 = tx * {T};",
-          # transposed operands: consecutive threads walk output ROWS (their unit stride)
+          f"    const int c0 = tx * {T};"]
+    if vec:
+        V = vec
+        vpr = T // V                      # vectors per tile row
+        passes = T * T // V // BLOCK
+        L += [f"    if (r0 + {T} <= H && c0 + {T} <= W) {{",
+              "#pragma unroll",
+              f"        for (int k = 0; k < {passes}; ++k) {{",
+              f"            const int e = threadIdx.x + k * {BLOCK};",
+              f"            const int lc = e / {vpr};",
+              f"            const int vr = e - lc * {vpr};"]
+        for i, k in enumerate(leaf_kind):
+            if k[0] == "t":
+                vt = VEC16[prog.leaves[i]][0]
+                ptr = f"(const {vt}*)(a{i} + (long long)(c0 + lc) * cs{i} + (r0 + vr * {V}))"
+                L.append(f"            const {vt} w{i} = {_ld(nt_load, ptr)};")
+                for q in range(V):
+                    L.append(f"            tt{i}[lc * {T + 1} + vr * {V} + {q}] = w{i}[{q}];")
+        L += ["        }", "        __syncthreads();",
+              "#pragma unroll",
+              f"        for (int k = 0; k < {passes}; ++k) {{",
+              f"            const int e = threadIdx.x + k * {BLOCK};",
+              f"            const int lr = e / {vpr};",
+              f"            const int vc = e - lr * {vpr};",
+              "            const long long i = r0 + lr;",
+              f"            const int j = c0 + vc * {V};"]
+        for i, k in enumerate(leaf_kind):
+            if k[0] == "d":
+                vt = VEC16[prog.leaves[i]][0]
+                L.append(f"            const {vt} d{i} = "
+                         f"{_ld(nt_load, f'(const {vt}*)(a{i} + i * rs{i} + j)')};")
+        for o, dt in enumerate(out_dtypes):
+            L.append(f"            {VEC16[dt][0]} R{o};")
+        for q in range(V):
+            vargs = []
+            for i, k in enumerate(leaf_kind):
+                if k[0] == "t":
+                    vargs.append(f"tt{i}[(vc * {V} + {q}) * {T + 1} + lr]")
+                elif k[0] == "d":
+                    vargs.append(f"d{i}[{q}]")
+                else:
+                    vargs.append(f"a{i}[0]")
+            decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+            call = vargs + [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
+            sets = " ".join(f"R{o}[{q}] = t{o};" for o in range(n_out))
+            L.append(f"            {{ {decl} dr_body({', '.join(call)}); {sets} }}")
+        for o, dt in enumerate(out_dtypes):
+            L.append("            " + _st(nt_store, f"R{o}", f"({VEC16[dt][0]}*)(o{o} + i * ors{o} + j)"))
+        L += ["        }", "        return;", "    }"]
+    L += [# transposed operands: consecutive threads walk output ROWS (their unit stride)
           "#pragma unroll",
           f"    for (int k = 0; k < {per_thread}; ++k) {{",
           f"        const int e = threadIdx.x + k * {BLOCK};",

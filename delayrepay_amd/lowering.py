@@ -36,6 +36,7 @@ TUNE = {
     "xcd": 1,         # vectorised stencil: give each XCD a contiguous band of tiles
     "sntl": 0,        # vectorised stencil: non-temporal loads / stores
     "snts": 1,
+    "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
 }
 for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
@@ -301,10 +302,29 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         if lds_bytes <= 64 * 1024:
             H, W = mshape
             low.kind = "tile2dt"
-            low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place)
+            # 16 bytes per lane on both sides when every array has the same element
+            # size and all rows (of the operands' own layouts) start 16-byte aligned
+            sizes = {cg.ITEMSIZE[c] for c in list(prog.leaves) + list(out_codes)}
+            vec = 16 // sizes.pop() if len(sizes) == 1 and sizes <= {4, 8} and TUNE["tvec"] else 0
+            if vec and all(c in cg.VEC16 for c in list(prog.leaves) + list(out_codes)):
+                pitches = [(st[1] if k[0] == "t" else st[0], a.offset)
+                           for a, k, st in zip(leaves, kinds, m_leaf) if k[0] != "b"]
+                pitches += [(st[0], ptr // cg.ITEMSIZE[c]) for ptr, st, c in zip(out_ptrs, m_out, out_codes)
+                            if ptr % cg.ITEMSIZE[c] == 0]
+                if len(pitches) != len(out_ptrs) + sum(k[0] != "b" for k in kinds) \
+                        or any(pitch % vec or first % vec for pitch, first in pitches):
+                    vec = 0
+            else:
+                vec = 0
+            out_bytes = sum(H * W * cg.ITEMSIZE[c] for c in out_codes)
+            in_bytes = sum(H * W * cg.ITEMSIZE[c] for c, k in zip(prog.leaves, kinds) if k[0] != "b")
+            nts = bool(vec and TUNE["nts"]) and in_bytes + out_bytes > TUNE["cache_mib"] << 20
+            ntl = bool(vec and TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
+            low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place, vec, ntl, nts)
 
             def emit():
-                return cg.emit_tile_transpose(prog, kinds, out_codes, restrict=not in_place)
+                return cg.emit_tile_transpose(prog, kinds, out_codes, restrict=not in_place,
+                                              vec=vec, nt_load=ntl, nt_store=nts)
             low.emit = emit
             tiles_x = -(-W // cg.T_TILE)
             low.grid = tiles_x * -(-H // cg.T_TILE)
