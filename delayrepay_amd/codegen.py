@@ -56,7 +56,16 @@ typedef double f8x2 __attribute__((ext_vector_type(2)));
 typedef int i4x4 __attribute__((ext_vector_type(4)));
 typedef long long i8x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u4x4 __attribute__((ext_vector_type(4)));
+typedef float f4x4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef double f8x2u __attribute__((ext_vector_type(2), aligned(8)));
+typedef int i4x4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef long long i8x2u __attribute__((ext_vector_type(2), aligned(8)));
+typedef unsigned int u4x4u __attribute__((ext_vector_type(4), aligned(4)));
 """
+# The `...u` types are the same vectors at element alignment: global memory takes 16-byte
+# accesses at any 4-byte address (measured on MI355X: 6.2-6.6 TB/s for a copy shifted by one
+# to three floats against 6.7 TB/s aligned, and 3.5 TB/s with one element per lane), so
+# views that do not start on a 16-byte boundary, or whose rows do not, still move vectors.
 
 
 def dtype_code(dtype):
@@ -312,17 +321,19 @@ def _st(nt, val, ptr):
 
 
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
-              reduce_op=None):
+              reduce_op=None, unaligned=False):
     """Contiguous 1-D kernel.
 
     leaf_class  per leaf 'c' (contiguous, same length as the output) or 'b'
                 (single element broadcast to every position)
-    vec         True: 16-byte vector accesses (all pointers 16-byte aligned and
-                all element types 4 or 8 bytes wide); False: one element per access
+    vec         True: 16-byte vector accesses (all element types 4 or 8 bytes wide);
+                False: one element per access
+    unaligned   some pointer is not 16-byte aligned: vectors at element alignment
     reduce_op   None, or 'add' | 'maximum' | 'minimum': the single root is
                 reduced instead of stored; the output is one partial per block
     """
     rs = "__restrict__ " if restrict else ""
+    ua = "u" if unaligned else ""
     n_leaf, n_out = len(prog.leaves), len(out_dtypes)
     red_dt = out_dtypes[0] if reduce_op else None
     if vec:
@@ -367,6 +378,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                 continue
             if vec:
                 vt, per = VEC16[dt]
+                vt += ua
                 chunks = E // per
                 for ch in range(chunks):
                     ptr = f"(const {vt}*)a{i} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
@@ -405,6 +417,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
         if vec and not reduce_op:
             for o, dt in enumerate(out_dtypes):
                 vt, per = VEC16[dt]
+                vt += ua
                 chunks = E // per
                 for ch in range(chunks):
                     ptr = f"({vt}*)o{o} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
@@ -655,7 +668,7 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
 
 def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_per_thread,
                      phase_group, phase_out, restrict=True, nt_load=False, nt_store=False,
-                     xcd_bands=True, nouter=1):
+                     xcd_bands=True, nouter=1, unaligned=False):
     """Vectorised 2-D tiled kernel for the aligned case: every output's row stride
     is a multiple of the 16-byte vector width VW and all outputs start at the same
     address phase (`phase_out` = address of output [0, 0] / itemsize, mod VW).
@@ -762,7 +775,7 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
     L.append("        if (inner) {")
     for i, k in enumerate(leaf_kind):
         if k[0] == "dv":
-            lvt = VEC16[prog.leaves[i]][0]
+            lvt = VEC16[prog.leaves[i]][0] + ("u" if unaligned else "")
             ptr = f"(const {lvt}*)(a{i} + base{i} + jf)"
             L.append(f"            const {lvt} D{i} = {_ld(nt_load, ptr)};")
     for o, dt in enumerate(out_dtypes):
@@ -772,7 +785,8 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
         sets = " ".join(f"R{o}[{e}] = t{o};" for o in range(n_out))
         L.append(f"            {{ {decl} dr_body({', '.join(args + tail_args)}); {sets} }}")
     for o, dt in enumerate(out_dtypes):
-        L.append("            " + _st(nt_store, f"R{o}", f"({VEC16[dt][0]}*)(o{o} + obase{o} + jf)"))
+        ovt = VEC16[dt][0] + ("u" if unaligned else "")
+        L.append("            " + _st(nt_store, f"R{o}", f"({ovt}*)(o{o} + obase{o} + jf)"))
     L.append("        } else {")
     for e in range(VW):
         args = [operand(i, k, e, False) for i, k in enumerate(leaf_kind)]
@@ -904,7 +918,7 @@ T_TILE = 64      # square tile edge: both the transposed read and the write coal
 
 
 def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_load=False,
-                        nt_store=False):
+                        nt_store=False, unaligned=False):
     """2-D tiled kernel for expressions in which some operand is walked along the
     output's rows by its unit stride (a transposed view).
 
@@ -961,7 +975,7 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
               f"            const int vr = e - lc * {vpr};"]
         for i, k in enumerate(leaf_kind):
             if k[0] == "t":
-                vt = VEC16[prog.leaves[i]][0]
+                vt = VEC16[prog.leaves[i]][0] + ("u" if unaligned else "")
                 ptr = f"(const {vt}*)(a{i} + (long long)(c0 + lc) * cs{i} + (r0 + vr * {V}))"
                 L.append(f"            const {vt} w{i} = {_ld(nt_load, ptr)};")
                 for q in range(V):
@@ -976,7 +990,7 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
               f"            const int j = c0 + vc * {V};"]
         for i, k in enumerate(leaf_kind):
             if k[0] == "d":
-                vt = VEC16[prog.leaves[i]][0]
+                vt = VEC16[prog.leaves[i]][0] + ("u" if unaligned else "")
                 L.append(f"            const {vt} d{i} = "
                          f"{_ld(nt_load, f'(const {vt}*)(a{i} + i * rs{i} + j)')};")
         for o, dt in enumerate(out_dtypes):
@@ -995,7 +1009,8 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
             sets = " ".join(f"R{o}[{q}] = t{o};" for o in range(n_out))
             L.append(f"            {{ {decl} dr_body({', '.join(call)}); {sets} }}")
         for o, dt in enumerate(out_dtypes):
-            L.append("            " + _st(nt_store, f"R{o}", f"({VEC16[dt][0]}*)(o{o} + i * ors{o} + j)"))
+            ovt = VEC16[dt][0] + ("u" if unaligned else "")
+            L.append("            " + _st(nt_store, f"R{o}", f"({ovt}*)(o{o} + i * ors{o} + j)"))
         L += ["        }", "        return;", "    }"]
     L += [# transposed operands: consecutive threads walk output ROWS (their unit stride)
           "#pragma unroll",

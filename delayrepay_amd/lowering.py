@@ -36,6 +36,7 @@ TUNE = {
     "xcd": 1,         # vectorised stencil: give each XCD a contiguous band of tiles
     "sntl": 0,        # vectorised stencil: non-temporal loads / stores
     "snts": 1,
+    "uvec": 1,        # 16-byte accesses at element alignment where 16-byte alignment is missing
     "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
 }
@@ -136,7 +137,8 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         if not reduce_op:
             widths_ok = widths_ok and all(cg.ITEMSIZE[c] in (4, 8) for c in out_codes)
             align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
-        vec = widths_ok and align_ok and n >= 64
+        vec = widths_ok and n >= 64 and (align_ok or bool(TUNE["uvec"]))
+        ua = vec and not align_ok      # vectors at element alignment
         unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
         in_bytes = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
         footprint = in_bytes
@@ -150,11 +152,11 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         ntl = bool(TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
         low.kind = "flat"
         low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
-                   unroll, ntl, nts)
+                   unroll, ntl, nts, ua)
 
         def emit():
             src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
-                                  restrict=not in_place, reduce_op=reduce_op)
+                                  restrict=not in_place, reduce_op=reduce_op, unaligned=ua)
             return src
         low.emit = emit
         if vec:
@@ -224,34 +226,46 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                 kinds[i] = ("b",) if not any(s) else ("d",) if s[-1] == 1 else ("r",)
         kinds = tuple(kinds)
         low.kind = "tile2d"
-        vec_ok = False
+        vec_ok = ua = False
         if TUNE["svec"] and out_codes:
             gsize = cg.ITEMSIZE[group[0]] if group is not None else cg.ITEMSIZE[out_codes[0]]
             vw = 16 // gsize if gsize in (4, 8) else 0
-            vec_ok = (vw > 0 and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
-                      and all(st % vw == 0 for s in m_out for st in s[:-1])
+            same_size = vw > 0 and all(cg.ITEMSIZE[c] == gsize for c in out_codes)
+            vec_ok = (same_size and all(st % vw == 0 for s in m_out for st in s[:-1])
                       and len({(p // gsize) % vw for p in out_ptrs}) == 1
                       and (group is None or g_args[0] % vw == 0))
+
+            def row_aligned(i, phase):
+                return (all(st % vw == 0 for st in m_leaf[i][:-1])
+                        and (leaves[i].ptr // gsize) % vw == phase)
+            sized = [k[0] == "d" and cg.ITEMSIZE[prog.leaves[i]] == gsize
+                     for i, k in enumerate(kinds)]
+            missed = True
+            if vec_ok:
+                ph_o = (out_ptrs[0] // gsize) % vw
+                dv = [d and row_aligned(i, ph_o) for i, d in enumerate(sized)]
+                missed = dv != sized        # some operand would fall back to element loads
+            if group is None and same_size and TUNE["uvec"] and W >= 4 * vw and missed:
+                # without a halo group nothing ties the tiles to 16-byte boundaries: rows of
+                # any pitch and phase move as vectors at element alignment
+                vec_ok = ua = True
+                ph_o = 0
+                dv = sized
         if vec_ok:
-            ph_o = (out_ptrs[0] // gsize) % vw
             ph_g = (g_ptr // gsize) % vw if group is not None else 0
             # direct operands whose rows share the outputs' alignment load as vectors
-            kinds = tuple(
-                ("dv",) if (k[0] == "d" and cg.ITEMSIZE[prog.leaves[i]] == gsize
-                            and all(st % vw == 0 for st in m_leaf[i][:-1])
-                            and (leaves[i].ptr // gsize) % vw == ph_o) else k
-                for i, k in enumerate(kinds))
+            kinds = tuple(("dv",) if d else k for d, k in zip(dv, kinds))
             gpr, rpt = TUNE["gpr"], TUNE["rpt"]
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
             bands = bool(TUNE["xcd"])
             low.key = ("tile2dv", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o,
-                       gpr, rpt, sntl, snts, bands, nouter)
+                       gpr, rpt, sntl, snts, bands, nouter, ua)
             tw, th = gpr * vw, (cg.BLOCK // gpr) * rpt
 
             def emit():
                 return cg.emit_stencil_vec(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o,
                                            restrict=not in_place, nt_load=sntl, nt_store=snts,
-                                           xcd_bands=bands, nouter=nouter)[0]
+                                           xcd_bands=bands, nouter=nouter, unaligned=ua)[0]
             tiles_x = -(-(W + ph_o) // tw)     # tiles start `ph_o` columns left of the view
         else:
             low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune, nouter)
@@ -306,25 +320,29 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             # size and all rows (of the operands' own layouts) start 16-byte aligned
             sizes = {cg.ITEMSIZE[c] for c in list(prog.leaves) + list(out_codes)}
             vec = 16 // sizes.pop() if len(sizes) == 1 and sizes <= {4, 8} and TUNE["tvec"] else 0
+            ua = False
             if vec and all(c in cg.VEC16 for c in list(prog.leaves) + list(out_codes)):
                 pitches = [(st[1] if k[0] == "t" else st[0], a.offset)
                            for a, k, st in zip(leaves, kinds, m_leaf) if k[0] != "b"]
                 pitches += [(st[0], ptr // cg.ITEMSIZE[c]) for ptr, st, c in zip(out_ptrs, m_out, out_codes)
                             if ptr % cg.ITEMSIZE[c] == 0]
-                if len(pitches) != len(out_ptrs) + sum(k[0] != "b" for k in kinds) \
-                        or any(pitch % vec or first % vec for pitch, first in pitches):
+                if len(pitches) != len(out_ptrs) + sum(k[0] != "b" for k in kinds):
                     vec = 0
+                elif any(pitch % vec or first % vec for pitch, first in pitches):
+                    ua = True               # vectors at element alignment
+                    vec = vec if TUNE["uvec"] else 0
             else:
                 vec = 0
             out_bytes = sum(H * W * cg.ITEMSIZE[c] for c in out_codes)
             in_bytes = sum(H * W * cg.ITEMSIZE[c] for c, k in zip(prog.leaves, kinds) if k[0] != "b")
             nts = bool(vec and TUNE["nts"]) and in_bytes + out_bytes > TUNE["cache_mib"] << 20
             ntl = bool(vec and TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
-            low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place, vec, ntl, nts)
+            ua = bool(ua and vec)
+            low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place, vec, ntl, nts, ua)
 
             def emit():
                 return cg.emit_tile_transpose(prog, kinds, out_codes, restrict=not in_place,
-                                              vec=vec, nt_load=ntl, nt_store=nts)
+                                              vec=vec, nt_load=ntl, nt_store=nts, unaligned=ua)
             low.emit = emit
             tiles_x = -(-W // cg.T_TILE)
             low.grid = tiles_x * -(-H // cg.T_TILE)

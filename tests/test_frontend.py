@@ -208,11 +208,25 @@ def test_contiguous_is_flat_and_vectorised():
     assert hip.lower_only(2.0 * leaf((256, 256)) + leaf((256, 256)))[0].key == low.key
 
 
-def test_misaligned_view_uses_scalar_flat_kernel():
+def test_misaligned_view_moves_vectors_at_element_alignment():
     base = hip.placeholder((1 << 12,), np.float32)
     low, src = hip.lower_only(NPArray(base[1:]) * 2.0)
-    assert low.kind == "flat" and "f4x4*)" not in src.split('extern "C"')[1]
+    kernel = src.split('extern "C"')[1]
+    assert low.kind == "flat" and "f4x4*)" not in kernel and "(const f4x4u*)a0" in kernel
     assert hip._kernel_name(low).startswith("dr_flat_") and hip._kernel_name(low) in src
+    aligned = hip.lower_only(NPArray(base[4:]) * 2.0)[1].split('extern "C"')[1]
+    assert "(const f4x4*)a0" in aligned and "f4x4u" not in aligned
+    # rows whose pitch is not a multiple of 16 bytes: vector tiles all the same
+    m = NPArray(hip.placeholder((1022, 1022), np.float32, strides=(1024, 1), offset=1025))
+    low, src = hip.lower_only(m * 2.0 + m)
+    assert low.key[0] == "tile2dv" and "(const f4x4u*)(a0" in src and "(f4x4u*)(o0" in src
+    hip.compile_source(src)
+    hip.set_tune(uvec=0)
+    try:
+        low, src = hip.lower_only(NPArray(base[1:]) * 2.0)
+        assert "f4x4u*)" not in src.split('extern "C"')[1]
+    finally:
+        hip.set_tune(uvec=1)
 
 
 def test_broadcast_scalar_leaf_and_mixed_dtypes():
