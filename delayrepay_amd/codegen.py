@@ -575,7 +575,8 @@ def _base_names(leaf_kind, n_out):
     return names + [(f"obase{o}", f"oos{o}") for o in range(n_out)]
 
 
-def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=True, nouter=1):
+def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=True, nouter=1,
+                 xcd_bands=True):
     """2-D tiled kernel; operands that are shifted views of one buffer are staged
     through an LDS halo tile.
 
@@ -619,12 +620,14 @@ def emit_stencil(prog, leaf_kind, group, out_dtypes, tile_w, tile_h, restrict=Tr
          f"void dr_kernel({', '.join(params)})", "{"]
     if group is not None:
         L.append(f"    __shared__ {CTYPE[gdt]} tile[{LH * LW}];")
-    L += [  # contiguous band of tiles per XCD (blocks are dealt round-robin to XCDs)
-         "    const int nb = gridDim.x;",
-         f"    const int xcd = blockIdx.x % {N_XCD};",
-         f"    const int slot = blockIdx.x / {N_XCD};",
-         f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;",
-         "    const int ty = t / tiles_x;",
+    if xcd_bands:   # contiguous band of tiles per XCD (blocks are dealt round-robin to XCDs)
+        L += ["    const int nb = gridDim.x;",
+              f"    const int xcd = blockIdx.x % {N_XCD};",
+              f"    const int slot = blockIdx.x / {N_XCD};",
+              f"    const int t = xcd * (nb / {N_XCD}) + min(xcd, nb % {N_XCD}) + slot;"]
+    else:
+        L.append("    const int t = blockIdx.x;")
+    L += ["    const int ty = t / tiles_x;",
          "    const int tx = t - ty * tiles_x;",
          f"    const int r0 = ty * {tile_h};",
          f"    const int c0 = tx * {tile_w};"]
