@@ -245,7 +245,8 @@ def main():
             "kernel_GBps": round(wl["nbytes"] / kernel_ms / 1e6, 1),
             "roofline_frac": round(wl["nbytes"] / kernel_ms / 1e6 / HBM_PEAK_GBPS, 4),
             # what limits the kernel (rocprofv3 VALUBusy / traffic in profiles/)
-            "bound": "fp64 VALU (VALUBusy 92%), not HBM" if name == "bs64" else "hbm",
+            "bound": {"bs64": "fp64 vector ALU (VALUBusy 89%), not HBM",
+                      "bs32": "fp32 vector ALU (VALUBusy ~100%) and HBM"}.get(name, "hbm"),
             "first_call_ms": round(first_ms, 2),
             "compile_ms": round((c1["compile_ns"] - c0["compile_ns"]) / 1e6, 2),
             "input_gen_s": round(t_gen, 2),
