@@ -22,6 +22,7 @@ TUNE = {
     "ax_blocks": 4096,   # axis reductions: blocks ('col') / waves ('row') worth of work to
     "ax_waves": 32768,   # aim for before the reduced extent is cut into slices
     "ax_rows": 4,        # 'row' strategy: outputs per wave (grid-stride), to amortise set-up
+    "ax_short": 64,      # reduced unit-stride extents up to this length: a lane per output
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
     "nts": 1,         # allow non-temporal stores }
@@ -425,6 +426,26 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
     inner_kept = any(s[-1] == 1 for s in ksets)
     inner_red = any(s[-1] == 1 for s in rsets)
     strategy = "col" if (inner_kept and not inner_red) else "row"
+    if (strategy == "row" and slices is None and R <= TUNE["ax_short"] and K >= 4096
+            and len(kmerged) == 1 and len(rmerged) == 1
+            and all(r[0] in (0, 1) for r in rsets) and K < 2 ** 40):
+        # many short rows: a lane per output walking its own row, no combining step
+        kinds = tuple("v" if r[0] == 1 else "k" for r in rsets)
+        low = Lowered()
+        low.lds = 0
+        low.fin_count = 0
+        low.kind = "axis_short"
+        low.key = ("axis_short", prog.key(), kinds, acc, reduce_op, R)
+
+        def emit_short():
+            return cg.emit_short_rows(prog, kinds, acc, reduce_op, R)
+        low.emit = emit_short
+        low.grid = -(-K // cg.BLOCK)
+        low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+                   + "q" + "q" * len(leaves))
+        low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+        low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets]
+        return low, 1, K, "short"
     # enough independent pieces to fill the device: cut the reduced extent into slices
     if slices is not None:
         S = slices

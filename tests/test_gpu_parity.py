@@ -20,6 +20,7 @@ import pytest
 
 import delayrepay_amd as dr
 from delayrepay_amd import hip
+from delayrepay_amd.delayarray import ReduceEx
 from oracle import numpy_oracle as orc
 from oracle.numpy_oracle import OracleArray
 from tests.helpers import bits_equal, golden, ulp_distance
@@ -722,3 +723,36 @@ def test_slices_transposes_and_rolls_of_lazy_expressions():
     for _ in range(60):
         big, rbig = big + 1.0, rbig + np.float32(1.0)
     assert _same(big[1:3].get(), rbig[1:3]) and "array" in big.__dict__
+
+
+def test_reductions_over_short_rows():
+    """Many short rows: a lane per output, the row length compiled in."""
+    rs = np.random.RandomState(21)
+    for shape, dt in [((50000, 3), np.float32), ((4096, 16), np.float64), ((70001, 7), np.float32),
+                      ((8192, 64), np.float32), ((5000, 33), np.int32)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
+        assert low.kind == "axis_short" and low.key[-1] == shape[1]
+        tol = dict(rtol=1e-5, atol=1e-5) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
+        assert np.allclose(dr.sum(a * a, axis=1).get(), (h * h).sum(axis=1), **tol)
+        assert dr.sum(a * a, axis=1).get().dtype == (h * h).sum(axis=1).dtype
+        assert np.array_equal(dr.max(a, axis=1).get(), h.max(axis=1))
+        assert np.array_equal(dr.min(a, axis=-1).get(), h.min(axis=-1))
+        if dt != np.int32:
+            assert np.allclose(dr.mean(a, axis=1).get(), h.mean(axis=1), **tol)
+    # operands constant along the row, one row for all, and rows with a pitch
+    h = rs.uniform(-1, 1, (20000, 8)).astype(np.float32)
+    w, v = rs.uniform(0, 1, (20000, 1)).astype(np.float32), rs.uniform(0, 1, 8).astype(np.float32)
+    a, W, V = dr.array(h), dr.array(w), dr.array(v)
+    assert np.allclose(dr.sum(a * W + V, axis=1).get(), (h * w + v).sum(axis=1), rtol=1e-5, atol=1e-5)
+    assert np.allclose(dr.sum(a[:, 1:6] * 2.0, axis=1).get(), (h[:, 1:6] * 2.0).sum(axis=1), rtol=1e-5,
+                       atol=1e-5)
+    assert hip.lower_only(ReduceEx(np.add, a[:, 1:6] * 2.0, (1,)))[0].kind == "axis_short"
+    assert np.allclose(dr.sum(a, axis=1, keepdims=True).get(), h.sum(axis=1, keepdims=True), rtol=1e-5,
+                       atol=1e-5)
+    hip.set_tune(ax_short=0)                      # the wave-per-row kernel gives the same numbers
+    try:
+        assert np.allclose(dr.sum(a * W + V, axis=1).get(), (h * w + v).sum(axis=1), rtol=1e-5, atol=1e-5)
+    finally:
+        hip.set_tune(ax_short=64)
