@@ -915,6 +915,96 @@ def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
     return "\n".join(src) + "\n"
 
 
+def emit_narrow_cols(prog, leaf_kind, acc_dt, op, K):
+    """Reduction over the rows of a dense row-major matrix with few columns (K is a
+    compile-time constant, K <= 64): the matrix is read as one contiguous stream, each
+    lane keeps the columns it meets in its own accumulators, and lanes holding the
+    same columns are combined once at the end.
+
+    A wave uses LW = (64 / KC) * KC lanes, KC = K / V units per row, V elements per
+    16-byte unit (V = 1 when K is not a multiple of that); chunk number w covers units
+    [w LW, (w+1) LW), so lane l always sees columns (l mod KC) V ... + V - 1.  A wave
+    takes four consecutive chunks at a time.
+
+    leaf_kind  per leaf 'd' (dense R x K), 'w' (one row of K for all), 'b' (one element)
+    Parameters: leaf pointers, partials pointer, scalars, U (units in the matrix).
+    Output: one partial per block and column, [block][K]."""
+    ct = CTYPE[acc_dt]
+    widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "d"}
+    V = 16 // widths.pop() if len(widths) == 1 and widths <= {4, 8} else 1
+    if K % V:
+        V = 1
+    KC = K // V
+    LW = (WAVE // KC) * KC
+    waves = BLOCK // WAVE
+    src = [PREAMBLE, emit_body(prog, [acc_dt])]
+    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
+    params.append(f"{ct}* __restrict__ out")
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params.append("const long long U")
+    call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
+    ident = _identity(op, acc_dt)
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{",
+         f"    __shared__ {ct} red[{waves}][{WAVE * V}];",
+         f"    const int lane = threadIdx.x & {WAVE - 1};",
+         "    const int wave = threadIdx.x >> 6;",
+         f"    const bool live = lane < {LW};",
+         f"    const int cls = lane % {KC};"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        for e in range(V):
+            if kind == "w":
+                L.append(f"    const {CTYPE[dt]} w{i}_{e} = a{i}[cls * {V} + {e}];")
+        if kind == "b":
+            L.append(f"    const {CTYPE[dt]} b{i} = a{i}[0];")
+    for e in range(V):
+        L.append(f"    {ct} acc{e} = {ident};")
+    UN = 4      # chunks in flight per wave: loads first, then arithmetic
+    L += [f"    const long long nw = (long long)gridDim.x * {waves};",
+          f"    for (long long g = (long long)blockIdx.x * {waves} + wave; g * {UN * LW} < U; g += nw) {{"]
+    for j in range(UN):
+        L.append(f"        const long long u{j} = (g * {UN} + {j}) * {LW} + lane;")
+        L.append(f"        const bool ok{j} = live && u{j} < U;")
+        for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+            if kind == "d":
+                if V > 1:
+                    vt = VEC16[dt][0] + "u"
+                    L.append(f"        {VEC16[dt][0]} X{i}_{j} = {{}};")
+                    L.append(f"        if (ok{j}) X{i}_{j} = *(const {vt}*)(a{i} + u{j} * {V});")
+                else:
+                    L.append(f"        {CTYPE[dt]} X{i}_{j} = 0;")
+                    L.append(f"        if (ok{j}) X{i}_{j} = a{i}[u{j}];")
+    for j in range(UN):
+        L.append(f"        if (ok{j}) {{")
+        for e in range(V):
+            args = []
+            for i, kind in enumerate(leaf_kind):
+                if kind == "d":
+                    args.append(f"X{i}_{j}[{e}]" if V > 1 else f"X{i}_{j}")
+                elif kind == "w":
+                    args.append(f"w{i}_{e}")
+                else:
+                    args.append(f"b{i}")
+            L.append(f"            {{ {ct} t0; dr_body({', '.join(args + call_tail)}); "
+                     f"acc{e} = {_combine(op, f'acc{e}', 't0')}; }}")
+        L.append("        }")
+    L.append("    }")
+    for e in range(V):
+        L.append(f"    red[wave][lane * {V} + {e}] = acc{e};")
+    L += ["    __syncthreads();",
+          f"    if (threadIdx.x < {K}) {{",
+          f"        const int cc = threadIdx.x / {V};",
+          f"        const int e = threadIdx.x - cc * {V};",
+          f"        {ct} tot = {ident};",
+          f"        for (int w = 0; w < {waves}; ++w)",
+          f"            for (int l = cc; l < {LW}; l += {KC})",
+          f"                tot = {_combine(op, 'tot', f'red[w][l * {V} + e]')};",
+          f"        out[(long long)blockIdx.x * {K} + threadIdx.x] = tot;",
+          "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n", V, LW
+
+
 def emit_short_rows(prog, leaf_kind, acc_dt, op, R):
     """Reduction over a short unit-stride last dimension: a lane owns one output and
     walks its own row of R elements (R is a compile-time constant) with 16-byte loads

@@ -22,6 +22,7 @@ TUNE = {
     "ax_blocks": 4096,   # axis reductions: blocks ('col') / waves ('row') worth of work to
     "ax_waves": 32768,   # aim for before the reduced extent is cut into slices
     "ax_rows": 4,        # 'row' strategy: outputs per wave (grid-stride), to amortise set-up
+    "ax_narrow": 64,     # kept unit-stride extents up to this many columns: stream the matrix
     "ax_short": 64,      # reduced unit-stride extents up to this length: a lane per output
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
@@ -426,6 +427,39 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
     inner_kept = any(s[-1] == 1 for s in ksets)
     inner_red = any(s[-1] == 1 for s in rsets)
     strategy = "col" if (inner_kept and not inner_red) else "row"
+    if (strategy == "col" and slices in (None, 1) and 2 <= K <= TUNE["ax_narrow"]
+            and (R >= 4096 or slices == 1)
+            and len(kmerged) == 1 and len(rmerged) == 1 and R * K < 2 ** 40
+            and all((k[0], r[0]) in ((1, K), (1, 0), (0, 0)) for k, r in zip(ksets, rsets))
+            and any((k[0], r[0]) == (1, K) for k, r in zip(ksets, rsets))):
+        # a dense matrix with few columns, summed over its rows: read it as one stream
+        kinds = tuple("d" if r[0] == K else "w" if k[0] == 1 else "b" for k, r in zip(ksets, rsets))
+        low = Lowered()
+        low.lds = 0
+        low.fin_count = 0
+        low.kind = "axis_narrow"
+        low.key = ("axis_narrow", prog.key(), kinds, acc, reduce_op, K)
+
+        def emit_narrow():
+            return cg.emit_narrow_cols(prog, kinds, acc, reduce_op, K)[0]
+        low.emit = emit_narrow
+        widths = {cg.ITEMSIZE[c] for c, kd in zip(prog.leaves, kinds) if kd == "d"}
+        V = 16 // widths.pop() if len(widths) == 1 and widths <= {4, 8} else 1
+        V = V if K % V == 0 else 1
+        KC = K // V
+        LW = (cg.WAVE // KC) * KC
+        U = R * KC
+        per_block = (cg.BLOCK // cg.WAVE) * LW
+        # several passes of four chunks per wave; the partials, one row of K per block,
+        # are a narrow matrix again and one more block of this kernel finishes them
+        # (which bounds their number: that block walks S * KC units alone)
+        S = 1 if slices == 1 else max(1, min(-(-U // (per_block * 4 * 4)), TUNE["ax_blocks"],
+                                             max(256, 16384 // KC)))
+        low.grid = S
+        low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars) + "q")
+        low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+        low.scal, low.tail = list(scalars), [U]
+        return low, S, K, "col"
     if (strategy == "row" and slices is None and R <= TUNE["ax_short"] and K >= 4096
             and len(kmerged) == 1 and len(rmerged) == 1
             and all(r[0] in (0, 1) for r in rsets) and K < 2 ** 40):

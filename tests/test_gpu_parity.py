@@ -756,3 +756,38 @@ def test_reductions_over_short_rows():
         assert np.allclose(dr.sum(a * W + V, axis=1).get(), (h * w + v).sum(axis=1), rtol=1e-5, atol=1e-5)
     finally:
         hip.set_tune(ax_short=64)
+
+
+def test_reductions_over_the_rows_of_narrow_matrices():
+    """Few columns, many rows: the matrix is read as one stream, lanes keep their columns."""
+    rs = np.random.RandomState(22)
+    for shape, dt in [((50000, 3), np.float32), ((8192, 16), np.float64), ((70001, 7), np.float32),
+                      ((5000, 64), np.float32), ((20000, 33), np.int32), ((4096, 2), np.float64)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (0,)))[0]
+        assert low.kind == "axis_narrow" and low.key[-1] == shape[1]
+        ref = (h.astype(np.float64) ** 2).sum(axis=0)
+        tol = dict(rtol=2e-5) if dt == np.float32 else dict(rtol=1e-13)
+        got = dr.sum(a * a, axis=0).get()
+        assert got.dtype == (h * h).sum(axis=0).dtype and np.allclose(got, ref, **tol)
+        assert np.array_equal(dr.max(a, axis=0).get(), h.max(axis=0))
+        assert np.array_equal(dr.min(a, axis=0).get(), h.min(axis=0))
+        if dt != np.int32:
+            assert np.allclose(dr.mean(a, axis=0).get(), h.astype(np.float64).mean(axis=0),
+                               rtol=tol["rtol"], atol=1e-6)
+            assert np.allclose(dr.var(a, axis=0).get(), h.astype(np.float64).var(axis=0), rtol=1e-4)
+    # one row of weights for all rows, a scalar array, keepdims; fewer rows take the general kernel
+    h = rs.uniform(0, 1, (30000, 12)).astype(np.float32)
+    w, c = rs.uniform(0, 1, 12).astype(np.float32), np.float32(0.5)
+    a, W = dr.array(h), dr.array(w)
+    ex = a * W + dr.array(np.array([c]))
+    assert hip.lower_only(ReduceEx(np.add, ex, (0,)))[0].kind == "axis_narrow"
+    assert np.allclose(dr.sum(ex, axis=0).get(), (h.astype(np.float64) * w + c).sum(axis=0), rtol=2e-5)
+    assert np.allclose(dr.sum(a, axis=0, keepdims=True).get(), h.sum(axis=0, keepdims=True), rtol=2e-5)
+    assert hip.lower_only(ReduceEx(np.add, dr.array(h[:100]) * 1.0, (0,)))[0].kind == "axis_col"
+    assert hip.lower_only(ReduceEx(np.add, a[:, :5] * 1.0, (0,)))[0].kind == "axis_col"   # not dense
+    assert np.allclose(dr.sum(a[:, :5] * 1.0, axis=0).get(), h[:, :5].sum(axis=0), rtol=2e-5)
+    # three dimensions: the leading two merge into the rows
+    h3 = rs.uniform(-1, 1, (300, 200, 6))
+    assert np.allclose(dr.sum(dr.array(h3), axis=(0, 1)).get(), h3.sum(axis=(0, 1)), rtol=1e-12, atol=1e-10)
