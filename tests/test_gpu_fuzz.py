@@ -122,11 +122,30 @@ def test_random_expression(seed):
     assert bits_equal(got, np.asarray(ref)), (seed, shape, mode)
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_random_expression_on_skinny_matrices(seed):
+    """Many rows, few columns: the shapes that have reduction kernels of their own."""
+    rs = np.random.RandomState(5000 + seed)
+    shape = (int(rs.choice([4096, 4100, 9001])), int(rs.choice([2, 3, 7, 16, 33, 64])))
+    with np.errstate(all="ignore"):
+        d, o = random_expr(rs, shape, depth=int(rs.randint(1, 4)))
+        anchor_d, anchor_o = full_shape_leaf(rs, shape)
+        d, o = d + anchor_d, o + anchor_o
+        mode = rs.randint(4)
+        if mode == 0:
+            got, ref = d.get(), o.get()
+        else:
+            axis = int(rs.randint(2))
+            fn = (dr.max, np.max) if mode == 1 else (dr.min, np.min)
+            got, ref = fn[0](d, axis=axis).get(), fn[1](o.a, axis=axis)
+    assert bits_equal(got, np.asarray(ref)), (seed, shape, mode)
+
+
 def test_fuzz_reached_every_kernel_shape():
     """Runs after the cases above: the kernel cache must hold every shape kind."""
     kinds = {}
     for key in hip._KERNELS:
         kinds[key[0]] = kinds.get(key[0], 0) + 1
     print("kernel kinds compiled:", kinds)
-    for kind in ("flat", "nd", "tile2d", "tile2dv", "tile2dt", "axis"):
+    for kind in ("flat", "nd", "tile2d", "tile2dv", "tile2dt", "axis", "axis_short", "axis_narrow"):
         assert kinds.get(kind, 0) > 0, kind
