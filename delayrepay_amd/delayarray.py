@@ -821,6 +821,8 @@ def _over_views(root, view):
     to be evaluated first."""
     shape = tuple(root.shape)
     fb = _backend.fallback
+    if getattr(fb, "broadcast_to", None) is None:
+        return None
     memo = {}
     budget = [PUSH_VIEWS_UP_TO]
     new_shape = tuple(view(np.broadcast_to(np.empty((), dtype=bool), shape)).shape)
