@@ -16,16 +16,25 @@ Differences in what is emitted:
     expressions produce identical source and hit the kernel cache (the
     reference embeds a global serial number, delayarray.py:150-152).
 
-Kernel shapes (all 256-thread blocks = 4 wave64, grid-stride):
-  flat     contiguous operands, 128-bit loads/stores, several vectors in
-           flight per thread, optional non-temporal access, scalar tail;
-  nd       arbitrary strides / broadcasting, one element per thread-iteration;
-  stencil  2-D operands that are shifted views of one buffer: the union of the
-           shifted tiles is staged once through LDS (halo tile), tiles are
-           assigned to XCDs in contiguous bands;
+Kernel shapes (all 256-thread blocks = 4 wave64):
+  flat      contiguous operands: one run of 256 16-byte vectors per block, optional
+            non-temporal access, scalar tail; supplies the element index to
+            index-valued leaves (`arange`, `linspace`)          emit_flat
+  tile2d    N-d operands whose last dimension has unit or zero stride; shifted views
+            of one buffer are staged once through an LDS halo tile, tiles go to XCDs
+            in contiguous bands                     emit_stencil, emit_stencil_vec
+  tile2dt   some operand is a transposed matrix: 64x64 LDS transpose, diagonal tile
+            order                                               emit_tile_transpose
+  nd        arbitrary strides / broadcasting, one element per thread-iteration
+                                                                emit_nd
+  axis_*    reductions along some axes: col / row (sliced, two passes), short rows
+            (a lane per output), narrow matrices (streamed, per-lane columns)
+                           emit_axis_reduce, emit_short_rows, emit_narrow_cols
   + an optional reduction tail on flat/nd: per-thread accumulators, wave64
     shuffle tree, LDS across the 4 waves, one partial per block, and a
     one-block finalize kernel (no atomics, deterministic).
+Vector accesses use 16-byte types at element alignment where 16-byte alignment is
+missing; float64 `log`, `erf`, `exp` come from `mathlib`.
 """
 import numpy as np
 

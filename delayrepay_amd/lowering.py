@@ -405,9 +405,12 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
 def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices=None):
     """Kernel choice for reducing over `axes` of the (broadcast) `shape`.
 
-    Returns (first pass, S): when S > 1 the first pass writes S partial results
-    per output ([slice][output] for 'col', [output][slice] for 'row') and the
-    caller runs a second reduction over them."""
+    Returns (first pass, S, K, strategy): when S > 1 the first pass writes S partial
+    results per output ([slice][output] for 'col', [output][slice] for 'row') and the
+    caller runs a second reduction over them (`slices=1` asks for that second pass).
+    Matrices with one short side have kernels of their own: `axis_narrow` (few kept
+    columns, dense rows reduced; its partials are laid out like 'col') and
+    `axis_short` (short contiguous rows reduced; no partials)."""
     kept = [d for d in range(len(shape)) if d not in axes]
     full = [broadcast_strides(a, shape) for a in leaves]
     kshape = [shape[d] for d in kept]
