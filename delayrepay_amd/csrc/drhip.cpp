@@ -121,6 +121,8 @@ int drhip_device_info_get(drhip_device_info* out) {
     out->clock_khz = g_prop.clockRate;
     out->mem_clock_khz = g_prop.memoryClockRate;
     out->mem_bus_bits = g_prop.memoryBusWidth;
+    int major = 0, minor = 0;
+    if (hiprtcVersion(&major, &minor) == HIPRTC_SUCCESS) out->hiprtc_version = major * 1000 + minor;
     return 0;
 }
 

@@ -265,8 +265,9 @@ def _load_or_compile(source):
     use_disk = "DELAYREPAY_NO_DISK_CACHE" not in os.environ
     path = None
     if use_disk:
-        arch = hiprt.device_info()["arch"]
-        digest = hashlib.sha256("\0".join([source, arch] + COMPILE_OPTS).encode()).hexdigest()
+        info = hiprt.device_info()
+        digest = hashlib.sha256("\0".join([source, info["arch"], str(info["hiprtc_version"])]
+                                          + COMPILE_OPTS).encode()).hexdigest()
         path = os.path.join(_cache_dir(), digest + ".co")
         if os.path.exists(path):
             try:

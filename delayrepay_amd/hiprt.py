@@ -34,7 +34,7 @@ class DeviceInfo(C.Structure):
         ("clock_khz", C.c_int32),
         ("mem_clock_khz", C.c_int32),
         ("mem_bus_bits", C.c_int32),
-        ("reserved", C.c_int32),
+        ("hiprtc_version", C.c_int32),
     ]
 
 
@@ -143,7 +143,7 @@ def device_info():
     info = DeviceInfo()
     _check(lib().drhip_device_info_get(C.byref(info)))
     return {f: (getattr(info, f).decode() if isinstance(getattr(info, f), bytes) else getattr(info, f))
-            for f, _ in DeviceInfo._fields_ if f != "reserved"}
+            for f, _ in DeviceInfo._fields_}
 
 
 def malloc(nbytes):

@@ -53,7 +53,7 @@ typedef struct drhip_device_info {
     int32_t  clock_khz;
     int32_t  mem_clock_khz;
     int32_t  mem_bus_bits;
-    int32_t  reserved;
+    int32_t  hiprtc_version; /* major * 1000 + minor of the run-time compiler   */
 } drhip_device_info;
 int drhip_device_info_get(drhip_device_info* out);
 
