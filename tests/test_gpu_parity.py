@@ -791,3 +791,32 @@ def test_reductions_over_the_rows_of_narrow_matrices():
     # three dimensions: the leading two merge into the rows
     h3 = rs.uniform(-1, 1, (300, 200, 6))
     assert np.allclose(dr.sum(dr.array(h3), axis=(0, 1)).get(), h3.sum(axis=(0, 1)), rtol=1e-12, atol=1e-10)
+
+
+def test_own_float64_functions_stay_within_two_ulp_of_numpy_on_the_device():
+    """The device build differs from the host build checked in test_mathlib.py in two
+    places (reciprocal seed + Newton steps, multiply-add with a scalar-register
+    constant); libm and SciPy are within 1 resp. 2.6 ulp of the true value themselves."""
+    from scipy.special import erf
+    rs = np.random.RandomState(31)
+    n = 1 << 20
+    cases = {
+        "log": (np.log, np.concatenate([rs.uniform(1e-6, 1e6, n), np.exp(rs.uniform(-700, 700, n)),
+                                        1 + rs.uniform(-1e-6, 1e-6, n // 4),
+                                        [5e-324, 1e-310, 2.2250738585072014e-308, 1.7976931348623157e308]]), 2),
+        "exp": (np.exp, np.concatenate([rs.uniform(-20, 20, n), rs.uniform(-708, 709, n),
+                                        rs.uniform(-1e-3, 1e-3, n // 4)]), 2),
+        "erf": (erf, np.concatenate([rs.uniform(-6.5, 6.5, n), rs.uniform(-1, 1, n),
+                                     10.0 ** rs.uniform(-300, 0, n // 4)]), 4),
+    }
+    for name, (fn, x, bar) in cases.items():
+        got, ref = fn(dr.array(x)).get(), fn(x)
+        d = np.abs(got - ref) / np.spacing(np.abs(ref))
+        print(name, "worst ulp distance from the host library:", d.max())
+        assert d.max() <= bar, (name, x[d.argmax()], d.max())
+    hip.set_tune(dmath=0)          # the device library's versions, for comparison
+    try:
+        x = rs.uniform(0.1, 10, 1 << 16)
+        assert np.max(np.abs(np.log(dr.array(x)).get() - np.log(x)) / np.spacing(np.abs(np.log(x)))) <= 2
+    finally:
+        hip.set_tune(dmath=1)
