@@ -379,6 +379,22 @@ class record:
 
 _STAMP = 0            # bumped whenever tunables or the fusion mode change
 _RECENT = collections.deque(maxlen=int(os.environ.get("DELAYREPAY_KEEP", "16")))
+_RECENT_BYTES = int(os.environ.get("DELAYREPAY_KEEP_BYTES", str(8 << 30)))
+
+
+def _remember(node):
+    """Keep `node` alive so that the same expression, built again, finds its nodes in
+    the hash-cons table and its plan on the root.  A kept root also keeps its cached
+    result, so the memory held this way is bounded as well as the count."""
+    _RECENT.append(node)
+    held = 0
+    for k in range(len(_RECENT) - 1, -1, -1):       # newest first
+        arr = _RECENT[k].__dict__.get("array")
+        held += getattr(arr, "nbytes", 0)
+        if held > _RECENT_BYTES and k < len(_RECENT) - 1:
+            for _ in range(k + 1):
+                _RECENT.popleft()
+            break
 
 
 def forget():
@@ -648,7 +664,7 @@ def run(ex):
             root = _trace_root(tracer, ex)
             plan = _make_plan(tracer, [root])
         d["_plan"] = plan
-        _RECENT.append(ex)
+        _remember(ex)
     else:
         STATS["plan_hits"] += 1
     out = _launch_fresh(plan)[0]
@@ -677,7 +693,7 @@ def run_multi(exs):
             roots = [_trace_root(tracer, exs[i]) for i in idxs]
             plan = _make_plan(tracer, roots)
             first["_multi"] = (key, plan, [exs[i] for i in idxs])
-            _RECENT.append(exs[idxs[0]])
+            _remember(exs[idxs[0]])
         outs = _launch_fresh(plan)
         deps = plan.deps()
         for i, out in zip(idxs, outs):
@@ -788,7 +804,7 @@ def run_into(ex, dst):
         root = _trace_root(tracer, ex)
         plan = _plan_write(tracer, root, dst)
         d["_into"] = (key, plan, dst.buf)     # holding the buffer keeps its id unique
-        _RECENT.append(ex)
+        _remember(ex)
     _write(plan, dst)
 
 

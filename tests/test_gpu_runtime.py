@@ -164,3 +164,19 @@ def test_recorded_launches_replay_as_a_hip_graph():
             hiprt.memcpy_d2d(total.ptr, total.ptr, 8)
     finally:
         hiprt.Graph.end()
+
+
+def test_recent_roots_are_bounded_by_the_memory_their_results_hold(monkeypatch):
+    import delayrepay_amd as dr
+    x = dr.array(np.ones(1 << 18))                       # 2 MiB results
+    monkeypatch.setattr(hip, "_RECENT_BYTES", 5 << 20)
+    hip.forget()
+    kept = []
+    for k in range(8):
+        node = x * float(k + 2)
+        kept.append(node.get()[0])
+        del node
+    assert kept == [float(k + 2) for k in range(8)]
+    held = sum(n.__dict__["array"].nbytes for n in hip._RECENT if "array" in n.__dict__)
+    assert len(hip._RECENT) <= 4 and held <= (5 << 20) + (2 << 20)
+    hip.forget()
