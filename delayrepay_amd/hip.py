@@ -728,6 +728,10 @@ def _plan_write(tracer, root, dst):
     shape = dst.shape
     for a in tracer.leaves:
         _broadcast_strides(a, shape)  # raises when the value does not fit the destination
+    for gen in tracer.gen_shapes:     # generated leaves have a shape too
+        if tuple(numpy.broadcast_shapes(gen, shape)) != tuple(shape):
+            raise ValueError(f"could not broadcast input array from shape {tuple(gen)} "
+                             f"into shape {tuple(shape)}")
     hazard = False
     d_lo, d_hi = _extent(dst)
     for a in tracer.leaves:

@@ -680,6 +680,8 @@ def test_constant_arrays_stay_lazy_until_written():
                       (lambda: dr.full_like(dr.array(a), 1.5, dtype=np.float64), np.full_like(a, 1.5, dtype=np.float64)),
                       (lambda: dr.zeros(4096, dtype=bool), np.zeros(4096, bool))]:
         assert _same(make().get(), ref)
+    with pytest.raises(ValueError):                                # shapes are still checked
+        dr.array(np.zeros(6000))[:] = dr.zeros(5000) + 1.0
     # the Jacobi set-up of configuration C4 starts from zeros and writes the interior
     u = dr.zeros((64, 64), dtype=np.float32)
     u[1:-1, 1:-1] = dr.array(a[:62, :62])
