@@ -822,3 +822,25 @@ def test_own_float64_functions_stay_within_two_ulp_of_numpy_on_the_device():
         assert np.max(np.abs(np.log(dr.array(x)).get() - np.log(x)) / np.spacing(np.abs(np.log(x)))) <= 2
     finally:
         hip.set_tune(dmath=1)
+
+
+def test_generated_leaves_behave_like_arrays_everywhere():
+    assert float(dr.sum(dr.ones(10000))) == 10000.0
+    assert float(dr.max(dr.arange(10000))) == 9999
+    assert np.array_equal(dr.ones((300, 400)).T.get(), np.ones((400, 300)))
+    assert np.array_equal(dr.zeros(5000)[10:20].get(), np.zeros(10))
+    assert dr.ones(5000).astype(np.float32).get().dtype == np.float32
+    assert np.array_equal(dr.arange(5000).reshape(50, 100).get(), np.arange(5000).reshape(50, 100))
+    assert np.array_equal(dr.where(dr.arange(5000) > 10, 1.0, 0.0).get(), np.where(np.arange(5000) > 10, 1.0, 0.0))
+    assert abs(float(dr.mean(dr.linspace(0, 1, 5000))) - 0.5) < 1e-12
+    assert np.array_equal(dr.sum(dr.ones((300, 400)), axis=0).get(), np.full(400, 300.0))
+    assert np.array_equal(dr.sum(dr.ones((5000, 4)), axis=1).get(), np.full(5000, 4.0))
+    assert np.array_equal(dr.sum(dr.ones((5000, 4)) * dr.array(np.arange(4.0)), axis=0).get(), np.arange(4.0) * 5000)
+    a = dr.arange(6000); b = a.copy(); assert np.array_equal(b.get(), np.arange(6000))
+    assert len(dr.zeros((5000, 3))) == 5000 and dr.zeros((5000, 3)).ndim == 2
+    z = dr.zeros(5000); z += 1; assert np.array_equal(z.get(), np.ones(5000))
+    e, f = dr.evaluate(dr.ones(5000) * 2, dr.arange(5000) + 1)
+    assert np.array_equal(e.get(), np.full(5000, 2.0)) and np.array_equal(f.get(), np.arange(5000) + 1)
+    assert np.array_equal(np.roll(dr.arange(5000) * 1, 3).get(), np.roll(np.arange(5000), 3))
+    assert repr(dr.arange(5000)).startswith("[   0    1    2")
+    assert np.array_equal(np.asarray(dr.arange(5000)), np.arange(5000))
