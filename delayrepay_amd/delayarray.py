@@ -1141,6 +1141,49 @@ for _name in ("empty", "empty_like", "eye", "identity", "ones", "ones_like", "ze
         globals()[_name] = cast(_fn)
 del _name, _fn
 
+Shape = tuple          # (rows, columns), as annotated in delayarray.py:159
+
+
+def is_matrix_matrix(left, right):
+    """Shapes of a matrix-matrix product (delayarray.py:454-455)."""
+    return len(left) > 1 and len(right) > 1
+
+
+def is_matrix_vector(left, right):
+    """Shapes of a matrix-vector product (delayarray.py:458-459)."""
+    return len(left) > 1 and len(right) == 1
+
+
+def _triangle(lower):
+    def tri_part(m, k=0):
+        """`numpy.tril` / `numpy.triu` (delayarray.py:642-643) as a lazy `where` over the
+        row and column indices: fused with whatever produces `m`, no mask array."""
+        m = arg_to_numpy_ex(m)
+        if m.ndim < 2:
+            raise ValueError("tril/triu need an array of at least two dimensions")
+        rows, cols = m.shape[-2:]
+        r = NPArray(_backend.fallback.asarray(np.arange(rows).reshape(rows, 1)))
+        c = NPArray(_backend.fallback.asarray(np.arange(cols)))
+        keep = (c - r <= int(k)) if lower else (c - r >= int(k))
+        return where(keep, m, m.dtype.type(0))
+    tri_part.__name__ = "tril" if lower else "triu"
+    return tri_part
+
+
+tril = _triangle(True)
+triu = _triangle(False)
+if "asmatrix" not in globals():
+    def asmatrix(data, dtype=None):
+        """2-d view of the data as a leaf (delayarray.py:624 wraps `numpy.asmatrix`; the
+        matrix subclass itself has no device counterpart)."""
+        arr = arg_to_numpy_ex(data if dtype is None else np.asarray(_unwrap_host(data), dtype=dtype))
+        return arr if arr.ndim == 2 else arr.reshape((1, -1) if arr.ndim < 2 else arr.shape)
+
+
+def _unwrap_host(obj):
+    return obj.get() if isinstance(obj, DelayArray) else obj
+
+
 # Generated leaves: constant and index-valued arrays stay lazy when the backend can
 # compute them inside a kernel.  Arrays shorter than this are made at once, as before.
 GENERATE_FROM = 4096

@@ -247,3 +247,20 @@ class TestEagerRoutines:
         npt.assert_allclose(np.var(a), a0.var(), rtol=1e-12)
         npt.assert_allclose(a.var(), a0.var(), rtol=1e-12)
         npt.assert_allclose(float(a.sum()), a0.sum(), rtol=1e-13)
+
+
+def test_tril_triu_asmatrix_and_shape_helpers():
+    """delayarray.py:454-459,624,642-643."""
+    import delayrepay as dnp
+    h = np.random.RandomState(3).uniform(-1, 1, (130, 70)).astype(np.float32)
+    a = dnp.array(h)
+    for k in (-3, 0, 1, 40):
+        assert np.array_equal(dnp.tril(a, k).get(), np.tril(h, k))
+        assert np.array_equal(dnp.triu(a * 2, k).get(), np.triu(h * 2, k))
+    lazy = dnp.tril(a + 1)
+    assert "array" not in lazy.__dict__ and lazy.dtype == np.float32
+    h3 = np.arange(2 * 5 * 6.0).reshape(2, 5, 6)
+    assert np.array_equal(dnp.triu(dnp.array(h3), 1).get(), np.triu(h3, 1))
+    assert dnp.asmatrix(dnp.array(np.arange(4.0))).shape == (1, 4)
+    assert dnp.is_matrix_matrix((3, 4), (4, 5)) and dnp.is_matrix_vector((3, 4), (4,))
+    assert not dnp.is_matrix_vector((3, 4), (4, 5))
