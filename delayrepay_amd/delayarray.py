@@ -252,7 +252,7 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         computed, and shifted slices of one expression fuse into one stencil."""
         key = _unwrap(key)
         if "array" not in self.__dict__ and type(self) in _ELEMENTWISE and _basic_key(key):
-            res = _over_views(self, lambda arr: arr[key])
+            res = _over_views(self, lambda arr: arr[key], key)
             if res is not None:
                 return res
         return NPArray(self._force()[key])
@@ -814,7 +814,7 @@ def _basic_key(key):
     return all(k is None or k is Ellipsis or isinstance(k, (slice, int, np.integer)) for k in key)
 
 
-def _over_views(root, view):
+def _over_views(root, view, key=None):
     """The unevaluated element-wise expression `root` rebuilt over `view(leaf)` of each
     leaf, every leaf first broadcast to the root's shape (so one view function serves
     all of them); None when the expression is too large or holds something that has
@@ -826,6 +826,8 @@ def _over_views(root, view):
     memo = {}
     budget = [PUSH_VIEWS_UP_TO]
     new_shape = tuple(view(np.broadcast_to(np.empty((), dtype=bool), shape)).shape)
+    sl = key[0] if isinstance(key, tuple) and len(key) == 1 else key
+    sl = sl if isinstance(sl, slice) and len(shape) == 1 else None
 
     def walk(node):
         hit = memo.get(id(node))
@@ -839,6 +841,15 @@ def _over_views(root, view):
             res = NPArray(view(fb.broadcast_to(node._force(), shape)))
         elif kind is FullEx and arr is None:
             res = FullEx(new_shape, node.val, node.dtype)
+        elif kind is IotaEx and arr is None and sl is not None and node.shape == shape \
+                and shape[0] <= (1 << 24 if node.dtype == np.float32 else 1 << 53):
+            # a slice of 0, 1, 2, ... is start + step * (0, 1, 2, ...): still no memory
+            picked = range(shape[0])[sl]
+            res = IotaEx(len(picked), node.dtype)
+            if picked.step != 1:
+                res = res * node.dtype.type(picked.step)
+            if picked.start != 0:
+                res = res + node.dtype.type(picked.start)
         elif kind in _ELEMENTWISE:
             budget[0] -= 1
             if budget[0] < 0:

@@ -844,3 +844,20 @@ def test_generated_leaves_behave_like_arrays_everywhere():
     assert np.array_equal(np.roll(dr.arange(5000) * 1, 3).get(), np.roll(np.arange(5000), 3))
     assert repr(dr.arange(5000)).startswith("[   0    1    2")
     assert np.array_equal(np.asarray(dr.arange(5000)), np.arange(5000))
+
+
+def test_slices_of_generated_grids_stay_generated():
+    n = 1 << 20
+    g = dr.linspace(-2.0, 2.0, n, dtype=np.float32)
+    p = ((0.5 * g + 1.0) * g - 3.0) * g
+    lap = (p[:-2] + p[2:]) - 2.0 * p[1:-1]
+    hg = np.linspace(-2.0, 2.0, n, dtype=np.float32)
+    hp = ((np.float32(0.5) * hg + 1) * hg - 3) * hg
+    assert len(hip.lower_only(lap)[0].srcs) == 0                 # nothing is read
+    before = hip.STATS["launches"]
+    got = lap.get()
+    assert hip.STATS["launches"] - before == 1
+    assert _same(got, (hp[:-2] + hp[2:]) - np.float32(2.0) * hp[1:-1])
+    a = dr.arange(100000)
+    assert _same((a * 3)[5:90000:7].get(), (np.arange(100000) * 3)[5:90000:7])
+    assert _same((a * 3)[::-1][:10].get(), (np.arange(100000) * 3)[::-1][:10])
