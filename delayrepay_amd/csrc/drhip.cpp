@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -127,10 +128,17 @@ int drhip_device_info_get(drhip_device_info* out) {
 }
 
 // ---- pool ------------------------------------------------------------------
+// One host thread drives the library, but an array's finaliser may run on whichever
+// thread happens to collect it, while the driving thread is inside another call (a
+// Python caller drops its interpreter lock for the duration of a foreign call): the
+// pool's tables are therefore guarded.  Recursive: an out-of-memory drhip_malloc trims.
+static std::recursive_mutex g_pool_mutex;
+#define POOL_LOCK() std::lock_guard<std::recursive_mutex> pool_lock_(g_pool_mutex)
 
 int drhip_malloc(void** dptr, size_t nbytes) {
     NEED_INIT();
     if (!dptr) return fail(DRHIP_EINVAL, "drhip_malloc", "null dptr");
+    POOL_LOCK();
     const size_t c = size_class(nbytes);
     g_pool.st.n_mallocs++;
     auto it = g_pool.free_lists.find(c);
@@ -164,6 +172,7 @@ int drhip_malloc(void** dptr, size_t nbytes) {
 int drhip_free(void* dptr) {
     if (!dptr) return 0;
     NEED_INIT();
+    POOL_LOCK();
     auto it = g_pool.live.find(dptr);
     if (it == g_pool.live.end())
         return fail(DRHIP_EINVAL, "drhip_free", "pointer was not returned by drhip_malloc");
@@ -177,12 +186,14 @@ int drhip_free(void* dptr) {
 
 int drhip_pool_stats(drhip_pool_stats_t* out) {
     if (!out) return fail(DRHIP_EINVAL, "drhip_pool_stats", "null out");
+    POOL_LOCK();
     *out = g_pool.st;
     return 0;
 }
 
 int drhip_pool_trim(void) {
     NEED_INIT();
+    POOL_LOCK();
     HIP_TRY(hipStreamSynchronize(g_stream));
     for (auto& kv : g_pool.free_lists) {
         for (void* p : kv.second) {

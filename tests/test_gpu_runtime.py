@@ -180,3 +180,34 @@ def test_recent_roots_are_bounded_by_the_memory_their_results_hold(monkeypatch):
     held = sum(n.__dict__["array"].nbytes for n in hip._RECENT if "array" in n.__dict__)
     assert len(hip._RECENT) <= 4 and held <= (5 << 20) + (2 << 20)
     hip.forget()
+
+
+def test_pool_survives_finalisers_running_on_other_threads():
+    """Foreign calls drop the interpreter lock, so frees issued by another thread's
+    garbage collection can overlap the driving thread's allocations."""
+    import threading
+    hiprt.init()
+    before = hiprt.pool_stats()
+    errors = []
+
+    def churn(seed):
+        try:
+            sizes = [256 << (k % 9) for k in range(seed, seed + 400)]
+            held = []
+            for n in sizes:
+                held.append(hiprt.malloc(n))
+                if len(held) > 16:
+                    hiprt.free(held.pop(0))
+            for p in held:
+                hiprt.free(p)
+        except Exception as exc:      # noqa: BLE001
+            errors.append(exc)
+    threads = [threading.Thread(target=churn, args=(k,)) for k in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    after = hiprt.pool_stats()
+    assert not errors
+    assert after["bytes_in_use"] == before["bytes_in_use"]
+    assert after["n_mallocs"] - before["n_mallocs"] == 6 * 400
