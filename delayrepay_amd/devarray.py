@@ -16,6 +16,7 @@ import numpy.lib.mixins
 
 from . import hiprt
 
+_CHECKED_DTYPES = set()
 SUPPORTED_DTYPES = ("float32", "float64", "int32", "int64", "bool", "uint8", "uint32")
 
 
@@ -88,8 +89,10 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
     def __init__(self, shape, dtype, buf=None, offset=0, strides=None):
         self.shape = tuple(int(d) for d in shape)
         self.dtype = np.dtype(dtype)
-        if self.dtype.name not in SUPPORTED_DTYPES:
-            raise TypeError(f"dtype {self.dtype} is not supported on the device")
+        if self.dtype not in _CHECKED_DTYPES:        # `dtype.name` is slow: look once per dtype
+            if self.dtype.name not in SUPPORTED_DTYPES:
+                raise TypeError(f"dtype {self.dtype} is not supported on the device")
+            _CHECKED_DTYPES.add(self.dtype)
         self._strides = _contiguous_strides(self.shape) if strides is None else tuple(strides)
         self.offset = int(offset)
         size = 1
@@ -191,11 +194,36 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
     # ---- views -----------------------------------------------------------
 
     def _view(self, shape, strides, offset):
-        return ndarray(shape, self.dtype, self.buf, offset, strides)
+        view = ndarray.__new__(ndarray)     # same buffer and dtype: nothing to validate
+        view.shape = tuple(shape)
+        view.dtype = self.dtype
+        view._strides = tuple(strides)
+        view.offset = offset
+        size = 1
+        for d in view.shape:
+            size *= d
+        view.size = size
+        view.buf = self.buf
+        return view
 
     def __getitem__(self, key):
         if not isinstance(key, tuple):
             key = (key,)
+        # the same few slices of one array come back every pass of an iterative loop
+        try:
+            token = tuple((k.start, k.stop, k.step) if type(k) is slice else k for k in key)
+            cache = self.__dict__.setdefault("_views", {})
+            hit = cache.get(token)
+            if hit is not None:
+                return hit
+        except TypeError:            # an unhashable index: no caching
+            token = cache = None
+        view = self._index(key)
+        if cache is not None and len(cache) < 32:
+            cache[token] = view
+        return view
+
+    def _index(self, key):
         n_specified = sum(1 for k in key if k is not None and k is not Ellipsis)
         if n_specified > self.ndim:
             raise IndexError("too many indices for array")
