@@ -21,6 +21,7 @@ Per configuration:
                       of the reference's CPU backend) on this machine's host cores
 """
 import argparse
+import contextlib
 import json
 import os
 import statistics
@@ -58,7 +59,8 @@ def parse():
     ap.add_argument("--workload", default="all",
                     help="horner (headline) | saxpy | bs32 | bs64 | jacobi | sumsq | all (these six); "
                          "dot | axis0 | axis1 | rowbcast | transpose | grid | next (these six: the "
-                         "operations either side of the five configurations)")
+                         "operations either side of the five configurations); "
+                         "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before each timed region (clock ramp-up)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0,
@@ -156,6 +158,18 @@ def main():
                         step=lambda: hip.run(horner_expr(c, g)),
                         cpu=lambda: orc.horner(c, np.linspace(-2.0, 2.0, m, dtype=np.float32)),
                         cpu_frac=1 / 16)
+        if name in ("matmul32", "matmul64"):
+            N = 8192
+            dt = np.float32 if name == "matmul32" else np.float64
+            ha, hb = rs.standard_normal((N, N)).astype(dt), rs.standard_normal((N, N)).astype(dt)
+            a, b = dr.array(ha), dr.array(hb)
+            m = 1024        # CPU sample: a 1024^3 product (NumPy's BLAS, all host cores)
+            return dict(dtype="f32" if dt == np.float32 else "f64", n=N * N,
+                        nbytes=3 * N * N * ha.itemsize, flops=2 * N ** 3, direct="matmul_mfma_kernel",
+                        mfma_peak=157.3 if dt == np.float32 else 78.6,
+                        desc=f"a @ b {np.dtype(dt).name} 8192^3 (eager matrix product on the matrix cores)",
+                        step=lambda: a.dot(b)._force(),
+                        cpu=lambda: ha[:m, :m] @ hb[:m, :m], cpu_frac=(m / N) ** 2)
         if name in ("axis0", "axis1", "rowbcast", "transpose"):
             N = 16384
             ha = rs.standard_normal((N, N)).astype(np.float32)
@@ -208,17 +222,22 @@ def main():
         ms_per_step = wall / K * 1e3
         # kernel duration: record the launches of one step (two for the ping-pong
         # stencil, which alternates between two buffers), replay them back to back
-        with hip.record() as plan:
+        if wl.get("direct"):     # a library kernel, launched without the fusion machinery
+            plan = step
+        with (hip.record() if not wl.get("direct") else contextlib.nullcontext()) as rec:
             keep = step()
             if wl.get("pair"):
                 keep = step()
+        if not wl.get("direct"):
+            plan = rec
         names_by_func = {}
         for kern in hip._KERNELS.values():
             nm = kern.source.split('extern "C" __global__')[-1].split("void ")[1].split("(")[0]
             names_by_func[kern.func] = nm
             if kern.finalize:
                 names_by_func[kern.finalize] = nm + "_fin"
-        kernel_names = sorted({names_by_func.get(f, "?") for f, _, _, _ in plan.launches})
+        kernel_names = [wl["direct"]] if wl.get("direct") else \
+            sorted({names_by_func.get(f, "?") for f, _, _, _ in plan.launches})
         steps_per_replay = 2 if wl.get("pair") else 1
         reps = max(1, K // steps_per_replay)
         t_warm = time.perf_counter()
@@ -246,7 +265,11 @@ def main():
             "roofline_frac": round(wl["nbytes"] / kernel_ms / 1e6 / HBM_PEAK_GBPS, 4),
             # what limits the kernel (rocprofv3 VALUBusy / traffic in profiles/)
             "bound": {"bs64": "fp64 vector ALU (VALUBusy 89%), not HBM",
-                      "bs32": "fp32 vector ALU (VALUBusy ~100%) and HBM"}.get(name, "hbm"),
+                      "bs32": "fp32 vector ALU (VALUBusy ~100%) and HBM",
+                      "matmul32": "mfma", "matmul64": "mfma"}.get(name, "hbm"),
+            **({"TFLOPs": round(wl["flops"] / kernel_ms / 1e9, 1),
+                "mfma_frac": round(wl["flops"] / kernel_ms / 1e9 / wl["mfma_peak"], 4),
+                "mfma_peak_TFLOPs": wl["mfma_peak"]} if wl.get("flops") else {}),
             "first_call_ms": round(first_ms, 2),
             "compile_ms": round((c1["compile_ns"] - c0["compile_ns"]) / 1e6, 2),
             "input_gen_s": round(t_gen, 2),

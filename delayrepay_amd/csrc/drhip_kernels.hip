@@ -86,6 +86,149 @@ __global__ __launch_bounds__(kBlock) void matmul_kernel(const T* __restrict__ A,
         }
 }
 
+// ---- the same product on the matrix cores -----------------------------------------
+// A 256-thread block owns a 128x128 tile of C; its four waves own 64x64 quarters and
+// keep them in MFMA accumulators (float: 2x2 tiles of v_mfma_f32_32x32x2f32, double:
+// 4x4 tiles of v_mfma_f64_16x16x4f64).  A and B pass through LDS TK deep, A stored
+// k-major so that both operands are read with consecutive lanes on consecutive
+// addresses; the next k-slab is fetched from global memory into registers while the
+// current one is multiplied (two LDS buffers, one barrier per slab).
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef double f64x2u __attribute__((ext_vector_type(2), aligned(8)));
+
+template <typename T> struct Mfma;
+template <> struct Mfma<float> {
+    static constexpr int MT = 32, MK = 2, TILES = 2, NACC = 16, V = 4, TK = 16;
+    using acc_t = f32x16;
+    using vec_t = f32x4;
+    using vecu_t = f32x4u;
+    static __device__ __forceinline__ acc_t mac(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+    // accumulator register v of lane l holds C[row(v, l)][l % 32]
+    static __device__ __forceinline__ int row(int v, int lane) {
+        return (v / 4) * 8 + (lane / 32) * 4 + (v % 4);
+    }
+};
+template <> struct Mfma<double> {
+    static constexpr int MT = 16, MK = 4, TILES = 4, NACC = 4, V = 2, TK = 8;
+    using acc_t = f64x4;
+    using vec_t = f64x2;
+    using vecu_t = f64x2u;
+    static __device__ __forceinline__ acc_t mac(double a, double b, acc_t c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int row(int v, int lane) { return 4 * v + lane / 16; }
+};
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void matmul_mfma_kernel(const T* __restrict__ A,
+                                                             const T* __restrict__ B,
+                                                             T* __restrict__ C, long M, long N,
+                                                             long K, long lda, long ldb,
+                                                             long ldc) {
+    using P = Mfma<T>;
+    constexpr int MT = P::MT, MK = P::MK, TI = P::TILES, V = P::V, TK = P::TK;
+    constexpr int BM = 2 * TI * MT, BN = BM, PAD = 4;      // 128 x 128
+    constexpr int A_VECS = BM * TK / V / kBlock;            // vectors per thread and slab: 2
+    constexpr int B_VECS = TK * BN / V / kBlock;
+    __shared__ __attribute__((aligned(16))) T As[2][TK][BM + PAD];
+    __shared__ __attribute__((aligned(16))) T Bs[2][TK][BN + PAD];   // rows are 16-byte multiples
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long row0 = (long)blockIdx.y * BM, col0 = (long)blockIdx.x * BN;
+    const int wrow = (wave >> 1) * TI * MT, wcol = (wave & 1) * TI * MT;
+    typename P::acc_t acc[TI][TI];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TI; ++j)
+#pragma unroll
+            for (int v = 0; v < P::NACC; ++v) acc[i][j][v] = T(0);
+
+    typename P::vec_t ra[A_VECS], rb[B_VECS];
+    auto fetch = [&](long k0) {
+#pragma unroll
+        for (int p = 0; p < A_VECS; ++p) {
+            const int idx = threadIdx.x + p * kBlock;
+            const int r = idx / (TK / V), kq = (idx % (TK / V)) * V;
+            const long gr = row0 + r, gk = k0 + kq;
+            if (gr < M && gk + V <= K) {
+                ra[p] = *(const typename P::vecu_t*)(A + gr * lda + gk);
+            } else {
+#pragma unroll
+                for (int q = 0; q < V; ++q)
+                    ra[p][q] = (gr < M && gk + q < K) ? A[gr * lda + gk + q] : T(0);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < B_VECS; ++p) {
+            const int idx = threadIdx.x + p * kBlock;
+            const int k = idx / (BN / V), c = (idx % (BN / V)) * V;
+            const long gk = k0 + k, gc = col0 + c;
+            if (gk < K && gc + V <= N) {
+                rb[p] = *(const typename P::vecu_t*)(B + gk * ldb + gc);
+            } else {
+#pragma unroll
+                for (int q = 0; q < V; ++q)
+                    rb[p][q] = (gk < K && gc + q < N) ? B[gk * ldb + gc + q] : T(0);
+            }
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < A_VECS; ++p) {
+            const int idx = threadIdx.x + p * kBlock;
+            const int r = idx / (TK / V), kq = (idx % (TK / V)) * V;
+#pragma unroll
+            for (int q = 0; q < V; ++q) As[buf][kq + q][r] = ra[p][q];
+        }
+#pragma unroll
+        for (int p = 0; p < B_VECS; ++p) {
+            const int idx = threadIdx.x + p * kBlock;
+            const int k = idx / (BN / V), c = (idx % (BN / V)) * V;
+            *(typename P::vec_t*)&Bs[buf][k][c] = rb[p];
+        }
+    };
+
+    const long slabs = (K + TK - 1) / TK;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (long s = 0; s < slabs; ++s) {
+        const int buf = (int)(s & 1);
+        if (s + 1 < slabs) fetch((s + 1) * TK);
+#pragma unroll
+        for (int ks = 0; ks < TK / MK; ++ks) {
+            const int k = ks * MK + lane / MT;
+            T a[TI], b[TI];
+#pragma unroll
+            for (int i = 0; i < TI; ++i) a[i] = As[buf][k][wrow + i * MT + lane % MT];
+#pragma unroll
+            for (int j = 0; j < TI; ++j) b[j] = Bs[buf][k][wcol + j * MT + lane % MT];
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < TI; ++j) acc[i][j] = P::mac(a[i], b[j], acc[i][j]);
+        }
+        if (s + 1 < slabs) stage(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TI; ++j)
+#pragma unroll
+            for (int v = 0; v < P::NACC; ++v) {
+                const long r = row0 + wrow + i * MT + P::row(v, lane);
+                const long c = col0 + wcol + j * MT + lane % MT;
+                if (r < M && c < N) C[r * ldc + c] = acc[i][j][v];
+            }
+}
+
 unsigned fill_grid(size_t n) {
     size_t b = (n + kBlock - 1) / kBlock;
     const size_t cap = 256u * 16u;
@@ -113,6 +256,18 @@ extern "C" void drhip_k_launch_copy(void* dst, const void* src, size_t nvec, uns
 extern "C" void drhip_k_launch_matmul(int is_double, const void* A, const void* B, void* C, long M,
                                       long N, long K, long lda, long ldb, long ldc,
                                       hipStream_t s) {
+    if (M >= 64 && N >= 64 && K >= 8) {   // enough of a 128x128 tile to be worth the matrix cores
+        dim3 grid((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128));
+        if (is_double)
+            hipLaunchKernelGGL(matmul_mfma_kernel<double>, grid, dim3(kBlock), 0, s,
+                               (const double*)A, (const double*)B, (double*)C, M, N, K, lda, ldb,
+                               ldc);
+        else
+            hipLaunchKernelGGL(matmul_mfma_kernel<float>, grid, dim3(kBlock), 0, s,
+                               (const float*)A, (const float*)B, (float*)C, M, N, K, lda, ldb,
+                               ldc);
+        return;
+    }
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
     if (is_double)
         hipLaunchKernelGGL(matmul_kernel<double>, grid, dim3(kBlock), 0, s, (const double*)A,

@@ -102,7 +102,9 @@ int drhip_copy_kernel(void* dst_dev, const void* src_dev, size_t nbytes,
 
 /* Row-major C[m,n] = A[m,k] * B[k,n] in float (is_double = 0) or double, leading
  * dimensions in elements.  Replaces `_backend.fallback.dot` = cupy.dot -> cuBLAS
- * (delayarray.py:85) for matrix operands; eager, not part of the fused path. */
+ * (delayarray.py:85) for matrix operands; eager, not part of the fused path.
+ * Products with at least 64 rows and columns run on the matrix cores (128x128 tiles
+ * of MFMA accumulators), smaller ones on a 64x64 vector-ALU tile. */
 int drhip_matmul(int is_double, const void* a, const void* b, void* c, int64_t m, int64_t n,
                  int64_t k, int64_t lda, int64_t ldb, int64_t ldc);
 

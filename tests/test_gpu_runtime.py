@@ -211,3 +211,21 @@ def test_pool_survives_finalisers_running_on_other_threads():
     assert not errors
     assert after["bytes_in_use"] == before["bytes_in_use"]
     assert after["n_mallocs"] - before["n_mallocs"] == 6 * 400
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 3e-6), (np.float64, 1e-14)])
+def test_matrix_product_on_the_matrix_cores(dtype, tol):
+    """Full and ragged 128x128 tiles, short and long inner dimensions, both kernels."""
+    import delayrepay_amd as dr
+    rs = np.random.RandomState(8)
+    for m, k, n in [(128, 16, 128), (64, 8, 64), (130, 33, 257), (600, 777, 513), (65, 1000, 300),
+                    (256, 7, 256), (63, 100, 500), (1, 64, 64), (300, 5, 1)]:
+        a, b = rs.standard_normal((m, k)).astype(dtype), rs.standard_normal((k, n)).astype(dtype)
+        got = dr.array(a).dot(dr.array(b)).get()
+        ref = a.astype(np.float64) @ b.astype(np.float64)
+        assert got.shape == ref.shape and got.dtype == dtype
+        assert np.abs(got - ref).max() <= tol * max(1.0, k / 64) * np.abs(ref).max(), (m, k, n)
+    v = rs.standard_normal(777).astype(dtype)
+    a = rs.standard_normal((600, 777)).astype(dtype)
+    assert np.allclose((dr.array(a) @ dr.array(v)).get(), a @ v, rtol=1e-4 if dtype == np.float32 else 1e-12,
+                       atol=1e-4 if dtype == np.float32 else 1e-12)
