@@ -149,3 +149,98 @@ def test_fuzz_reached_every_kernel_shape():
     print("kernel kinds compiled:", kinds)
     for kind in ("flat", "nd", "tile2d", "tile2dv", "tile2dt", "axis", "axis_short", "axis_narrow"):
         assert kinds.get(kind, 0) > 0, kind
+
+
+# ---- random view geometries: offsets, row pitches, steps, transposes, broadcast axes ------------
+
+GEO_DTYPES = [np.float32, np.float64, np.int32, np.int64]
+
+
+def geo_leaf(rs, shape, dtype):
+    """(lazy leaf, host array) with the same random geometry on both sides."""
+    nd = len(shape)
+    kind = rs.randint(7)
+
+    def both(host, view):
+        dev = dr.array(host)
+        return view(dev), view(host)
+
+    if kind == 1:                                   # starts off a 16-byte boundary
+        off = int(rs.randint(1, 4))
+        n = int(np.prod(shape))
+        host = make_host(rs, (n + off,), dtype)
+        return both(host, lambda a: a[off:].reshape(shape))
+    if kind == 2 and nd >= 2:                       # rows with a pitch, shifted start
+        pad = int(rs.randint(1, 6))
+        host = make_host(rs, shape[:-1] + (shape[-1] + pad,), dtype)
+        lo = int(rs.randint(0, pad + 1))
+        return both(host, lambda a: a[..., lo:lo + shape[-1]])
+    if kind == 3:                                   # stretched along one axis
+        k = int(rs.randint(nd))
+        host = make_host(rs, tuple(1 if i == k else d for i, d in enumerate(shape)), dtype)
+        return both(host, lambda a: a)
+    if kind == 4 and nd >= 2:                       # lower rank
+        host = make_host(rs, shape[1:], dtype)
+        return both(host, lambda a: a)
+    if kind == 5 and nd == 2:                       # transposed
+        host = make_host(rs, (shape[1], shape[0]), dtype)
+        return both(host, lambda a: a.T)
+    if kind == 6:                                   # every second element
+        host = make_host(rs, tuple(2 * d for d in shape), dtype)
+        key = tuple(slice(int(rs.randint(2)), None, 2) for _ in shape)
+        return both(host, lambda a: a[key])
+    host = make_host(rs, shape, dtype)
+    return both(host, lambda a: a)
+
+
+def geo_expr(rs, shape, depth):
+    if depth == 0:
+        return geo_leaf(rs, shape, GEO_DTYPES[rs.randint(len(GEO_DTYPES))])
+    op = rs.randint(8)
+    d, h = geo_expr(rs, shape, depth - 1)
+    if op == 0:
+        return d * 2.5, h * 2.5
+    if op == 1:
+        return np.sqrt(np.abs(d) + 1.0), np.sqrt(np.abs(h) + 1.0)
+    if op == 2:
+        return dr.where(d > 0, d, 1), np.where(h > 0, h, 1)
+    if op == 3:
+        return (d + 0).astype(np.float32), (h + 0).astype(np.float32)
+    d2, h2 = geo_expr(rs, shape, depth - 1)
+    if op == 4:
+        return d + d2, h + h2
+    if op == 5:
+        return d * d2, h * h2
+    if op == 6:
+        return np.maximum(d, d2), np.maximum(h, h2)
+    return d - d2, h - h2
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_random_geometry_matches_numpy(seed):
+    rs = np.random.RandomState(9000 + seed)
+    nd = int(rs.randint(1, 4))
+    shape = tuple(int(rs.choice([1, 3, 16, 33, 64, 130, 1030])) for _ in range(nd))
+    if np.prod(shape) > 1 << 21:
+        shape = shape[:2]
+    with np.errstate(all="ignore"):
+        d, h = geo_expr(rs, shape, int(rs.randint(0, 4)))
+        anchor = make_host(rs, shape, np.float32)
+        d, h = d + dr.array(anchor), h + anchor
+        mode = rs.randint(4)
+        if mode == 0 or len(shape) < 2:
+            got, ref = d.get(), h
+        elif mode == 1:
+            got, ref = np.asarray(dr.max(d).get()), np.asarray(np.max(h))
+        elif mode == 2:
+            axis = int(rs.randint(len(shape)))
+            got, ref = dr.min(d, axis=axis).get(), np.min(h, axis=axis)
+        else:                                       # into a view with a pitch
+            pad = tuple(s + 2 for s in shape)
+            host = make_host(rs, pad, np.float64)
+            dst_d, dst_h = dr.array(host), host.copy()
+            key = tuple(slice(1, 1 + s) for s in shape)
+            dst_d[key] = d
+            dst_h[key] = h
+            got, ref = dst_d.get(), dst_h
+    assert got.dtype == np.asarray(ref).dtype and bits_equal(got, np.asarray(ref)), (seed, shape, mode)
