@@ -813,7 +813,7 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
 
 # ---- reduction along some axes ------------------------------------------------
 
-def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
+def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy, row_vec=None):
     """Reduce the (fused) expression over `rdim` merged dimensions, keeping `kdim`.
 
     The reduced extent R may be cut into S slices of RS elements; the kernel then
@@ -827,6 +827,9 @@ def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
                     reduced extent and meet with a shuffle tree.  Coalesced when the
                     fastest-varying dimension is reduced (sum over the last axis).
                     Partials: [output][slice].
+    row_vec         ('row' with one reduced dimension only) per leaf 'v' (unit stride
+                    along the reduced dimension: 16-byte loads at element alignment)
+                    or 'k' (constant along it)
     Parameters: leaf pointers, output pointer, scalars, K, R, S, RS, kept dims,
     reduced dims, then per leaf its kept strides and its reduced strides."""
     ct = CTYPE[acc_dt]
@@ -905,13 +908,40 @@ def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy):
               "        const long long sl = o - g * S;"]
         L += decompose("g", "dk", "k", kdim, "bk", 8)
         L += [f"        {ct} acc = {ident};",
-              "        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;",
-              "#pragma unroll 4",
-              f"        for (long long r = sl * RS + lane; r < r_end; r += {WAVE}) {{"]
-        L += decompose("r", "dr", "r", rdim, "br", 12)
-        L += [f"            {ct} t0; dr_body({', '.join(args + call_tail)});",
-              f"            acc = {_combine(op, 'acc', 't0')};",
-              "        }",
+              "        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;"]
+        if row_vec:
+            widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, row_vec) if k == "v"}
+            V = 16 // widths.pop()
+            for i, (dt, k) in enumerate(zip(prog.leaves, row_vec)):
+                if k == "k":
+                    L.append(f"        const {CTYPE[dt]} c{i} = a{i}[bk{i}];")
+            L += ["        long long r = sl * RS + (long long)lane * " + str(V) + ";",
+                  "#pragma unroll 2",
+                  f"        for (; r + {V} <= r_end; r += {WAVE * V}) {{"]
+            for i, (dt, k) in enumerate(zip(prog.leaves, row_vec)):
+                if k == "v":
+                    vt = VEC16[dt][0] + "u"
+                    L.append(f"            const {vt} X{i} = *(const {vt}*)(a{i} + bk{i} + r);")
+            for e in range(V):
+                vargs = [f"X{i}[{e}]" if k == "v" else f"c{i}" for i, k in enumerate(row_vec)]
+                L.append(f"            {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
+                         f"acc = {_combine(op, 'acc', 't0')}; }}")
+            L.append("        }")
+            # exactly one lane is left with r < r_end: the one whose next vector would
+            # straddle the end; it finishes the row element by element
+            sargs = [f"a{i}[bk{i} + r]" if k == "v" else f"c{i}" for i, k in enumerate(row_vec)]
+            L += ["        for (; r < r_end; ++r) {",
+                  f"            {ct} t0; dr_body({', '.join(sargs + call_tail)});",
+                  f"            acc = {_combine(op, 'acc', 't0')};",
+                  "        }"]
+        else:
+            L += ["#pragma unroll 4",
+                  f"        for (long long r = sl * RS + lane; r < r_end; r += {WAVE}) {{"]
+            L += decompose("r", "dr", "r", rdim, "br", 12)
+            L += [f"            {ct} t0; dr_body({', '.join(args + call_tail)});",
+                  f"            acc = {_combine(op, 'acc', 't0')};",
+                  "        }"]
+        L += [
               "#pragma unroll",
               f"        for (int off = {WAVE // 2}; off > 0; off >>= 1) {{",
               f"            const {ct} other = {shfl};",

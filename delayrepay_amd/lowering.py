@@ -498,10 +498,19 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
     low.fin_count = 0
     low.kind = "axis_" + strategy
     kdim, rdim = len(kmerged), len(rmerged)
-    low.key = ("axis", prog.key(), kdim, rdim, acc, reduce_op, strategy)
+    row_vec = None
+    # short rows gain from 16-byte loads (256 elements: 59% -> 73% of peak), long ones do
+    # not (16384: 73% -> 70%): a wave's 256-byte loads already stream them
+    if (strategy == "row" and rdim == 1 and TUNE["uvec"] and RS <= 512
+            and all(r[0] in (0, 1) for r in rsets)):
+        widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == 1}
+        if len(widths) == 1 and widths <= {4, 8} and all(
+                c in cg.VEC16 for c, r in zip(prog.leaves, rsets) if r[0] == 1):
+            row_vec = tuple("v" if r[0] == 1 else "k" for r in rsets)
+    low.key = ("axis", prog.key(), kdim, rdim, acc, reduce_op, strategy, row_vec)
 
     def emit():
-        return cg.emit_axis_reduce(prog, kdim, rdim, acc, reduce_op, strategy)
+        return cg.emit_axis_reduce(prog, kdim, rdim, acc, reduce_op, strategy, row_vec)
     low.emit = emit
     if strategy == "col":
         low.grid = max(1, min(-(-K // cg.WAVE) * S, 1 << 20))

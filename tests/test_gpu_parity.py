@@ -861,3 +861,23 @@ def test_slices_of_generated_grids_stay_generated():
     a = dr.arange(100000)
     assert _same((a * 3)[5:90000:7].get(), (np.arange(100000) * 3)[5:90000:7])
     assert _same((a * 3)[::-1][:10].get(), (np.arange(100000) * 3)[::-1][:10])
+
+
+def test_row_reductions_with_vector_loads_and_ragged_ends():
+    """A wave per row, 16-byte loads at element alignment; the row length need not be a
+    multiple of the vector, nor the row start aligned."""
+    rs = np.random.RandomState(23)
+    for shape, dt in [((3000, 100), np.float32), ((2000, 257), np.float64), ((1500, 515), np.float32),
+                      ((700, 130), np.int32)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
+        assert low.kind == "axis_row" and low.key[-1] == ("v",)
+        tol = dict(rtol=2e-5, atol=1e-5) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
+        assert np.allclose(dr.sum(a * a, axis=1).get(), (h.astype(np.float64) ** 2).sum(axis=1), **tol)
+        assert np.array_equal(dr.max(a, axis=1).get(), h.max(axis=1))
+        assert np.array_equal(dr.min(a[:, 3:-2], axis=1).get(), h[:, 3:-2].min(axis=1))
+    h = rs.uniform(0, 1, (900, 300)).astype(np.float32)
+    w = rs.uniform(0, 1, (900, 1)).astype(np.float32)
+    got = dr.sum(dr.array(h) * dr.array(w) + 1.0, axis=1).get()
+    assert np.allclose(got, (h.astype(np.float64) * w + 1.0).sum(axis=1), rtol=2e-5)
