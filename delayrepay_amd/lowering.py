@@ -23,7 +23,7 @@ TUNE = {
     "ax_waves": 32768,   # aim for before the reduced extent is cut into slices
     "ax_rows": 4,        # 'row' strategy: outputs per wave (grid-stride), to amortise set-up
     "ax_narrow": 64,     # kept unit-stride extents up to this many columns: stream the matrix
-    "ax_short": 64,      # reduced unit-stride extents up to this length: a lane per output
+    "ax_short": 192,     # reduced unit-stride extents up to this length: a lane per output
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
     "nts": 1,         # allow non-temporal stores }

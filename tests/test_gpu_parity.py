@@ -757,7 +757,7 @@ def test_reductions_over_short_rows():
     try:
         assert np.allclose(dr.sum(a * W + V, axis=1).get(), (h * w + v).sum(axis=1), rtol=1e-5, atol=1e-5)
     finally:
-        hip.set_tune(ax_short=64)
+        hip.set_tune(ax_short=192)
 
 
 def test_reductions_over_the_rows_of_narrow_matrices():
@@ -867,8 +867,8 @@ def test_row_reductions_with_vector_loads_and_ragged_ends():
     """A wave per row, 16-byte loads at element alignment; the row length need not be a
     multiple of the vector, nor the row start aligned."""
     rs = np.random.RandomState(23)
-    for shape, dt in [((3000, 100), np.float32), ((2000, 257), np.float64), ((1500, 515), np.float32),
-                      ((700, 130), np.int32)]:
+    for shape, dt in [((3000, 200), np.float32), ((2000, 257), np.float64), ((1500, 515), np.float32),
+                      ((700, 230), np.int32)]:
         h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
         a = dr.array(h)
         low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
