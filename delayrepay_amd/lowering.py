@@ -427,8 +427,12 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
     for d in rmerged:
         R *= d
     # coalescing decides the strategy: which side holds the unit-stride dimension
-    inner_kept = any(s[-1] == 1 for s in ksets)
-    inner_red = any(s[-1] == 1 for s in rsets)
+    # (judged by the operands that carry the traffic: a column of weights beside a matrix
+    # must not turn a sum over rows into the strategy for sums along rows)
+    big = max([a.size for a in leaves], default=0)
+    heavy = [i for i, a in enumerate(leaves) if a.size == big]
+    inner_kept = any(ksets[i][-1] == 1 for i in heavy)
+    inner_red = any(rsets[i][-1] == 1 for i in heavy)
     strategy = "col" if (inner_kept and not inner_red) else "row"
     if (strategy == "col" and slices in (None, 1) and 2 <= K <= TUNE["ax_narrow"]
             and (R >= 4096 or slices == 1)

@@ -881,3 +881,16 @@ def test_row_reductions_with_vector_loads_and_ragged_ends():
     w = rs.uniform(0, 1, (900, 1)).astype(np.float32)
     got = dr.sum(dr.array(h) * dr.array(w) + 1.0, axis=1).get()
     assert np.allclose(got, (h.astype(np.float64) * w + 1.0).sum(axis=1), rtol=2e-5)
+
+
+def test_reduction_strategy_follows_the_operands_that_carry_the_traffic():
+    """A column of weights beside a matrix (unit stride along the reduced axis) must not
+    switch a sum over rows to the kernel for sums along rows."""
+    rs = np.random.RandomState(24)
+    h, w = rs.uniform(0, 1, (3000, 500)), rs.uniform(0, 1, (3000, 1))
+    a, W = dr.array(h), dr.array(w)
+    assert hip.lower_only(ReduceEx(np.add, a * W, (0,)))[0].kind == "axis_col"
+    assert np.allclose(dr.sum(a * W, axis=0).get(), (h * w).sum(axis=0), rtol=1e-13)
+    r = rs.uniform(0, 1, (1, 500))
+    assert hip.lower_only(ReduceEx(np.add, a * dr.array(r), (1,)))[0].kind == "axis_row"
+    assert np.allclose(dr.sum(a * dr.array(r), axis=1).get(), (h * r).sum(axis=1), rtol=1e-13)
