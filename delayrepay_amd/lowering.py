@@ -39,6 +39,9 @@ TUNE = {
                       # or unaligned rows, 2: always, 0: never)
     "sntl": 0,        # vectorised stencil: non-temporal loads / stores
     "snts": 1,
+    "s3": 1,          # 3-D shifted views of one buffer: LDS window (0: read every view directly)
+    "s3_gpr": 16,     # 3-D window: 16-byte column groups per tile row (tile rows = 256 / s3_gpr)
+    "s3_tz": 4,       # 3-D window: planes per tile
     "uvec": 1,        # 16-byte accesses at element alignment where 16-byte alignment is missing
     "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
@@ -109,6 +112,103 @@ def grid_cap():
             return 256 * TUNE["bpc"]
         _CUS = hiprt.device_info()["compute_units"]
     return _CUS * TUNE["bpc"]
+
+
+def _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_ptrs, scal_fmt,
+                     scal_vals, in_place):
+    """3-D expression with >= 2 operands that are shifted views of one buffer: stage the
+    buffer's window in LDS (`codegen.emit_stencil3d`).  Returns None when the layout does
+    not qualify (the general tiled kernel then reads every view directly)."""
+    groups = {}
+    for i, (a, s) in enumerate(zip(leaves, m_leaf)):
+        if s[2] == 1 and s[0] > 0 and s[1] > 0:
+            groups.setdefault((id(a.buf), s[0], s[1], prog.leaves[i]), []).append(i)
+    best = max(groups.values(), key=len) if groups else []
+    if len(best) < 2 or not out_codes:
+        return None
+    gcode = prog.leaves[best[0]]
+    gsize = cg.ITEMSIZE[gcode]
+    if gsize not in (4, 8) or gcode not in cg.VEC16:
+        return None
+    vw = 16 // gsize
+    pz, py = m_leaf[best[0]][0], m_leaf[best[0]][1]
+    aligned = (all(cg.ITEMSIZE[c] == gsize for c in out_codes)
+               and all(st % vw == 0 for st_ in m_out for st in st_[:-1])
+               and len({(p // gsize) % vw for p in out_ptrs}) == 1
+               and all(p % gsize == 0 for p in out_ptrs)
+               and pz % vw == 0 and py % vw == 0)
+    if not aligned:
+        return None
+    ref_off = min(leaves[i].offset for i in best)
+    shifts = {}
+    for i in best:
+        d = leaves[i].offset - ref_off
+        dz, r = divmod(d, pz)
+        if r > pz // 2:
+            dz, r = dz + 1, r - pz
+        dy, dx = divmod(r, py)
+        if dx > py // 2:
+            dy, dx = dy + 1, dx - py
+        if dz * pz + dy * py + dx != d:
+            return None
+        shifts[i] = (dz, dy, dx)
+    dz_max = max(v[0] for v in shifts.values())
+    dy_min, dy_max = min(v[1] for v in shifts.values()), max(v[1] for v in shifts.values())
+    dx_min, dx_max = min(v[2] for v in shifts.values()), max(v[2] for v in shifts.values())
+    if min(v[0] for v in shifts.values()) < 0 or dz_max > 4 or dy_max - dy_min > 8 \
+            or dx_max - dx_min > 16:
+        return None
+    gpr, tz = TUNE["s3_gpr"], TUNE["s3_tz"]
+    ty = cg.BLOCK // gpr
+    Z, Y, W = mshape
+    g_buf = leaves[best[0]].buf
+    g_ptr = g_buf.ptr + ref_off * gsize
+    ph_o = (out_ptrs[0] // gsize) % vw
+    ph_g = (g_ptr // gsize) % vw
+    kinds = []
+    for i, st in enumerate(m_leaf):
+        if i in shifts:
+            kinds.append(("g",) + shifts[i])
+        elif not any(st):
+            kinds.append(("b",))
+        elif st[-1] == 1:
+            dv = (cg.ITEMSIZE[prog.leaves[i]] == gsize and st[0] % vw == 0 and st[1] % vw == 0
+                  and (leaves[i].ptr // gsize) % vw == ph_o)
+            kinds.append(("dv",) if dv else ("d",))
+        else:
+            kinds.append(("r",))
+    kinds = tuple(kinds)
+    group = (gcode, dz_max, dy_min, dy_max, dx_min, dx_max)
+    lds_bytes = cg.emit_stencil3d(prog, kinds, group, out_codes, gpr, tz, ph_g, ph_o)[4]
+    tiles_x = -(-(W + ph_o) // (gpr * vw))
+    tiles_y, tiles_z = -(-Y // ty), -(-Z // tz)
+    if lds_bytes > 64 * 1024 or tiles_x * tiles_y * tiles_z >= 2 ** 31 or max(Z, Y, W) >= 2 ** 31 - 4096:
+        return None
+    snts = bool(TUNE["snts"])
+    bands = TUNE["xcd"] != 0
+    low.kind = "tile3d"
+    low.key = ("tile3d", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o, gpr, tz,
+               snts, bands)
+
+    def emit():
+        return cg.emit_stencil3d(prog, kinds, group, out_codes, gpr, tz, ph_g, ph_o,
+                                 restrict=not in_place, nt_store=snts, xcd_bands=bands)[0]
+    low.emit = emit
+    low.grid = tiles_x * tiles_y * tiles_z
+    srcs = [(a.buf, a.offset * a.dtype.itemsize) for a, k in zip(leaves, kinds) if k[0] != "g"]
+    srcs.append((g_buf, ref_off * gsize))
+    fmt = "@" + "P" * (len(srcs) + len(out_ptrs)) + scal_fmt + "iii" + "qqqq" + "ii"
+    tail = [Z, Y, W, pz, py, -ref_off, g_buf.nbytes // gsize - ref_off, tiles_x, tiles_y]
+    for k, st in zip(kinds, m_leaf):
+        if k[0] in ("d", "dv", "r"):
+            fmt += "qq"
+            tail += [st[0], st[1]]
+    for st in m_out:
+        fmt += "qq"
+        tail += [st[0], st[1]]
+    low.fmt = fmt
+    low.srcs, low.scal, low.tail = srcs, scal_vals, tail
+    return low
 
 
 def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, reduce_op,
@@ -189,6 +289,11 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     rows = 1
     for d in mshape[:-1]:
         rows *= d
+    if tiled and ndim == 3 and TUNE["lds"] and TUNE["svec"] and TUNE["s3"]:
+        low3 = _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_ptrs,
+                                scal_fmt, scal_vals, in_place)
+        if low3 is not None:
+            return low3
     if tiled and rows < 2 ** 31 and mshape[-1] < 2 ** 31 - 4096:
         H, W = rows, mshape[-1]
         tw, th = TUNE["tw"], TUNE["th"]

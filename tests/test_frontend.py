@@ -241,7 +241,7 @@ def test_broadcast_scalar_leaf_and_mixed_dtypes():
 def test_strided_and_broadcast_operands_use_nd():
     a, b = leaf((64, 1, 32), np.float64), leaf((1, 48, 32), np.float32)
     low, src = hip.lower_only(a * b + 1)         # unit inner stride: tiled, rows = 64 * 48
-    assert low.kind == "tile2d" and "rem_o % od1" in src
+    assert low.kind == "tile2d" and "rem_o / e1" in src
     hip.compile_source(src)
     col = leaf((64, 1))
     low, src = hip.lower_only(leaf((64, 32)) * col)          # column broadcast: one load per row
@@ -387,3 +387,19 @@ def test_views_of_lazy_expressions_are_pushed_to_the_leaves():
     low, src = hip.lower_only((a * 2).T)
     assert low.kind == "tile2dt"
     assert e.T.shape == (1024, 512) and "array" not in e.__dict__
+
+
+def test_three_dimensional_shifted_views_lower_to_the_lds_window():
+    n = 128
+    u = NPArray(hip.placeholder((n, n, n), np.float32))
+    rhs = (u[:-2, 1:-1, 1:-1] + u[2:, 1:-1, 1:-1] + u[1:-1, :-2, 1:-1] + u[1:-1, 2:, 1:-1]
+           + u[1:-1, 1:-1, :-2] + u[1:-1, 1:-1, 2:]) * (1 / 6.0)
+    dst = hip.placeholder((n - 2,) * 3, np.float32, strides=(n * n, n, 1), offset=n * n + n + 1)
+    low, src = hip.lower_only(rhs, dst=dst)
+    assert low.kind == "tile3d" and len(low.srcs) == 1 and "__shared__ f4x4 tile[" in src
+    shifts = sorted(k[1:] for k in low.key[2])
+    assert shifts == [(0, 0, 0), (1, -1, 0), (1, 0, -1), (1, 0, 1), (1, 1, 0), (2, 0, 0)]
+    hip.compile_source(src)
+    odd = NPArray(hip.placeholder((n, n, n - 1), np.float32))      # rows not 16-byte multiples
+    low, src = hip.lower_only(odd[:-2, 1:-1, 1:-1] + odd[2:, 1:-1, 1:-1])
+    assert low.kind == "tile2d"

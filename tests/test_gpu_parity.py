@@ -894,3 +894,55 @@ def test_reduction_strategy_follows_the_operands_that_carry_the_traffic():
     r = rs.uniform(0, 1, (1, 500))
     assert hip.lower_only(ReduceEx(np.add, a * dr.array(r), (1,)))[0].kind == "axis_row"
     assert np.allclose(dr.sum(a * dr.array(r), axis=1).get(), (h * r).sum(axis=1), rtol=1e-13)
+
+
+def _laplace3d(u, f=None, c=1 / 6.0):
+    s = (u[:-2, 1:-1, 1:-1] + u[2:, 1:-1, 1:-1] + u[1:-1, :-2, 1:-1] + u[1:-1, 2:, 1:-1]
+         + u[1:-1, 1:-1, :-2] + u[1:-1, 1:-1, 2:])
+    return c * s if f is None else c * (s + f)
+
+
+@pytest.mark.parametrize("shape,dtype", [((40, 36, 64), np.float32), ((33, 50, 132), np.float32),
+                                         ((20, 24, 40), np.float64), ((9, 9, 260), np.float32)])
+def test_stencils_in_three_dimensions_go_through_the_lds_window(shape, dtype):
+    rs = np.random.RandomState(41)
+    h = rs.uniform(0, 1, shape).astype(dtype)
+    src_term = rs.uniform(0, 1, tuple(s - 2 for s in shape)).astype(dtype)
+    u, ref = dr.array(h), h.copy()
+    c = dtype(1 / 6.0) if dtype == np.float32 else 1 / 6.0
+    kinds_before = {k[0] for k in hip._KERNELS}
+    for _ in range(3):                                        # in place: ping-pong buffers
+        u[1:-1, 1:-1, 1:-1] = _laplace3d(u)
+        ref[1:-1, 1:-1, 1:-1] = _laplace3d(ref, c=c)
+    assert u.get().tobytes() == ref.tobytes()
+    assert "tile3d" in {k[0] for k in hip._KERNELS} | kinds_before
+    # into another array, with a source term read directly and a row-constant operand
+    F = dr.array(src_term)
+    col = rs.uniform(0, 1, (shape[1] - 2, 1)).astype(dtype)
+    v = dr.array(np.zeros(shape, dtype))
+    v[1:-1, 1:-1, 1:-1] = _laplace3d(u, F) + dr.array(col)
+    expect = np.zeros(shape, dtype)
+    expect[1:-1, 1:-1, 1:-1] = _laplace3d(ref, src_term, c=c) + col
+    assert v.get().tobytes() == expect.tobytes()
+    # a fresh result, 27 points, wider reach along x
+    w = (u[:-2, :-2, :-4] + u[1:-1, 1:-1, 2:-2] * 2 + u[2:, 2:, 4:] + u[2:, :-2, 1:-3]).get()
+    r = ref[:-2, :-2, :-4] + ref[1:-1, 1:-1, 2:-2] * 2 + ref[2:, 2:, 4:] + ref[2:, :-2, 1:-3]
+    assert w.tobytes() == r.tobytes()
+
+
+def test_three_dimensional_stencil_layouts_that_do_not_qualify_still_match():
+    rs = np.random.RandomState(42)
+    h = rs.uniform(0, 1, (20, 30, 63)).astype(np.float32)       # row pitch not a multiple of 16 bytes
+    u, ref = dr.array(h), h.copy()
+    u[1:-1, 1:-1, 1:-1] = _laplace3d(u)
+    ref[1:-1, 1:-1, 1:-1] = _laplace3d(ref, c=np.float32(1 / 6.0))
+    assert u.get().tobytes() == ref.tobytes()
+    hip.set_tune(s3=0)
+    try:
+        h = rs.uniform(0, 1, (20, 30, 64)).astype(np.float32)
+        u, ref = dr.array(h), h.copy()
+        u[1:-1, 1:-1, 1:-1] = _laplace3d(u)
+        ref[1:-1, 1:-1, 1:-1] = _laplace3d(ref, c=np.float32(1 / 6.0))
+        assert u.get().tobytes() == ref.tobytes()
+    finally:
+        hip.set_tune(s3=1)
