@@ -237,7 +237,7 @@ def main():
             if kern.finalize:
                 names_by_func[kern.finalize] = nm + "_fin"
         kernel_names = [wl["direct"]] if wl.get("direct") else \
-            sorted({names_by_func.get(f, "?") for f, _, _, _ in plan.launches})
+            sorted({names_by_func.get(f, "?") for f, *_ in plan.launches})
         steps_per_replay = 2 if wl.get("pair") else 1
         reps = max(1, K // steps_per_replay)
         t_warm = time.perf_counter()

@@ -30,6 +30,10 @@ extern "C" void drhip_k_launch_matmul(int is_double, const void* A, const void* 
 extern "C" int drhip_k_cumsum(int kind, void* temp, size_t* temp_bytes, const void* in, void* out,
                               size_t n, hipStream_t s);
 
+extern "C" int drhip_k_scratch_init(int device);
+extern "C" void* drhip_k_scratch_ptr(int device);
+extern "C" size_t drhip_k_scratch_bytes(void);
+
 namespace {
 
 thread_local std::string t_err;
@@ -102,6 +106,9 @@ int drhip_init(int device) {
     HIP_TRY(hipSetDevice(device));
     HIP_TRY(hipGetDeviceProperties(&g_prop, device));
     HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    // address of the static scratch array on this device (drhip_launch_scratch)
+    if (int rc = drhip_k_scratch_init(device))
+        return fail(rc, "hipGetSymbolAddress(scratch)", hipGetErrorString((hipError_t)rc));
     g_arch = g_prop.gcnArchName;
     g_device = device;
     g_init = true;
@@ -402,6 +409,26 @@ int drhip_launch(void* func, unsigned grid_x, unsigned block_x, unsigned lds_byt
                                   g_stream, nullptr, extra));
     g_cnt.n_launches++;
     return 0;
+}
+
+size_t drhip_scratch_bytes(void) { return drhip_k_scratch_bytes(); }
+
+int drhip_launch_scratch(void* func, unsigned grid_x, unsigned block_x, unsigned lds_bytes,
+                         const void* args, size_t args_bytes, size_t scratch_arg_offset,
+                         size_t scratch_bytes) {
+    NEED_INIT();
+    unsigned char block[DRHIP_MAX_ARGS_BYTES];
+    if (!args || args_bytes > sizeof block)
+        return fail(DRHIP_EINVAL, "drhip_launch_scratch", "argument block missing or larger than DRHIP_MAX_ARGS_BYTES");
+    if (scratch_arg_offset % sizeof(void*) || scratch_arg_offset + sizeof(void*) > args_bytes)
+        return fail(DRHIP_EINVAL, "drhip_launch_scratch", "scratch pointer slot outside the argument block or misaligned");
+    if (scratch_bytes > drhip_k_scratch_bytes())
+        return fail(DRHIP_EINVAL, "drhip_launch_scratch", "request exceeds the static scratch array (drhip_scratch_bytes())");
+    void* ptr = drhip_k_scratch_ptr(g_device);
+    if (!ptr) return fail(DRHIP_ENOTINIT, "drhip_launch_scratch", "scratch address was not resolved");
+    memcpy(block, args, args_bytes);
+    memcpy(block + scratch_arg_offset, &ptr, sizeof ptr);
+    return drhip_launch(func, grid_x, block_x, lds_bytes, block, args_bytes);
 }
 
 // ---- graphs ----------------------------------------------------------------

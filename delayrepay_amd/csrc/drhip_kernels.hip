@@ -237,6 +237,39 @@ unsigned fill_grid(size_t n) {
 
 }  // namespace
 
+// ---- static scratch memory ----------------------------------------------------------
+// Device memory for drhip_launch_scratch: partial results of reductions for callers that
+// cannot allocate.  One array per GPU (each device that loads this code object holds its
+// own copy at its own address) until the process ends.  In host code the array's name is
+// only a handle for hipGetSymbolAddress, never a device address: the address is looked up
+// once per device and everything else works with that pointer.
+#define DRHIP_SCRATCH_BYTES (4u << 20)
+static __device__ __align__(256) unsigned char scratch[DRHIP_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+// Look up the address of `scratch` on `device`, which must be the current device.
+extern "C" int drhip_k_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    if (g_scratch_ptr[device]) return 0;
+    void* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
+
+// Device address of the scratch array on `device` (null before drhip_k_scratch_init).
+extern "C" void* drhip_k_scratch_ptr(int device) {
+    return (device >= 0 && device < kMaxDevices) ? g_scratch_ptr[device] : nullptr;
+}
+
+extern "C" size_t drhip_k_scratch_bytes(void) { return DRHIP_SCRATCH_BYTES; }
+
 extern "C" void drhip_k_launch_fill32(void* dst, uint32_t v, size_t n, hipStream_t s) {
     hipLaunchKernelGGL(fill_kernel<uint32_t>, dim3(fill_grid(n)), dim3(kBlock), 0, s,
                        (uint32_t*)dst, v, n);

@@ -326,7 +326,7 @@ class Replay:
     pipeline; it keeps the recorded outputs and scratch buffers alive."""
 
     def __init__(self):
-        self.launches = []      # (function, grid, lds bytes, packed arguments)
+        self.launches = []      # (function, grid, lds bytes, packed arguments, scratch slot, bytes)
         self.keep = []
         self._scratch = []
         self._graph = None
@@ -335,8 +335,14 @@ class Replay:
         if self._graph is not None:
             self._graph.launch()
             return
-        for func, grid, lds, args in self.launches:
-            hiprt.launch(func, grid, cg.BLOCK, lds, args, len(args))
+        self._issue_all()
+
+    def _issue_all(self):
+        for func, grid, lds, args, slot, scratch in self.launches:
+            if slot is None:
+                hiprt.launch(func, grid, cg.BLOCK, lds, args, len(args))
+            else:
+                hiprt.launch_scratch(func, grid, cg.BLOCK, lds, args, len(args), slot, scratch)
 
     def as_graph(self):
         """Capture the recorded launches into a HIP graph; later calls replay the
@@ -344,8 +350,7 @@ class Replay:
         if self._graph is None and self.launches:
             hiprt.Graph.begin()
             try:
-                for func, grid, lds, args in self.launches:
-                    hiprt.launch(func, grid, cg.BLOCK, lds, args, len(args))
+                self._issue_all()
             finally:
                 graph = hiprt.Graph.end()
             self._graph = graph
@@ -435,6 +440,32 @@ class Plan:
         return tuple((buf, buf.version) for buf in seen.values()) + lazy
 
 
+def _issue(func, grid, args, slot=None, scratch=0):
+    """Launch (and record) one kernel.  `slot`: byte offset of the pointer parameter
+    that takes the library's static scratch array, of which the kernel uses
+    `scratch` bytes; None for a kernel without one."""
+    if slot is None:
+        hiprt.launch(func, grid, cg.BLOCK, 0, args, len(args))
+    else:
+        hiprt.launch_scratch(func, grid, cg.BLOCK, 0, args, len(args), slot, scratch)
+    if _RECORDING is not None:
+        _RECORDING.launches.append((func, grid, 0, args, slot, scratch))
+    STATS["launches"] += 1
+
+
+_SCRATCH_BYTES = hiprt.scratch_bytes()
+
+
+def _partials(nbytes):
+    """Where a reduction's partial results go: the library's static scratch array when
+    they fit (nothing is allocated; launches on the one stream are ordered, so the
+    finalising kernel has read them before the next reduction writes), else a pooled
+    block.  Returns (pointer to pack, whether it is the static array)."""
+    if nbytes <= _SCRATCH_BYTES and TUNE["static_scratch"]:
+        return 0, True
+    return hiprt.malloc(nbytes), False
+
+
 def _fire(plan, out_ptrs, reduce_out=None):
     """Compile on first use, pack the argument block, launch."""
     low = plan.low
@@ -442,42 +473,44 @@ def _fire(plan, out_ptrs, reduce_out=None):
     if kern is None:
         kern = plan.kern = _kernel_for(low, reduce_out is not None)
     ptrs = [buf.ptr + off for buf, off in low.srcs]
+    slot = 8 * len(ptrs)         # the partials pointer follows the source pointers
     if plan.second is not None:
-        # two-pass axis reduction: partials into pooled scratch, then reduce those
+        # two-pass axis reduction: partials into scratch memory, then reduce those
         low2 = plan.second
         kern2 = plan.kern2
         if kern2 is None:
             kern2 = plan.kern2 = _kernel_for(low2, False)
-        scratch = hiprt.malloc(plan.scratch)
+        scratch, static = _partials(plan.scratch)
         args = kern.packer.pack(*ptrs, scratch, *low.scal, *low.tail)
-        hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
         args2 = kern2.packer.pack(scratch, *out_ptrs, *low2.tail)
-        hiprt.launch(kern2.func, low2.grid, cg.BLOCK, 0, args2, len(args2))
-        if _RECORDING is not None:
-            _RECORDING.launches += [(kern.func, low.grid, 0, args), (kern2.func, low2.grid, 0, args2)]
-            _RECORDING._scratch.append(scratch)
+        if static:
+            _issue(kern.func, low.grid, args, slot, plan.scratch)
+            _issue(kern2.func, low2.grid, args2, 0, plan.scratch)
         else:
-            hiprt.free(scratch)
-        STATS["launches"] += 2
-        return
-    if reduce_out is not None:
-        partial = hiprt.malloc(low.fin_count * cg.ITEMSIZE[plan.acc])
+            _issue(kern.func, low.grid, args)
+            _issue(kern2.func, low2.grid, args2)
+            if _RECORDING is not None:
+                _RECORDING._scratch.append(scratch)
+            else:
+                hiprt.free(scratch)  # stream-ordered: safe to recycle once queued
+    elif reduce_out is not None:
+        nbytes = low.fin_count * cg.ITEMSIZE[plan.acc]
+        partial, static = _partials(nbytes)
         args = kern.packer.pack(*ptrs, partial, *low.scal, *low.tail)
-        hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
         fin = struct.pack("@PPi", partial, reduce_out, low.fin_count)
-        hiprt.launch(kern.finalize, 1, cg.BLOCK, 0, fin, len(fin))
-        if _RECORDING is not None:
-            _RECORDING.launches += [(kern.func, low.grid, 0, args), (kern.finalize, 1, 0, fin)]
-            _RECORDING._scratch.append(partial)
+        if static:
+            _issue(kern.func, low.grid, args, slot, nbytes)
+            _issue(kern.finalize, 1, fin, 0, nbytes)
         else:
-            hiprt.free(partial)  # stream-ordered: safe to recycle once queued
-        STATS["launches"] += 2
+            _issue(kern.func, low.grid, args)
+            _issue(kern.finalize, 1, fin)
+            if _RECORDING is not None:
+                _RECORDING._scratch.append(partial)
+            else:
+                hiprt.free(partial)
     else:
         args = kern.packer.pack(*ptrs, *out_ptrs, *low.scal, *low.tail)
-        hiprt.launch(kern.func, low.grid, cg.BLOCK, 0, args, len(args))
-        if _RECORDING is not None:
-            _RECORDING.launches.append((kern.func, low.grid, 0, args))
-        STATS["launches"] += 1
+        _issue(kern.func, low.grid, args)
 
 
 # ---------------------------------------------------------------------------

@@ -83,6 +83,9 @@ _SIGNATURES = {
     "drhip_get_function": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]),
     "drhip_compile_log": (C.c_char_p, []),
     "drhip_launch": (C.c_int, [C.c_void_p, C.c_uint, C.c_uint, C.c_uint, C.c_void_p, C.c_size_t]),
+    "drhip_launch_scratch": (C.c_int, [C.c_void_p, C.c_uint, C.c_uint, C.c_uint, C.c_void_p,
+                                       C.c_size_t, C.c_size_t, C.c_size_t]),
+    "drhip_scratch_bytes": (C.c_size_t, []),
     "drhip_graph_begin": (C.c_int, []),
     "drhip_graph_end": (C.c_int, [C.POINTER(C.c_void_p)]),
     "drhip_graph_launch": (C.c_int, [C.c_void_p]),
@@ -249,6 +252,19 @@ def launch(func, grid, block, lds_bytes, argbuf, nbytes):
     rc = _lib.drhip_launch(func, grid, block, lds_bytes, argbuf, nbytes)
     if rc:
         _check(rc)
+
+
+def launch_scratch(func, grid, block, lds_bytes, argbuf, nbytes, slot_offset, scratch_bytes):
+    """`launch` with the library's static scratch array in the pointer slot at
+    `slot_offset` of the argument block; allocates nothing."""
+    rc = _lib.drhip_launch_scratch(func, grid, block, lds_bytes, argbuf, nbytes, slot_offset,
+                                   scratch_bytes)
+    if rc:
+        _check(rc)
+
+
+def scratch_bytes():
+    return lib().drhip_scratch_bytes()
 
 
 def sync():

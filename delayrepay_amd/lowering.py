@@ -17,6 +17,7 @@ TUNE = {
     "unroll": 1,      # 16-byte vectors per thread and chunk in flat element-wise kernels
     "red_unroll": 4,  # the same for flat kernels with a reduction tail
     "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
+    "static_scratch": 1,  # partial results go to the library's static scratch array if they fit
     "flat_cap": 0,    # most blocks of a flat element-wise kernel (0: one chunk per block)
     "bpc": 8,         # resident blocks per CU that bound the grid of `nd` kernels
     "ax_blocks": 4096,   # axis reductions: blocks ('col') / waves ('row') worth of work to

@@ -141,6 +141,27 @@ const char* drhip_compile_log(void);
 int drhip_launch(void* func, unsigned grid_x, unsigned block_x,
                  unsigned lds_bytes, const void* args, size_t args_bytes);
 
+/* drhip_launch for a kernel that needs device scratch memory (the partial results a
+ * reduction kernel hands to its finalising kernel), for callers that cannot allocate:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference (whose reductions are CuPy library calls,
+ * delayarray.py:516-518).  The call allocates nothing: the scratch memory is one static
+ * device array of drhip_scratch_bytes() bytes (4 MiB) that every GPU the library runs on
+ * holds until the process ends.  Its address on the current device is written into the
+ * pointer slot at byte offset `scratch_arg_offset` of the argument block (a multiple of
+ * 8; the slot's previous contents are ignored), then the kernel is launched exactly as
+ * drhip_launch would.  The kernel may use the first `scratch_bytes` bytes; a request
+ * above drhip_scratch_bytes(), or an argument block above DRHIP_MAX_ARGS_BYTES, is
+ * refused with DRHIP_EINVAL.  All calls on a GPU share the array and it keeps the last
+ * call's contents: a kernel must write what it later reads (nothing is cleared), work
+ * queued through this library is ordered by its one stream, and users of the array that
+ * overlap on one GPU by any other route race. */
+#define DRHIP_MAX_ARGS_BYTES 4096
+int drhip_launch_scratch(void* func, unsigned grid_x, unsigned block_x, unsigned lds_bytes,
+                         const void* args, size_t args_bytes, size_t scratch_arg_offset,
+                         size_t scratch_bytes);
+size_t drhip_scratch_bytes(void);
+
 /* ---- HIP graphs -----------------------------------------------------------
  * Capture the launches issued between begin and end into a graph and replay
  * them with one call: for launch-bound loops (small arrays, many sweeps).  The
