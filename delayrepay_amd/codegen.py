@@ -108,6 +108,10 @@ _INFIX = {"add": "+", "subtract": "-", "multiply": "*", "divide": "/", "true_div
 _COMPARE = {"greater": ">", "less": "<", "greater_equal": ">=", "less_equal": "<=",
             "equal": "==", "not_equal": "!="}
 
+# arithmetic ufuncs whose bool loop is a logical operation (None: NumPy raises TypeError)
+_BOOL_ARITH = {"add": "|", "maximum": "|", "fmax": "|", "multiply": "&", "minimum": "&",
+               "fmin": "&", "subtract": None, "negative": None}
+
 # results are bool; arithmetic happens in the operands' common type
 _PREDICATES = {"isnan", "isinf", "isfinite", "logical_not", "logical_and", "logical_or",
                "logical_xor"}
@@ -127,6 +131,14 @@ def op_expr(name, dt, args):
     """C expression computing ufunc `name` in arithmetic type `dt` on `args`
     (C expressions already converted to `dt`)."""
     is_float = dt in ("f4", "f8")
+    if dt == "b1" and name in _BOOL_ARITH:
+        # NumPy's bool arithmetic is logical: True + True is True (a byte value of 2
+        # in a bool array would break later comparisons); subtraction does not exist
+        op = _BOOL_ARITH[name]
+        if op is None:
+            raise TypeError(f"numpy boolean {name} is not supported, as in NumPy "
+                            "(use bitwise or logical operations instead)")
+        return f"(unsigned char)({args[0]} {op} {args[1]})"
     if name in _INFIX:
         if name in ("divide", "true_divide") and not is_float:
             raise NotImplementedError("integer division has no float result type here")

@@ -34,6 +34,7 @@ import numpy as np
 import numpy.lib.mixins
 
 from . import backend as be
+from .promote import PY_DESCR, result_dtype, scalar_descr
 
 _backend = be.backend
 
@@ -262,6 +263,13 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         to the backend as one fused kernel writing straight into the destination
         (the reference evaluates it to a temporary first, delayarray.py:114-121)."""
         arr = self._force()
+        # written to by hand, the result is an array in its own right from now on: it
+        # must not be recomputed (and the write lost) when one of its inputs changes
+        d = self.__dict__
+        if "_deps" in d:
+            d.pop("_deps", None)
+            d.pop("_plan", None)
+            d.pop("_multi", None)
         key = _unwrap(key)
         if isinstance(item, DelayArray) and "array" not in item.__dict__:
             _backend.run_into(item, arr[key])
@@ -375,10 +383,7 @@ def calc_shape(left, right, op=None):
     return tuple(np.broadcast_shapes(left, right))
 
 
-_RESOLVE_CACHE = {}
-
-
-_PY_DESCR = {bool: ("py", "b"), int: ("py", "i"), float: ("py", "f"), complex: ("py", "c")}
+_PY_DESCR = PY_DESCR
 _ARRAY_DESCR = {}
 
 
@@ -393,44 +398,7 @@ def _descr(node):
         return _ARRAY_DESCR.setdefault(dt, ("a", dt.str))
 
 
-def _scalar_descr(val):
-    d = _PY_DESCR.get(type(val))
-    if d is not None:
-        return d
-    if isinstance(val, np.generic):
-        return ("np", val.dtype.str)
-    if isinstance(val, numbers.Integral):
-        return ("py", "i")
-    if isinstance(val, numbers.Real):
-        return ("py", "f")
-    return ("py", "c")
-
-
-_PY_PROBE = {"b": True, "i": 1, "f": 1.0, "c": 1j}
-
-
-def result_dtype(func, descrs):
-    """dtype NumPy gives `func` on operands described by `descrs` (weak Python
-    scalars included); decided by NumPy itself on empty arrays."""
-    key = (func, descrs)
-    try:
-        return _RESOLVE_CACHE[key]
-    except KeyError:
-        pass
-    probes = []
-    for kind, code in descrs:
-        if kind == "a":
-            probes.append(np.empty(0, dtype=code))
-        elif kind == "np":
-            probes.append(np.dtype(code).type(1))
-        else:
-            probes.append(_PY_PROBE[code])
-    if all(kind != "a" for kind, _ in descrs):
-        probes[0] = np.empty(0, dtype=np.asarray(probes[0]).dtype)
-    with np.errstate(all="ignore"):
-        dt = func(*probes).dtype
-    _RESOLVE_CACHE[key] = dt
-    return dt
+_scalar_descr = scalar_descr
 
 
 def calc_type(func, children):
@@ -645,9 +613,21 @@ _ELEMENTWISE = (BinaryNumpyEx, BinaryFuncEx, UnaryFuncEx, WhereEx, CastEx)
 
 def pow_ex(func, left, right):
     """`x ** k` with a Python-int k >= 2 becomes k-1 left-associated multiplies
-    (delayarray.py:316-324); k <= 1 returns x itself, as the reference does."""
+    (delayarray.py:316-324), k == 1 is x itself.  The reference returns x for every
+    k <= 1 as well; here k <= 0 gives what NumPy's `**` gives: `x**0` is ones,
+    `x**-1` is `1/x` (correctly rounded, NumPy's own shortcut), other negative k go to
+    `power`; an integer array to a negative power is an error, as in NumPy."""
     exponent = right.val if isinstance(right, Scalar) else None
     if not isinstance(exponent, int) or isinstance(exponent, bool):
+        return BinaryFuncEx(func, left, right)
+    if exponent < 1:
+        integral = left.dtype.kind in "iu"
+        if exponent < 0 and (integral or left.dtype.kind == "b"):
+            raise ValueError("Integers to negative integer powers are not allowed.")
+        if exponent == 0 and integral:
+            return left * 0 + 1
+        if exponent == -1 and left.dtype.kind == "f":
+            return UnaryFuncEx(np.reciprocal, left)
         return BinaryFuncEx(func, left, right)
     ex = left
     for _ in range(exponent - 1):

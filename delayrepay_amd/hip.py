@@ -22,6 +22,7 @@ import hashlib
 import os
 import struct
 import sys
+import warnings
 
 import numpy
 
@@ -29,6 +30,8 @@ from . import codegen as cg
 from . import hiprt
 from .devarray import Buffer, ndarray, placeholder  # noqa: F401
 from .codegen import Program, dtype_code, code_dtype
+from .promote import result_dtype, scalar_descr
+from .visitor import Visitor
 from .lowering import (TUNE, Lowered, broadcast_strides as _broadcast_strides, lower as _lower,
                        lower_axis_reduce as _lower_axis_reduce)
 
@@ -41,7 +44,8 @@ COMPILE_OPTS = [
 ]
 
 _FUSED = "DELAY_UNFUSED" not in os.environ
-STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0}
+STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0,
+         "disk_write_failures": 0}
 
 _COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal") \
     + tuple(cg._PREDICATES)
@@ -90,14 +94,7 @@ def _scalar_value(value, code):
         return code_dtype(code).type(value).item()
 
 
-_FE = None          # the front-end module, bound on first use (it imports this one)
 _CODES = {}
-
-
-def _bind_frontend():
-    global _FE
-    from . import delayarray
-    _FE = delayarray
 
 
 def _code_of(dtype):
@@ -107,10 +104,29 @@ def _code_of(dtype):
         return _CODES.setdefault(dtype, dtype_code(dtype))
 
 
-class Tracer:
-    """Collects leaves, scalar parameters and SSA operations of one or more roots."""
+def _kind(node):
+    """Node kind = its class name, the way the reference's backends tell nodes apart
+    (delayrepay/visitor.py:18-21): any front end whose node classes carry these names
+    and fields can hand its DAG to this backend."""
+    return node.__class__.__name__
+
+
+class Tracer(Visitor):
+    """Walks the DAG of one or more roots once (memoised by node identity) and
+    collects leaves, typed scalar parameters and SSA operations.
+
+    Dispatch is by class name through `Visitor.visit_<ClassName>`, as in the
+    reference's emitter (delayrepay/cuda.py:46-88): `BinaryNumpyEx`, `UnaryFuncEx`,
+    `BinaryFuncEx`, `NPArray`, `Scalar`, plus this repository's `WhereEx`, `CastEx`,
+    `ReduceEx`, `FullEx`, `IotaEx`.  Only `children`, `func`, `val` and `array` of a node
+    are read; every statement's type is derived here with NumPy's promotion rules
+    (`promote.result_dtype`) from the leaves' dtypes, so a front end that stores no
+    dtype on a scalar, or a sibling's dtype on an interior node
+    (delayrepay/delayarray.py:434-452,462-467), gets NumPy's result all the same.
+    Each handler returns (operand reference, dtype code)."""
 
     def __init__(self, evaluated=None):
+        super().__init__()
         self.leaves = []
         self.leaf_codes = []
         self._leaf_index = {}
@@ -125,6 +141,9 @@ class Tracer:
         self.iotas = []           # index-valued generated leaves
 
     def leaf(self, arr):
+        if not isinstance(arr, ndarray):
+            raise TypeError(f"a leaf of the expression holds a {type(arr).__name__}, not a device "
+                            "array of this backend")
         code = _code_of(arr.dtype)
         key = (id(arr.buf), arr.offset, arr.shape, arr._strides, code)
         idx = self._leaf_index.get(key)
@@ -158,72 +177,101 @@ class Tracer:
         hit = memo.get(nid)
         if hit is not None:
             return hit
-        if _FE is None:
-            _bind_frontend()
-        kind = type(node)
         arr = self._evaluated.get(nid) if self._evaluated else None
         if arr is None:
             arr = node.__dict__.get("array")
-            if arr is not None and kind is not _FE.NPArray:
+            if arr is not None and _kind(node) != "NPArray":
                 deps = node.__dict__.get("_deps")
                 if deps is not None and any(buf.version != ver for buf, ver in deps):
                     arr = None  # stale: recompute inside this kernel
         if arr is not None:
             res = self.leaf(arr)
             self.leaf_nodes.append((node, arr, node.__dict__.get("_deps")))
-        elif kind is _FE.BinaryNumpyEx or kind is _FE.BinaryFuncEx or kind is _FE.UnaryFuncEx:
-            func = node.func
-            name = func.__name__
-            result = _code_of(node.dtype)
-            compute = result
-            if name in _COMPARES:     # arithmetic in the operands' common type, bool out
-                descrs = tuple(_FE._descr(c) for c in node.children)
-                compute = dtype_code(_FE.result_dtype(
-                    numpy.add if len(descrs) == 2 else numpy.positive, descrs))
-                if compute == "b1" and name not in cg._PREDICATES:
-                    compute = "u1"
-            elif name not in cg.SUPPORTED_UFUNCS:
-                raise NotImplementedError(f"ufunc {name!r} cannot be fused by the HIP backend")
-            refs = []
-            for child in node.children:
-                if type(child) is _FE.Scalar:
-                    refs.append(self.scalar(child.val, compute, id(child))[0])
-                else:
-                    refs.append(self.visit(child)[0])
-            self.ops.append((name, compute, result, tuple(refs)))
-            res = (("v", len(self.ops) - 1), result)
-        elif kind is _FE.WhereEx:
-            result = _code_of(node.dtype)
-            refs = []
-            for pos, child in enumerate(node.children):
-                if type(child) is _FE.Scalar:
-                    code = result if pos else dtype_code(numpy.asarray(child.val).dtype)
-                    refs.append(self.scalar(child.val, code, id(child))[0])
-                else:
-                    refs.append(self.visit(child)[0])
-            self.ops.append(("where", result, result, tuple(refs)))
-            res = (("v", len(self.ops) - 1), result)
-        elif kind is _FE.Scalar:
-            res = self.scalar(node.val, dtype_code(numpy.asarray(node.val).dtype), nid)
-        elif kind is _FE.CastEx:
-            ref, code = self.visit(node.children[0])
-            target = dtype_code(node.dtype)
-            res = self.op("cast", target, target, [ref]) if code != target else (ref, code)
-        elif kind is _FE.ReduceEx:
-            res = self.leaf(node._force())
-        elif kind is _FE.FullEx:      # a constant array is a scalar parameter
-            res = self.scalar(node.val, _code_of(node.dtype), nid)
-            self.gen_shapes.append(node.shape)
-            self.leaf_nodes.append((node, None, None))   # the plan holds while it stays unwritten
-        elif kind is _FE.IotaEx:      # the element index, converted
-            code = _code_of(node.dtype)
-            res = self.op("iota", code, code, [])
-            self.gen_shapes.append(node.shape)
-            self.iotas.append((res[0][1], node))
-            self.leaf_nodes.append((node, None, None))
         else:
-            raise NotImplementedError(f"{kind.__name__} nodes cannot be evaluated by the HIP backend")
+            res = Visitor.visit(self, node)
         memo[nid] = res
+        return res
+
+    def default_visit(self, node):
+        raise NotImplementedError(f"{_kind(node)} nodes cannot be evaluated by the HIP backend")
+
+    # -- operands of an interior node ---------------------------------------------
+
+    def _operands(self, children):
+        """[(child, reference-or-None, descriptor)]: array-valued children are traced,
+        numbers are left for the consumer (a weak scalar takes the consumer's type)."""
+        out = []
+        for child in children:
+            if _kind(child) == "Scalar":
+                out.append((child, None, scalar_descr(child.val)))
+            else:
+                ref, code = self.visit(child)
+                out.append((child, ref, ("a", code)))
+        return out
+
+    def _call(self, node):
+        func = node.func
+        name = func.__name__
+        operands = self._operands(node.children)
+        descrs = tuple(d for _, _, d in operands)
+        if name not in cg.SUPPORTED_UFUNCS and name not in _COMPARES:
+            raise NotImplementedError(f"ufunc {name!r} cannot be fused by the HIP backend")
+        result = dtype_code(result_dtype(func, descrs))
+        compute = result
+        if name in _COMPARES:     # arithmetic in the operands' common type, bool out
+            compute = dtype_code(result_dtype(numpy.add if len(descrs) == 2 else numpy.positive,
+                                              descrs))
+            if compute == "b1" and name not in cg._PREDICATES:
+                compute = "u1"
+        refs = [ref if ref is not None else self.scalar(child.val, compute, id(child))[0]
+                for child, ref, _ in operands]
+        self.ops.append((name, compute, result, tuple(refs)))
+        return ("v", len(self.ops) - 1), result
+
+    visit_BinaryNumpyEx = _call
+    visit_BinaryFuncEx = _call
+    visit_UnaryFuncEx = _call
+
+    def visit_NPArray(self, node):
+        res = self.leaf(node.array)
+        self.leaf_nodes.append((node, node.array, None))
+        return res
+
+    def visit_Scalar(self, node):
+        return self.scalar(node.val, dtype_code(numpy.asarray(node.val).dtype), id(node))
+
+    def visit_WhereEx(self, node):
+        operands = self._operands(node.children)
+        result = dtype_code(result_dtype(numpy.add, (operands[1][2], operands[2][2])))
+        refs = []
+        for pos, (child, ref, _) in enumerate(operands):
+            if ref is None:
+                code = result if pos else dtype_code(numpy.asarray(child.val).dtype)
+                ref = self.scalar(child.val, code, id(child))[0]
+            refs.append(ref)
+        return self.op("where", result, result, refs)
+
+    def visit_CastEx(self, node):
+        ref, code = self.visit(node.children[0])
+        target = dtype_code(node.dtype)
+        return self.op("cast", target, target, [ref]) if code != target else (ref, code)
+
+    def visit_ReduceEx(self, node):
+        # a reduction inside a larger expression is evaluated on its own first
+        return self.leaf(node._force())
+
+    def visit_FullEx(self, node):      # a constant array is a scalar parameter
+        res = self.scalar(node.val, _code_of(node.dtype), id(node))
+        self.gen_shapes.append(node.shape)
+        self.leaf_nodes.append((node, None, None))   # the plan holds while it stays unwritten
+        return res
+
+    def visit_IotaEx(self, node):      # the element index, converted
+        code = _code_of(node.dtype)
+        res = self.op("iota", code, code, [])
+        self.gen_shapes.append(node.shape)
+        self.iotas.append((res[0][1], node))
+        self.leaf_nodes.append((node, None, None))
         return res
 
     def materialise_indices(self):
@@ -286,8 +334,15 @@ def _load_or_compile(source):
             with open(tmp, "wb") as fh:
                 fh.write(code)
             os.replace(tmp, path)
-        except OSError:
-            pass
+        except OSError as exc:
+            # not fatal, but every process would then recompile every kernel: say so once
+            STATS["disk_write_failures"] += 1
+            if STATS["disk_write_failures"] == 1:
+                warnings.warn(f"delayrepay_amd: cannot write the kernel cache under "
+                              f"{_cache_dir()!r} ({exc}); kernels will be recompiled by every "
+                              "process.  Set DELAYREPAY_CACHE_DIR to a writable directory or "
+                              "DELAYREPAY_NO_DISK_CACHE=1 to silence this.", RuntimeWarning,
+                              stacklevel=2)
     return module
 
 
@@ -323,19 +378,51 @@ class Replay:
     """Kernel launches recorded by `record()`: calling the object issues them again
     with the same arguments (same inputs, same outputs), without tracing, lowering
     or allocating.  Used to time kernels back to back and to re-run a fixed
-    pipeline; it keeps the recorded outputs and scratch buffers alive."""
+    pipeline; it keeps the recorded outputs and scratch buffers alive.
+
+    The recorded argument blocks hold device addresses.  Every replay bumps the write
+    version of each buffer the recorded launches write, so results cached from those
+    buffers are recomputed afterwards.  An update that reads what it overwrites goes
+    through the buffer's second allocation and swaps the two addresses; a recording
+    must therefore hold an even number of such updates per buffer (checked when the
+    recording ends), and a replay refuses to run if a buffer's current address is not
+    the one it was recorded with."""
 
     def __init__(self):
         self.launches = []      # (function, grid, lds bytes, packed arguments, scratch slot, bytes)
         self.keep = []
+        self.written = []       # (buffer, whether the write swapped its two allocations)
+        self._pinned = []       # (buffer, address it must have when a replay starts)
         self._scratch = []
         self._graph = None
 
+    def _seal(self):
+        swaps = {}
+        for buf, swapped in self.written:
+            if swapped:
+                swaps[id(buf)] = (buf, swaps.get(id(buf), (buf, 0))[1] + 1)
+        for buf, count in swaps.values():
+            if count % 2:
+                raise RuntimeError(
+                    "hip.record(): an odd number of updates that read what they overwrite was "
+                    "recorded for one array; record such sweeps in pairs, so that a replay "
+                    "ends in the allocation it started in")
+            self._pinned.append((buf, buf.ptr))
+
     def __call__(self):
+        for buf, ptr in self._pinned:
+            if buf.ptr != ptr:
+                raise RuntimeError("replay refused: an array written by the recording has been "
+                                   "swapped to its other allocation since it was recorded")
         if self._graph is not None:
             self._graph.launch()
-            return
-        self._issue_all()
+        else:
+            self._issue_all()
+        for buf, swapped in self.written:
+            if swapped:
+                buf.version += 1
+            else:
+                buf.touch()
 
     def _issue_all(self):
         for func, grid, lds, args, slot, scratch in self.launches:
@@ -378,7 +465,9 @@ class record:
 
     def __exit__(self, *exc):
         global _RECORDING
-        _RECORDING = None
+        rec, _RECORDING = _RECORDING, None
+        if exc[0] is None:
+            rec._seal()
         return False
 
 
@@ -433,11 +522,21 @@ class Plan:
         return True
 
     def deps(self):
+        """What the result just computed depends on, as (buffer, version) pairs: the
+        buffers of the leaves and, for a leaf that is itself a cached result, what
+        that result was computed from.  The cached leaf is refreshed in place when its
+        own inputs change, which does not touch its buffer's version, so only the
+        transitive closure tells a later reader that this result is stale too."""
         seen = {}
         for arr in self.leaves:
-            seen[id(arr.buf)] = arr.buf
-        lazy = tuple((node, 0) for node, arr, _ in self.checks if arr is None)   # generated leaves
-        return tuple((buf, buf.version) for buf in seen.values()) + lazy
+            seen[id(arr.buf)] = (arr.buf, arr.buf.version)
+        for node, arr, deps in self.checks:
+            if arr is None:                 # a generated leaf, still lazy
+                seen[id(node)] = (node, 0)
+            elif deps is not None:
+                for dep in deps:
+                    seen.setdefault(id(dep[0]), dep)
+        return tuple(seen.values())
 
 
 def _issue(func, grid, args, slot=None, scratch=0):
@@ -649,29 +748,26 @@ def _launch_fresh(plan):
 
 
 def _trace_root(tracer, node):
-    if _FE is None:
-        _bind_frontend()
-    if type(node) is _FE.ReduceEx and "array" not in node.__dict__:
+    if _kind(node) == "ReduceEx" and "array" not in node.__dict__:
         raise TypeError("a reduction must be the root of its own evaluation")
     return tracer.visit(node)
 
 
 def _run_unfused(ex, evaluated):
     """One kernel per interior node, children first."""
-    from .delayarray import NPArray, Scalar, ReduceEx
     nid = id(ex)
     if nid in evaluated:
         return evaluated[nid]
-    if isinstance(ex, NPArray):
+    if _kind(ex) == "NPArray":
         return ex.array
     for child in ex.children:
-        if not isinstance(child, (Scalar, NPArray)):
+        if _kind(child) not in ("Scalar", "NPArray"):
             _run_unfused(child, evaluated)
     tracer = Tracer(evaluated)
-    if isinstance(ex, ReduceEx):
+    if _kind(ex) == "ReduceEx":
         root = tracer.visit(ex.children[0])
         out = _launch_fresh(_make_plan(tracer, [root], reduce_op=ex.func.__name__,
-                                       axes=ex.axis))[0]
+                                       axes=getattr(ex, "axis", None)))[0]
     else:
         root = tracer.visit(ex)
         out = _launch_fresh(_make_plan(tracer, [root]))[0]
@@ -687,12 +783,11 @@ def run(ex):
     d = ex.__dict__
     plan = d.get("_plan")
     if plan is None or not plan.valid():
-        if _FE is None:
-            _bind_frontend()
         tracer = Tracer()
-        if type(ex) is _FE.ReduceEx:
+        if _kind(ex) == "ReduceEx":
             root = tracer.visit(ex.children[0])
-            plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__, axes=ex.axis)
+            plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__,
+                              axes=getattr(ex, "axis", None))
         else:
             root = _trace_root(tracer, ex)
             plan = _make_plan(tracer, [root])
@@ -823,6 +918,7 @@ def _write(plan, dst):
         buf.version += 1
     if _RECORDING is not None:
         _RECORDING.keep += [dst] + plan.leaves
+        _RECORDING.written.append((buf, plan.hazard))
 
 
 def run_into(ex, dst):
@@ -889,13 +985,13 @@ def run_reduce_product(a, b):
 def lower_only(exs, dst=None):
     """Trace and lower without touching the device: returns (Lowered, source).
     Works with placeholder arrays on a machine that has no GPU."""
-    from .delayarray import ReduceEx
     if not isinstance(exs, (list, tuple)):
         exs = [exs]
     tracer = Tracer()
-    if isinstance(exs[0], ReduceEx):
+    if _kind(exs[0]) == "ReduceEx":
         root = tracer.visit(exs[0].children[0])
-        low = _make_plan(tracer, [root], reduce_op=exs[0].func.__name__, axes=exs[0].axis).low
+        low = _make_plan(tracer, [root], reduce_op=exs[0].func.__name__,
+                         axes=getattr(exs[0], "axis", None)).low
     elif dst is not None:
         low = _plan_write(tracer, tracer.visit(exs[0]), dst).low
     else:

@@ -10,7 +10,8 @@ cpu.py:19-26); leaves are the arrays and Python scalars themselves
 (cpu.py:13-17).  Before that, the front end rewrites three things
 (delayrepay/delayarray.py:316-336): `square(x)` becomes `multiply(x, x)`, and
 `x ** k` for a Python-int k becomes k-1 left-associated multiplies (k <= 1 gives
-x).  Hence the reference's value of an expression is the value of the same Python
+x there; the restatement keeps that for k = 1 only and follows NumPy for k <= 0,
+where returning x is plainly a slip: x**0 would be x).  Hence the reference's value of an expression is the value of the same Python
 expression evaluated eagerly, node by node, on numpy.ndarrays with those rewrites
 applied.  `OracleArray` is exactly that evaluator; the named functions below state
 the five benchmark configurations directly in NumPy.
@@ -64,6 +65,10 @@ class OracleArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         if name == "square":                                   # delayarray.py:330-331
             return OracleArray(np.multiply(args[0], args[0]))
         if name == "power" and isinstance(args[1], int) and not isinstance(args[1], bool):
+            if args[1] < 1:
+                # the reference returns x itself for k <= 1 (delayarray.py:316-324), which
+                # is x**1; for k <= 0 the restatement follows NumPy's `**` instead
+                return OracleArray(np.asarray(args[0]) ** args[1])
             acc = args[0]                                      # delayarray.py:316-324
             for _ in range(args[1] - 1):
                 acc = np.multiply(acc, args[0])

@@ -112,6 +112,34 @@ def test_rewrites_follow_the_reference():
     assert a.astype(np.float32) is a                         # same dtype: same leaf
 
 
+def test_powers_below_one_follow_numpy_not_the_reference():
+    a = leaf((16,))
+    zero = a ** 0                                # the reference would hand back `a`
+    assert zero is not a and isinstance(zero, BinaryFuncEx) and zero.func is np.power
+    inv = a ** -1
+    assert isinstance(inv, UnaryFuncEx) and inv.func is np.reciprocal
+    assert isinstance(a ** -2, BinaryFuncEx)
+    ints = leaf((16,), np.int32)
+    with pytest.raises(ValueError, match="negative integer powers"):
+        ints ** -1
+    ones = ints ** 0
+    assert ones is not ints and ones.dtype == np.int32
+    low, src = hip.lower_only(ones)
+    hip.compile_source(src)
+
+
+def test_bool_arithmetic_is_logical():
+    p, q = leaf((64,), np.bool_), leaf((64,), np.bool_)
+    _, src = hip.lower_only(p + q)
+    assert "l0 | l1" in src.replace("(", " ").replace(")", " ") or "|" in src
+    _, src = hip.lower_only(p * q)
+    assert "&" in src
+    with pytest.raises(TypeError, match="boolean"):
+        hip.lower_only(UnaryFuncEx(np.negative, p))
+    with pytest.raises(TypeError):
+        p - q                                    # NumPy itself refuses to type this
+
+
 def test_dtype_and_shape_inference_is_numpys():
     f32, f64, i64 = leaf((4, 5)), leaf((4, 5), np.float64), leaf((4, 5), np.int64)
     assert (f32 * 0.3).dtype == np.float32                 # weak Python scalar

@@ -10,6 +10,8 @@ import pytest
 import delayrepay as dnp
 from delayrepay import NPArray, array, full, ones, sum  # noqa: A004
 
+from .helpers import bits_equal, ulp_distance
+
 pytestmark = pytest.mark.gpu
 SIZE = 64
 
@@ -183,6 +185,71 @@ class TestSurface:
         assert np.all(b.get() == 11)       # the reference would return the stale 3s
         c = b + 1                          # an evaluated node is reused as a leaf
         assert np.all(c.get() == 12)
+
+    def test_astype_on_a_leaf_returns_a_new_leaf_and_leaves_the_old_one_alone(self):
+        """The reference converts the leaf in place and returns the same wrapper
+        (delayarray.py:401-408), so `a.astype(t)` without rebinding changes `a` under
+        every expression already built on it.  Here the call is NumPy's: a converted
+        copy.  The rebinding form of the reference's tests (tests/test.py:59-62,74-77)
+        behaves the same under both."""
+        a0 = np.arange(64.0) / 3
+        a = array(a0)
+        before = a * 2
+        b = a.astype(np.float32)
+        assert b is not a and b.dtype == np.float32 and a.dtype == np.float64
+        assert isinstance(b, NPArray)
+        assert np.array_equal(b.get(), a0.astype(np.float32))
+        assert np.array_equal(a.get(), a0)                       # untouched
+        assert np.array_equal(before.get(), a0 * 2)              # still float64 arithmetic
+        assert (b ** 2).get().dtype == np.float32
+        assert a.astype(np.float64) is a
+
+    def test_staleness_reaches_results_built_on_cached_results(self):
+        a = array(np.ones(16))
+        b = a * 2 + 1
+        assert np.all(b.get() == 3)
+        c = b + 1                          # evaluated while b is fresh: b is its leaf
+        assert np.all(c.get() == 4)
+        p, q = dnp.evaluate(b * 2, b - 1)
+        assert np.all(p.get() == 6) and np.all(q.get() == 2)
+        a[:] = 5.0
+        assert np.all(c.get() == 12)       # through b, although b's buffer was never written
+        assert np.all(b.get() == 11)
+        assert np.all(p.get() == 22) and np.all(q.get() == 10)
+
+    def test_a_write_into_an_evaluated_expression_survives(self):
+        x0 = np.arange(8.0)
+        x = array(x0.copy())
+        y = x * 2
+        y[0] = 5.0                         # forces y, then writes into its array
+        x[1] = 7.0
+        want = x0 * 2
+        want[0] = 5.0
+        assert np.array_equal(y.get(), want)       # not recomputed from the new x
+        assert np.array_equal((y + 1).get(), want + 1)
+
+    def test_powers_below_one(self):
+        x0 = np.random.RandomState(5).uniform(0.5, 3, 5000).astype(np.float32)
+        x0[:4] = [np.nan, np.inf, 0.0, -0.0]
+        x = array(x0)
+        with np.errstate(all="ignore"):
+            assert bits_equal((x ** 0).get(), x0 ** 0)
+            assert bits_equal((x ** -1).get(), x0 ** -1)
+            got, want = (x ** -2).get(), x0 ** -2
+        assert np.all(ulp_distance(got[4:], want[4:]) <= 2)
+        assert np.isnan(got[0]) and got[1] == 0 and np.isinf(got[2]) and np.isinf(got[3])
+        k = array(np.arange(-5, 5000, dtype=np.int32))
+        assert bits_equal((k ** 0).get(), np.arange(-5, 5000, dtype=np.int32) ** 0)
+
+    def test_bool_arithmetic_is_logical(self):
+        rs = np.random.RandomState(6)
+        p0, q0 = rs.rand(5000) < 0.5, rs.rand(5000) < 0.5
+        p, q = array(p0), array(q0)
+        for got, want in (((p + q).get(), p0 + q0), ((p * q).get(), p0 * q0),
+                          (np.maximum(p, q).get(), np.maximum(p0, q0)),
+                          (np.where(p + q, 1.0, 2.0).get(), np.where(p0 + q0, 1.0, 2.0))):
+            assert got.dtype == want.dtype and got.tobytes() == want.tobytes()
+        assert float(dnp.sum(p + q)) == float(np.sum(p0 + q0))
 
     def test_host_numpy_operands_are_uploaded(self):
         x = np.arange(8.0)

@@ -80,6 +80,21 @@ def test_compile_cache_levels(tmp_path, monkeypatch):
         hiprt.launch(fn, 0, 64, 0, args, len(args))    # bad geometry is refused on the host
 
 
+def test_unwritable_cache_directory_is_reported_once(tmp_path, monkeypatch):
+    blocker = tmp_path / "file_not_dir"
+    blocker.write_text("x")                          # a file where the directory should be
+    monkeypatch.setenv("DELAYREPAY_CACHE_DIR", str(blocker / "cache"))
+    monkeypatch.setitem(hip.STATS, "disk_write_failures", 0)
+    src = 'extern "C" __global__ void dr_kernel(float* o) { o[0] = %d.0f; }\n'
+    with pytest.warns(RuntimeWarning, match="cannot write the kernel cache"):
+        hip._load_or_compile(src % 1)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        hip._load_or_compile(src % 2)                # second failure: counted, not repeated
+    assert hip.STATS["disk_write_failures"] == 2
+
+
 def test_views_follow_numpy_basic_indexing():
     host = np.arange(7 * 9 * 5, dtype=np.float64).reshape(7, 9, 5)
     dev = ndarray.from_host(host)
@@ -164,6 +179,53 @@ def test_recorded_launches_replay_as_a_hip_graph():
             hiprt.memcpy_d2d(total.ptr, total.ptr, 8)
     finally:
         hiprt.Graph.end()
+
+
+def test_replays_invalidate_cached_results_and_keep_ping_pong_parity():
+    import delayrepay_amd as dr
+    from oracle import numpy_oracle as orc
+    rs = np.random.RandomState(22)
+    u0 = np.zeros((66, 130), np.float32)
+    u0[1:-1, 1:-1] = rs.uniform(0, 1, (64, 128))
+    u = dr.array(u0)
+
+    def sweep():
+        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+
+    sweep()
+    with pytest.raises(RuntimeError, match="pairs"):
+        with hip.record():
+            sweep()                          # one aliasing update: would end in the other allocation
+    done = 2
+    with hip.record() as plan:
+        sweep()
+        sweep()
+    done += 2
+    doubled = u * 2.0
+    assert np.array_equal(doubled.get(), orc.jacobi(u0, done) * np.float32(2))
+    plan()
+    done += 2
+    # the replay wrote u: the result cached on `doubled` is stale and is recomputed
+    assert np.array_equal(doubled.get(), orc.jacobi(u0, done) * np.float32(2))
+    sweep()                                  # an eager update leaves u in its other allocation
+    done += 1
+    with pytest.raises(RuntimeError, match="swapped"):
+        plan()
+    sweep()
+    done += 1
+    plan()
+    done += 2
+    assert np.array_equal(u.get(), orc.jacobi(u0, done))
+    # a plain (non-aliasing) recorded write bumps the version as well
+    v = dr.array(np.zeros(1000))
+    w = dr.array(np.arange(1000.0))
+    with hip.record() as fill:
+        v[:] = w + 1.0
+    total = v.sum()
+    assert float(total) == float(np.sum(np.arange(1000.0) + 1))
+    w[:] = 5.0
+    fill()
+    assert np.all(v.get() == 6.0) and float(v.sum()) == 6000.0
 
 
 def test_recent_roots_are_bounded_by_the_memory_their_results_hold(monkeypatch):
