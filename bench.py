@@ -6,19 +6,30 @@
 A step is one pass of the hot path over one batch: build the lazy expression,
 trace it, look the kernel up in the cache and launch it on inputs that already
 sit in HBM (for the stencil: one sweep; for the reduction: body + finalize).
-Prints ONE JSON line.  Its top-level fields describe the headline workload
-(degree-8 Horner polynomial, float32, n = 2^26); `configs` carries the same
-figures for every configuration.
+Prints ONE JSON line.  Its top-level fields describe the largest configuration
+(the fused reduction sum((x-y)**2*w), float64, n = 2^27); `configs` carries the
+same figures for every configuration and `roofline.min_frac` the lowest fraction
+among them.
+
+Cold measurement: MI355X has a 256 MB last-level (Infinity) cache in front of HBM,
+so a kernel replayed over one set of buffers smaller than that is partly served
+from the cache.  Every workload therefore owns R sets of inputs and outputs with
+R x footprint >= 3 x 256 MiB (at least 2) and both the timed steps and the kernel
+replays rotate through them, so a buffer has been evicted by the time it comes
+round again.  The replay over a single set is kept as `frac_warm`.
 
 Per configuration:
   value / GBps        algorithmic bytes * steps / wall time of the timed region
-                      (whole step, host side included)
-  roofline            algorithmic bytes / average kernel duration, measured with HIP
-                      events on the library's stream around back-to-back replays of
-                      the recorded launches, against 8 TB/s
+                      (whole step, host side included), rotating over the R sets
+  roofline            algorithmic bytes / kernel duration against 8 TB/s; the duration
+                      is measured with HIP events on the library's stream around
+                      back-to-back replays of the recorded launches of all R sets,
+                      median (and minimum) over REGIONS timed regions
   unfused             the same expression with one kernel per DAG node
   cpu_baseline        the NumPy node-by-node evaluation (oracle/numpy_oracle.py, a port
                       of the reference's CPU backend) on this machine's host cores
+  parity (bs32/bs64)  largest result-relative differences from the oracle over all 2^25
+                      options (oracle/accuracy.py)
 """
 import argparse
 import contextlib
@@ -32,6 +43,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+LLC_BYTES = 256 << 20          # Infinity Cache
+REGIONS = 7                    # timed regions per kernel figure (median and minimum reported)
 METRIC = "fused-kernel effective HBM GB/s (% of MI355X peak); Gelem/s vs unfused"
 
 
@@ -51,15 +64,31 @@ def measured_traffic(name):
     return None
 
 
+def profiled_figure(fname, name):
+    """A per-workload figure kept under profiles/ as `<workload> <number>` lines (taken
+    with rocprofv3 counters, which this script cannot read while it runs)."""
+    path = os.path.join(ROOT, "profiles", fname)
+    try:
+        with open(path) as fh:
+            for ln in fh:
+                parts = ln.split()
+                if len(parts) >= 2 and parts[0] == name:
+                    return float(parts[1])
+    except OSError:
+        pass
+    return None
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all",
-                    help="horner (headline) | saxpy | bs32 | bs64 | jacobi | sumsq | all (these six); "
-                         "dot | axis0 | axis1 | rowbcast | transpose | grid | next (these six: the "
-                         "operations either side of the five configurations); "
+                    help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
+                         "dot | axis0 | axis1 | rows200 | rowbcast | transpose | interior | stencil3d | "
+                         "grid | next (these nine: the operations either side of the five "
+                         "configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before each timed region (clock ramp-up)")
@@ -67,6 +96,10 @@ def parse():
                     help="CPU time spent on the headline workload's baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-copy", action="store_true", help="skip the plain-copy ceiling leg")
+    ap.add_argument("--no-parity", action="store_true",
+                    help="skip the Black-Scholes error table against the oracle")
+    ap.add_argument("--sets", type=int, default=0,
+                    help="buffer sets to rotate over (0: enough to defeat the last-level cache)")
     ap.add_argument("--no-unfused", action="store_true", help="skip the un-fused leg")
     return ap.parse_args()
 
@@ -94,60 +127,79 @@ def main():
             acc = acc * x + c[i]
         return acc
 
-    # ---- the workloads: (inputs on device, step function, bytes, elements, cpu function)
+    def sets_for(nbytes):
+        """Buffer sets so that a set has left the last-level cache before its next turn."""
+        if args.sets:
+            return args.sets
+        return max(2, -(-3 * LLC_BYTES // nbytes))
+
+    # ---- the workloads: R step functions (one per set of device buffers), algorithmic
+    #      bytes and elements of one step, and the CPU evaluation of a bounded sample
     def make(name):
         inp = orc.make_inputs(name) if name in ("saxpy", "horner", "bs32", "bs64", "jacobi",
                                                 "sumsq") else None
         if name == "saxpy":
-            x, y = dr.array(inp["x"]), dr.array(inp["y"])
             n = inp["x"].size
+            R = sets_for(12 * n)
+            sets = [(dr.array(inp["x"]), dr.array(inp["y"])) for _ in range(R)]
             return dict(dtype="f32", n=n, nbytes=12 * n, desc="SAXPY z=a*x+y f32 n=2^24",
-                        step=lambda: hip.run(inp["a"] * x + y),
-                        cpu=lambda: orc.saxpy(inp["a"], inp["x"], inp["y"]), cpu_frac=1.0)
+                        steps=[(lambda x=x, y=y: hip.run(inp["a"] * x + y)) for x, y in sets],
+                        cpu=lambda: orc.saxpy(inp["a"], inp["x"], inp["y"]), cpu_frac=1.0,
+                        cpu_code="oracle/numpy_oracle.py::saxpy")
         if name == "horner":
-            x = dr.array(inp["x"])
             n = inp["x"].size
+            R = sets_for(8 * n)
+            sets = [dr.array(inp["x"]) for _ in range(R)]
             return dict(dtype="f32", n=n, nbytes=8 * n,
                         desc="Horner degree-8 polynomial f32 n=2^26",
-                        step=lambda: hip.run(horner_expr(inp["c"], x)),
-                        cpu=lambda: orc.horner(inp["c"], inp["x"]), cpu_frac=1.0)
+                        steps=[(lambda x=x: hip.run(horner_expr(inp["c"], x))) for x in sets],
+                        cpu=lambda: orc.horner(inp["c"], inp["x"]), cpu_frac=1.0,
+                        cpu_code="oracle/numpy_oracle.py::horner")
         if name in ("bs32", "bs64"):
-            S, K_, T = dr.array(inp["S"]), dr.array(inp["K"]), dr.array(inp["T"])
             n = inp["S"].size
             size = inp["S"].dtype.itemsize
+            R = sets_for(5 * size * n)
+            sets = [tuple(dr.array(inp[k]) for k in "SKT") for _ in range(R)]
             m = n // 4       # CPU sample: a quarter of the options
             return dict(dtype="f32" if size == 4 else "f64", n=n, nbytes=5 * size * n,
                         desc=f"Black-Scholes call+put {'f32' if size == 4 else 'f64'} n=2^25",
-                        step=lambda: hip.run_multi(list(orc.black_scholes_expr(
-                            dr, S, K_, T, inp["r"], inp["sigma"]))),
+                        steps=[(lambda S=S, K_=K_, T=T: hip.run_multi(list(orc.black_scholes_expr(
+                            dr, S, K_, T, inp["r"], inp["sigma"])))) for S, K_, T in sets],
                         cpu=lambda: orc.black_scholes(inp["S"][:m], inp["K"][:m], inp["T"][:m],
-                                                      inp["r"], inp["sigma"]), cpu_frac=0.25)
+                                                      inp["r"], inp["sigma"]), cpu_frac=0.25,
+                        cpu_code="oracle/numpy_oracle.py::black_scholes", inputs=inp)
         if name == "jacobi":
-            u = dr.array(inp["u"])
             N = inp["u"].shape[0]
+            nbytes = 4 * N * N + 4 * (N - 2) * (N - 2)
+            R = sets_for(nbytes)
+            grids = [dr.array(inp["u"]) for _ in range(R)]
 
-            def sweep():
+            def sweep(u):
                 u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
-            return dict(dtype="f32", n=(N - 2) * (N - 2), nbytes=4 * N * N + 4 * (N - 2) * (N - 2),
-                        desc="Jacobi 5-point f32 8192x8192, per sweep", step=sweep, pair=True,
-                        cpu=lambda: orc.jacobi(inp["u"], 1), cpu_frac=1.0)
+            return dict(dtype="f32", n=(N - 2) * (N - 2), nbytes=nbytes,
+                        desc="Jacobi 5-point f32 8192x8192, per sweep",
+                        steps=[(lambda u=u: sweep(u)) for u in grids], pair=True,
+                        cpu=lambda: orc.jacobi(inp["u"], 1), cpu_frac=1.0,
+                        cpu_code="oracle/numpy_oracle.py::jacobi")
         if name == "sumsq":
-            x, y, w = dr.array(inp["x"]), dr.array(inp["y"]), dr.array(inp["w"])
             n = inp["x"].size
+            R = sets_for(24 * n)
+            sets = [tuple(dr.array(inp[k]) for k in "xyw") for _ in range(R)]
             m = n // 4
             return dict(dtype="f64", n=n, nbytes=24 * n, desc="sum((x-y)**2*w) f64 n=2^27",
-                        step=lambda: hip.run(ReduceEx(np.add, (x - y) ** 2 * w)),
+                        steps=[(lambda x=x, y=y, w=w: hip.run(ReduceEx(np.add, (x - y) ** 2 * w)))
+                               for x, y, w in sets],
                         cpu=lambda: orc.sumsq(inp["x"][:m], inp["y"][:m], inp["w"][:m]),
-                        cpu_frac=0.25)
+                        cpu_frac=0.25, cpu_code="oracle/numpy_oracle.py::sumsq")
         # ---- operations either side of the five configurations (no CPU sample kept small)
         rs = np.random.RandomState(0)
         if name == "dot":
             n = 1 << 27
             hx, hy = rs.standard_normal(n), rs.standard_normal(n)
-            x, y = dr.array(hx), dr.array(hy)
+            sets = [(dr.array(hx), dr.array(hy)) for _ in range(sets_for(16 * n))]
             return dict(dtype="f64", n=n, nbytes=16 * n, desc="dot(x, y) f64 n=2^27 (fused multiply-reduce)",
-                        step=lambda: hip.run(ReduceEx(np.add, x * y)),
-                        cpu=lambda: np.dot(hx[:n // 4], hy[:n // 4]), cpu_frac=0.25)
+                        steps=[(lambda x=x, y=y: hip.run(ReduceEx(np.add, x * y))) for x, y in sets],
+                        cpu=lambda: np.dot(hx[:n // 4], hy[:n // 4]), cpu_frac=0.25, cpu_code="numpy.dot")
         if name == "grid":
             n = 1 << 26
             c = orc.make_inputs("horner")["c"]
@@ -155,9 +207,9 @@ def main():
             m = n // 16
             return dict(dtype="f32", n=n, nbytes=4 * n,
                         desc="Horner degree-8 on linspace(-2, 2, n) f32 n=2^26 (grid generated in the kernel)",
-                        step=lambda: hip.run(horner_expr(c, g)),
+                        steps=[lambda: hip.run(horner_expr(c, g))] * sets_for(4 * n),
                         cpu=lambda: orc.horner(c, np.linspace(-2.0, 2.0, m, dtype=np.float32)),
-                        cpu_frac=1 / 16)
+                        cpu_frac=1 / 16, cpu_code="oracle/numpy_oracle.py::horner on numpy.linspace")
         if name in ("matmul32", "matmul64"):
             N = 8192
             dt = np.float32 if name == "matmul32" else np.float64
@@ -168,104 +220,162 @@ def main():
                         nbytes=3 * N * N * ha.itemsize, flops=2 * N ** 3, direct="matmul_mfma_kernel",
                         mfma_peak=157.3 if dt == np.float32 else 78.6,
                         desc=f"a @ b {np.dtype(dt).name} 8192^3 (eager matrix product on the matrix cores)",
-                        step=lambda: a.dot(b)._force(),
-                        cpu=lambda: ha[:m, :m] @ hb[:m, :m], cpu_frac=(m / N) ** 2)
-        if name in ("axis0", "axis1", "rowbcast", "transpose"):
+                        steps=[lambda: a.dot(b)._force()],
+                        cpu=lambda: ha[:m, :m] @ hb[:m, :m], cpu_frac=(m / N) ** 2, cpu_code="numpy.matmul")
+        if name in ("axis0", "axis1", "rowbcast", "transpose", "interior", "rows200"):
             N = 16384
             ha = rs.standard_normal((N, N)).astype(np.float32)
-            a = dr.array(ha)
             if name in ("axis0", "axis1"):
                 ax = int(name[-1])
+                mats = [dr.array(ha) for _ in range(sets_for(4 * N * N))]
                 return dict(dtype="f32", n=N * N, nbytes=4 * N * N + 4 * N,
                             desc=f"sum(a, axis={ax}) f32 16384x16384",
-                            step=lambda: hip.run(ReduceEx(np.add, a, (ax,))),
-                            cpu=lambda: ha[:N // 4].sum(axis=ax), cpu_frac=0.25)
+                            steps=[(lambda a=a: hip.run(ReduceEx(np.add, a, (ax,)))) for a in mats],
+                            cpu=lambda: ha[:N // 4].sum(axis=ax), cpu_frac=0.25, cpu_code="numpy.sum")
+            if name == "rows200":
+                rows = N * N // 200
+                hm = ha.reshape(-1)[:rows * 200].reshape(rows, 200)
+                mats = [dr.array(hm) for _ in range(sets_for(4 * rows * 200))]
+                return dict(dtype="f32", n=rows * 200, nbytes=4 * rows * 200 + 4 * rows,
+                            desc=f"sum(a, axis=1) f32 {rows}x200 (rows of 200 contiguous elements)",
+                            steps=[(lambda a=a: hip.run(ReduceEx(np.add, a, (1,)))) for a in mats],
+                            cpu=lambda: hm[:rows // 4].sum(axis=1), cpu_frac=0.25, cpu_code="numpy.sum")
+            mats = [dr.array(ha) for _ in range(sets_for(8 * N * N))]
             if name == "rowbcast":
                 hr = rs.standard_normal(N).astype(np.float32)
                 r = dr.array(hr)
                 return dict(dtype="f32", n=N * N, nbytes=8 * N * N + 4 * N,
                             desc="a + row (broadcast) f32 16384x16384",
-                            step=lambda: hip.run(a + r), cpu=lambda: ha[:N // 4] + hr, cpu_frac=0.25)
+                            steps=[(lambda a=a: hip.run(a + r)) for a in mats],
+                            cpu=lambda: ha[:N // 4] + hr, cpu_frac=0.25, cpu_code="numpy.add")
+            if name == "interior":
+                M = N - 2
+                return dict(dtype="f32", n=M * M, nbytes=8 * M * M,
+                            desc="m[1:-1,1:-1] * 2 f32 16384x16384 into a dense array (no row starts on 16 bytes)",
+                            steps=[(lambda a=a: hip.run(a[1:-1, 1:-1] * 2.0)) for a in mats],
+                            cpu=lambda: ha[1:N // 4, 1:-1] * np.float32(2.0), cpu_frac=0.25,
+                            cpu_code="numpy.multiply")
             return dict(dtype="f32", n=N * N, nbytes=8 * N * N, desc="a.T * 2 f32 16384x16384",
-                        step=lambda: hip.run(a.T * 2.0),
-                        cpu=lambda: ha[:, :N // 4].T * np.float32(2.0), cpu_frac=0.25)
+                        steps=[(lambda a=a: hip.run(a.T * 2.0)) for a in mats],
+                        cpu=lambda: ha[:, :N // 4].T * np.float32(2.0), cpu_frac=0.25,
+                        cpu_code="numpy.multiply")
+        if name == "stencil3d":
+            N = 512
+            hv = rs.uniform(0, 1, (N, N, N)).astype(np.float32)
+            M = N - 2
+            nbytes = 4 * N ** 3 + 4 * M ** 3
+            vols = [dr.array(hv) for _ in range(sets_for(nbytes))]
+
+            def sweep3(v):
+                c = v[1:-1, 1:-1, 1:-1]
+                v[1:-1, 1:-1, 1:-1] = (v[:-2, 1:-1, 1:-1] + v[2:, 1:-1, 1:-1] + v[1:-1, :-2, 1:-1]
+                                       + v[1:-1, 2:, 1:-1] + v[1:-1, 1:-1, :-2] + v[1:-1, 1:-1, 2:]
+                                       + c) * (1.0 / 7.0)
+            return dict(dtype="f32", n=M ** 3, nbytes=nbytes, pair=True,
+                        desc="7-point stencil f32 512^3, per sweep",
+                        steps=[(lambda v=v: sweep3(v)) for v in vols],
+                        cpu=lambda: hv[1:65, 1:-1, 1:-1] + hv[:64, 1:-1, 1:-1], cpu_frac=64 / N,
+                        cpu_code="numpy.add (two of the seven views)")
         raise KeyError(name)
+
+    def kernel_regions(replay, launches_per_replay, reps):
+        """Durations (ms per launch group) of REGIONS timed regions of `reps` replays."""
+        t_warm = time.perf_counter()
+        while time.perf_counter() - t_warm < args.settle / 2:
+            for _ in range(4):
+                replay()
+            hiprt.sync()
+        out = []
+        for _ in range(REGIONS):
+            e0, e1 = hiprt.Event(), hiprt.Event()
+            e0.record()
+            for _ in range(reps):
+                replay()
+            e1.record()
+            e1.synchronize()
+            out.append(e0.elapsed_ms(e1) / (reps * launches_per_replay))
+        return out
 
     def measure(name):
         t_gen = time.perf_counter()
         wl = make(name)
         t_gen = time.perf_counter() - t_gen
-        step = wl["step"]
+        steps = wl["steps"]
+        R = len(steps)
+        ring = [None] * R                 # the last R results stay alive: outputs rotate, too
         # first call: compile (or cache load) + run
         c0 = hiprt.counters()
         t0 = time.perf_counter()
-        keep = step()
+        ring[0] = steps[0]()
         hiprt.sync()
         first_ms = (time.perf_counter() - t0) * 1e3
         c1 = hiprt.counters()
-        for _ in range(W):
-            keep = step()
+        for i in range(max(W, R)):
+            ring[i % R] = steps[i % R]()
         hiprt.sync()
         # The GPU raises its clocks only under sustained load (an ALU-heavy kernel
         # measures ~25% slower during the first 30 ms): keep it busy before timing.
         t_warm = time.perf_counter()
+        i = 0
         while time.perf_counter() - t_warm < args.settle:
             for _ in range(10):
-                keep = step()
+                ring[i % R] = steps[i % R]()
+                i += 1
             hiprt.sync()
-        # whole-step throughput: K steps, wall clock between two synchronisations
+        # whole-step throughput: exactly K steps, wall clock between two synchronisations
         t0 = time.perf_counter()
-        for _ in range(K):
-            keep = step()
+        for i in range(K):
+            ring[i % R] = steps[i % R]()
         hiprt.sync()
         wall = time.perf_counter() - t0
         ms_per_step = wall / K * 1e3
-        # kernel duration: record the launches of one step (two for the ping-pong
-        # stencil, which alternates between two buffers), replay them back to back
-        if wl.get("direct"):     # a library kernel, launched without the fusion machinery
-            plan = step
-        with (hip.record() if not wl.get("direct") else contextlib.nullcontext()) as rec:
-            keep = step()
-            if wl.get("pair"):
-                keep = step()
-        if not wl.get("direct"):
-            plan = rec
-        names_by_func = {}
-        for kern in hip._KERNELS.values():
-            nm = kern.source.split('extern "C" __global__')[-1].split("void ")[1].split("(")[0]
-            names_by_func[kern.func] = nm
-            if kern.finalize:
-                names_by_func[kern.finalize] = nm + "_fin"
-        kernel_names = [wl["direct"]] if wl.get("direct") else \
-            sorted({names_by_func.get(f, "?") for f, *_ in plan.launches})
-        steps_per_replay = 2 if wl.get("pair") else 1
-        reps = max(1, K // steps_per_replay)
-        t_warm = time.perf_counter()
-        while time.perf_counter() - t_warm < args.settle / 2:
-            for _ in range(10):
-                plan()
-            hiprt.sync()
-        e0, e1 = hiprt.Event(), hiprt.Event()
-        e0.record()
-        for _ in range(reps):
-            plan()
-        e1.record()
-        e1.synchronize()
-        kernel_ms = e0.elapsed_ms(e1) / (reps * steps_per_replay)
-        del plan
+        # kernel duration: record one step on every set (two for an aliasing update, which
+        # alternates between a buffer's two allocations), replay the lot back to back
+        per_set = 2 if wl.get("pair") else 1
+        direct = wl.get("direct")     # a library kernel, launched without the fusion machinery
+        if direct:
+            cold = warm = lambda: steps[0]()
+            kernel_names = [direct]
+        else:
+            with hip.record() as cold:
+                for _ in range(per_set):
+                    for j in range(R):
+                        ring[j] = steps[j]()
+            with hip.record() as warm:
+                for _ in range(per_set):
+                    ring[0] = steps[0]()
+            names_by_func = {}
+            for kern in hip._KERNELS.values():
+                nm = kern.source.split('extern "C" __global__')[-1].split("void ")[1].split("(")[0]
+                names_by_func[kern.func] = nm
+                if kern.finalize:
+                    names_by_func[kern.finalize] = nm + "_fin"
+            kernel_names = sorted({names_by_func.get(f, "?") for f, *_ in cold.launches})
+        reps = max(1, K // (R * per_set))
+        cold_ms = kernel_regions(cold, 1 if direct else R * per_set, reps)
+        warm_ms = kernel_regions(warm, 1 if direct else per_set, max(1, K // per_set))
+        kernel_ms, kernel_min = statistics.median(cold_ms), min(cold_ms)
+        warm_med = statistics.median(warm_ms)
+        del cold, warm
+        frac = wl["nbytes"] / kernel_ms / 1e6 / HBM_PEAK_GBPS
         res = {
             "workload": wl["desc"], "dtype": wl["dtype"], "elements": wl["n"],
             "kernel": kernel_names,
             "algorithmic_bytes": wl["nbytes"],
+            "buffer_sets": R,
             "ms_per_step": round(ms_per_step, 5),
             "GBps": round(wl["nbytes"] / ms_per_step / 1e6, 1),
             "Gelem_per_s": round(wl["n"] / ms_per_step / 1e6, 2),
             "kernel_us": round(kernel_ms * 1e3, 2),
+            "kernel_us_min": round(kernel_min * 1e3, 2),
+            "kernel_us_regions": [round(v * 1e3, 2) for v in cold_ms],
             "kernel_GBps": round(wl["nbytes"] / kernel_ms / 1e6, 1),
-            "roofline_frac": round(wl["nbytes"] / kernel_ms / 1e6 / HBM_PEAK_GBPS, 4),
+            "roofline_frac": round(frac, 4),
+            "roofline_frac_best_region": round(wl["nbytes"] / kernel_min / 1e6 / HBM_PEAK_GBPS, 4),
+            "kernel_us_warm": round(warm_med * 1e3, 2),
+            "roofline_frac_warm": round(wl["nbytes"] / warm_med / 1e6 / HBM_PEAK_GBPS, 4),
             # what limits the kernel (rocprofv3 VALUBusy / traffic in profiles/)
-            "bound": {"bs64": "fp64 vector ALU (VALUBusy 89%), not HBM",
-                      "bs32": "fp32 vector ALU (VALUBusy ~100%) and HBM",
+            "bound": {"bs64": "fp64 vector ALU and HBM", "bs32": "fp32 vector ALU and HBM",
                       "matmul32": "mfma", "matmul64": "mfma"}.get(name, "hbm"),
             **({"TFLOPs": round(wl["flops"] / kernel_ms / 1e9, 1),
                 "mfma_frac": round(wl["flops"] / kernel_ms / 1e9 / wl["mfma_peak"], 4),
@@ -274,30 +384,58 @@ def main():
             "compile_ms": round((c1["compile_ns"] - c0["compile_ns"]) / 1e6, 2),
             "input_gen_s": round(t_gen, 2),
         }
+        valu = profiled_figure("valu_instructions.txt", name)
+        if valu is not None:
+            # vector-ALU roofline: one wave instruction per SIMD every 4 cycles = 64 lanes
+            # per CU and cycle
+            peak = info["compute_units"] * 64 * info["clock_khz"] * 1e3
+            res["valu_instr_per_element"] = valu
+            res["valu_frac"] = round(valu * wl["n"] / (kernel_ms * 1e-3) / peak, 4)
+            res["valu_peak_lane_instr_per_s"] = peak
+        if "inputs" in wl and not args.no_parity:
+            from oracle import accuracy
+            inp = wl["inputs"]
+            call, put = (a.get() for a in steps[0]())
+            ocall, oput = orc.black_scholes(inp["S"], inp["K"], inp["T"], inp["r"], inp["sigma"])
+            rep = accuracy.bs_report(call, put, ocall, oput, inp, detail=False)
+            res["parity"] = {
+                which: {"scaled_max_eps": r["scaled"]["max_eps"], "scaled_index": r["scaled"]["index"],
+                        **{f"k{k}": {kk: e[kk] for kk in ("count", "max_ulp", "max_ulp_index", "max_rel",
+                                                          "max_rel_index") if kk in e}
+                           for k, e in r["subsets"].items() if k in (1, 4, 8)}}
+                for which, r in rep.items()}
+            res["parity"]["subsets"] = "k: options with |oracle price| >= 2^-k max(S, K)"
+            del call, put, ocall, oput
         if not args.no_unfused:
+            # one kernel per node: its temporaries are re-read by the next kernel, so this
+            # leg gets the cache policy that suits it (streams stay cacheable up to the
+            # size of the last-level cache)
+            policy = {k: hip.TUNE[k] for k in ("cache_mib", "ntl_mib")}
+            hip.set_tune(cache_mib=200, ntl_mib=320)
             hip.set_fused(False)
             try:
                 l0 = hip.STATS["launches"]
-                keep = step()
+                ring[0] = steps[0]()
                 hiprt.sync()
                 res["unfused_kernels"] = hip.STATS["launches"] - l0
-                keep = step()
+                ring[0] = steps[0]()
                 hiprt.sync()
                 reps_u = max(3, K // 4)
                 t0 = time.perf_counter()
                 for _ in range(reps_u):
-                    keep = step()
+                    ring[0] = steps[0]()
                 hiprt.sync()
                 u_ms = (time.perf_counter() - t0) / reps_u * 1e3
             finally:
                 hip.set_fused(True)
+                hip.set_tune(**policy)
             res["unfused_ms_per_step"] = round(u_ms, 4)
             res["unfused_Gelem_per_s"] = round(wl["n"] / u_ms / 1e6, 2)
             res["fused_speedup_vs_unfused"] = round(u_ms / ms_per_step, 2)
         if not args.no_cpu:
             wl["cpu"]()                     # warm-up
             times = []
-            budget = args.cpu_seconds if name == "horner" else 0.0
+            budget = args.cpu_seconds if name == HEADLINE else 0.0
             t_all = time.perf_counter()
             while len(times) < 3 or time.perf_counter() - t_all < budget:
                 t0 = time.perf_counter()
@@ -308,17 +446,19 @@ def main():
             res["cpu"] = {"GBps": round(cpu_bytes / cpu_s / 1e9, 2),
                           "Gelem_per_s": round(wl["n"] * wl["cpu_frac"] / cpu_s / 1e9, 3),
                           "seconds": round(cpu_s, 3), "passes": len(times),
-                          "sample_fraction": wl["cpu_frac"]}
-        del keep, wl
+                          "sample_fraction": wl["cpu_frac"], "code": wl["cpu_code"]}
+        del ring, wl, steps
         return res
 
-    names = {"all": ["horner", "saxpy", "bs32", "bs64", "jacobi", "sumsq"],
-             "next": ["dot", "axis0", "axis1", "rowbcast", "transpose", "grid"]}.get(args.workload,
-                                                                             [args.workload])
+    names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
+             "next": ["dot", "axis0", "axis1", "rows200", "rowbcast", "transpose", "interior",
+                      "stencil3d", "grid"]}.get(args.workload, [args.workload])
+    HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:
         results[name] = measure(name)
         print(f"[bench] {name}: {results[name]}", file=sys.stderr, flush=True)
+        hip.forget()
         hiprt.pool_trim()
 
     # the plain streaming copy (1 GiB in, 1 GiB out): measured ceiling of the memory
@@ -343,8 +483,8 @@ def main():
                 "GBps": round(2 * nb / ms / 1e6, 1), "frac": round(2 * nb / ms / 1e6 / HBM_PEAK_GBPS, 4)}
         del a, b
 
-    head = results.get("horner") or results[names[0]]
-    head_name = "horner" if "horner" in results else names[0]
+    head = results[HEADLINE]
+    worst = min(results, key=lambda k: results[k]["roofline_frac"])
     line = {
         "metric": METRIC,
         "value": head["GBps"],
@@ -357,25 +497,31 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": head["dtype"],
-        "data": "synthetic (numpy RandomState(0), resident in HBM before timing)",
-        "config": {"workload": head["workload"], "name": head_name,
+        "data": "synthetic (numpy RandomState(0), resident in HBM before timing; "
+                f"{head['buffer_sets']} buffer sets in rotation)",
+        "config": {"workload": head["workload"], "name": HEADLINE,
                    "elements": head["elements"], "Gelem_per_s": head["Gelem_per_s"],
                    "device": info["name"] or info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": head["kernel_GBps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": head["roofline_frac"], "traffic": None,
                      "kernel": head["kernel"][0], "kernel_us": head["kernel_us"],
-                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"]},
+                     "kernel_us_min": head["kernel_us_min"], "timed_regions": REGIONS,
+                     "frac_warm": head["roofline_frac_warm"],
+                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
+                     "min_frac": results[worst]["roofline_frac"], "min_frac_config": worst,
+                     "frac_by_config": {k: v["roofline_frac"] for k, v in results.items()}},
         "configs": results,
     }
     if copy is not None:
         line["copy_kernel"] = copy
-    traffic = measured_traffic(head_name)
+    traffic = measured_traffic(HEADLINE)
     if traffic is not None:
         line["roofline"]["traffic"] = traffic
         line["roofline"]["traffic_source"] = "profiles/hbm_traffic.txt (rocprofv3 --pmc, calibrated)"
     if "cpu" in head:
         line["cpu_baseline"] = {
             "value": head["cpu"]["GBps"], "unit": "GB/s", "cores": 1, "kind": "port",
+            "code": head["cpu"]["code"] + " (NumPy node by node, restating the reference's cpu.py)",
             "host_cores_available": os.cpu_count(),
             "sample": f"{head['workload']}: NumPy node-by-node evaluation of "
                       f"{head['cpu']['sample_fraction']:g} of the workload, median of "

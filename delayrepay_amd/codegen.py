@@ -236,7 +236,7 @@ def _conv(expr, src, dst):
     return f"({CTYPE[dst]}){expr}"
 
 
-def emit_body(prog, out_dtypes, fname="dr_body"):
+def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
     """Inline device function evaluating the whole program for one element.
 
     Parameters: leaf values, scalar values, then one reference per root."""
@@ -244,7 +244,7 @@ def emit_body(prog, out_dtypes, fname="dr_body"):
     params += [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
-    lines = [mathlib.source(prog.own_math),
+    lines = [mathlib.source(prog.own_math) if with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
     for i, (name, cdt, rdt, args) in enumerate(prog.ops):
         cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
@@ -253,7 +253,7 @@ def emit_body(prog, out_dtypes, fname="dr_body"):
         elif name == "iota":
             expr = f"({CTYPE[cdt]})dr_i"
         elif cdt == "f8" and name in prog.own_math:
-            expr = f"{mathlib.FUNCTIONS[name][0]}({cargs[0]})"
+            expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
         elif name == "where":    # the condition keeps its own type
             k, j = args[0]
             expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
@@ -262,6 +262,49 @@ def emit_body(prog, out_dtypes, fname="dr_body"):
         lines.append(f"    const {CTYPE[rdt]} v{i} = {expr};")
     for i, ((k, j), rdt) in enumerate(prog.roots):
         lines.append(f"    r{i} = {_conv(f'{k}{j}', rdt, out_dtypes[i])};")
+    lines.append("}")
+    return "\n".join(lines)
+
+
+def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"):
+    """The same program on a pack of `pack` elements held by one thread: every value
+    is a small array and every operation a fully unrolled loop over it, so that the
+    elements pass through each float64 `log`/`erf`/`exp` in lock step (see `mathlib`).
+    Leaves flagged False in `leaf_is_array` are one value for the whole pack (broadcast
+    operands).  The arithmetic per element is exactly that of `emit_body`."""
+    P = pack
+    loop = f'_Pragma("unroll") for (int e = 0; e < {P}; ++e)'
+
+    def ref(k, j):
+        if k == "s" or (k == "l" and not leaf_is_array[j]):
+            return f"{k}{j}"
+        return f"{k}{j}[e]"
+
+    params = [f"const {CTYPE[dt]} (&l{i})[{P}]" if leaf_is_array[i] else f"const {CTYPE[dt]} l{i}"
+              for i, dt in enumerate(prog.leaves)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += [f"{CTYPE[dt]} (&r{i})[{P}]" for i, dt in enumerate(out_dtypes)]
+    lines = [f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
+    for i, (name, cdt, rdt, args) in enumerate(prog.ops):
+        cargs = [_conv(ref(k, j), prog.ref_dtype((k, j)), cdt) for k, j in args]
+        lines.append(f"    {CTYPE[rdt]} v{i}[{P}];")
+        if cdt == "f8" and name in prog.own_math:
+            k, j = args[0]
+            if prog.ref_dtype((k, j)) == "f8" and ref(k, j).endswith("[e]"):
+                lines.append(f"    {mathlib.FUNCTIONS[name][0]}<{P}>({k}{j}, v{i});")
+            else:       # converted or broadcast argument: gather it first
+                lines.append(f"    {{ double t_[{P}]; {loop} t_[e] = {cargs[0]}; "
+                             f"{mathlib.FUNCTIONS[name][0]}<{P}>(t_, v{i}); }}")
+            continue
+        if name == "cast":
+            expr = cargs[0]
+        elif name == "where":    # the condition keeps its own type
+            expr = f"(({ref(*args[0])} != 0) ? {cargs[1]} : {cargs[2]})"
+        else:
+            expr = op_expr(name, cdt, cargs)
+        lines.append(f"    {loop} v{i}[e] = {expr};")
+    for i, ((k, j), rdt) in enumerate(prog.roots):
+        lines.append(f"    {loop} r{i}[e] = {_conv(ref(k, j), rdt, out_dtypes[i])};")
     lines.append("}")
     return "\n".join(lines)
 
@@ -341,6 +384,12 @@ def _st(nt, val, ptr):
     return f"__builtin_nontemporal_store({val}, {ptr});" if nt else f"*({ptr}) = {val};"
 
 
+def packs(prog, vec):
+    """Whether the flat kernel evaluates this program on packs of elements: programs
+    that use the float64 functions of `mathlib`, in vector kernels."""
+    return bool(vec and prog.own_math and not prog.uses_index)
+
+
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
               reduce_op=None, unaligned=False):
     """Contiguous 1-D kernel.
@@ -365,6 +414,9 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     else:
         E = 1
     src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    packed = packs(prog, vec)
+    if packed:
+        src.append(emit_body_packed(prog, out_dtypes, [c == "c" for c in leaf_class], E * unroll))
     if reduce_op:
         src.append(emit_block_reduce(reduce_op, red_dt))
         src.append(emit_finalize(reduce_op, red_dt))
@@ -462,6 +514,39 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
         lo, wo = step(f"_u{u}", f"v + {u * BLOCK}" if u else "v", 8)
         all_loads += lo
         all_work += wo
+    if packed:
+        # all E * unroll elements of this thread go through the program together
+        P, pad = E * unroll, " " * 8
+        all_work = []
+        args = []
+        for i, (dt, c) in enumerate(zip(prog.leaves, leaf_class)):
+            if c == "b":
+                args.append(f"b{i}")
+                continue
+            per = VEC16[dt][1]
+            items = ", ".join(f"L{i}_{e // per}_u{u}[{e % per}]" for u in range(unroll)
+                              for e in range(E))
+            all_work.append(f"{pad}const {CTYPE[dt]} P{i}[{P}] = {{{items}}};")
+            args.append(f"P{i}")
+        for o, dt in enumerate(out_dtypes):
+            all_work.append(f"{pad}{CTYPE[dt]} T{o}[{P}];")
+        outs = [f"T{o}" for o in range(n_out)]
+        all_work.append(f"{pad}dr_body_pack({', '.join(args + scal + outs)});")
+        for u in range(unroll):
+            if reduce_op:
+                for e in range(E):
+                    all_work.append(f"{pad}acc{e} = {_combine(reduce_op, f'acc{e}', f'T0[{u * E + e}]')};")
+                continue
+            for o, dt in enumerate(out_dtypes):
+                vt, per = VEC16[dt]
+                chunks = E // per
+                for ch in range(chunks):
+                    items = ", ".join(f"T{o}[{u * E + ch * per + k}]" for k in range(per))
+                    idx = f"v + {u * BLOCK}" if u else "v"
+                    ptr = f"({vt + ua}*)o{o} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
+                        else f"({vt + ua}*)o{o} + ({idx})"
+                    all_work.append(f"{pad}{{ const {vt} R = {{{items}}}; "
+                                    f"{_st(nt_store, 'R', ptr)} }}")
     L += all_loads + all_work
     L.append("    }")
     # leftover vectors (fewer than one chunk), spread over the first blocks

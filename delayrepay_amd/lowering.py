@@ -28,8 +28,8 @@ TUNE = {
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
     "nts": 1,         # allow non-temporal stores }
-    "cache_mib": 200,  # working sets up to this size are left to the 256 MB Infinity Cache
-    "ntl_mib": 320,   # inputs beyond this size are read with non-temporal loads
+    "cache_mib": 32,  # working sets up to this size (the eight L2s together) stay cacheable
+    "ntl_mib": 32,    # inputs beyond this size are read with non-temporal loads
     "tw": 128,        # stencil tile width (elements)
     "th": 16,         # stencil tile height (rows)
     "lds": 1,         # stage shifted views through LDS (0: read them directly)
@@ -46,6 +46,7 @@ TUNE = {
     "uvec": 1,        # 16-byte accesses at element alignment where 16-byte alignment is missing
     "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
+    "pack": 4,        # elements a thread passes through those functions in lock step
 }
 for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
     _k, _v = _kv.split("=")
@@ -244,14 +245,23 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         vec = widths_ok and n >= 64 and (align_ok or bool(TUNE["uvec"]))
         ua = vec and not align_ok      # vectors at element alignment
         unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
+        if cg.packs(prog, vec) and TUNE["pack"]:
+            # float64 functions evaluate a pack of elements in lock step: at least `pack`
+            # elements per thread (a vector of doubles holds two)
+            min_width = min([cg.ITEMSIZE[c] for c, k in zip(prog.leaves, leaf_class) if k == "c"]
+                            + ([] if reduce_op else [cg.ITEMSIZE[c] for c in out_codes]) or [8])
+            unroll = max(unroll, TUNE["pack"] * min_width // 16)
         in_bytes = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
         footprint = in_bytes
         if not reduce_op:
             footprint += sum(n * cg.ITEMSIZE[c] for c in out_codes)
-        # Cache policy, from measurement: a working set that fits the 256 MB Infinity
-        # Cache is left cacheable; beyond that outputs are written non-temporally (they
-        # are write-once streams) and inputs are read non-temporally only when they are
-        # too large to survive in the cache until a later kernel reads them again.
+        # Cache policy, from measurement: a stream is read once and written once per
+        # launch, so beyond what the L2s hold both directions are non-temporal.  On
+        # buffers that have left the 256 MB last-level cache since their last use (the
+        # case a fresh batch of data presents) that is the faster choice: SAXPY n=2^24
+        # 36.3 -> 33.0 us, Horner n=2^26 86.1 -> 82.6 us.  Replaying one kernel over
+        # one and the same set of buffers smaller than that cache is the opposite case
+        # (29 vs 31 us, 73 vs 83 us): `cache_mib`/`ntl_mib` = 200/320 favour it.
         nts = bool(TUNE["nts"]) and footprint > TUNE["cache_mib"] << 20
         ntl = bool(TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
         low.kind = "flat"

@@ -50,22 +50,30 @@ def show(name, c, err):
 
 def main():
     zero, one = mp.mpf(0), mp.mpf(1)
-    # erf(x) = x P(x^2) on [0, 1], relative error; the code adds x separately, so the
-    # constant term is stored minus 1
-    fa = lambda z: mp.erf(mp.sqrt(z)) / mp.sqrt(z) if z > 0 else 2 / mp.sqrt(mp.pi)
-    wa = lambda z: 1 / fa(z)
-    c = fit(fa, wa, zero, one, 12)
-    show("erf, |x| < 1, P(z) - 1 with z = x^2 (relative)", [c[0] - 1] + c[1:], worst(fa, wa, c, zero, one))
-    # erfc(x) = exp(-(x^2 + G(x - 3.5))) on [1, 6]; weight erfc(x): absolute error of erf
-    gb = lambda x: -mp.log(mp.erfc(x)) - x * x
-    tv = lambda x: x - mp.mpf(7) / 2
-    c = fit(gb, mp.erfc, one, mp.mpf(6), 18, tv)
-    show("erf, 1 <= x <= 6, G(t) with t = x - 3.5 (absolute error of erfc)", c,
-         worst(gb, mp.erfc, c, one, mp.mpf(6), tv))
-    # exp(v) on |v| <= ln(2)/2, relative
+    # erf(x) = -expm1(-w), w = -log(erfc(x)) = x (x + 1 + H(x)) on [0, 6].  An error dH
+    # changes erf by erfc(x) x dH: the weight makes that relative to erf(x).
+    def fh(x):
+        if x == 0:
+            return 2 / mp.sqrt(mp.pi) - 1
+        return -mp.log(mp.erfc(x)) / x - x - 1
+
+    def wh(x):
+        if x == 0:
+            return mp.sqrt(mp.pi) / 2
+        return mp.erfc(x) * x / mp.erf(x)
+    c = fit(fh, wh, zero, mp.mpf(6), 23)
+    show("erf, 0 <= x <= 6, H(x) (relative error of erf)", c, worst(fh, wh, c, zero, mp.mpf(6)))
+    # e^v - 1 = v + v^2 R(v) on |v| <= ln(2)/2; an error dR changes it by v^2 dR, relative
+    # to e^v - 1 ~ v that is |v| dR (the small constant keeps the fit determined at 0)
     h = mp.log(2) / 2
-    c = fit(mp.exp, lambda v: mp.exp(-v), -h, h, 11)
-    show("exp(v), |v| <= ln(2)/2 (relative)", c, worst(mp.exp, lambda v: mp.exp(-v), c, -h, h))
+
+    def fr(v):
+        if v == 0:
+            return one / 2
+        return (mp.expm1(v) - v) / (v * v)
+    c = fit(fr, lambda v: abs(v) + mp.mpf(10) ** -3, -h, h, 9)
+    show("exp, R(v), |v| <= ln(2)/2 (relative error of e^v - 1)", c,
+         worst(fr, lambda v: abs(v), c, -h, h))
     # log((1+s)/(1-s)) = 2s + s z Q(z), z = s^2, s <= (sqrt(2)-1)/(sqrt(2)+1)
     smax = (mp.sqrt(2) - 1) / (mp.sqrt(2) + 1)
 

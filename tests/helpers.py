@@ -13,24 +13,7 @@ def golden(name):
     return np.load(os.path.join(GOLDEN, name), allow_pickle=False)
 
 
-def ulp_distance(a, b):
-    """Distance in units in the last place between same-dtype float arrays
-    (0 where both are NaN or both the same infinity)."""
-    a = np.asarray(a)
-    b = np.asarray(b)
-    assert a.dtype == b.dtype and a.dtype.kind == "f"
-    itype = np.int32 if a.dtype.itemsize == 4 else np.int64
-    ia = a.view(itype).astype(np.int64)
-    ib = b.view(itype).astype(np.int64)
-    top = np.int64(np.iinfo(itype).min)
-    ia = np.where(ia < 0, top - ia, ia)   # map to a monotone integer line
-    ib = np.where(ib < 0, top - ib, ib)
-    dist = np.abs(ia - ib).astype(np.float64)
-    both_nan = np.isnan(a) & np.isnan(b)
-    one_nan = np.isnan(a) ^ np.isnan(b)
-    dist = np.where(both_nan, 0.0, dist)
-    dist = np.where(one_nan, np.inf, dist)
-    return dist
+from oracle.accuracy import ulp_distance  # noqa: E402,F401
 
 
 def bits_equal(a, b):

@@ -3,7 +3,14 @@
 Bars (written out where they are applied):
   + - * / and sqrt expressions          bit-exact
   transcendental functions               <= 2 ulp in float32; <= 1e-13 relative in float64
-  Black-Scholes call/put                 |gpu - oracle| <= 4 eps(float32) resp. 1e-13 (float64)
+  Black-Scholes call/put                 result-relative: <= 1e-13 (float64) wherever the price
+                                         is >= 2^-8 max(S, K); float32: within 8 ulp of the
+                                         oracle where the price is >= max(S, K)/2 and no
+                                         farther from the true price than NumPy is (the
+                                         stated 2 ulp is beyond NumPy's own float32 error,
+                                         see `bs_bars`).  Everywhere, including options whose
+                                         terms cancel:
+                                         |gpu - oracle| <= 4 eps(float32) resp. 1e-13 (float64)
                                          times max(S, K).  The price is a difference of
                                          terms of that size, so ulps of the (possibly tiny)
                                          result would only measure cancellation, in NumPy as
@@ -135,12 +142,63 @@ def bs_check(cfg, n):
 @pytest.mark.parametrize("cfg", ["bs64", "bs32"])
 @pytest.mark.parametrize("n", [1, 1000, 65537])
 def test_black_scholes_within_tolerance(cfg, n):
-    bs_check(cfg, n)
+    call, put, inp = bs_check(cfg, n)
+    if n > 1:
+        bs_bars(cfg, call, put, inp)
+
+
+def bs_bars(cfg, call, put, inp):
+    """The result-relative bars, on the options where a result-relative figure means
+    something, and the table that shows where they stop meaning something.
+
+    float64: <= 1e-13 relative (the stated bar, literally) on every option whose price is
+    at least 2^-8 of max(S, K): 62 % of the calls and 95 % of the puts at n = 2^25,
+    measured maximum 4.9e-14.  Below that the two terms of the price cancel and the
+    figure grows in the CPU evaluation exactly as on the device (at 2^-16: 7e-12, with
+    the oracle itself 57 000 ulp from the 50-digit value); those are held by the bar
+    scaled with max(S, K) in `bs_check`.
+    float32: the stated 2 ulp cannot be met by any implementation, a correctly rounded
+    one included: on the best-conditioned options (price >= max(S, K) / 2) NumPy's own
+    float32 result is up to 4.6 (call) and 6.3 (put) ulp from the true price, so a perfect
+    device result would still be 4-6 ulp from the oracle.  What is asserted instead: the
+    device is within 8 / 16 / 40 ulp of the oracle on the subsets 2^-1 / 2^-2 / 2^-4
+    (measured 8 / 16 / 40: each is the sum of the two sides' own errors), and it is at
+    least as close to the true price (the float64 evaluation of the same inputs) as
+    NumPy's float32 result is, plus one ulp."""
+    from oracle import accuracy
+    ocall, oput = orc.black_scholes(inp["S"], inp["K"], inp["T"], inp["r"], inp["sigma"])
+    rep = accuracy.bs_report(call, put, ocall, oput, inp, detail=call.size >= 1 << 20)
+    print("\n" + accuracy.format_report(cfg, rep), flush=True)
+    for which in ("call", "put"):
+        sub = rep[which]["subsets"]
+        if cfg == "bs64":
+            for k in (1, 2, 4, 8):
+                if sub[k]["count"]:
+                    assert sub[k]["max_rel"] <= 1e-13, (which, k, sub[k])
+        else:
+            for k, bound in ((1, 8), (2, 16), (4, 40)):
+                if sub[k]["count"]:
+                    assert sub[k]["max_ulp"] <= bound, (which, k, sub[k])
+    if cfg == "bs32":
+        truth = orc.black_scholes(*(inp[k].astype(np.float64) for k in "SKT"), inp["r"], inp["sigma"])
+        scale = np.maximum(inp["S"], inp["K"]).astype(np.float64)
+        for which, got, ref, t in (("call", call, ocall, truth[0]), ("put", put, oput, truth[1])):
+            ulp = np.spacing(np.abs(t).astype(np.float32)).astype(np.float64)
+            for k in (1, 2, 4):
+                m = np.abs(t) >= scale * 2.0 ** -k
+                if m.any():
+                    e_dev = float(np.max(np.abs(got - t)[m] / ulp[m]))
+                    e_np = float(np.max(np.abs(ref - t)[m] / ulp[m]))
+                    print(f"  {which}, price >= 2^-{k} max(S,K): device {e_dev:.2f} ulp, NumPy float32 "
+                          f"{e_np:.2f} ulp from the float64 value", flush=True)
+                    assert e_dev <= e_np + 1.0, (which, k, e_dev, e_np)
+    return rep
 
 
 @pytest.mark.parametrize("cfg", ["bs64", "bs32"])
 def test_black_scholes_full_size_and_put_call_parity(cfg):
     call, put, inp = bs_check(cfg, 1 << 25)
+    bs_bars(cfg, call, put, inp)
     parity = inp["S"].astype(np.float64) - inp["K"] * np.exp(-inp["r"] * inp["T"].astype(np.float64))
     scale = np.maximum(inp["S"], inp["K"])
     tol = 8 * np.finfo(inp["S"].dtype).eps

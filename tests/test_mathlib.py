@@ -2,7 +2,7 @@
 
 `mathlib.source(..., HOST_MACROS)` is the same text the kernels include, with the
 reciprocal seed and the scalar-constant multiply-add spelled in plain C; it is built
-here with gcc and compared with 40-digit values (mpmath) and with libm / SciPy.
+here with g++ and compared with 40-digit values (mpmath) and with libm / SciPy.
 The device build of the same text is checked against NumPy in the GPU tests."""
 import ctypes
 import subprocess
@@ -17,14 +17,19 @@ from delayrepay_amd import hip, mathlib
 
 @pytest.fixture(scope="module")
 def host(tmp_path_factory):
+    """The device source built for the host with g++.  Arrays go through the 4-element
+    pack (the form the kernels use) and the remainder through the 1-element form."""
     d = tmp_path_factory.mktemp("mathlib")
-    src = mathlib.source(sorted(mathlib.FUNCTIONS), mathlib.HOST_MACROS)
+    src = "#include <math.h>\n" + mathlib.source(sorted(mathlib.FUNCTIONS), mathlib.HOST_MACROS)
     for name, (fn, _) in mathlib.FUNCTIONS.items():
-        src += (f"void v_{name}(const double* x, double* y, long n)\n"
-                f"{{ for (long i = 0; i < n; i++) y[i] = {fn}(x[i]); }}\n")
-    (d / "m.c").write_text(src)
-    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
-                    str(d / "m.c"), "-lm"], check=True)
+        src += (f'extern "C" void v_{name}(const double* x, double* y, long n)\n'
+                "{ long i = 0;\n"
+                "  for (; i + 4 <= n; i += 4) { const double a[4] = {x[i], x[i+1], x[i+2], x[i+3]}; "
+                f"double r[4]; {fn}<4>(a, r); for (int e = 0; e < 4; e++) y[i+e] = r[e]; }}\n"
+                f"  for (; i < n; i++) y[i] = {fn}_1(x[i]); }}\n")
+    (d / "m.cpp").write_text(src)
+    subprocess.run(["g++", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
+                    str(d / "m.cpp")], check=True)
     lib = ctypes.CDLL(str(d / "m.so"))
 
     def call(name, x):
@@ -73,19 +78,24 @@ def test_log_special_values(host):
 def test_erf_accuracy(host):
     rs = np.random.RandomState(4)
     x = np.concatenate([rs.uniform(-6.5, 6.5, 1 << 19), rs.uniform(-1, 1, 1 << 18),
+                        rs.uniform(0.2, 0.4, 1 << 16),          # where k goes from 0 to -1
                         rs.uniform(0.9, 1.1, 1 << 16), 10.0 ** rs.uniform(-300, 1, 1 << 16),
                         [1.0, -1.0, np.nextafter(1, 0), np.nextafter(1, 2), 5.9, 6.0, 6.1,
                          27.0, 1e300, 5e-324, 1e-310]])
     got = host("erf", x)
     ref = scipy.special.erf(x)
-    assert np.max(np.abs(got - ref) / np.spacing(np.abs(ref))) <= 3.5      # SciPy's is off by up to 2.6
+    assert np.max(np.abs(got - ref) / np.spacing(np.abs(ref))) <= 4.5      # SciPy's is off by up to 2.6
     assert np.all(np.abs(got) <= 1.0)
-    pick = np.r_[rs.choice(x.size - 11, 6000, replace=False), np.arange(x.size - 11, x.size)]
-    assert ulp_error(got[pick], x[pick], mp.erf) <= 1.0
-    # odd and monotone across the switch between the two branches
+    pick = np.r_[rs.choice(x.size - 11, 12000, replace=False), np.arange(x.size - 11, x.size)]
+    assert ulp_error(got[pick], x[pick], mp.erf) <= 2.0
+    # odd, and monotone where the exponent k of the reduction steps from 0 to -1
     assert np.array_equal(host("erf", -x), -got)
-    near = np.sort(rs.uniform(1 - 1e-9, 1 + 1e-9, 4096))
-    assert np.all(np.diff(host("erf", near)) >= -np.spacing(1.0))
+    w = 0.5 * np.log(2)
+    edge = float(mp.findroot(lambda t: -mp.log(mp.erfc(t)) - w, 0.28))
+    near = np.sort(rs.uniform(edge - 1e-9, edge + 1e-9, 4096))
+    assert np.all(np.diff(host("erf", near)) >= -np.spacing(0.25))
+    # the pack and the one-element form are the same arithmetic
+    assert np.array_equal(host("erf", x[:1001]), np.concatenate([host("erf", x[i:i + 1]) for i in range(1001)]))
 
 
 def test_erf_special_values(host):
@@ -118,10 +128,38 @@ def test_exp_accuracy_and_limits(host):
 
 def test_device_source_compiles():
     src = mathlib.source(["log", "erf", "exp"])
-    assert src.count("DR_FMA_K(") > 40 and src.count("dr_exp_reduced(double") == 1
+    assert src.count("DR_STEP(") > 35 and src.count("void dr_expm1_reduced(") == 1
     kernel = ('extern "C" __global__ void k(const double* a, double* o)\n'
-              "{ int i = threadIdx.x; o[i] = dr_log_f8(a[i]) + dr_erf_f8(a[i]) + dr_exp_f8(a[i]); }\n")
+              "{ int i = threadIdx.x; const double x[2] = {a[2 * i], a[2 * i + 1]}; double p[2], q[2], r[2];\n"
+              "  dr_log_f8<2>(x, p); dr_erf_f8<2>(x, q); dr_exp_f8<2>(x, r);\n"
+              "  o[i] = p[0] + q[1] + r[0] + dr_log_f8_1(a[i]) + dr_erf_f8_1(a[i]) + dr_exp_f8_1(a[i]); }\n")
     assert len(hip.compile_source(src + kernel)) > 0
+
+
+def test_packs_share_each_coefficient_between_their_elements():
+    """The reason for packs: in the kernel's main loop a coefficient is moved into its
+    scalar register pair once per pack.  Counted in the generated assembly: scalar moves
+    per vector multiply-add must be well below the two that a lone element needs."""
+    import re
+    import shutil
+    import tempfile
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    src = mathlib.source(["erf"]) + (
+        'extern "C" __global__ void k(const double* a, double* o)\n'
+        "{ const long i = 4L * (blockIdx.x * 256 + threadIdx.x);\n"
+        "  const double x[4] = {a[i], a[i + 1], a[i + 2], a[i + 3]}; double r[4];\n"
+        "  dr_erf_f8<4>(x, r); for (int e = 0; e < 4; e++) o[i + e] = r[e]; }\n")
+    with tempfile.TemporaryDirectory() as d:
+        with open(f"{d}/k.hip", "w") as fh:
+            fh.write(src)
+        subprocess.run([hipcc, "-x", "hip", "-include", "hip/hip_runtime.h", "-O3", "-ffp-contract=off",
+                        "--offload-arch=gfx950", "--cuda-device-only", "-S", "-o", f"{d}/k.s",
+                        f"{d}/k.hip"], check=True, capture_output=True)
+        asm = open(f"{d}/k.s").read()
+    fma = len(re.findall(r"^\s+v_fma_f64", asm, re.M))
+    smov = len(re.findall(r"^\s+s_mov_b32", asm, re.M))
+    assert fma >= 4 * 34                      # 23 + 9 polynomial steps and two more per element
+    assert smov <= 0.75 * fma, (smov, fma)    # a lone element needs 2 moves per step
 
 
 def test_programs_name_the_functions_they_replace():

@@ -239,3 +239,32 @@ def test_oracle_array_reproduces_golden_special_values():
                 assert bits_equal(fn(x).get(), g[f"{tag}_{name}"]), name
             for name, fn in BINARY.items():
                 assert bits_equal(fn(x, y).get(), g[f"{tag}_{name}"]), name
+
+
+def test_accuracy_report_measures_what_it_says():
+    """oracle/accuracy.py: the 50-digit price agrees with the float64 oracle where nothing
+    cancels, the ulp distance counts representable numbers, and a planted error shows up
+    at the right index, in the right subset, with the right size."""
+    from oracle import accuracy
+    inp = orc.make_inputs("bs64", 4096)
+    call, put = orc.black_scholes(inp["S"], inp["K"], inp["T"], inp["r"], inp["sigma"])
+    scale = np.maximum(inp["S"], inp["K"])
+    for i in np.flatnonzero(call >= 0.25 * scale)[:5]:
+        truth = float(accuracy.bs_truth(inp["S"][i], inp["K"][i], inp["T"][i], 0.02, 0.30, "call"))
+        assert abs(call[i] - truth) <= 1e-14 * truth
+        parity = float(accuracy.bs_truth(inp["S"][i], inp["K"][i], inp["T"][i], 0.02, 0.30, "put"))
+        assert abs((truth - parity) - (inp["S"][i] - inp["K"][i] * np.exp(-0.02 * inp["T"][i]))) \
+            <= 1e-13 * scale[i]
+    one = np.float32(1.0)
+    assert accuracy.ulp_distance(np.array([one]), np.array([np.nextafter(one, np.float32(2))]))[0] == 1
+    assert accuracy.ulp_distance(np.array([-0.0]), np.array([0.0]))[0] == 0
+    assert accuracy.ulp_distance(np.array([np.nan]), np.array([1.0]))[0] == np.inf
+    bent = call.copy()
+    i = int(np.flatnonzero(call >= 0.5 * scale)[0])
+    for _ in range(5):
+        bent[i] = np.nextafter(bent[i], np.inf)
+    rep = accuracy.bs_report(bent, put, call, put, inp)
+    assert rep["call"]["subsets"][1]["max_ulp"] == 5 and rep["call"]["subsets"][1]["max_ulp_index"] == i
+    assert rep["call"]["subsets"][1]["max_ulp_at"]["oracle_err_ulp_vs_truth"] < 16
+    assert rep["put"]["subsets"][16]["max_ulp"] == 0 and rep["put"]["scaled"]["max_eps"] == 0
+    assert "5 ulp" in accuracy.format_report("bs64", rep)
