@@ -87,7 +87,7 @@ def parse():
     ap.add_argument("--workload", default="all",
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
                          "dot | axis0 | axis1 | rows200 | rowbcast | transpose | interior | stencil3d | "
-                         "grid | next (these nine: the operations either side of the five "
+                         "grid | rand | next (these ten: the operations either side of the five "
                          "configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
@@ -210,6 +210,15 @@ def main():
                         steps=[lambda: hip.run(horner_expr(c, g))] * sets_for(4 * n),
                         cpu=lambda: orc.horner(c, np.linspace(-2.0, 2.0, m, dtype=np.float32)),
                         cpu_frac=1 / 16, cpu_code="oracle/numpy_oracle.py::horner on numpy.linspace")
+        if name == "rand":
+            n = 1 << 26
+            u = dr.random.device(0).random(n)                   # lazy: computed inside the kernel
+            m = n // 16
+            return dict(dtype="f64", n=n, nbytes=8 * n,
+                        desc="Philox-4x64-10 uniform doubles n=2^26 written to memory (generated in the kernel)",
+                        steps=[lambda: hip.run(u * 1.0)] * sets_for(8 * n),
+                        cpu=lambda: np.random.Generator(np.random.Philox(key=0)).random(m),
+                        cpu_frac=1 / 16, cpu_code="numpy.random.Generator(Philox).random")
         if name in ("matmul32", "matmul64"):
             N = 8192
             dt = np.float32 if name == "matmul32" else np.float64
@@ -452,7 +461,7 @@ def main():
 
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
              "next": ["dot", "axis0", "axis1", "rows200", "rowbcast", "transpose", "interior",
-                      "stencil3d", "grid"]}.get(args.workload, [args.workload])
+                      "stencil3d", "grid", "rand"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:

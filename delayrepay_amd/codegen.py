@@ -192,6 +192,74 @@ def op_expr(name, dt, args):
     raise NotImplementedError(f"ufunc {name!r} cannot be fused")
 
 
+# operations computed from the element index instead of from operands
+INDEX_OPS = ("iota", "philox_raw", "philox_f8")
+
+# Philox-4x64-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11),
+# the counter-based generator behind numpy.random.Philox.  Output r of the stream that
+# starts at the 256-bit counter (c0..c3) is word r % 4 of the block computed from
+# counter + r / 4 with the 128-bit key (k0, k1): ten rounds of two 64x64->128-bit
+# multiplications, the key bumped by the Weyl constants between rounds.
+PHILOX = """\
+typedef unsigned long long dr_u64;
+static __device__ __forceinline__ dr_u64 dr_mulhi64(dr_u64 a, dr_u64 b)
+{
+    return (dr_u64)(((unsigned __int128)a * b) >> 64);
+}
+/* the four outputs of block `blk` of the stream */
+static __device__ __forceinline__ void dr_philox_block(dr_u64 k0, dr_u64 k1, dr_u64 c0, dr_u64 c1,
+                                                       dr_u64 c2, dr_u64 c3, dr_u64 blk,
+                                                       dr_u64 (&x)[4])
+{
+    x[0] = c0 + blk;                      /* 256-bit counter + block number */
+    dr_u64 carry = x[0] < blk;
+    x[1] = c1 + carry;
+    carry = x[1] < carry;
+    x[2] = c2 + carry;
+    carry = x[2] < carry;
+    x[3] = c3 + carry;
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        const dr_u64 hi0 = dr_mulhi64(0xD2E7470EE14C6C93ULL, x[0]), lo0 = 0xD2E7470EE14C6C93ULL * x[0];
+        const dr_u64 hi1 = dr_mulhi64(0xCA5A826395121157ULL, x[2]), lo1 = 0xCA5A826395121157ULL * x[2];
+        x[0] = hi1 ^ x[1] ^ k0;
+        x[2] = hi0 ^ x[3] ^ k1;
+        x[1] = lo1;
+        x[3] = lo0;
+        k0 += 0x9E3779B97F4A7C15ULL;
+        k1 += 0xBB67AE8584CAA73BULL;
+    }
+}
+/* output r of the stream */
+static __device__ __forceinline__ dr_u64 dr_philox(dr_u64 k0, dr_u64 k1, dr_u64 c0, dr_u64 c1,
+                                                  dr_u64 c2, dr_u64 c3, dr_u64 r)
+{
+    dr_u64 x[4];
+    dr_philox_block(k0, k1, c0, c1, c2, c3, r >> 2, x);
+    const int lane = (int)(r & 3);
+    return lane == 0 ? x[0] : lane == 1 ? x[1] : lane == 2 ? x[2] : x[3];
+}
+"""
+
+
+def _philox_value(name, raw):
+    """int64 bits, or a double in [0, 1) from the top 53 bits (what
+    numpy.random.Generator.random makes of a raw output)."""
+    return f"(long long){raw}" if name == "philox_raw" else f"(double)({raw} >> 11) * 0x1p-53"
+
+
+def flat_elements(prog, leaf_class, out_dtypes, reduce_op):
+    """Elements one thread handles per vector step of the flat kernel: enough to fill a
+    16-byte vector of the narrowest streamed type; four when the program draws Philox
+    numbers, whose blocks hold four outputs (a thread then makes each block once)."""
+    widths = [ITEMSIZE[dt] for dt, c in zip(prog.leaves, leaf_class) if c == "c"]
+    if not reduce_op:
+        widths += [ITEMSIZE[dt] for dt in out_dtypes]
+    if any(name.startswith("philox") for name, _, _, _ in prog.ops):
+        widths.append(4)
+    return 16 // min(widths) if widths else 4
+
+
 class Program:
     """Straight-line SSA form of an expression DAG.
 
@@ -213,8 +281,8 @@ class Program:
         self.own_math = tuple(sorted({name for name, cdt, _, _ in self.ops
                                       if cdt == "f8" and name in mathlib.FUNCTIONS})) \
             if own_math else ()
-        # 'iota' operations read the element index: only the flat kernel supplies it
-        self.uses_index = any(name == "iota" for name, _, _, _ in self.ops)
+        # these operations read the element index: only the flat kernel supplies it
+        self.uses_index = any(name in INDEX_OPS for name, _, _, _ in self.ops)
 
     def key(self):
         return (self.leaves, self.scalars, self.ops, self.roots, self.own_math)
@@ -244,7 +312,9 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
     params += [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
+    uses_philox = any(name.startswith("philox") for name, _, _, _ in prog.ops)
     lines = [mathlib.source(prog.own_math) if with_math else "",
+             PHILOX if uses_philox and with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
     for i, (name, cdt, rdt, args) in enumerate(prog.ops):
         cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
@@ -252,6 +322,12 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
             expr = cargs[0]
         elif name == "iota":
             expr = f"({CTYPE[cdt]})dr_i"
+        elif name in ("philox_raw", "philox_f8"):
+            # operands: key (2 words), counter (4 words), position of element 0 in the stream
+            # (a seventh operand, when the draw starts inside a block: that offset)
+            words = ", ".join(f"(dr_u64){k}{j}" for k, j in args[:6])
+            pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
+            expr = _philox_value(name, f"dr_philox({words}, {pos}(dr_u64)dr_i)")
         elif cdt == "f8" and name in prog.own_math:
             expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
         elif name == "where":    # the condition keeps its own type
@@ -266,28 +342,51 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
     return "\n".join(lines)
 
 
-def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"):
+def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack", group=1):
     """The same program on a pack of `pack` elements held by one thread: every value
     is a small array and every operation a fully unrolled loop over it, so that the
     elements pass through each float64 `log`/`erf`/`exp` in lock step (see `mathlib`).
     Leaves flagged False in `leaf_is_array` are one value for the whole pack (broadcast
-    operands).  The arithmetic per element is exactly that of `emit_body`."""
+    operands).  The pack is made of groups of `group` consecutive elements; programs
+    that read the element index get the index of each group's first element in `dr_g`
+    (a multiple of `group`).  The arithmetic per element is exactly that of
+    `emit_body`."""
     P = pack
     loop = f'_Pragma("unroll") for (int e = 0; e < {P}; ++e)'
+    index = f"(dr_g[e / {group}] + e % {group})"
 
     def ref(k, j):
         if k == "s" or (k == "l" and not leaf_is_array[j]):
             return f"{k}{j}"
         return f"{k}{j}[e]"
 
-    params = [f"const {CTYPE[dt]} (&l{i})[{P}]" if leaf_is_array[i] else f"const {CTYPE[dt]} l{i}"
-              for i, dt in enumerate(prog.leaves)]
+    params = [f"const long long (&dr_g)[{P // group}]"] if prog.uses_index else []
+    params += [f"const {CTYPE[dt]} (&l{i})[{P}]" if leaf_is_array[i] else f"const {CTYPE[dt]} l{i}"
+               for i, dt in enumerate(prog.leaves)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]} (&r{i})[{P}]" for i, dt in enumerate(out_dtypes)]
     lines = [f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
     for i, (name, cdt, rdt, args) in enumerate(prog.ops):
         cargs = [_conv(ref(k, j), prog.ref_dtype((k, j)), cdt) for k, j in args]
         lines.append(f"    {CTYPE[rdt]} v{i}[{P}];")
+        if name == "iota":
+            lines.append(f"    {loop} v{i}[e] = ({CTYPE[cdt]}){index};")
+            continue
+        if name in ("philox_raw", "philox_f8"):
+            words = ", ".join(f"(dr_u64){k}{j}" for k, j in args[:6])
+            if len(args) == 6 and group == 4:
+                # the draw starts on a block and a group is four consecutive elements
+                # from a multiple of four: one block per group
+                for g in range(P // 4):
+                    vals = " ".join(f"v{i}[{4 * g + w}] = {_philox_value(name, f'x_[{w}]')};"
+                                    for w in range(4))
+                    lines.append(f"    {{ dr_u64 x_[4]; dr_philox_block({words}, (dr_u64)dr_g[{g}] >> 2, x_); "
+                                 f"{vals} }}")
+            else:
+                pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
+                raw = f"dr_philox({words}, {pos}(dr_u64){index})"
+                lines.append(f"    {loop} v{i}[e] = {_philox_value(name, raw)};")
+            continue
         if cdt == "f8" and name in prog.own_math:
             k, j = args[0]
             if prog.ref_dtype((k, j)) == "f8" and ref(k, j).endswith("[e]"):
@@ -386,8 +485,9 @@ def _st(nt, val, ptr):
 
 def packs(prog, vec):
     """Whether the flat kernel evaluates this program on packs of elements: programs
-    that use the float64 functions of `mathlib`, in vector kernels."""
-    return bool(vec and prog.own_math and not prog.uses_index)
+    that use the float64 functions of `mathlib` or draw Philox numbers, in vector
+    kernels."""
+    return bool(vec and (prog.own_math or any(name.startswith("philox") for name, _, _, _ in prog.ops)))
 
 
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
@@ -406,17 +506,12 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     ua = "u" if unaligned else ""
     n_leaf, n_out = len(prog.leaves), len(out_dtypes)
     red_dt = out_dtypes[0] if reduce_op else None
-    if vec:
-        widths = [ITEMSIZE[dt] for dt, c in zip(prog.leaves, leaf_class) if c == "c"]
-        if not reduce_op:
-            widths += [ITEMSIZE[dt] for dt in out_dtypes]
-        E = 16 // min(widths) if widths else 4
-    else:
-        E = 1
+    E = flat_elements(prog, leaf_class, out_dtypes, reduce_op) if vec else 1
     src = [PREAMBLE, emit_body(prog, out_dtypes)]
     packed = packs(prog, vec)
     if packed:
-        src.append(emit_body_packed(prog, out_dtypes, [c == "c" for c in leaf_class], E * unroll))
+        src.append(emit_body_packed(prog, out_dtypes, [c == "c" for c in leaf_class], E * unroll,
+                                    group=E))
     if reduce_op:
         src.append(emit_block_reduce(reduce_op, red_dt))
         src.append(emit_finalize(reduce_op, red_dt))
@@ -519,6 +614,10 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
         P, pad = E * unroll, " " * 8
         all_work = []
         args = []
+        if prog.uses_index:
+            bases = ", ".join(f"(v + {u * BLOCK}) * {E}" if u else f"v * {E}" for u in range(unroll))
+            all_work.append(f"{pad}const long long G[{unroll}] = {{{bases}}};")
+            args.append("G")
         for i, (dt, c) in enumerate(zip(prog.leaves, leaf_class)):
             if c == "b":
                 args.append(f"b{i}")

@@ -41,6 +41,20 @@ class CpuVisitor(Visitor):
         arr = node.__dict__.get("array")
         return arr if arr is not None else numpy.arange(node.shape[0]).astype(node.dtype)
 
+    def visit_RandEx(self, node):
+        arr = node.__dict__.get("array")
+        if arr is not None:
+            return arr
+        # numpy.random.Philox steps its counter before it makes a block, so the block
+        # that holds output `pos` is made from `counter + pos // 4`, entered one lower
+        first, skip = divmod(node.pos, 4)
+        start = (node.counter + first - 1) % (1 << 256)
+        bits = numpy.random.Philox(key=node.key, counter=start)
+        raw = bits.random_raw(skip + node.shape[0])[skip:]
+        if node.dtype == numpy.int64:
+            return raw.view(numpy.int64)
+        return (raw >> numpy.uint64(11)) * (1.0 / 9007199254740992.0)
+
     def visit_CastEx(self, node):
         return self.visit(node.children[0]).astype(node.dtype)
 

@@ -785,6 +785,29 @@ class IotaEx(_Generated):
         return f"iota{self._count}"
 
 
+class RandEx(_Generated):
+    """`n` consecutive outputs of a Philox-4x64-10 stream (`numpy.random.Philox` with
+    the same key and counter), starting `pos` outputs into it: raw 64-bit words (dtype
+    int64, the same bits as NumPy's uint64) or doubles in [0, 1) made from their top 53
+    bits as `numpy.random.Generator.random` makes them.  Every element is a function of
+    its index alone, so inside a 1-d expression of the same length it is computed in
+    the kernel and costs no memory traffic; made by `random.device(seed)`."""
+
+    def __init__(self, n, key, counter, pos, dtype):
+        super().__init__()
+        self.shape = (int(n),)
+        self.dtype = np.dtype(dtype)
+        if self.dtype not in (np.int64, np.float64):
+            raise TypeError("a Philox stream yields int64 words or float64 numbers")
+        self.key = int(key)
+        self.counter = int(counter)        # counter of the block that holds output 0
+        self.pos = int(pos)
+
+    @property
+    def name(self):
+        return f"rand{self._count}"
+
+
 PUSH_VIEWS_UP_TO = 48     # interior nodes; larger expressions are evaluated once, then viewed
 
 

@@ -95,6 +95,7 @@ def _scalar_value(value, code):
 
 
 _CODES = {}
+_M64 = (1 << 64) - 1
 
 
 def _code_of(dtype):
@@ -264,6 +265,18 @@ class Tracer(Visitor):
         res = self.scalar(node.val, _code_of(node.dtype), id(node))
         self.gen_shapes.append(node.shape)
         self.leaf_nodes.append((node, None, None))   # the plan holds while it stays unwritten
+        return res
+
+    def visit_RandEx(self, node):      # a stretch of a Philox stream, from the element index
+        words = [node.key & _M64, node.key >> 64] + [(node.counter >> (64 * k)) & _M64 for k in range(4)]
+        refs = [self.scalar(w - (1 << 64) if w >> 63 else w, "i8")[0] for w in words]
+        if node.pos:        # the draw starts inside a block
+            refs.append(self.scalar(node.pos, "i8", ("pos", id(node)))[0])
+        code = _code_of(node.dtype)
+        res = self.op("philox_raw" if code == "i8" else "philox_f8", code, code, refs)
+        self.gen_shapes.append(node.shape)
+        self.iotas.append((res[0][1], node))
+        self.leaf_nodes.append((node, None, None))
         return res
 
     def visit_IotaEx(self, node):      # the element index, converted

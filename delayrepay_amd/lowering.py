@@ -248,9 +248,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         if cg.packs(prog, vec) and TUNE["pack"]:
             # float64 functions evaluate a pack of elements in lock step: at least `pack`
             # elements per thread (a vector of doubles holds two)
-            min_width = min([cg.ITEMSIZE[c] for c, k in zip(prog.leaves, leaf_class) if k == "c"]
-                            + ([] if reduce_op else [cg.ITEMSIZE[c] for c in out_codes]) or [8])
-            unroll = max(unroll, TUNE["pack"] * min_width // 16)
+            unroll = max(unroll, TUNE["pack"] // cg.flat_elements(prog, leaf_class, out_codes, reduce_op))
         in_bytes = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
         footprint = in_bytes
         if not reduce_op:
@@ -273,13 +271,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                                   restrict=not in_place, reduce_op=reduce_op, unaligned=ua)
             return src
         low.emit = emit
-        if vec:
-            widths = [cg.ITEMSIZE[c] for c, k in zip(prog.leaves, leaf_class) if k == "c"]
-            if not reduce_op:
-                widths += [cg.ITEMSIZE[c] for c in out_codes]
-            E = 16 // min(widths) if widths else 4
-        else:
-            E = 1
+        E = cg.flat_elements(prog, leaf_class, out_codes, reduce_op) if vec else 1
         chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
         cap = TUNE["red_blocks"] if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
         low.grid = min(chunks, cap)

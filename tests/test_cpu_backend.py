@@ -54,6 +54,17 @@ SCRIPT = textwrap.dedent("""
     assert np.array_equal(np.where(a > 5, a, 0.0).get(), np.where(np.arange(12.0).reshape(3, 4) > 5,
                                                                    np.arange(12.0).reshape(3, 4), 0.0))
 
+    # the device generator's stream is NumPy's Philox stream, call after call
+    gen, ref = dnp.random.device(99), np.random.Generator(np.random.Philox(key=99))
+    for size in (5, 4096, 3, (6, 7)):
+        assert np.array_equal(gen.random(size).get(), ref.random(size))
+    assert np.array_equal(gen.uniform(-3.0, 5.0, 1001).get(), ref.uniform(-3.0, 5.0, 1001))
+    raw = gen.random_raw(10).get()
+    assert raw.dtype == np.int64 and np.array_equal(raw.view(np.uint64), ref.bit_generator.random_raw(10))
+    big = dnp.random.device(3, counter=(1 << 256) - 2)
+    assert np.array_equal(big.random(20).get(),
+                          np.random.Generator(np.random.Philox(key=3, counter=(1 << 256) - 2)).random(20))
+
     # generated leaves: long constant / index arrays stay lazy and give NumPy's exact bits
     from delayrepay.delayarray import FullEx, WhereEx, BinaryNumpyEx
     same = lambda got, ref: (got.dtype == ref.dtype and got.shape == ref.shape

@@ -436,3 +436,26 @@ def test_three_dimensional_shifted_views_lower_to_the_lds_window():
     odd = NPArray(hip.placeholder((n, n, n - 1), np.float32))      # rows not 16-byte multiples
     low, src = hip.lower_only(odd[:-2, 1:-1, 1:-1] + odd[2:, 1:-1, 1:-1])
     assert low.kind == "tile2d"
+
+
+def test_device_random_numbers_cost_no_operand():
+    """`random.device(seed)`: the Philox stream is computed from the element index, so an
+    expression over its arrays reads nothing; successive draws continue the stream."""
+    from delayrepay_amd.delayarray import RandEx
+    gen = dr.random.device(2024)
+    u = gen.random(1 << 16)
+    v = gen.uniform(-1.0, 1.0, 1 << 16)
+    assert isinstance(u, RandEx) and "array" not in u.__dict__
+    assert (u.pos, v.children[1].children[1].pos) == (0, 0)      # each draw starts on its own block
+    assert v.children[1].children[1].counter == u.counter + (1 << 14)
+    low, src = hip.lower_only(u * u + v)
+    assert low.kind == "flat" and low.srcs == []                 # 0 bytes read per element
+    assert src.count("dr_philox(") == 3 and "unsigned __int128" in src
+    hip.compile_source(src)
+    odd = dr.random.device(1)
+    odd.random(3)
+    w = odd.random_raw(1 << 12)                                   # starts in the middle of a block
+    assert (w.pos, w.dtype) == (3, np.int64)
+    hip.compile_source(hip.lower_only(w)[1])
+    with pytest.raises(ValueError):
+        dr.random.device(-1)

@@ -1004,3 +1004,47 @@ def test_three_dimensional_stencil_layouts_that_do_not_qualify_still_match():
         assert u.get().tobytes() == ref.tobytes()
     finally:
         hip.set_tune(s3=1)
+
+
+# ---- device random numbers (Philox-4x64-10) ----------------------------------------------
+
+@pytest.mark.parametrize("seed,counter", [(0, 0), (20261125, 0), ((1 << 128) - 1, (1 << 256) - 3),
+                                          (5, (1 << 64) - 1000)])
+def test_device_random_stream_is_numpys_philox(seed, counter):
+    """Integer work, so bit-exact: raw outputs equal `Philox(key, counter).random_raw`,
+    doubles equal `Generator(Philox).random`, over successive draws of awkward lengths
+    (the stream position stops inside a block, the counter carries into the next word,
+    the last elements go through the kernel's leftover and tail paths)."""
+    gen = dr.random.device(seed, counter)
+    ref = np.random.Generator(np.random.Philox(key=seed, counter=counter))
+    for n in (1, 3, 4097, (1 << 20) + 3, 70001):
+        raw = gen.random_raw(n).get()
+        assert raw.dtype == np.int64
+        assert np.array_equal(raw.view(np.uint64), ref.bit_generator.random_raw(n)), n
+    for n in (5, 1 << 16, (1 << 18) + 1):
+        assert np.array_equal(gen.random(n).get(), ref.random(n)), n
+    assert np.array_equal(gen.uniform(-2.5, 7.0, 100003).get(), ref.uniform(-2.5, 7.0, 100003))
+    assert np.array_equal(gen.random((33, 65)).get(), ref.random((33, 65)))
+
+
+def test_device_random_numbers_fuse_without_memory_traffic():
+    gen = dr.random.device(11)
+    ref = np.random.Generator(np.random.Philox(key=11))
+    n = 1 << 22
+    u, v = gen.random(n), gen.random(n)
+    inside = (u * u + v * v) < 1.0                  # Monte-Carlo pi: no array is ever stored
+    low, _ = hip.lower_only(ReduceEx(np.add, inside))
+    assert low.srcs == []
+    launches = hip.STATS["launches"]
+    hits = int(dr.sum(inside))
+    assert hip.STATS["launches"] == launches + 2     # fused body + finalize
+    a, b = ref.random(n), ref.random(n)
+    assert hits == int(np.sum((a * a + b * b) < 1.0))
+    # asked for on its own, or used in another shape, the node becomes an ordinary array
+    w = gen.random(6000)
+    col = w.reshape(6000, 1) * dr.array(np.ones((1, 3)))
+    assert np.array_equal(col.get(), ref.random(6000)[:, None] * np.ones((1, 3)))
+    x = gen.random(5000)
+    y = x[10:20] + 1.0
+    want = ref.random(5000)
+    assert np.array_equal(y.get(), want[10:20] + 1.0) and np.array_equal(x.get(), want)

@@ -268,3 +268,23 @@ def test_accuracy_report_measures_what_it_says():
     assert rep["call"]["subsets"][1]["max_ulp_at"]["oracle_err_ulp_vs_truth"] < 16
     assert rep["put"]["subsets"][16]["max_ulp"] == 0 and rep["put"]["scaled"]["max_eps"] == 0
     assert "5 ulp" in accuracy.format_report("bs64", rep)
+
+
+def test_philox_restatement_against_numpy_and_the_published_vectors():
+    """oracle/philox.py: known-answer vectors of Philox-4x64-10 (all-zero and all-ones
+    counter and key, from the generator's reference distribution), NumPy's generator for
+    keys and counters that exercise every word and the carry out of the counter, and the
+    53-bit doubles across two calls of one Generator."""
+    from oracle import philox
+    assert philox.block(0, 0) == [0x16554d9eca36314c, 0xdb20fe9d672d0fdc,
+                                  0xd7e772cee186176b, 0x7e68b68aec7ba23b]
+    assert philox.block((1 << 256) - 1, (1 << 128) - 1) == [
+        0x87b092c3013fe90b, 0x438c3c67be8d0224, 0x9cc7d7c69cd777b6, 0xa09caebf594f0ba0]
+    for key, ctr in ((0, 0), (12345, 0), ((1 << 128) - 5, (1 << 256) - 2),
+                     (987654321 << 70, 3 << 190), (1, (1 << 64) - 2), (2, (1 << 128) - 1)):
+        ref = np.random.Philox(key=key, counter=ctr).random_raw(23)
+        assert [int(v) for v in ref] == philox.stream(key, ctr, 23), (key, ctr)
+    gen = np.random.Generator(np.random.Philox(key=7))
+    drawn = list(gen.random(10)) + list(gen.random(7))          # 17 outputs: not a multiple of 4
+    assert drawn == philox.doubles(philox.stream(7, 0, 17))
+    assert philox.stream(7, 0, 5, skip=9) == philox.stream(7, 0, 14)[9:]
