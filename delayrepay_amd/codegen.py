@@ -34,11 +34,11 @@ Kernel shapes (all 256-thread blocks = 4 wave64):
     shuffle tree, LDS across the 4 waves, one partial per block, and a
     one-block finalize kernel (no atomics, deterministic).
 Vector accesses use 16-byte types at element alignment where 16-byte alignment is
-missing; float64 `log`, `erf`, `exp` come from `mathlib`.
+missing; `log`, `erf`, `exp` come from `mathlib` (float64) and `mathlib32` (float32).
 """
 import numpy as np
 
-from . import mathlib
+from . import mathlib, mathlib32
 
 BLOCK = 256          # threads per block: 4 wave64
 WAVE = 64
@@ -270,9 +270,9 @@ class Program:
     roots    list of (ref, dtype code)
     """
 
-    __slots__ = ("leaves", "scalars", "ops", "roots", "own_math", "uses_index")
+    __slots__ = ("leaves", "scalars", "ops", "roots", "own_math", "own_math32", "uses_index")
 
-    def __init__(self, leaves, scalars, ops, roots, own_math=True):
+    def __init__(self, leaves, scalars, ops, roots, own_math=True, own_math32=True):
         self.leaves = tuple(leaves)
         self.scalars = tuple(scalars)
         self.ops = tuple(ops)
@@ -281,11 +281,15 @@ class Program:
         self.own_math = tuple(sorted({name for name, cdt, _, _ in self.ops
                                       if cdt == "f8" and name in mathlib.FUNCTIONS})) \
             if own_math else ()
+        # float32 functions taken from `mathlib32`
+        self.own_math32 = tuple(sorted({name for name, cdt, _, _ in self.ops
+                                        if cdt == "f4" and name in mathlib32.FUNCTIONS})) \
+            if own_math32 else ()
         # these operations read the element index: only the flat kernel supplies it
         self.uses_index = any(name in INDEX_OPS for name, _, _, _ in self.ops)
 
     def key(self):
-        return (self.leaves, self.scalars, self.ops, self.roots, self.own_math)
+        return (self.leaves, self.scalars, self.ops, self.roots, self.own_math, self.own_math32)
 
     def ref_dtype(self, ref):
         kind, i = ref
@@ -314,6 +318,7 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
     uses_philox = any(name.startswith("philox") for name, _, _, _ in prog.ops)
     lines = [mathlib.source(prog.own_math) if with_math else "",
+             mathlib32.source(prog.own_math32) if with_math else "",
              PHILOX if uses_philox and with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
     for i, (name, cdt, rdt, args) in enumerate(prog.ops):
@@ -330,6 +335,8 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
             expr = _philox_value(name, f"dr_philox({words}, {pos}(dr_u64)dr_i)")
         elif cdt == "f8" and name in prog.own_math:
             expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
+        elif cdt == "f4" and name in prog.own_math32:
+            expr = f"{mathlib32.FUNCTIONS[name][0]}({cargs[0]})"
         elif name == "where":    # the condition keeps its own type
             k, j = args[0]
             expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
@@ -399,6 +406,8 @@ def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"
             expr = cargs[0]
         elif name == "where":    # the condition keeps its own type
             expr = f"(({ref(*args[0])} != 0) ? {cargs[1]} : {cargs[2]})"
+        elif cdt == "f4" and name in prog.own_math32:
+            expr = f"{mathlib32.FUNCTIONS[name][0]}({cargs[0]})"
         else:
             expr = op_expr(name, cdt, cargs)
         lines.append(f"    {loop} v{i}[e] = {expr};")

@@ -299,7 +299,7 @@ class Tracer(Visitor):
         self.iotas = []
 
     def program(self, roots):
-        return Program(self.leaf_codes, self.scalar_codes, self.ops, roots, TUNE["dmath"])
+        return Program(self.leaf_codes, self.scalar_codes, self.ops, roots, TUNE["dmath"], TUNE["smath"])
 
 
 # ---------------------------------------------------------------------------

@@ -46,6 +46,7 @@ TUNE = {
     "uvec": 1,        # 16-byte accesses at element alignment where 16-byte alignment is missing
     "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
+    "smath": 1,       # float32 log/erf/exp from `mathlib32` (0: the device library's)
     "pack": 4,        # elements a thread passes through those functions in lock step
 }
 for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):

@@ -13,7 +13,7 @@ import pytest
 
 import delayrepay_amd as dr
 from delayrepay_amd import codegen as cg
-from delayrepay_amd import hip, hiprt, mathlib
+from delayrepay_amd import hip, hiprt, mathlib, mathlib32
 from delayrepay_amd.delayarray import (BinaryFuncEx, BinaryNumpyEx, CastEx, FullEx, IotaEx, NPArray,
                                        ReduceEx, Scalar, UnaryFuncEx, Memoiser)
 
@@ -348,7 +348,9 @@ def test_every_supported_ufunc_generates_compilable_source(name, dtype):
     hip.compile_source(src)
     expect = ("f" if dtype == np.float32 else "")
     if dtype == np.float64 and name in mathlib.FUNCTIONS:
-        assert f"{mathlib.FUNCTIONS[name][0]}(" in src
+        assert f"{mathlib.FUNCTIONS[name][0]}<" in src and f"{mathlib.FUNCTIONS[name][0]}_1(" in src
+    elif dtype == np.float32 and name in mathlib32.FUNCTIONS:
+        assert f"{mathlib32.FUNCTIONS[name][0]}(" in src
     elif name in cg._FLOAT_FUNCS1:
         assert f"{cg._FLOAT_FUNCS1[name]}{expect}(" in src
 

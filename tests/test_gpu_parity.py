@@ -270,6 +270,46 @@ def test_transcendentals_on_dense_random_arguments(dtype):
             assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-300)) <= 1e-13, name
 
 
+@pytest.mark.parametrize("name", ["erf", "exp", "log"])
+def test_float32_functions_over_the_bit_patterns(name):
+    """The device's own float32 `erf`, `exp`, `log` (hardware 2^x and log2 inside) against
+    SciPy / NumPy evaluated in float64 and rounded: every 7th float32 bit pattern (613
+    million arguments, denormals, infinities and NaNs among them) plus every float32 of
+    the intervals where the method changes.  Bar: 2 ulp of the correctly rounded result
+    (exp, log: 1 ulp on denormal results, which have fewer bits)."""
+    from scipy.special import erf
+    fn = {"erf": erf, "exp": np.exp, "log": np.log}[name]
+    worst = 0.0
+
+    def check(bits):
+        nonlocal worst
+        x = bits.view(np.float32)
+        got = fn(dr.array(x)).get()
+        with np.errstate(all="ignore"):
+            exact = fn(x.astype(np.float64))
+            want = exact.astype(np.float32)
+        fin = np.isfinite(want)
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])   # infinities
+        err = ulp_distance(got[fin], want[fin])
+        k = int(err.argmax()) if err.size else 0
+        assert err.size == 0 or err[k] <= 2, (name, x[fin][k], got[fin][k], want[fin][k])
+        worst = max(worst, float(err.max()) if err.size else 0.0)
+
+    step = 7
+    for lo in range(0, 1 << 32, 1 << 29):
+        check(np.arange(lo, lo + (1 << 29), step, dtype=np.uint64).astype(np.uint32))
+    dense = {"erf": [(0.86, 0.89), (3.9, 4.1), (0.0, 1e-6)],
+             "exp": [(86.0, 89.0), (-104.5, -86.0), (-1e-3, 1e-3)],
+             "log": [(0.99, 1.01), (1e-39, 2e-38)]}[name]
+    for a, b in dense:
+        for sign in ((1, -1) if name != "log" else (1,)):
+            lo, hi = sorted(np.array([a, b], np.float32).view(np.uint32).astype(np.int64))
+            span = np.arange(lo, min(hi, lo + (1 << 25)), dtype=np.int64).astype(np.uint32)
+            check(span if sign > 0 else span | np.uint32(1 << 31))
+    print(f"\n  float32 {name}: worst {worst:.0f} ulp from the correctly rounded result", flush=True)
+
+
 # ---- C4 Jacobi and other shifted-slice stencils --------------------------------------------
 
 def jacobi_sweeps(u, sweeps):

@@ -183,3 +183,112 @@ def test_coefficients_are_the_ones_the_fit_script_prints(capsys):
     printed |= {"-" + h for h in printed}                       # -ln 2 (hi, lo)
     assert used - printed == {"0x1.6a09e667f3bcdp-1"}            # sqrt(1/2)
     assert float.fromhex("0x1.6a09e667f3bcdp-1") == np.sqrt(0.5)
+
+
+# ---- float32 functions (mathlib32) ---------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def host32(tmp_path_factory):
+    """`mathlib32` built for the host: the two hardware functions (2^x, log2 x) are taken
+    from libm here, so this checks the argument reductions, the polynomials and the
+    special cases; the device's own 1-ulp versions are measured in the GPU tests."""
+    from delayrepay_amd import mathlib32
+    d = tmp_path_factory.mktemp("mathlib32")
+    src = "#include <math.h>\n" + mathlib32.source(sorted(mathlib32.FUNCTIONS), mathlib32.HOST_MACROS)
+    for name, (fn, _) in mathlib32.FUNCTIONS.items():
+        src += (f"void v_{name}(const float* x, float* y, long n)\n"
+                f"{{ for (long i = 0; i < n; i++) y[i] = {fn}(x[i]); }}\n")
+    (d / "m.c").write_text(src)
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
+                    str(d / "m.c"), "-lm"], check=True)
+    lib = ctypes.CDLL(str(d / "m.so"))
+
+    def call(name, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        y = np.empty_like(x)
+        getattr(lib, "v_" + name)(x.ctypes.data_as(ctypes.c_void_p),
+                                  y.ctypes.data_as(ctypes.c_void_p), ctypes.c_long(x.size))
+        return y
+    return call
+
+
+def ulp32(got, exact64):
+    """Error of float32 results in float32 ulps of the exact value (given in float64)."""
+    scale = np.spacing(np.abs(exact64).astype(np.float32)).astype(np.float64)
+    return np.abs(got.astype(np.float64) - exact64) / scale
+
+
+def test_float32_erf(host32):
+    rs = np.random.RandomState(6)
+    x = np.concatenate([rs.uniform(-4.5, 4.5, 1 << 20), rs.uniform(-1, 1, 1 << 19),
+                        rs.uniform(0.87, 0.88, 1 << 16), 10.0 ** rs.uniform(-44, 0, 1 << 16),
+                        [0.875, np.nextafter(np.float32(0.875), 0), 3.9, 4.0, 4.1, 1e-45, 1e30]]
+                       ).astype(np.float32)
+    got = host32("erf", x)
+    exact = scipy.special.erf(x.astype(np.float64))
+    assert ulp32(got, exact).max() <= 1.5
+    assert np.all(np.abs(got) <= 1.0) and np.array_equal(host32("erf", -x), -got)
+    near = np.sort(rs.uniform(0.8749, 0.8751, 4096).astype(np.float32))      # across the switch
+    assert np.all(np.diff(host32("erf", near)) >= -np.spacing(np.float32(0.5)))
+    sp = host32("erf", [0.0, -0.0, np.inf, -np.inf, np.nan, 40.0, -40.0])
+    assert sp[0] == 0 and not np.signbit(sp[0]) and sp[1] == 0 and np.signbit(sp[1])
+    assert sp[2] == 1 and sp[3] == -1 and np.isnan(sp[4]) and sp[5] == 1 and sp[6] == -1
+
+
+def test_float32_exp(host32):
+    rs = np.random.RandomState(7)
+    x = np.concatenate([rs.uniform(-104, 89, 1 << 20), rs.uniform(-1, 1, 1 << 18),
+                        [0.0, -0.0, 88.72283, 88.72284, -87.33654, -103.97, -104.1, 87.0, -87.0]]
+                       ).astype(np.float32)
+    got = host32("exp", x)
+    with np.errstate(over="ignore", under="ignore"):
+        exact = np.exp(x.astype(np.float64))
+    normal = (exact >= np.finfo(np.float32).tiny) & (exact <= np.finfo(np.float32).max)
+    assert ulp32(got[normal], exact[normal]).max() <= 1.0
+    small = exact < np.finfo(np.float32).tiny
+    assert np.max(np.abs(got[small].astype(np.float64) - exact[small]) / 1.401298464324817e-45) <= 1.0
+    with np.errstate(over="ignore"):
+        assert np.array_equal(np.isinf(got), np.isinf(np.exp(x)))
+    sp = host32("exp", [np.inf, -np.inf, np.nan, 89.0, 1e30, -105.0, -1e30, 0.0])
+    assert sp[0] == np.inf and sp[1] == 0 and np.isnan(sp[2]) and sp[3] == np.inf
+    assert sp[4] == np.inf and sp[5] == 0 and sp[6] == 0 and sp[7] == 1.0
+
+
+def test_float32_log(host32):
+    rs = np.random.RandomState(8)
+    x = np.concatenate([rs.uniform(1e-6, 1e6, 1 << 19), np.exp(rs.uniform(-103, 88, 1 << 19)),
+                        rs.uniform(0.5, 2, 1 << 19), 1 + rs.uniform(-1e-3, 1e-3, 1 << 16),
+                        [1e-45, 1.1754944e-38, 1e-40, 1.0, np.nextafter(np.float32(1), 2),
+                         np.nextafter(np.float32(1), 0), 3.4028235e38]]).astype(np.float32)
+    got = host32("log", x)
+    exact = np.log(x.astype(np.float64))
+    nz = exact != 0
+    # the stand-in log2f is itself up to 0.8 ulp off, and that error passes straight through
+    assert ulp32(got[nz], exact[nz]).max() <= 1.6 and np.all(got[~nz] == 0)
+    sp = host32("log", [0.0, -0.0, -1.0, -np.inf, np.inf, np.nan, 1.0])
+    assert sp[0] == -np.inf and sp[1] == -np.inf
+    assert np.isnan(sp[2]) and np.isnan(sp[3]) and np.isnan(sp[5])
+    assert sp[4] == np.inf and sp[6] == 0.0 and not np.signbit(sp[6])
+
+
+def test_float32_device_source_compiles_to_the_hardware_functions():
+    import re
+    import shutil
+    import tempfile
+    from delayrepay_amd import mathlib32
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    src = mathlib32.source(["erf", "exp", "log"]) + (
+        'extern "C" __global__ void k(const float* a, float* o)\n'
+        "{ const int i = blockIdx.x * 256 + threadIdx.x;\n"
+        "  o[i] = dr_erf_f4(a[i]) + dr_exp_f4(a[i]) * dr_log_f4(a[i]); }\n")
+    assert len(hip.compile_source(src)) > 0
+    with tempfile.TemporaryDirectory() as d:
+        with open(f"{d}/k.hip", "w") as fh:
+            fh.write(src)
+        subprocess.run([hipcc, "-x", "hip", "-include", "hip/hip_runtime.h", "-O3", "-ffp-contract=off",
+                        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                        "--offload-arch=gfx950", "--cuda-device-only", "-S", "-o", f"{d}/k.s",
+                        f"{d}/k.hip"], check=True, capture_output=True)
+        asm = open(f"{d}/k.s").read()
+    assert len(re.findall(r"^\s+v_exp_f32", asm, re.M)) >= 2 and len(re.findall(r"^\s+v_log_f32", asm, re.M)) >= 1
+    assert not re.findall(r"^\s+v_pk_\w+_f32", asm, re.M)
