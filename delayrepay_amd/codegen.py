@@ -308,7 +308,7 @@ def _conv(expr, src, dst):
     return f"({CTYPE[dst]}){expr}"
 
 
-def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
+def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=False):
     """Inline device function evaluating the whole program for one element.
 
     Parameters: leaf values, scalar values, then one reference per root."""
@@ -317,7 +317,7 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True):
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
     uses_philox = any(name.startswith("philox") for name, _, _, _ in prog.ops)
-    lines = [mathlib.source(prog.own_math) if with_math else "",
+    lines = [mathlib.source(prog.own_math, lds=lds_tables) if with_math else "",
              mathlib32.source(prog.own_math32) if with_math else "",
              PHILOX if uses_philox and with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
@@ -516,7 +516,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     n_leaf, n_out = len(prog.leaves), len(out_dtypes)
     red_dt = out_dtypes[0] if reduce_op else None
     E = flat_elements(prog, leaf_class, out_dtypes, reduce_op) if vec else 1
-    src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    src = [PREAMBLE, emit_body(prog, out_dtypes, lds_tables=True)]
     packed = packs(prog, vec)
     if packed:
         src.append(emit_body_packed(prog, out_dtypes, [c == "c" for c in leaf_class], E * unroll,
@@ -537,6 +537,8 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     L.append(f'extern "C" __global__ __launch_bounds__({BLOCK})')
     L.append(f"void dr_kernel({', '.join(params)})")
     L.append("{")
+    if mathlib.tables(prog.own_math):
+        L.append("    DR_STAGE_TABLES();      // the functions' tables, from memory into LDS")
     for i, c in enumerate(leaf_class):
         if c == "b":
             L.append(f"    const {CTYPE[prog.leaves[i]]} b{i} = a{i}[0];")

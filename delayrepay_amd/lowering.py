@@ -10,6 +10,7 @@ ElementwiseKernel does its own (contiguous-or-generic) indexing (cuda.py:35-43).
 import os
 
 from . import codegen as cg
+from . import mathlib
 from . import hiprt
 
 # Tunables; part of every cache key.  DELAYREPAY_TUNE="unroll=2,bpc=16" overrides.
@@ -46,6 +47,7 @@ TUNE = {
     "uvec": 1,        # 16-byte accesses at element alignment where 16-byte alignment is missing
     "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
+    "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
     "smath": 1,       # float32 log/erf/exp from `mathlib32` (0: the device library's)
     "pack": 4,        # elements a thread passes through those functions in lock step
 }
@@ -275,6 +277,11 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         E = cg.flat_elements(prog, leaf_class, out_codes, reduce_op) if vec else 1
         chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
         cap = TUNE["red_blocks"] if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
+        if mathlib.tables(prog.own_math) and not TUNE["flat_cap"]:
+            # the workgroup copies the functions' tables into LDS first: let it stay for
+            # several chunks (Black-Scholes float64: 262 us with a chunk per workgroup, 244 us
+            # with 4096 to 8192 workgroups, 251 us with 1024)
+            cap = min(cap, TUNE["table_blocks"])
         low.grid = min(chunks, cap)
         n_out_ptr = 1 if reduce_op else len(out_ptrs)
         low.fmt = "@" + "P" * (len(ptrs) + n_out_ptr) + scal_fmt + "q"
