@@ -1,4 +1,4 @@
-"""Double-precision `log`, `erf` and `exp` for the generated kernels.
+"""Double-precision `log`, `erf`, `exp` and `sqrt` for the generated kernels.
 
 The device library's versions cost 97, 105 and 41 vector instructions per element
 (counted in gfx950 code), which makes a Black-Scholes kernel in float64 wait on the
@@ -6,7 +6,8 @@ fp64 pipes rather than on memory.  These cost about 25, 20 and 25.  Black-Schole
 float64, n = 2^25, microseconds per launch on MI355X (vector instructions per option):
 device library 398 (379); polynomial `log`/`erf`/`exp`, one element at a time 305 (254);
 the same on packs of four 299 (245); `log` from a table 293 (227); `erf` from a table
-read in memory 405, read in LDS 262, with workgroups that stay for eight chunks 241 (153).
+read in memory 405, read in LDS 262, with workgroups that stay for eight chunks 241 (153);
+with the short `sqrt` 240.
 
 `log` and `erf` are table driven.  `log`: x = 2^k z, z in [0.706, 1.412) falls into one of
 256 intervals with centre c, log x = k ln 2 + log c + log1p(z/c - 1); 1/c and log c come
@@ -21,7 +22,11 @@ a double to within a small fraction of an ulp, so that the table adds almost no 
 of its own.  Every lane reads its own row: through the vector memory path that is slow, so
 flat kernels copy the tables into LDS first (`source(..., lds=True)`, `DR_STAGE_TABLES`);
 other kernel shapes read them in memory.  `exp` is 2^k (1 + m) with k = rint(x / ln 2),
-m = e^v - 1 = v + v^2 R(v), R of degree 9.
+m = e^v - 1 = v + v^2 R(v), R of degree 9.  `sqrt` is the compiler's own correctly rounded
+expansion without its rescaling and special-case selects (10 instructions instead of 21);
+arguments that need those take the compiler's path, which a wave skips when none of its
+lanes does (tested per wave: a per-lane condition is folded into selects and both
+versions run).
 
 Packs.  A 64-bit polynomial coefficient reaches `v_fma_f64` through a scalar register
 pair (`DR_FMA_K`), which takes two scalar moves.  Every function is a template over P
@@ -43,6 +48,8 @@ fits on Chebyshev nodes in 50-digit arithmetic).
 DEVICE_MACROS = """\
 #define DR_FN static __device__ __forceinline__
 #define DR_TABLE static __device__ const
+#define DR_RSQ64(x) __builtin_amdgcn_rsq(x)
+#define DR_ANY_LANE(p) (__builtin_amdgcn_ballot_w64(p) != 0)
 /* p * z + k with the constant k in a scalar register pair.  The compiler prefers the
    two-address v_fmac_f64 for a Horner step and then copies every 64-bit constant into
    the accumulator with two v_mov_b32, which triples the cost of a polynomial. */
@@ -53,6 +60,15 @@ DEVICE_MACROS = """\
 HOST_MACROS = """\
 #define DR_FN static inline
 #define DR_TABLE static const
+/* a 24-bit estimate of 1/sqrt(x), like the hardware's */
+static inline double dr_rsq64_host(double x)
+{
+    int ex;
+    const double mant = frexp(1.0 / sqrt(x), &ex);
+    return ldexp((double)(float)mant, ex);
+}
+#define DR_RSQ64(x) dr_rsq64_host(x)
+#define DR_ANY_LANE(p) (p)
 #define DR_FMA_K(p, z, k) __builtin_fma(p, z, k)
 """
 
@@ -562,11 +578,44 @@ DR_FN void dr_erf_f8(const double (&x)[P], double (&out)[P])
         out[e] = __builtin_copysign(p[e], x[e]);
 }"""
 
+SQRT_F8 = r"""
+/* Correctly rounded square root: reciprocal square root estimate, one coupled step for
+   g ~ sqrt(x) and h ~ 1/(2 sqrt(x)), two residual corrections d = x - g^2, g += d h; the
+   last fused operation rounds once.  This is the compiler's own expansion of sqrt for
+   arguments that need no rescaling; zero, negative, infinite, NaN and arguments below
+   2^-767 (whose estimate would lose bits) go to that expansion, on a path a wave skips
+   when none of its lanes needs it. */
+template <int P>
+DR_FN void dr_sqrt_f8(const double (&x)[P], double (&out)[P])
+{
+    _Pragma("unroll") for (int e = 0; e < P; ++e) {
+        const double y = DR_RSQ64(x[e]);
+        double g = x[e] * y;
+        double h = 0.5 * y;
+        const double r = __builtin_fma(-h, g, 0.5);
+        g = __builtin_fma(g, r, g);
+        h = __builtin_fma(h, r, h);
+        double d = __builtin_fma(-g, g, x[e]);
+        g = __builtin_fma(d, h, g);
+        d = __builtin_fma(-g, g, x[e]);
+        out[e] = __builtin_fma(d, h, g);
+    }
+    bool rare = false;
+    _Pragma("unroll") for (int e = 0; e < P; ++e)
+        rare |= !(x[e] >= 0x1p-767 && x[e] < __builtin_inf());
+    if (DR_ANY_LANE(rare)) {        /* one test per wave: the compiler must not fold this into selects */
+        _Pragma("unroll") for (int e = 0; e < P; ++e)
+            if (!(x[e] >= 0x1p-767 && x[e] < __builtin_inf()))
+                out[e] = __builtin_sqrt(x[e]);
+    }
+}"""
+
 # ufunc name -> (device function template, sources it needs in order), float64 only
 FUNCTIONS = {
     "log": ("dr_log_f8", (STEP, LOG_TABLE, LOG_CORE, LOG_F8)),
     "erf": ("dr_erf_f8", (ERF_TABLE, ERF_F8)),
     "exp": ("dr_exp_f8", (STEP, EXPM1_REDUCED, EXP_F8)),
+    "sqrt": ("dr_sqrt_f8", (SQRT_F8,)),
 }
 
 # Where the functions read their tables.  In memory (the default): every lane's 16-byte

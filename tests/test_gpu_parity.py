@@ -270,6 +270,30 @@ def test_transcendentals_on_dense_random_arguments(dtype):
             assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-300)) <= 1e-13, name
 
 
+def test_float64_sqrt_is_ieee_on_the_device():
+    """The short float64 square root (reciprocal square root estimate by hardware, then
+    the compiler's own correction steps) must give IEEE sqrt's bits: random arguments over
+    every exponent, neighbours of perfect squares, and the arguments that take the guarded
+    path (below 2^-767, denormals, zeros, infinity, NaN, negative)."""
+    rs = np.random.RandomState(12)
+    m = rs.uniform(1, 4, 1 << 22)
+    exact = np.floor(rs.uniform(1, 2 ** 26, 1 << 18)) ** 2
+    x = np.concatenate([m, np.ldexp(m, rs.randint(-1074, 1020, m.size)), exact, np.nextafter(exact, 0),
+                        np.nextafter(exact, np.inf), rs.uniform(0, 1e-300, 1 << 12),
+                        rs.randint(0, 1 << 62, 1 << 22).astype(np.uint64).view(np.float64),
+                        [0.0, -0.0, np.inf, -np.inf, np.nan, -1.0, 4.0, 2.0, 1e-320, 5e-324, 2.0 ** -767,
+                         np.nextafter(2.0 ** -767, 0), 1.7976931348623157e308]])
+    with np.errstate(invalid="ignore"):
+        want = np.sqrt(x)
+    assert bits_equal(np.sqrt(dr.array(x)).get(), want)
+    # inside a larger expression (the packed form) and in the general-stride kernel
+    y = rs.uniform(0.5, 2, x.size)
+    with np.errstate(invalid="ignore"):
+        assert bits_equal((np.sqrt(dr.array(x)) * dr.array(y) + 1.0).get(), np.sqrt(x) * y + 1.0)
+        x2 = x[:1 << 20].reshape(1 << 10, 1 << 10)
+        assert bits_equal(np.sqrt(dr.array(x2)[::2, 1::3]).get(), np.sqrt(x2[::2, 1::3]))
+
+
 @pytest.mark.parametrize("name", ["erf", "exp", "log"])
 def test_float32_functions_over_the_bit_patterns(name):
     """The device's own float32 `erf`, `exp`, `log` (hardware 2^x and log2 inside) against

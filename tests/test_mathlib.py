@@ -137,15 +137,33 @@ def test_exp_accuracy_and_limits(host):
     assert got[4] == np.inf and got[5] == 0 and got[6] == 0 and got[7] == 1.0
 
 
+def test_sqrt_is_correctly_rounded(host):
+    """The short square root against IEEE sqrt (NumPy's is the hardware instruction):
+    equal bits on random arguments over the whole exponent range, on arguments next to
+    perfect squares (where the rounding is decided by the last residual), and on the
+    arguments that take the compiler's own path."""
+    rs = np.random.RandomState(9)
+    m = rs.uniform(1, 4, 1 << 20)
+    exact = np.floor(rs.uniform(1, 2 ** 26, 1 << 16)) ** 2
+    x = np.concatenate([m, np.ldexp(m, rs.randint(-766, 1020, m.size)), exact, np.nextafter(exact, 0),
+                        np.nextafter(exact, np.inf), rs.uniform(0, 1e-300, 1 << 12),
+                        [0.0, -0.0, np.inf, 4.0, 2.0, 1e-320, 5e-324, 2.0 ** -767, np.nextafter(2.0 ** -767, 0),
+                         1.7976931348623157e308]])
+    got = host("sqrt", x)
+    assert got.tobytes() == np.sqrt(x).tobytes()
+    bad = host("sqrt", [-1.0, -np.inf, np.nan])
+    assert np.all(np.isnan(bad))
+
+
 def test_device_source_compiles():
     for lds in (False, True):
-        src = mathlib.source(["log", "erf", "exp"], lds=lds)
+        src = mathlib.source(["log", "erf", "exp", "sqrt"], lds=lds)
         assert src.count("DR_STEP(") >= 13 and src.count("void dr_expm1_reduced(") == 1
         assert ("__shared__ double dr_erf_tab_lds[960]" in src) == lds
         stage = "DR_STAGE_TABLES(); " if lds else ""
         kernel = ('extern "C" __global__ void k(const double* a, double* o)\n'
                   "{ " + stage + "int i = threadIdx.x; const double x[2] = {a[2 * i], a[2 * i + 1]}; double p[2], q[2], r[2];\n"
-                  "  dr_log_f8<2>(x, p); dr_erf_f8<2>(x, q); dr_exp_f8<2>(x, r);\n"
+                  "  dr_log_f8<2>(x, p); dr_erf_f8<2>(x, q); dr_exp_f8<2>(x, r); dr_sqrt_f8<2>(q, q);\n"
                   "  o[i] = p[0] + q[1] + r[0] + dr_log_f8_1(a[i]) + dr_erf_f8_1(a[i]) + dr_exp_f8_1(a[i]); }\n")
         assert len(hip.compile_source(src + kernel)) > 0
 
@@ -161,8 +179,8 @@ def test_packs_share_each_coefficient_between_their_elements():
     src = mathlib.source(["exp"]) + (
         'extern "C" __global__ void k(const double* a, double* o)\n'
         "{ const long i = 4L * (blockIdx.x * 256 + threadIdx.x);\n"
-        "  const double x[4] = {a[i], a[i + 1], a[i + 2], a[i + 3]}; double r[4];\n"
-        "  dr_exp_f8<4>(x, r); for (int e = 0; e < 4; e++) o[i + e] = r[e]; }\n")
+        "  const double x[4] = {a[i], a[i + 1], a[i + 2], a[i + 3]}; double r[4], k[4];\n"
+        "  dr_expm1_reduced<4>(x, r, k); for (int e = 0; e < 4; e++) o[i + e] = r[e] + k[e]; }\n")
     with tempfile.TemporaryDirectory() as d:
         with open(f"{d}/k.hip", "w") as fh:
             fh.write(src)
