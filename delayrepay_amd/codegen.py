@@ -1453,6 +1453,93 @@ def emit_short_rows(prog, leaf_kind, acc_dt, op, R):
     return "\n".join(src) + "\n"
 
 
+def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
+    """Reduction over a unit-stride last dimension of R elements (a compile-time
+    constant) by groups of G lanes (G a power of two, 8..64): a wave holds 64 / G rows at a
+    time, lane j of a group takes the 16-byte units j, j + G, ... of its row (a group reads
+    16 G contiguous bytes per step), and the group's lanes meet in log2 G butterfly steps.
+    A whole wave per row leaves lanes idle whenever a row is not a multiple of 256 elements
+    (200 floats: 22 % of the lanes, then six combining steps for one output); groups of
+    eight waste a tenth as many unit slots, combine in three steps and store eight adjacent
+    outputs per wave.
+
+    leaf_kind  per leaf 'v' (unit stride along the row) or 'k' (constant along it)
+    Parameters: leaf pointers, output pointer, scalars, K, then per leaf the stride
+    between rows (elements)."""
+    ct = CTYPE[acc_dt]
+    nl = len(prog.leaves)
+    widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "v"}
+    V = 16 // widths.pop() if len(widths) == 1 and widths <= {4, 8} else 1
+    units = -(-R // V)                     # 16-byte units per row, the last one maybe partial
+    steps = -(-units // G)
+    per_wave = WAVE // G
+    src = [PREAMBLE, emit_body(prog, [acc_dt])]
+    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
+    params.append(f"{ct}* __restrict__ out")
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params.append("const long long K")
+    params += [f"const long long sk{i}" for i in range(nl)]
+    call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
+    shfl = "__shfl_xor(acc, off, 64)"
+    if acc_dt in ("u1", "b1"):
+        shfl = f"({ct})__shfl_xor((int)acc, off, 64)"
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{",
+         f"    const int sub = threadIdx.x & {G - 1};",
+         f"    const int grp = (threadIdx.x & {WAVE - 1}) >> {G.bit_length() - 1};",
+         f"    const long long stride = (long long)gridDim.x * {BLOCK // WAVE * per_wave};",
+         f"    for (long long first = ((long long)blockIdx.x * {BLOCK // WAVE} + (threadIdx.x >> 6)) * "
+         f"{per_wave}; first < K; first += stride) {{",
+         "        const long long row = first + grp;",
+         "        const long long k = row < K ? row : K - 1;      // idle groups re-read the last row"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind == "v":
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+        else:
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+    L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
+
+    def element(args, pad):
+        return (f"{pad}{{ {ct} t0; dr_body({', '.join(args + call_tail)}); "
+                f"acc = {_combine(op, 'acc', 't0')}; }}")
+
+    full = R // V                          # units that are whole
+    for j in range(steps):
+        lo = j * G                         # this step covers units lo .. lo + G - 1
+        if lo + G <= full:
+            cond, pad = None, "        "
+        else:
+            cond, pad = f"        if ({lo} + sub < {full}) {{", "            "
+        if lo < full:
+            if cond:
+                L.append(cond)
+            for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+                if kind == "v":
+                    vt = (VEC16[dt][0] + "u") if V > 1 else CTYPE[dt]
+                    L.append(f"{pad}const {vt} X{j}_{i} = *(const {vt}*)(row{i} + ({lo} + sub) * {V});")
+            for e in range(V):
+                L.append(element([(f"X{j}_{i}[{e}]" if V > 1 else f"X{j}_{i}") if kind == "v" else f"c{i}"
+                                  for i, kind in enumerate(leaf_kind)], pad))
+            if cond:
+                L.append("        }")
+        if full * V < R and lo <= full < lo + G:
+            # the partial unit at the end of the row: its lane takes the elements one by one
+            L.append(f"        if (sub == {full - lo}) {{")
+            for r in range(full * V, R):
+                L.append(element([f"row{i}[{r}]" if kind == "v" else f"c{i}"
+                                  for i, kind in enumerate(leaf_kind)], "            "))
+            L.append("        }")
+    L += ["#pragma unroll",
+          f"        for (int off = {G // 2}; off > 0; off >>= 1) {{",
+          f"            const {ct} other = {shfl};",
+          f"            acc = {_combine(op, 'acc', 'other')};",
+          "        }",
+          "        if (sub == 0 && row < K) out[row] = acc;",
+          "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"
+
+
 # ---- 2-D kernel with transposed operands ------------------------------------------
 
 T_TILE = 64      # square tile edge: both the transposed read and the write coalesce

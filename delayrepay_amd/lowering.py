@@ -25,7 +25,10 @@ TUNE = {
     "ax_waves": 32768,   # aim for before the reduced extent is cut into slices
     "ax_rows": 4,        # 'row' strategy: outputs per wave (grid-stride), to amortise set-up
     "ax_narrow": 64,     # kept unit-stride extents up to this many columns: stream the matrix
-    "ax_short": 192,     # reduced unit-stride extents up to this length: a lane per output
+    "ax_short": 28,      # reduced unit-stride extents up to this length: a lane per output
+    "ax_group": 2048,    # ... and up to this length: a group of 8 to 64 lanes per output
+    "ax_group_lanes": 0,  # force the group size (0: the one that wastes the fewest unit slots)
+    "ax_group_steps": 8,  # most 16-byte units a lane of such a group takes from its row
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
     "nts": 1,         # allow non-temporal stores }
@@ -603,6 +606,39 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
         low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
         low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets]
         return low, 1, K, "short"
+    if (strategy == "row" and slices is None and TUNE["ax_short"] < R <= TUNE["ax_group"]
+            and K >= 1024 and len(kmerged) == 1 and len(rmerged) == 1 and TUNE["uvec"]
+            and all(r[0] in (0, 1) for r in rsets) and K < 2 ** 40):
+        widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == 1}
+        if len(widths) == 1 and widths <= {4, 8} and all(
+                c in cg.VEC16 for c, r in zip(prog.leaves, rsets) if r[0] == 1):
+            # rows of a few hundred elements: a group of lanes per row, sized to the row
+            V = 16 // next(iter(widths))
+            units = -(-R // V)
+            # measured (float32, 2^28 elements, % of 8 TB/s, groups of 8 / 16 lanes): rows of
+            # 32: 72 / 56, 100: 76 / 70, 128: 75 / 75, 200: 75 / 77, 250: 76 / 78, 1000: 75 / 76;
+            # a whole wave per row: 200: 55, 250: 50, 333: 52; a lane per row: 32: 71, 100: 50
+            G = 8 if units <= 32 else 16
+            while -(-units // G) > TUNE["ax_group_steps"] and G < cg.WAVE:
+                G *= 2
+            G = TUNE["ax_group_lanes"] or G
+            kinds = tuple("v" if r[0] == 1 else "k" for r in rsets)
+            low = Lowered()
+            low.lds = 0
+            low.fin_count = 0
+            low.kind = "axis_group"
+            low.key = ("axis_group", prog.key(), kinds, acc, reduce_op, R, G)
+
+            def emit_group():
+                return cg.emit_group_rows(prog, kinds, acc, reduce_op, R, G)
+            low.emit = emit_group
+            rows_per_block = (cg.BLOCK // cg.WAVE) * (cg.WAVE // G)
+            low.grid = max(1, min(-(-K // rows_per_block // TUNE["ax_rows"]), 1 << 20))
+            low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+                       + "q" + "q" * len(leaves))
+            low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+            low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets]
+            return low, 1, K, "group"
     # enough independent pieces to fill the device: cut the reduced extent into slices
     if slices is not None:
         S = slices

@@ -147,7 +147,8 @@ def test_fuzz_reached_every_kernel_shape():
     for key in hip._KERNELS:
         kinds[key[0]] = kinds.get(key[0], 0) + 1
     print("kernel kinds compiled:", kinds)
-    for kind in ("flat", "nd", "tile2d", "tile2dv", "tile2dt", "axis", "axis_short", "axis_narrow"):
+    for kind in ("flat", "nd", "tile2d", "tile2dv", "tile2dt", "axis", "axis_short", "axis_narrow",
+                 "axis_group"):
         assert kinds.get(kind, 0) > 0, kind
 
 

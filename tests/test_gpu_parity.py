@@ -857,7 +857,10 @@ def test_reductions_over_short_rows():
         h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
         a = dr.array(h)
         low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
-        assert low.kind == "axis_short" and low.key[-1] == shape[1]
+        if shape[1] <= 28:
+            assert low.kind == "axis_short" and low.key[-1] == shape[1]
+        else:
+            assert low.kind == "axis_group" and low.key[-2:] == (shape[1], 8)
         tol = dict(rtol=1e-5, atol=1e-5) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
         assert np.allclose(dr.sum(a * a, axis=1).get(), (h * h).sum(axis=1), **tol)
         assert dr.sum(a * a, axis=1).get().dtype == (h * h).sum(axis=1).dtype
@@ -879,7 +882,42 @@ def test_reductions_over_short_rows():
     try:
         assert np.allclose(dr.sum(a * W + V, axis=1).get(), (h * w + v).sum(axis=1), rtol=1e-5, atol=1e-5)
     finally:
-        hip.set_tune(ax_short=192)
+        hip.set_tune(ax_short=28)
+
+
+def test_reductions_over_rows_of_a_few_hundred_elements():
+    """Rows too long for a lane and too short for a wave: a group of lanes per row
+    (8 lanes up to 32 16-byte units per row, 16 beyond, more when a lane would otherwise
+    take more than 8 units), the row length compiled in."""
+    rs = np.random.RandomState(23)
+    cases = [((9000, 100), np.float32, 8), ((6001, 200), np.float32, 16), ((4100, 250), np.float32, 16),
+             ((3000, 333), np.float64, 32), ((2500, 257), np.int32, 16), ((1500, 1000), np.float32, 32),
+             ((1100, 2048), np.float32, 64), ((2000, 131), np.float64, 16), ((1024, 29), np.float32, 8)]
+    for shape, dt, lanes in cases:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
+        assert low.kind == "axis_group" and low.key[-2:] == (shape[1], lanes), (shape, low.key[-2:])
+        tol = dict(rtol=2e-5, atol=1e-4) if dt == np.float32 else dict(rtol=1e-12, atol=1e-12)
+        assert np.allclose(dr.sum(a * a, axis=1).get(), (h * h).sum(axis=1), **tol), shape
+        assert dr.sum(a * a, axis=1).get().dtype == (h * h).sum(axis=1).dtype
+        assert np.array_equal(dr.max(a, axis=1).get(), h.max(axis=1))
+        assert np.array_equal(dr.min(a, axis=-1).get(), h.min(axis=-1))
+    # operands constant along the row, one row for all, rows with a pitch, a misaligned start
+    h = rs.uniform(-1, 1, (5000, 210)).astype(np.float32)
+    w, v = rs.uniform(0, 1, (5000, 1)).astype(np.float32), rs.uniform(0, 1, 210).astype(np.float32)
+    a, W, V = dr.array(h), dr.array(w), dr.array(v)
+    assert np.allclose(dr.sum(a * W + V, axis=1).get(), (h * w + v).sum(axis=1), rtol=2e-5, atol=1e-4)
+    part = ReduceEx(np.add, a[:, 3:204] * 2.0, (1,))
+    assert hip.lower_only(part)[0].kind == "axis_group"
+    assert np.allclose(dr.sum(a[:, 3:204] * 2.0, axis=1).get(), (h[:, 3:204] * 2.0).sum(axis=1), rtol=2e-5,
+                       atol=1e-4)
+    assert np.array_equal(dr.max(a[1:4999:3, 5:205], axis=1).get(), h[1:4999:3, 5:205].max(axis=1))
+    hip.set_tune(ax_group=0)                      # the wave-per-row kernel gives the same numbers
+    try:
+        assert np.allclose(dr.sum(a * W + V, axis=1).get(), (h * w + v).sum(axis=1), rtol=2e-5, atol=1e-4)
+    finally:
+        hip.set_tune(ax_group=2048)
 
 
 def test_reductions_over_the_rows_of_narrow_matrices():
@@ -985,16 +1023,29 @@ def test_slices_of_generated_grids_stay_generated():
     assert _same((a * 3)[::-1][:10].get(), (np.arange(100000) * 3)[::-1][:10])
 
 
-def test_row_reductions_with_vector_loads_and_ragged_ends():
-    """A wave per row, 16-byte loads at element alignment; the row length need not be a
-    multiple of the vector, nor the row start aligned."""
+@pytest.mark.parametrize("groups", [True, False])
+def test_row_reductions_with_vector_loads_and_ragged_ends(groups):
+    """A wave per row (fewer than 1024 rows, or rows beyond 2048 elements) or a group of lanes
+    per row, 16-byte loads at element alignment; the row length need not be a multiple of
+    the vector, nor the row start aligned."""
     rs = np.random.RandomState(23)
+    hip.set_tune(ax_group=2048 if groups else 0)
+    try:
+        _row_reduction_cases(rs, groups)
+    finally:
+        hip.set_tune(ax_group=2048)
+
+
+def _row_reduction_cases(rs, groups):
     for shape, dt in [((3000, 200), np.float32), ((2000, 257), np.float64), ((1500, 515), np.float32),
                       ((700, 230), np.int32)]:
         h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
         a = dr.array(h)
         low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
-        assert low.kind == "axis_row" and low.key[-1] == ("v",)
+        if groups and shape[0] >= 1024:
+            assert low.kind == "axis_group"
+        else:
+            assert low.kind == "axis_row" and low.key[-1] == ("v",)
         tol = dict(rtol=2e-5, atol=1e-5) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
         assert np.allclose(dr.sum(a * a, axis=1).get(), (h.astype(np.float64) ** 2).sum(axis=1), **tol)
         assert np.array_equal(dr.max(a, axis=1).get(), h.max(axis=1))
@@ -1014,7 +1065,7 @@ def test_reduction_strategy_follows_the_operands_that_carry_the_traffic():
     assert hip.lower_only(ReduceEx(np.add, a * W, (0,)))[0].kind == "axis_col"
     assert np.allclose(dr.sum(a * W, axis=0).get(), (h * w).sum(axis=0), rtol=1e-13)
     r = rs.uniform(0, 1, (1, 500))
-    assert hip.lower_only(ReduceEx(np.add, a * dr.array(r), (1,)))[0].kind == "axis_row"
+    assert hip.lower_only(ReduceEx(np.add, a * dr.array(r), (1,)))[0].kind in ("axis_row", "axis_group")
     assert np.allclose(dr.sum(a * dr.array(r), axis=1).get(), (h * r).sum(axis=1), rtol=1e-13)
 
 
