@@ -1023,8 +1023,8 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
     return "\n".join(src) + "\n", TW, TH, lds_bytes
 
 
-def emit_stencil3d(prog, leaf_kind, group, out_dtypes, groups_per_row, planes, phase_group,
-                   phase_out, restrict=True, nt_store=True, xcd_bands=True):
+def emit_stencil3d(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_per_thread,
+                   phase_group, phase_out, restrict=True, nt_store=True, xcd_bands=True, depth=1):
     """Vectorised 3-D tiled kernel: operands that are shifted views of one buffer are
     staged through an LDS window of the buffer, like `emit_stencil_vec` does in two
     dimensions.  Without it a 7-point stencil fetches six vectors per four outputs
@@ -1036,29 +1036,49 @@ def emit_stencil3d(prog, leaf_kind, group, out_dtypes, groups_per_row, planes, p
                the last dimension; ('b',) single element broadcast
     group      (dtype code, dz_max, dy_min, dy_max, dx_min, dx_max): dz in [0, dz_max]
 
-    A block owns TW = groups_per_row * VW columns, TY = 256 / groups_per_row rows and
-    `planes` planes; a thread computes VW adjacent outputs in each plane of its row, so
-    the values it reads from the planes above and below are shared between its
-    outputs.  Alignment works as in the 2-D kernel: tiles start `phase_out` columns
-    left of the view, the first and last column group of a row take element stores.
+    A block owns TW = groups_per_row * VW columns and TY = rows_per_thread * 256 /
+    groups_per_row rows, and walks ZC planes (a launch parameter) with a ring of window
+    planes in LDS: every plane of the buffer is fetched once per block instead of once
+    per plane that uses it (a window of 4 + 2 planes re-reads half the volume).  The
+    ring holds dz_max + 2 planes rounded up to a power of two: a plane goes from registers
+    to the ring slot of the plane that was retired one step earlier, so one barrier per
+    plane is enough.  The next `depth` planes are in flight in registers meanwhile (the
+    loop over planes is unrolled `depth` times, each copy with its own registers).
+    A thread computes VW adjacent outputs in each of its rows; the body runs once per
+    output, also in the first and last column group of a row, where only the loads of
+    directly read operands and the stores are done element by element.
+    Measured on 512^3 float32 (7-point, microseconds per sweep): 4 planes x 16 rows x 64
+    columns without the ring 262; ring with tiles of 32 x 64: 235, 8 x 256: 211 (depth 1;
+    2 and 3 planes in flight: 218, 223).  What bounds it is the number of cache lines a
+    compute unit requests per line it stores, not the bytes from HBM (1.08 x algorithmic):
+    a tile of 8 x 256 asks for 10 rows x 10 lines and stores 64, a copy asks for 64 and
+    stores 64; 164 / 128 of the copy kernel's time is what the 8 x 256 tile takes, and
+    the other shapes follow the same ratio.  Alignment works
+    as in the 2-D kernel: tiles start `phase_out` columns left of the view, the first
+    and last column group of a row take element stores.
     Parameters: directly read leaves, group pointer, outputs, scalars, Z, Y, W, group
-    plane and row stride, [glo, ghi) element range of the buffer relative to the group
-    pointer, tiles_x, tiles_y, then plane and row stride of every directly read leaf and
-    of every output."""
+    plane and row stride, first and last 16-byte aligned vector of the buffer (glo, ghi;
+    in elements relative to the group pointer), tiles_x, tiles_y, ZC, then plane and row stride of every directly read leaf
+    and of every output."""
     rs = "__restrict__ " if restrict else ""
     gdt, dz_max, dy_min, dy_max, dx_min, dx_max = group
     vt, VW = VEC16[gdt]
     ct = CTYPE[gdt]
     n_out = len(out_dtypes)
     GPR = groups_per_row
-    TY = BLOCK // GPR
-    TZ = planes
+    RY = BLOCK // GPR
+    RPT = rows_per_thread
+    TY = RY * RPT
     TW = GPR * VW
     ph = (phase_group - phase_out + dx_min) % VW
     LW = -(-(TW + dx_max - dx_min + ph) // VW) * VW
     LWV = LW // VW
     WY = TY + dy_max - dy_min
-    WZ = TZ + dz_max
+    PV = WY * LWV                     # 16-byte vectors per window plane
+    NV = -(-PV // BLOCK)              # of them per thread
+    NS = 2
+    while NS < dz_max + 2:
+        NS *= 2
     src = [PREAMBLE, emit_body(prog, out_dtypes)]
     params = [f"const {CTYPE[dt]}* {rs}a{i}" for i, dt in enumerate(prog.leaves)
               if leaf_kind[i][0] != "g"]
@@ -1067,15 +1087,35 @@ def emit_stencil3d(prog, leaf_kind, group, out_dtypes, groups_per_row, planes, p
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += ["const int Z", "const int Y", "const int W", "const long long gps",
                "const long long grs", "const long long glo", "const long long ghi",
-               "const int tiles_x", "const int tiles_y"]
+               "const int tiles_x", "const int tiles_y", "const int ZC"]
     for i, k in enumerate(leaf_kind):
         if k[0] in ("d", "dv", "r"):
             params += [f"const long long os{i}_0", f"const long long os{i}_1"]
     for o in range(n_out):
         params += [f"const long long oos{o}_0", f"const long long oos{o}_1"]
+
+    def fetch(plane, ind, cur="cur0"):
+        """`cur` <- this thread's vectors of buffer plane `plane`.  A vector that is not
+        wholly inside the buffer is read from the nearest aligned place that is: only
+        outputs outside the view would use its values, and those are not stored.  No branch
+        surrounds the loads, so the compiler counts outstanding loads exactly instead of
+        waiting for all of them at every join.  For the same reason the planes past the
+        last one the block needs are fetched too (as that last plane again, from L2)."""
+        return [ind + "#pragma unroll",
+                ind + f"for (int q = 0; q < {NV}; ++q) {{",
+                ind + f"    const long long lin = wlin[q] + (long long)min({plane}, zlast) * gps;",
+                ind + f"    {cur}[q] = *(const {vt}*)(gp + min(max(lin, glo), ghi));",
+                ind + "}"]
+
+    def stash(slot, ind, cur="cur0"):
+        return [ind + "#pragma unroll",
+                ind + f"for (int q = 0; q < {NV}; ++q)",
+                ind + f"    if (threadIdx.x + q * {BLOCK} < {PV}) "
+                      f"tile[({slot}) * {PV} + threadIdx.x + q * {BLOCK}] = {cur}[q];"]
+
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{",
-         f"    __shared__ {vt} tile[{WZ * WY * LWV}];",
+         f"    __shared__ {vt} tile[{NS * PV}];",
          "    const int nb = gridDim.x;",
          f"    const int xcd = blockIdx.x % {N_XCD};",
          f"    const int slot = blockIdx.x / {N_XCD};",
@@ -1085,82 +1125,106 @@ def emit_stencil3d(prog, leaf_kind, group, out_dtypes, groups_per_row, planes, p
          "    const int tx = t - tyz * tiles_x;",
          "    const int tz = tyz / tiles_y;",
          "    const int ty = tyz - tz * tiles_y;",
-         f"    const int z0 = tz * {TZ};",
+         "    const int z0 = tz * ZC;",
+         "    const int nk = min(ZC, Z - z0);",
+         f"    const int zlast = z0 + nk - 1 + {dz_max};      // last plane of the buffer the block needs",
          f"    const int y0 = ty * {TY};",
          f"    const int j0 = tx * {TW} - {phase_out};      // first output column of the tile",
          f"    const int cs = j0 + ({dx_min}) - {ph};       // buffer column held in LDS column 0",
-         f"    for (int idx = threadIdx.x; idx < {WZ * WY * LWV}; idx += {BLOCK}) {{",
-         f"        const int wr = idx / {LWV};",
-         f"        const int lv = idx - wr * {LWV};",
-         f"        const int wz = wr / {WY};",
-         f"        const int wy = wr - wz * {WY};",
-         f"        const long long lin = (long long)(z0 + wz) * gps + (long long)(y0 + wy + ({dy_min})) * grs "
-         f"+ cs + lv * {VW};",
-         f"        {vt} val;",
-         f"        if (lin >= glo && lin + {VW} <= ghi) {{",
-         f"            val = *(const {vt}*)(gp + lin);",
-         "        } else {",
+         f"    long long wlin[{NV}];                         // this thread's window vectors in a plane",
          "#pragma unroll",
-         f"            for (int e = 0; e < {VW}; ++e)",
-         f"                val[e] = (lin + e >= glo && lin + e < ghi) ? gp[lin + e] : ({ct})0;",
-         "        }",
-         "        tile[idx] = val;",
+         f"    for (int q = 0; q < {NV}; ++q) {{",
+         f"        const int idx = threadIdx.x + q * {BLOCK};",
+         f"        const int wy = idx / {LWV};",
+         f"        const int lv = idx - wy * {LWV};",
+         f"        wlin[q] = (long long)(y0 + wy + ({dy_min})) * grs + cs + lv * {VW};",
          "    }",
-         "    __syncthreads();",
-         f"    const {ct}* ts = (const {ct}*)tile;",
-         f"    const int g = threadIdx.x % {GPR};",
-         f"    const int ly = threadIdx.x / {GPR};",
-         "    const int y = y0 + ly;",
-         f"    const int jf = j0 + g * {VW};                // first of this thread's {VW} columns",
-         f"    const bool inner = jf >= 0 && jf + {VW} <= W;",
-         "    if (y >= Y) return;",
-         "#pragma unroll",
-         f"    for (int k = 0; k < {TZ}; ++k) {{",
-         "        const int z = z0 + k;",
-         "        if (z >= Z) break;"]
-    for i, kd in enumerate(leaf_kind):
-        if kd[0] in ("d", "dv", "r"):
-            L.append(f"        const long long base{i} = (long long)z * os{i}_0 + (long long)y * os{i}_1;")
-    for o in range(n_out):
-        L.append(f"        const long long obase{o} = (long long)z * oos{o}_0 + (long long)y * oos{o}_1;")
+         "    " + " ".join(f"{vt} cur{u}[{NV}];" for u in range(depth)),
+         f"    for (int p = 0; p < {dz_max}; ++p) {{"]
+    L += fetch("z0 + p", "        ") + stash("p", "        ") + ["    }"]
+    for u in range(depth):
+        L += fetch(f"z0 + {dz_max + u}", "    ", f"cur{u}")
+    L += [f"    const {ct}* ts = (const {ct}*)tile;",
+          f"    const int g = threadIdx.x % {GPR};",
+          f"    const int ly = threadIdx.x / {GPR};",
+          f"    const int jf = j0 + g * {VW};                // first of this thread's {VW} columns",
+          f"    const bool inner = jf >= 0 && jf + {VW} <= W;",
+          f"    for (int k0 = 0; k0 < nk; k0 += {depth}) {{"]
+    decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+    tail_args = [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
 
-    def operand(i, kd, e, vector_path):
+    def operand(i, kd, e):
         if kd[0] == "g":
             _, dz, dy, dx = kd
-            return (f"ts[((k + {dz}) * {WY} + ly + {dy - dy_min}) * {LW} + g * {VW} + "
+            return (f"ts[sl{dz} + (lyr + {dy - dy_min}) * {LW} + g * {VW} + "
                     f"{e + dx - dx_min + ph}]")
-        if kd[0] == "dv" and vector_path:
-            return f"D{i}[{e}]"
         if kd[0] in ("d", "dv"):
-            return f"a{i}[base{i} + jf + {e}]"
+            return f"D{i}[{e}]"
         if kd[0] == "r":
             return f"a{i}[base{i}]"
         return f"a{i}[0]"
 
-    decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
-    tail_args = [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
-    L.append("        if (inner) {")
-    for i, kd in enumerate(leaf_kind):
-        if kd[0] == "dv":
-            lvt = VEC16[prog.leaves[i]][0]
-            L.append(f"            const {lvt} D{i} = *(const {lvt}*)(a{i} + base{i} + jf);")
-    for o, dt in enumerate(out_dtypes):
-        L.append(f"            {VEC16[dt][0]} R{o};")
-    for e in range(VW):
-        args = [operand(i, kd, e, True) for i, kd in enumerate(leaf_kind)]
-        sets = " ".join(f"R{o}[{e}] = t{o};" for o in range(n_out))
-        L.append(f"            {{ {decl} dr_body({', '.join(args + tail_args)}); {sets} }}")
-    for o, dt in enumerate(out_dtypes):
-        L.append("            " + _st(nt_store, f"R{o}", f"({VEC16[dt][0]}*)(o{o} + obase{o} + jf)"))
-    L.append("        } else {")
-    for e in range(VW):
-        args = [operand(i, kd, e, False) for i, kd in enumerate(leaf_kind)]
-        stores = " ".join(f"o{o}[obase{o} + jf + {e}] = t{o};" for o in range(n_out))
-        L.append(f"            if (jf + {e} >= 0 && jf + {e} < W) "
-                 f"{{ {decl} dr_body({', '.join(args + tail_args)}); {stores} }}")
-    L += ["        }", "    }", "}"]
+    for u in range(depth):
+        L += ["        {",
+              f"        const int k = k0 + {u};",
+              "        if (k >= nk) break;"]
+        L += stash(f"(k + {dz_max}) & {NS - 1}", "        ", f"cur{u}")
+        L += ["        __syncthreads();"]
+        L += fetch(f"z0 + k + {depth + dz_max}", "        ", f"cur{u}")
+        L += ["        const int z = z0 + k;"]
+        for dz in sorted({kd[1] for kd in leaf_kind if kd[0] == "g"}):
+            L.append(f"        const int sl{dz} = ((k + {dz}) & {NS - 1}) * {PV * VW};")
+        L += ["#pragma unroll",
+              f"        for (int r = 0; r < {RPT}; ++r) {{",
+              f"            const int lyr = ly + r * {RY};",
+              "            const int y = y0 + lyr;",
+              "            if (y >= Y) break;"]
+        for i, kd in enumerate(leaf_kind):
+            if kd[0] in ("d", "dv", "r"):
+                L.append(f"            const long long base{i} = (long long)z * os{i}_0 + (long long)y * os{i}_1;")
+        for o in range(n_out):
+            L.append(f"            const long long obase{o} = (long long)z * oos{o}_0 + (long long)y * oos{o}_1;")
+        # operands read directly: whole vectors where the thread's columns are all inside
+        # the view, single elements (0 outside) in the first and last column group of a row
+        for i, kd in enumerate(leaf_kind):
+            if kd[0] in ("d", "dv"):
+                lct = CTYPE[prog.leaves[i]]
+                L.append(f"            {lct} D{i}[{VW}];")
+        direct = [i for i, kd in enumerate(leaf_kind) if kd[0] in ("d", "dv")]
+        if direct:
+            L.append("            if (inner) {")
+            for i in direct:
+                if leaf_kind[i][0] == "dv":
+                    lvt = VEC16[prog.leaves[i]][0]
+                    L.append(f"                const {lvt} V{i} = *(const {lvt}*)(a{i} + base{i} + jf);")
+                    L.append(f"                " + " ".join(f"D{i}[{e}] = V{i}[{e}];" for e in range(VW)))
+                else:
+                    L.append(f"                " + " ".join(f"D{i}[{e}] = a{i}[base{i} + jf + {e}];"
+                                                             for e in range(VW)))
+            L.append("            } else {")
+            for i in direct:
+                lct = CTYPE[prog.leaves[i]]
+                for e in range(VW):
+                    L.append(f"                D{i}[{e}] = (jf + {e} >= 0 && jf + {e} < W) "
+                             f"? a{i}[base{i} + jf + {e}] : ({lct})0;")
+            L.append("            }")
+        for o, dt in enumerate(out_dtypes):
+            L.append(f"            {VEC16[dt][0]} R{o};")
+        for e in range(VW):
+            args = [operand(i, kd, e) for i, kd in enumerate(leaf_kind)]
+            sets = " ".join(f"R{o}[{e}] = t{o};" for o in range(n_out))
+            L.append(f"            {{ {decl} dr_body({', '.join(args + tail_args)}); {sets} }}")
+        L.append("            if (inner) {")
+        for o, dt in enumerate(out_dtypes):
+            L.append("                " + _st(nt_store, f"R{o}", f"({VEC16[dt][0]}*)(o{o} + obase{o} + jf)"))
+        L.append("            } else {")
+        for e in range(VW):
+            stores = " ".join(f"o{o}[obase{o} + jf + {e}] = R{o}[{e}];" for o in range(n_out))
+            L.append(f"                if (jf + {e} >= 0 && jf + {e} < W) {{ {stores} }}")
+        L += ["            }", "        }", "        }"]
+    L += ["    }", "}"]
     src.append("\n".join(L))
-    return "\n".join(src) + "\n", TW, TY, TZ, WZ * WY * LW * ITEMSIZE[gdt]
+    return "\n".join(src) + "\n", TW, TY, NS, NS * PV * VW * ITEMSIZE[gdt]
 
 
 # ---- reduction along some axes ------------------------------------------------

@@ -45,8 +45,10 @@ TUNE = {
     "sntl": 0,        # vectorised stencil: non-temporal loads / stores
     "snts": 1,
     "s3": 1,          # 3-D shifted views of one buffer: LDS window (0: read every view directly)
-    "s3_gpr": 16,     # 3-D window: 16-byte column groups per tile row (tile rows = 256 / s3_gpr)
-    "s3_tz": 4,       # 3-D window: planes per tile
+    "s3_gpr": 64,     # 3-D window: 16-byte column groups per tile row (tile rows = 256 / s3_gpr)
+    "s3_rpt": 2,      # 3-D window: tile rows per thread (tile rows = s3_rpt * 256 / s3_gpr)
+    "s3_zc": 0,       # 3-D window: planes a block walks; 0 = fewest rounds of resident blocks
+    "s3_depth": 1,    # 3-D window: planes in flight in registers
     "uvec": 1,        # 16-byte accesses at element alignment where 16-byte alignment is missing
     "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
@@ -147,32 +149,44 @@ def _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_pt
                and pz % vw == 0 and py % vw == 0)
     if not aligned:
         return None
-    ref_off = min(leaves[i].offset for i in best)
-    shifts = {}
-    for i in best:
-        d = leaves[i].offset - ref_off
-        dz, r = divmod(d, pz)
-        if r > pz // 2:
-            dz, r = dz + 1, r - pz
-        dy, dx = divmod(r, py)
-        if dx > py // 2:
-            dy, dx = dy + 1, dx - py
-        if dz * pz + dy * py + dx != d:
-            return None
-        shifts[i] = (dz, dy, dx)
+    def shifts_of(members):
+        ref = min(leaves[i].offset for i in members)
+        out = {}
+        for i in members:
+            d = leaves[i].offset - ref
+            dz, r = divmod(d, pz)
+            if r > pz // 2:
+                dz, r = dz + 1, r - pz
+            dy, dx = divmod(r, py)
+            if dx > py // 2:
+                dy, dx = dy + 1, dx - py
+            if dz * pz + dy * py + dx != d:
+                return ref, None
+            out[i] = (dz, dy, dx)
+        return ref, out
+
+    ref_off, shifts = shifts_of(best)
+    if shifts is None:
+        return None
     dz_max = max(v[0] for v in shifts.values())
     dy_min, dy_max = min(v[1] for v in shifts.values()), max(v[1] for v in shifts.values())
     dx_min, dx_max = min(v[2] for v in shifts.values()), max(v[2] for v in shifts.values())
     if min(v[0] for v in shifts.values()) < 0 or dz_max > 4 or dy_max - dy_min > 8 \
             or dx_max - dx_min > 16:
         return None
-    gpr, tz = TUNE["s3_gpr"], TUNE["s3_tz"]
-    ty = cg.BLOCK // gpr
+    gpr, rpt, zc, depth = TUNE["s3_gpr"], TUNE["s3_rpt"], TUNE["s3_zc"], TUNE["s3_depth"]
+    ty = cg.BLOCK // gpr * rpt
     Z, Y, W = mshape
     g_buf = leaves[best[0]].buf
     g_ptr = g_buf.ptr + ref_off * gsize
     ph_o = (out_ptrs[0] // gsize) % vw
     ph_g = (g_ptr // gsize) % vw
+    # first and last aligned 16-byte vector inside the buffer, relative to the group pointer
+    v_lo = -ref_off + (ref_off - ph_g) % vw
+    v_hi = g_buf.nbytes // gsize - ref_off - vw
+    v_hi -= (v_hi + ph_g) % vw
+    if v_hi < v_lo:
+        return None
     kinds = []
     for i, st in enumerate(m_leaf):
         if i in shifts:
@@ -187,26 +201,40 @@ def _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_pt
             kinds.append(("r",))
     kinds = tuple(kinds)
     group = (gcode, dz_max, dy_min, dy_max, dx_min, dx_max)
-    lds_bytes = cg.emit_stencil3d(prog, kinds, group, out_codes, gpr, tz, ph_g, ph_o)[4]
+    lds_bytes = cg.emit_stencil3d(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o)[4]
     tiles_x = -(-(W + ph_o) // (gpr * vw))
-    tiles_y, tiles_z = -(-Y // ty), -(-Z // tz)
+    tiles_y = -(-Y // ty)
+    if zc <= 0:
+        # Blocks walk their planes in step, so what counts is how many rounds of resident
+        # blocks the grid takes and how long a round is: planes walked plus the planes
+        # fetched before the first output.
+        slots = grid_cap() // TUNE["bpc"] * max(1, min(8, (160 * 1024) // max(lds_bytes, 1)))
+        best = None
+        for chunks in range(1, max(1, Z // 8) + 1):
+            c = -(-Z // chunks)
+            rounds = -(-(tiles_x * tiles_y * -(-Z // c)) // slots)
+            cost = rounds * (c + dz_max + 2)
+            if best is None or cost < best[0]:
+                best = (cost, c)
+        zc = best[1]
+    tiles_z = -(-Z // zc)
     if lds_bytes > 64 * 1024 or tiles_x * tiles_y * tiles_z >= 2 ** 31 or max(Z, Y, W) >= 2 ** 31 - 4096:
         return None
     snts = bool(TUNE["snts"])
     bands = TUNE["xcd"] != 0
     low.kind = "tile3d"
-    low.key = ("tile3d", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o, gpr, tz,
-               snts, bands)
+    low.key = ("tile3d", prog.key(), kinds, group, tuple(out_codes), in_place, ph_g, ph_o, gpr, rpt,
+               snts, bands, depth)
 
     def emit():
-        return cg.emit_stencil3d(prog, kinds, group, out_codes, gpr, tz, ph_g, ph_o,
-                                 restrict=not in_place, nt_store=snts, xcd_bands=bands)[0]
+        return cg.emit_stencil3d(prog, kinds, group, out_codes, gpr, rpt, ph_g, ph_o,
+                                 restrict=not in_place, nt_store=snts, xcd_bands=bands, depth=depth)[0]
     low.emit = emit
     low.grid = tiles_x * tiles_y * tiles_z
     srcs = [(a.buf, a.offset * a.dtype.itemsize) for a, k in zip(leaves, kinds) if k[0] != "g"]
     srcs.append((g_buf, ref_off * gsize))
-    fmt = "@" + "P" * (len(srcs) + len(out_ptrs)) + scal_fmt + "iii" + "qqqq" + "ii"
-    tail = [Z, Y, W, pz, py, -ref_off, g_buf.nbytes // gsize - ref_off, tiles_x, tiles_y]
+    fmt = "@" + "P" * (len(srcs) + len(out_ptrs)) + scal_fmt + "iii" + "qqqq" + "iii"
+    tail = [Z, Y, W, pz, py, v_lo, v_hi, tiles_x, tiles_y, zc]
     for k, st in zip(kinds, m_leaf):
         if k[0] in ("d", "dv", "r"):
             fmt += "qq"
