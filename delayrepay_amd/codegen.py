@@ -940,6 +940,9 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
         params += ["const long long grs", "const long long glo", "const long long ghi"]
     params.append("const int tiles_x")
     params += _outer_params(leaf_kind, n_out, nouter)
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "dv":       # elements of the operand's buffer before and from its pointer
+            params += [f"const long long lo{i}", f"const long long hi{i}"]
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{"]
     if group is not None:
@@ -982,41 +985,57 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
           "        if (i >= H) break;"]
     L += _row_bases(nouter, _base_names(leaf_kind, n_out), 8)
 
-    def operand(i, k, e, vector_path):
+    def operand(i, k, e):
         if k[0] == "g":
             _, dy, dx = k
             return f"ts[(lr + {dy}) * {LW} + g * {VW} + {e + dx - dx_min + ph}]"
-        if k[0] == "dv" and vector_path:
-            return f"D{i}[{e}]"
         if k[0] in ("d", "dv"):
-            return f"a{i}[base{i} + jf + {e}]"
+            return f"D{i}[{e}]"
         if k[0] == "r":
             return f"a{i}[base{i}]"
         return f"a{i}[0]"
 
     decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
     tail_args = [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
-    L.append("        if (inner) {")
+    # Directly read operands.  The first and last column group of a row hold columns outside
+    # the view: their vectors are loaded whole where the operand's buffer reaches that far
+    # (an interior view: always), element by element otherwise; the body then runs once per
+    # output and only the stores are masked.  Evaluating such groups element by element,
+    # loads included, cost every wave of a short row eight more memory instructions.
     for i, k in enumerate(leaf_kind):
         if k[0] == "dv":
             lvt = VEC16[prog.leaves[i]][0] + ("u" if unaligned else "")
             ptr = f"(const {lvt}*)(a{i} + base{i} + jf)"
-            L.append(f"            const {lvt} D{i} = {_ld(nt_load, ptr)};")
+            L += [f"        {VEC16[prog.leaves[i]][0]} D{i};",
+                  f"        if (inner || (base{i} + jf >= lo{i} && base{i} + jf + {VW} <= hi{i})) {{",
+                  f"            D{i} = {_ld(nt_load, ptr)};",
+                  "        } else {"]
+            L += [f"            D{i}[{e}] = (jf + {e} >= 0 && jf + {e} < W) ? a{i}[base{i} + jf + {e}] "
+                  f": ({CTYPE[prog.leaves[i]]})0;" for e in range(VW)]
+            L.append("        }")
+        elif k[0] == "d":
+            ct_i = CTYPE[prog.leaves[i]]
+            L.append(f"        {ct_i} D{i}[{VW}];")
+            L.append("        if (inner) {")
+            L.append("            " + " ".join(f"D{i}[{e}] = a{i}[base{i} + jf + {e}];" for e in range(VW)))
+            L.append("        } else {")
+            L += [f"            D{i}[{e}] = (jf + {e} >= 0 && jf + {e} < W) ? a{i}[base{i} + jf + {e}] "
+                  f": ({ct_i})0;" for e in range(VW)]
+            L.append("        }")
     for o, dt in enumerate(out_dtypes):
-        L.append(f"            {VEC16[dt][0]} R{o};")
+        L.append(f"        {VEC16[dt][0]} R{o};")
     for e in range(VW):
-        args = [operand(i, k, e, True) for i, k in enumerate(leaf_kind)]
+        args = [operand(i, k, e) for i, k in enumerate(leaf_kind)]
         sets = " ".join(f"R{o}[{e}] = t{o};" for o in range(n_out))
-        L.append(f"            {{ {decl} dr_body({', '.join(args + tail_args)}); {sets} }}")
+        L.append(f"        {{ {decl} dr_body({', '.join(args + tail_args)}); {sets} }}")
+    L.append("        if (inner) {")
     for o, dt in enumerate(out_dtypes):
         ovt = VEC16[dt][0] + ("u" if unaligned else "")
         L.append("            " + _st(nt_store, f"R{o}", f"({ovt}*)(o{o} + obase{o} + jf)"))
     L.append("        } else {")
     for e in range(VW):
-        args = [operand(i, k, e, False) for i, k in enumerate(leaf_kind)]
-        stores = " ".join(f"o{o}[obase{o} + jf + {e}] = t{o};" for o in range(n_out))
-        L.append(f"            if (jf + {e} >= 0 && jf + {e} < W) "
-                 f"{{ {decl} dr_body({', '.join(args + tail_args)}); {stores} }}")
+        stores = " ".join(f"o{o}[obase{o} + jf + {e}] = R{o}[{e}];" for o in range(n_out))
+        L.append(f"            if (jf + {e} >= 0 && jf + {e} < W) {{ {stores} }}")
     L += ["        }", "    }", "}"]
     src.append("\n".join(L))
     lds_bytes = LH * LW * ITEMSIZE[first] if group is not None else 0

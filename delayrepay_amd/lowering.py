@@ -40,6 +40,8 @@ TUNE = {
     "svec": 1,        # aligned stencils: 16-byte loads into LDS and 16-byte stores
     "gpr": 64,        # vectorised stencil: 16-byte column groups per tile row
     "rpt": 2,         # vectorised stencil: consecutive rows per thread
+    "row_gpr": 256,   # vector tiles without a halo group: most column groups per block (0: as
+                      # the stencil tiles)
     "xcd": 1,         # vector tiles: a contiguous band of tiles per XCD (1: with a halo group
                       # or unaligned rows, 2: always, 0: never)
     "sntl": 0,        # vectorised stencil: non-temporal loads / stores
@@ -407,6 +409,23 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             kinds = tuple(("dv",) if d else k for d, k in zip(dv, kinds))
             gpr, rpt = TUNE["gpr"], TUNE["rpt"]
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
+            streams = all(any(st[:-1]) for st, k in zip(m_leaf, kinds) if k[0] in ("d", "dv"))
+            if group is None and TUNE["row_gpr"] and streams:
+                # Nothing is shared between rows: a block takes one stretch of a row, as
+                # long as the row allows (up to 4 KB), like a chunk of a flat kernel, and
+                # the streams follow the flat kernels' cache policy.  An interior view of
+                # 16384^2 float32, percent of the HBM peak: tiles of 8 rows x 256 columns
+                # 66, with non-temporal loads 69, 2 rows x 512: 76, 1 row x 1024: 80
+                # (a flat copy: 81); more rows per thread are slower (4: 70).  An operand that
+                # repeats from row to row keeps the taller tile, whose rows share it in L1.
+                gpr = 16
+                while gpr < TUNE["row_gpr"] and gpr * vw < W + ph_o:
+                    gpr *= 2
+                rpt = 1
+                in_bytes = sum(a.nbytes for a, k in zip(leaves, kinds) if k[0] in ("d", "dv"))
+                out_bytes = sum(n * cg.ITEMSIZE[c] for c in out_codes)
+                snts = bool(TUNE["nts"]) and in_bytes + out_bytes > TUNE["cache_mib"] << 20
+                sntl = bool(TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
             # A band of consecutive tiles per XCD pays where neighbouring tiles meet in L2:
             # halo rows, or rows that do not start on 16-byte boundaries, whose first and
             # last cache lines are shared with the next tile (3-D inner slice: 66% vs 57%).
@@ -456,6 +475,10 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             for s in m_out:
                 fmt += "q" * nouter
                 tail_vals += list(s[:-1])
+            for a, k in zip(leaves, kinds):
+                if vec_ok and k[0] == "dv":
+                    fmt += "qq"
+                    tail_vals += [-a.offset, a.buf.nbytes // a.dtype.itemsize - a.offset]
             low.fmt = fmt
             low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
             return low

@@ -282,6 +282,29 @@ def test_strided_and_broadcast_operands_use_nd():
     assert hip.lower_only(NPArray(m[::2, ::3]) * 2.0)[0].kind == "nd"
 
 
+def test_views_without_shared_rows_stream_row_by_row():
+    """No halo group: a block takes one stretch of one row (up to 1024 float32), the streams
+    are non-temporal beyond the cache sizes, and the first and last column group of a row
+    load whole vectors where the operand's buffer allows."""
+    n = 16384
+    m = NPArray(hip.placeholder((n, n), np.float32))
+    low, src = hip.lower_only(m[1:-1, 1:-1] * 2.0)
+    assert low.kind == "tile2d" and low.key[0] == "tile2dv"
+    gpr, rpt, ntl, nts = low.key[8:12]
+    assert (gpr, rpt, ntl, nts) == (256, 1, True, True)
+    assert low.grid == 16 * (n - 2) and "lo0" in src and "__builtin_nontemporal_load" in src
+    assert low.tail[-2:] == [-(n + 1), n * n - (n + 1)]
+    hip.compile_source(src)
+    u = NPArray(hip.placeholder((64, 64, 64), np.float32))       # short rows: 62 -> 16 groups
+    dst = hip.placeholder((62, 62, 62), np.float32, strides=(4096, 64, 1), offset=4096 + 64 + 1)
+    low, src = hip.lower_only(u[1:-1, 1:-1, 1:-1] * 2.0, dst=dst)
+    assert low.key[8:10] == (16, 1) and "__builtin_nontemporal_load" not in src
+    hip.compile_source(src)
+    row = NPArray(hip.placeholder((n,), np.float32))             # repeats from row to row:
+    low, src = hip.lower_only(m + row)                            # the taller tile shares it
+    assert low.key[0] == "tile2dv" and low.key[8:10] == (64, 2)
+
+
 def test_shifted_views_lower_to_lds_stencil():
     n = 512
     u = NPArray(hip.placeholder((n, n), np.float32))
