@@ -1629,14 +1629,14 @@ T_TILE = 64      # square tile edge: both the transposed read and the write coal
 
 
 def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_load=False,
-                        nt_store=False, unaligned=False):
+                        nt_store=False, unaligned=False, tile=(T_TILE, T_TILE)):
     """2-D tiled kernel for expressions in which some operand is walked along the
     output's rows by its unit stride (a transposed view).
 
-    leaf_kind  per leaf: ('t',) unit stride along output dimension 0: its 64x64 tile
-               is read along its own contiguous direction into LDS and read back
-               transposed (rows padded by one word, so neither side has bank
-               conflicts); ('d',) unit stride along output dimension 1, read directly;
+    leaf_kind  per leaf: ('t',) unit stride along output dimension 0: its tile (TR output
+               rows x TC output columns, `tile`) is read along its own contiguous
+               direction, TR elements at a time, into LDS and read back transposed
+               (rows padded by one word, so neither side has bank conflicts); ('d',) unit stride along output dimension 1, read directly;
                ('b',) single element broadcast
     vec        0, or the number of elements in 16 bytes when every array has that
                element size, 16-byte aligned rows and row strides: tiles that lie
@@ -1647,8 +1647,8 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
     row stride."""
     rs = "__restrict__ " if restrict else ""
     n_out = len(out_dtypes)
-    T = T_TILE
-    per_thread = T * T // BLOCK
+    TR, TC = tile
+    per_thread = TR * TC // BLOCK
     src = [PREAMBLE, emit_body(prog, out_dtypes)]
     params = [f"const {CTYPE[dt]}* {rs}a{i}" for i, dt in enumerate(prog.leaves)]
     params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
@@ -1665,20 +1665,21 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
          f"void dr_kernel({', '.join(params)})", "{"]
     for i, k in enumerate(leaf_kind):
         if k[0] == "t":
-            L.append(f"    __shared__ {CTYPE[prog.leaves[i]]} tt{i}[{T * (T + 1)}];")
+            L.append(f"    __shared__ {CTYPE[prog.leaves[i]]} tt{i}[{TC * (TR + 1)}];")
     # Diagonal order: blocks that run at the same time differ in both tile coordinates.
     # With row-major order they would share r0, and the transposed operand's tiles
     # (rows a power-of-two pitch apart) would all fall into the same few memory channels.
     L += ["    const int band = blockIdx.x / tiles_x;",
           "    const int tx = blockIdx.x - band * tiles_x;",
-          f"    const int ty = (band + tx) % ((H + {T - 1}) / {T});",
-          f"    const int r0 = ty * {T};",
-          f"    const int c0 = tx * {T};"]
+          f"    const int ty = (band + tx) % ((H + {TR - 1}) / {TR});",
+          f"    const int r0 = ty * {TR};",
+          f"    const int c0 = tx * {TC};"]
     if vec:
         V = vec
-        vpr = T // V                      # vectors per tile row
-        passes = T * T // V // BLOCK
-        L += [f"    if (r0 + {T} <= H && c0 + {T} <= W) {{",
+        vpr = TR // V                     # vectors per column of the tile (operand's rows)
+        vpc = TC // V                     # vectors per row of the tile (output's rows)
+        passes = TR * TC // V // BLOCK
+        L += [f"    if (r0 + {TR} <= H && c0 + {TC} <= W) {{",
               "#pragma unroll",
               f"        for (int k = 0; k < {passes}; ++k) {{",
               f"            const int e = threadIdx.x + k * {BLOCK};",
@@ -1690,13 +1691,13 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
                 ptr = f"(const {vt}*)(a{i} + (long long)(c0 + lc) * cs{i} + (r0 + vr * {V}))"
                 L.append(f"            const {vt} w{i} = {_ld(nt_load, ptr)};")
                 for q in range(V):
-                    L.append(f"            tt{i}[lc * {T + 1} + vr * {V} + {q}] = w{i}[{q}];")
+                    L.append(f"            tt{i}[lc * {TR + 1} + vr * {V} + {q}] = w{i}[{q}];")
         L += ["        }", "        __syncthreads();",
               "#pragma unroll",
               f"        for (int k = 0; k < {passes}; ++k) {{",
               f"            const int e = threadIdx.x + k * {BLOCK};",
-              f"            const int lr = e / {vpr};",
-              f"            const int vc = e - lr * {vpr};",
+              f"            const int lr = e / {vpc};",
+              f"            const int vc = e - lr * {vpc};",
               "            const long long i = r0 + lr;",
               f"            const int j = c0 + vc * {V};"]
         for i, k in enumerate(leaf_kind):
@@ -1710,7 +1711,7 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
             vargs = []
             for i, k in enumerate(leaf_kind):
                 if k[0] == "t":
-                    vargs.append(f"tt{i}[(vc * {V} + {q}) * {T + 1} + lr]")
+                    vargs.append(f"tt{i}[(vc * {V} + {q}) * {TR + 1} + lr]")
                 elif k[0] == "d":
                     vargs.append(f"d{i}[{q}]")
                 else:
@@ -1727,25 +1728,25 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
           "#pragma unroll",
           f"    for (int k = 0; k < {per_thread}; ++k) {{",
           f"        const int e = threadIdx.x + k * {BLOCK};",
-          f"        const int lc = e / {T};",
-          f"        const int lr = e - lc * {T};",
+          f"        const int lc = e / {TR};",
+          f"        const int lr = e - lc * {TR};",
           "        if (r0 + lr < H && c0 + lc < W) {"]
     for i, k in enumerate(leaf_kind):
         if k[0] == "t":
-            L.append(f"            tt{i}[lc * {T + 1} + lr] = a{i}[(long long)(c0 + lc) * cs{i} + (r0 + lr)];")
+            L.append(f"            tt{i}[lc * {TR + 1} + lr] = a{i}[(long long)(c0 + lc) * cs{i} + (r0 + lr)];")
     L += ["        }", "    }", "    __syncthreads();",
           "#pragma unroll",
           f"    for (int k = 0; k < {per_thread}; ++k) {{",
           f"        const int e = threadIdx.x + k * {BLOCK};",
-          f"        const int lr = e / {T};",
-          f"        const int lc = e - lr * {T};",
+          f"        const int lr = e / {TC};",
+          f"        const int lc = e - lr * {TC};",
           "        const int i = r0 + lr;",
           "        const int j = c0 + lc;",
           "        if (i < H && j < W) {"]
     args = []
     for i, k in enumerate(leaf_kind):
         if k[0] == "t":
-            args.append(f"tt{i}[lc * {T + 1} + lr]")
+            args.append(f"tt{i}[lc * {TR + 1} + lr]")
         elif k[0] == "d":
             args.append(f"a{i}[(long long)i * rs{i} + j]")
         else:

@@ -53,6 +53,8 @@ TUNE = {
     "s3_depth": 1,    # 3-D window: planes in flight in registers
     "uvec": 1,        # 16-byte accesses at element alignment where 16-byte alignment is missing
     "tvec": 1,        # transpose tiles: 16-byte global accesses where alignment allows
+    "t_rows": 0,      # transpose tiles: output rows (= contiguous elements of the operand) and
+    "t_cols": 0,      # output columns per tile (powers of two; 0: 128 bytes by 1 KB)
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
     "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
     "smath": 1,       # float32 log/erf/exp from `mathlib32` (0: the device library's)
@@ -489,8 +491,18 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                   and any(s[0] == 1 and s[1] != 1 for s in m_leaf))
     if transposed:
         kinds = tuple(("b",) if s == [0, 0] else ("d",) if s[1] == 1 else ("t",) for s in m_leaf)
-        lds_bytes = sum((cg.T_TILE + 1) * cg.T_TILE * cg.ITEMSIZE[c]
+        # Tile: 128 bytes of the transposed operand's rows by 1 KB of the output's rows.  What
+        # is written contiguously counts for more than what is read contiguously; float32
+        # 16384^2, percent of the HBM peak: 64 x 64 elements 66, 128 x 64: 67, 64 x 128: 68,
+        # 32 x 256: 73, 16 x 512: 60, 32 x 384: 64.
+        widest = max(cg.ITEMSIZE[c] for c in list(prog.leaves) + list(out_codes))
+        t_r, t_c = TUNE["t_rows"] or 128 // widest, TUNE["t_cols"] or 1024 // widest
+        lds_bytes = sum((t_r + 1) * t_c * cg.ITEMSIZE[c]
                         for c, k in zip(prog.leaves, kinds) if k[0] == "t")
+        if lds_bytes > 64 * 1024:
+            t_r = t_c = cg.T_TILE
+            lds_bytes = sum((t_r + 1) * t_c * cg.ITEMSIZE[c]
+                            for c, k in zip(prog.leaves, kinds) if k[0] == "t")
         if lds_bytes <= 64 * 1024:
             H, W = mshape
             low.kind = "tile2dt"
@@ -516,14 +528,16 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             nts = bool(vec and TUNE["nts"]) and in_bytes + out_bytes > TUNE["cache_mib"] << 20
             ntl = bool(vec and TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
             ua = bool(ua and vec)
-            low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place, vec, ntl, nts, ua)
+            low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place, vec, ntl, nts, ua,
+                       t_r, t_c)
 
             def emit():
                 return cg.emit_tile_transpose(prog, kinds, out_codes, restrict=not in_place,
-                                              vec=vec, nt_load=ntl, nt_store=nts, unaligned=ua)
+                                              vec=vec, nt_load=ntl, nt_store=nts, unaligned=ua,
+                                              tile=(t_r, t_c))
             low.emit = emit
-            tiles_x = -(-W // cg.T_TILE)
-            low.grid = tiles_x * -(-H // cg.T_TILE)
+            tiles_x = -(-W // t_c)
+            low.grid = tiles_x * -(-H // t_r)
             fmt = "@" + "P" * (len(leaves) + len(out_ptrs)) + scal_fmt + "iii"
             tail_vals = [H, W, tiles_x]
             for k, s in zip(kinds, m_leaf):
