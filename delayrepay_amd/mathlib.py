@@ -6,8 +6,11 @@ fp64 pipes rather than on memory.  These cost about 25, 20 and 25.  Black-Schole
 float64, n = 2^25, microseconds per launch on MI355X (vector instructions per option):
 device library 398 (379); polynomial `log`/`erf`/`exp`, one element at a time 305 (254);
 the same on packs of four 299 (245); `log` from a table 293 (227); `erf` from a table
-read in memory 405, read in LDS 262, with workgroups that stay for eight chunks 241 (153);
-with the short `sqrt` 240.
+read in memory 405, read in LDS 262, with workgroups that stay for eight chunks 241;
+with the short `sqrt` 240 (138).  At that point the kernel moves its bytes at 85 % of a
+plain copy's rate; the vector unit is busy 59 % of the time and LDS 43 %, more than half
+of that in bank conflicts between the lanes' table rows (rocprofv3 `SQ_ACTIVE_INST_VALU`,
+`SQ_LDS_IDX_ACTIVE`, `SQ_LDS_BANK_CONFLICT`).
 
 `log` and `erf` are table driven.  `log`: x = 2^k z, z in [0.706, 1.412) falls into one of
 256 intervals with centre c, log x = k ln 2 + log c + log1p(z/c - 1); 1/c and log c come
