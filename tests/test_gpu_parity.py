@@ -1103,6 +1103,38 @@ def test_stencils_in_three_dimensions_go_through_the_lds_window(shape, dtype):
     assert w.tobytes() == r.tobytes()
 
 
+@pytest.mark.parametrize("tune", [dict(), dict(s3_zc=8), dict(s3_zc=5, s3_depth=2), dict(s3_gpr=16, s3_rpt=1),
+                                  dict(s3_gpr=32, s3_rpt=2, s3_depth=3)])
+def test_ring_of_window_planes_at_the_ends_of_the_buffer(tune):
+    """Views that begin at the first and end at the last element of the buffer (window
+    vectors beyond either end are read from the nearest vector inside), stencils that reach
+    one plane only, walks cut into stretches of planes that do not divide the extent, more
+    than one plane in flight."""
+    rs = np.random.RandomState(43)
+    hip.set_tune(**tune)
+    try:
+        for shape, dt in (((37, 21, 72), np.float32), ((19, 11, 36), np.float64), ((3, 3, 12), np.float32)):
+            h = rs.uniform(-1, 1, shape).astype(dt)
+            u = dr.array(h)
+            for expr in (lambda a: a[:-1, :-1, :-4] + a[1:, 1:, 4:] - a[:-1, 1:, :-4],   # both ends
+                         lambda a: a[:-2, 1:-1, 4:-4] + a[2:, 1:-1, 4:-4] * 2,           # planes only
+                         lambda a: a[:-1, 1:, 4:] - a[1:, :-1, :-4]):                     # one plane
+                low = hip.lower_only(expr(u))[0]
+                assert low.kind == "tile3d" or shape[0] == 3, (shape, low.kind)
+                got = expr(u).get()
+                assert got.tobytes() == expr(h).tobytes(), (tune, shape, dt)
+        h = rs.uniform(-1, 1, (67, 20, 40)).astype(np.float32)
+        u, ref = dr.array(h), h.copy()
+        launched = set(hip._KERNELS)
+        for _ in range(2):
+            u[1:-1, 1:-1, 1:-1] = _laplace3d(u)
+            ref[1:-1, 1:-1, 1:-1] = _laplace3d(ref, c=np.float32(1 / 6.0))
+        assert u.get().tobytes() == ref.tobytes()
+        assert {k[0] for k in set(hip._KERNELS) - launched} <= {"tile3d"}
+    finally:
+        hip.set_tune(s3_zc=0, s3_depth=1, s3_gpr=64, s3_rpt=2)
+
+
 def test_three_dimensional_stencil_layouts_that_do_not_qualify_still_match():
     rs = np.random.RandomState(42)
     h = rs.uniform(0, 1, (20, 30, 63)).astype(np.float32)       # row pitch not a multiple of 16 bytes
