@@ -15,7 +15,8 @@ from . import hiprt
 
 # Tunables; part of every cache key.  DELAYREPAY_TUNE="unroll=2,bpc=16" overrides.
 TUNE = {
-    "unroll": 1,      # 16-byte vectors per thread and chunk in flat element-wise kernels
+    "unroll": 0,      # 16-byte vectors per thread and chunk in flat element-wise kernels
+                      # (0: by the number of streams, see `lower`)
     "red_unroll": 4,  # the same for flat kernels with a reduction tail
     "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
     "static_scratch": 1,  # partial results go to the library's static scratch array if they fit
@@ -283,7 +284,18 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         vec = widths_ok and n >= 64 and (align_ok or bool(TUNE["uvec"]))
         ua = vec and not align_ok      # vectors at element alignment
         unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
-        if cg.packs(prog, vec) and TUNE["pack"]:
+        packed = bool(cg.packs(prog, vec) and TUNE["pack"])
+        if not unroll and packed:
+            unroll = 1          # the pack below decides
+        elif not unroll:
+            # More streams want more vectors in flight per thread.  Percent of the HBM peak
+            # with 1 / 2 / 4 vectors: one load and one store (Horner) 81.4 / 80.0 / 79.9; two
+            # loads and one store (SAXPY, 2^24) 76.3 / 78.9 / 78.8; three float64 loads and
+            # two stores with a trivial body 75.0 / 77.6 / 78.8, with Black-Scholes' float32
+            # body 73.2 / 73.5 / 71.7.
+            streams = sum(c == "c" for c in leaf_class) + len(out_codes)
+            unroll = 1 if streams <= 2 else 2
+        if packed:
             # float64 functions evaluate a pack of elements in lock step: at least `pack`
             # elements per thread (a vector of doubles holds two)
             unroll = max(unroll, TUNE["pack"] // cg.flat_elements(prog, leaf_class, out_codes, reduce_op))
