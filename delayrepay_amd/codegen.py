@@ -1623,6 +1623,74 @@ def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
     return "\n".join(src) + "\n"
 
 
+def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4):
+    """Reduction over a long unit-stride last dimension: a block per (row, slice) streams
+    its stretch of the row like a flat reduction (256 lanes x 16 bytes x `unroll` per step,
+    one accumulator per vector element), combines through `dr_block_reduce` and writes one
+    value.  A wave per row reads 256 bytes per instruction and keeps far fewer bytes in
+    flight (sum over axis 1 of 16384^2 float32: 74 % of the HBM peak against the 87 % of a
+    flat reduction).
+
+    leaf_kind  per leaf 'v' (unit stride along the row) or 'k' (constant along it)
+    Parameters: leaf pointers, output pointer, scalars, K, R, S, RS, then per leaf the
+    stride between rows (elements).  Output layout [row][slice]."""
+    ct = CTYPE[acc_dt]
+    nl = len(prog.leaves)
+    widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "v"}
+    V = 16 // widths.pop()
+    src = [PREAMBLE, emit_body(prog, [acc_dt]), emit_block_reduce(op, acc_dt)]
+    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
+    params.append(f"{ct}* __restrict__ out")
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += ["const long long K", "const long long R", "const long long S", "const long long RS"]
+    params += [f"const long long sk{i}" for i in range(nl)]
+    call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
+    ident = _identity(op, acc_dt)
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{",
+         "    for (long long o = blockIdx.x; o < K * S; o += gridDim.x) {",
+         "        const long long k = o / S;",
+         "        const long long sl = o - k * S;",
+         "        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind == "v":
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+        else:
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+    L += [f"        {ct} acc[{V}];",
+          "#pragma unroll",
+          f"        for (int e = 0; e < {V}; ++e) acc[e] = {ident};",
+          f"        long long r = sl * RS + (long long)threadIdx.x * {V};",
+          f"#pragma unroll {unroll}",
+          f"        for (; r + {V} <= r_end; r += {BLOCK * V}) {{"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind == "v":
+            vt = VEC16[dt][0] + "u"
+            L.append(f"            const {vt} X{i} = __builtin_nontemporal_load((const {vt}*)(row{i} + r));")
+    for e in range(V):
+        vargs = [f"X{i}[{e}]" if kind == "v" else f"c{i}" for i, kind in enumerate(leaf_kind)]
+        L.append(f"            {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
+                 f"acc[{e}] = {_combine(op, f'acc[{e}]', 't0')}; }}")
+    L.append("        }")
+    # exactly one thread is left with r < r_end: the one whose next vector would straddle
+    # the end of the stretch; it takes those elements one by one
+    sargs = [f"row{i}[r]" if kind == "v" else f"c{i}" for i, kind in enumerate(leaf_kind)]
+    L += ["        for (; r < r_end; ++r) {",
+          f"            {ct} t0; dr_body({', '.join(sargs + call_tail)});",
+          f"            acc[0] = {_combine(op, 'acc[0]', 't0')};",
+          "        }"]
+    accs = [f"acc[{e}]" for e in range(V)]
+    while len(accs) > 1:
+        accs = [f"({_combine(op, accs[i], accs[i + 1])})" if i + 1 < len(accs) else accs[i]
+                for i in range(0, len(accs), 2)]
+    L += [f"        {ct} total = dr_block_reduce({accs[0]});",
+          "        if (threadIdx.x == 0) out[o] = total;",
+          "        __syncthreads();          // the block reduction's LDS words are reused",
+          "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"
+
+
 # ---- 2-D kernel with transposed operands ------------------------------------------
 
 T_TILE = 64      # square tile edge: both the transposed read and the write coalesce

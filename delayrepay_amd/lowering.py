@@ -31,6 +31,7 @@ TUNE = {
     "ax_group_lanes": 0,  # force the group size (0: the one that wastes the fewest unit slots)
     "ax_group_steps": 8,  # most 16-byte units a lane of such a group takes from its row
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
+    "ax_block": 4096,    # reduced unit-stride extents from this length: a block per row slice
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
     "nts": 1,         # allow non-temporal stores }
     "cache_mib": 32,  # working sets up to this size (the eight L2s together) stay cacheable
@@ -716,6 +717,33 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
             low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
             low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets]
             return low, 1, K, "group"
+    if (strategy == "row" and slices is None and len(rmerged) == 1 and len(kmerged) == 1
+            and R >= TUNE["ax_block"] > 0 and TUNE["uvec"] and all(r[0] in (0, 1) for r in rsets)):
+        widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == 1}
+        if len(widths) == 1 and widths <= {4, 8} and all(
+                c in cg.VEC16 for c, r in zip(prog.leaves, rsets) if r[0] == 1):
+            # long rows: a block per row (or per slice of a row, while there are too few rows
+            # to fill the device), streamed like a flat reduction
+            V = 16 // next(iter(widths))
+            S = max(1, min(-(-TUNE["ax_blocks"] // K), R // TUNE["ax_block"], TUNE["ax_slices"]))
+            RS = -(-R // S)
+            S = -(-R // RS)
+            kinds = tuple("v" if r[0] == 1 else "k" for r in rsets)
+            low = Lowered()
+            low.lds = 0
+            low.fin_count = 0
+            low.kind = "axis_block"
+            low.key = ("axis_block", prog.key(), kinds, acc, reduce_op)
+
+            def emit_block():
+                return cg.emit_block_rows(prog, kinds, acc, reduce_op)
+            low.emit = emit_block
+            low.grid = max(1, min(K * S, 1 << 20))
+            low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+                       + "qqqq" + "q" * len(leaves))
+            low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+            low.scal, low.tail = list(scalars), [K, R, S, RS] + [k[0] for k in ksets]
+            return low, S, K, "row"
     # enough independent pieces to fill the device: cut the reduced extent into slices
     if slices is not None:
         S = slices

@@ -1056,6 +1056,31 @@ def _row_reduction_cases(rs, groups):
     assert np.allclose(got, (h.astype(np.float64) * w + 1.0).sum(axis=1), rtol=2e-5)
 
 
+def test_reductions_over_long_rows_take_a_block_per_row_slice():
+    """Rows from 4096 elements: a block streams a row (or a slice of it, when there are too
+    few rows to fill the device) like a flat reduction; lengths that are not multiples of the
+    vector, rows that start off 16 bytes, an operand constant along the row."""
+    rs = np.random.RandomState(29)
+    for shape, dt in [((300, 4096), np.float32), ((129, 5003), np.float64), ((3, 1 << 20), np.float32),
+                      ((40, 4099), np.int32), ((1, 70001), np.float64)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
+        assert low.kind == "axis_block", (shape, low.kind)
+        tol = dict(rtol=2e-5, atol=1e-4) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
+        assert np.allclose(dr.sum(a * a, axis=1).get(), (h.astype(np.float64) ** 2).sum(axis=1), **tol)
+        assert np.array_equal(dr.max(a, axis=1).get(), h.max(axis=1))
+        assert np.array_equal(dr.min(a[:, 3:-2], axis=1).get(), h[:, 3:-2].min(axis=1))
+        if dt == np.int32:
+            assert np.array_equal(dr.sum(a, axis=1).get(), h.sum(axis=1))
+    h = rs.uniform(0, 1, (50, 6000)).astype(np.float32)
+    w = rs.uniform(0, 1, (50, 1)).astype(np.float32)
+    got = dr.sum(dr.array(h) * dr.array(w) + 1.0, axis=1).get()
+    assert np.allclose(got, (h.astype(np.float64) * w + 1.0).sum(axis=1), rtol=2e-5)
+    m = dr.mean(dr.array(h), axis=1).get()
+    assert np.allclose(m, h.mean(axis=1, dtype=np.float64), rtol=2e-5)
+
+
 def test_reduction_strategy_follows_the_operands_that_carry_the_traffic():
     """A column of weights beside a matrix (unit stride along the reduced axis) must not
     switch a sum over rows to the kernel for sums along rows."""
