@@ -1623,6 +1623,74 @@ def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
     return "\n".join(src) + "\n"
 
 
+def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8):
+    """Reduction over the rows of a matrix whose kept dimension has unit stride: a block owns
+    256 x V adjacent columns (V the elements of a 16-byte vector: 4 KB of every row) and a
+    slice of rows, and walks the rows with `unroll` loads in flight per lane; every lane
+    keeps its own V columns, so nothing is combined inside the block.  Blocks with adjacent
+    column tiles are adjacent in launch order: together they read whole rows.
+
+    leaf_kind  per leaf 'v' (unit stride along the kept dimension) or 'k' (constant along it)
+    Parameters: leaf pointers, output pointer, scalars, K, R, S, RS, then per leaf the
+    stride between rows (elements).  Output layout [slice][column]."""
+    ct = CTYPE[acc_dt]
+    nl = len(prog.leaves)
+    widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "v"}
+    V = 16 // widths.pop()
+    TK = BLOCK * V
+    src = [PREAMBLE, emit_body(prog, [acc_dt])]
+    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
+    params.append(f"{ct}* __restrict__ out")
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += ["const long long K", "const long long R", "const long long S", "const long long RS"]
+    params += [f"const long long sr{i}" for i in range(nl)]
+    call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
+    ident = _identity(op, acc_dt)
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{",
+         f"    const long long ktiles = (K + {TK - 1}) / {TK};",
+         "    for (long long b = blockIdx.x; b < ktiles * S; b += gridDim.x) {",
+         "        const long long sl = b / ktiles;",
+         f"        const long long g = (b - sl * ktiles) * {TK} + (long long)threadIdx.x * {V};",
+         "        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;",
+         f"        {ct} acc[{V}];",
+         "#pragma unroll",
+         f"        for (int e = 0; e < {V}; ++e) acc[e] = {ident};",
+         f"        if (g + {V} <= K) {{",
+         f"#pragma unroll {unroll}",
+         "            for (long long r = sl * RS; r < r_end; ++r) {"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind == "v":
+            vt = VEC16[dt][0] + "u"
+            L.append(f"                const {vt} X{i} = __builtin_nontemporal_load((const {vt}*)(a{i} + g + r * sr{i}));")
+        else:
+            L.append(f"                const {CTYPE[dt]} c{i} = a{i}[r * sr{i}];")
+    for e in range(V):
+        vargs = [f"X{i}[{e}]" if kind == "v" else f"c{i}" for i, kind in enumerate(leaf_kind)]
+        L.append(f"                {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
+                 f"acc[{e}] = {_combine(op, f'acc[{e}]', 't0')}; }}")
+    sargs = [f"a{i}[g + e + r * sr{i}]" if kind == "v" else f"a{i}[r * sr{i}]"
+             for i, kind in enumerate(leaf_kind)]
+    L += ["            }",
+          "        } else if (g < K) {          // the vector that straddles the last column",
+          "            for (long long r = sl * RS; r < r_end; ++r) {",
+          "#pragma unroll",
+          f"                for (int e = 0; e < {V}; ++e) {{",
+          "                    if (g + e < K) {",
+          f"                        {ct} t0; dr_body({', '.join(sargs + call_tail)});",
+          f"                        acc[e] = {_combine(op, 'acc[e]', 't0')};",
+          "                    }",
+          "                }",
+          "            }",
+          "        }",
+          "#pragma unroll",
+          f"        for (int e = 0; e < {V}; ++e)",
+          "            if (g + e < K) out[sl * K + g + e] = acc[e];",
+          "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"
+
+
 def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4):
     """Reduction over a long unit-stride last dimension: a block per (row, slice) streams
     its stretch of the row like a flat reduction (256 lanes x 16 bytes x `unroll` per step,

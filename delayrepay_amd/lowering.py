@@ -32,6 +32,9 @@ TUNE = {
     "ax_group_steps": 8,  # most 16-byte units a lane of such a group takes from its row
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ax_block": 4096,    # reduced unit-stride extents from this length: a block per row slice
+    "ax_stream": 256,    # kept unit-stride extents of 256 vectors or more: blocks to aim for, one
+                         # per compute unit (0: off)
+    "ax_stream_unroll": 8,   # ... and rows in flight per lane
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
     "nts": 1,         # allow non-temporal stores }
     "cache_mib": 32,  # working sets up to this size (the eight L2s together) stay cacheable
@@ -717,6 +720,38 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
             low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
             low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets]
             return low, 1, K, "group"
+    if (strategy == "col" and slices is None and len(rmerged) == 1 and len(kmerged) == 1
+            and TUNE["ax_stream"] > 0 and TUNE["uvec"] and all(k[0] in (0, 1) for k in ksets)):
+        widths = {cg.ITEMSIZE[c] for c, k in zip(prog.leaves, ksets) if k[0] == 1}
+        if len(widths) == 1 and widths <= {4, 8} and all(
+                c in cg.VEC16 for c, k in zip(prog.leaves, ksets) if k[0] == 1):
+            V = 16 // next(iter(widths))
+            ktiles = -(-K // (cg.BLOCK * V))
+            if K >= cg.BLOCK * V and R >= 64:
+                # long rows kept: blocks of 256 lanes x one vector stream whole rows together.
+                # Sum over axis 0 of 16384^2 float32, percent of the HBM peak by blocks in the
+                # grid: 128: 77, 256 (one per compute unit): 80, 512: 79, 1024: 77, 2048: 65,
+                # 4096: 61; a lane per column with four waves on four rows (`col`): 72.
+                S = max(1, min(-(-TUNE["ax_stream"] // ktiles), R // 32, TUNE["ax_slices"]))
+                RS = -(-R // S)
+                S = -(-R // RS)
+                kinds = tuple("v" if k[0] == 1 else "k" for k in ksets)
+                low = Lowered()
+                low.lds = 0
+                low.fin_count = 0
+                low.kind = "axis_stream"
+                unroll = TUNE["ax_stream_unroll"]
+                low.key = ("axis_stream", prog.key(), kinds, acc, reduce_op, unroll)
+
+                def emit_stream():
+                    return cg.emit_col_stream(prog, kinds, acc, reduce_op, unroll)
+                low.emit = emit_stream
+                low.grid = max(1, min(ktiles * S, 1 << 20))
+                low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+                           + "qqqq" + "q" * len(leaves))
+                low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+                low.scal, low.tail = list(scalars), [K, R, S, RS] + [r[0] for r in rsets]
+                return low, S, K, "col"
     if (strategy == "row" and slices is None and len(rmerged) == 1 and len(kmerged) == 1
             and R >= TUNE["ax_block"] > 0 and TUNE["uvec"] and all(r[0] in (0, 1) for r in rsets)):
         widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == 1}

@@ -1081,6 +1081,31 @@ def test_reductions_over_long_rows_take_a_block_per_row_slice():
     assert np.allclose(m, h.mean(axis=1, dtype=np.float64), rtol=2e-5)
 
 
+def test_reductions_over_the_rows_of_wide_matrices_stream_whole_rows():
+    """Kept rows of 256 vectors or more: a block owns 256 lanes x one vector of columns and
+    walks a slice of rows; widths that are not multiples of the vector, views that start off
+    16 bytes, an operand constant along the kept dimension, integer sums, extrema."""
+    rs = np.random.RandomState(31)
+    for shape, dt in [((5000, 1024), np.float32), ((300, 3001), np.float64), ((64, 1030), np.float32),
+                      ((2000, 2050), np.int32), ((70, 4096), np.float64)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (0,)))[0]
+        assert low.kind == "axis_stream", (shape, low.kind)
+        tol = dict(rtol=2e-5, atol=1e-4) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
+        assert np.allclose(dr.sum(a * a, axis=0).get(), (h.astype(np.float64) ** 2).sum(axis=0), **tol)
+        assert np.array_equal(dr.max(a, axis=0).get(), h.max(axis=0))
+        assert np.array_equal(dr.min(a[1:-1, 3:-2], axis=0).get(), h[1:-1, 3:-2].min(axis=0))
+        if dt == np.int32:
+            assert np.array_equal(dr.sum(a, axis=0).get(), h.sum(axis=0))
+    h = rs.uniform(0, 1, (900, 1500)).astype(np.float32)
+    w = rs.uniform(0, 1, (900, 1)).astype(np.float32)
+    got = dr.sum(dr.array(h) * dr.array(w) + 1.0, axis=0).get()
+    assert np.allclose(got, (h.astype(np.float64) * w + 1.0).sum(axis=0), rtol=2e-5)
+    v = dr.var(dr.array(h), axis=0).get()
+    assert np.allclose(v, h.astype(np.float64).var(axis=0), rtol=1e-4)
+
+
 def test_reduction_strategy_follows_the_operands_that_carry_the_traffic():
     """A column of weights beside a matrix (unit stride along the reduced axis) must not
     switch a sum over rows to the kernel for sums along rows."""
