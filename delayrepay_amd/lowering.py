@@ -17,8 +17,8 @@ from . import hiprt
 TUNE = {
     "unroll": 0,      # 16-byte vectors per thread and chunk in flat element-wise kernels
                       # (0: by the number of streams, see `lower`)
-    "red_unroll": 4,  # the same for flat kernels with a reduction tail
-    "red_blocks": 4096,  # most blocks (= partial results) of a reduction kernel
+    "red_unroll": 0,  # the same for flat kernels with a reduction tail } 0: see `lower`
+    "red_blocks": 0,  # most blocks (= partial results) of a reduction kernel }
     "static_scratch": 1,  # partial results go to the library's static scratch array if they fit
     "flat_cap": 0,    # most blocks of a flat element-wise kernel (0: one chunk per block)
     "bpc": 8,         # resident blocks per CU that bound the grid of `nd` kernels
@@ -288,6 +288,22 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         vec = widths_ok and n >= 64 and (align_ok or bool(TUNE["uvec"]))
         ua = vec and not align_ok      # vectors at element alignment
         unroll = TUNE["red_unroll"] if reduce_op else TUNE["unroll"]
+        red_cap = TUNE["red_blocks"]
+        if reduce_op and not (unroll and red_cap):
+            # A stream that is only read is fastest with one block per compute unit and six
+            # to eight 16-byte loads in flight per lane.  sum((x-y)**2*w), float64, 2^27,
+            # percent of the HBM peak: 4096 blocks x 4 vectors per operand 86.4; 256 blocks x
+            # 1 / 2 / 3 vectors 65.8 / 89.3 / 86.6; 384 blocks 81.6; 128 blocks 72.3.  dot of
+            # two operands: 256 blocks x 2 / 4 vectors 77.5 / 89.5.  A body with many
+            # operations per element needs more waves than that to keep the vector unit busy.
+            n_in = max(1, sum(c == "c" for c in leaf_class))
+            cheap = {"floor", "ceil", "trunc", "rint", "copysign", "fmax", "fmin"}
+            cost = sum(10 if (name in cg._FLOAT_FUNCS1 or name in cg._FLOAT_FUNCS2 or name in
+                              ("divide", "true_divide", "reciprocal")) and name not in cheap else 1
+                       for name, _, _, _ in prog.ops)
+            light = cost <= 4 * n_in + 4
+            unroll = unroll or (max(1, min(8, 8 // n_in)) if light else 4)
+            red_cap = red_cap or (grid_cap() // TUNE["bpc"] if light else 4096)
         packed = bool(cg.packs(prog, vec) and TUNE["pack"])
         if not unroll and packed:
             unroll = 1          # the pack below decides
@@ -327,7 +343,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         low.emit = emit
         E = cg.flat_elements(prog, leaf_class, out_codes, reduce_op) if vec else 1
         chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
-        cap = TUNE["red_blocks"] if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
+        cap = red_cap if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
         if mathlib.tables(prog.own_math) and not TUNE["flat_cap"]:
             # the workgroup copies the functions' tables into LDS first: let it stay for
             # several chunks (Black-Scholes float64: 262 us with a chunk per workgroup, 244 us
