@@ -730,7 +730,9 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
                 return cg.emit_group_rows(prog, kinds, acc, reduce_op, R, G)
             low.emit = emit_group
             rows_per_block = (cg.BLOCK // cg.WAVE) * (cg.WAVE // G)
-            low.grid = max(1, min(-(-K // rows_per_block // TUNE["ax_rows"]), 1 << 20))
+            # one pass over the rows per wave (rows of 200 float32: 80.6 % of the HBM peak; four
+            # passes 76.5, sixteen 72.9)
+            low.grid = max(1, min(-(-K // rows_per_block), 1 << 20))
             low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
                        + "q" + "q" * len(leaves))
             low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
