@@ -32,7 +32,6 @@ Per configuration:
                       options (oracle/accuracy.py)
 """
 import argparse
-import contextlib
 import json
 import os
 import statistics

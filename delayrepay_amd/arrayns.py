@@ -9,7 +9,7 @@ import numpy
 
 from . import hiprt
 from .devarray import ndarray
-from .hip import assign, materialise, run, run_reduce_product
+from .hip import assign, materialise, run_reduce_product
 
 
 def _upload(fn):

@@ -8,7 +8,6 @@ returns views of the same buffer, as the front end's `__getitem__` /
 `__setitem__` expect (delayarray.py:114-128).  All data movement and compute
 goes through libdrhip; nothing here computes on the host.
 """
-import ctypes
 import numbers
 
 import numpy as np

@@ -21,7 +21,6 @@ import collections
 import hashlib
 import os
 import struct
-import sys
 import warnings
 
 import numpy
@@ -32,7 +31,7 @@ from .devarray import Buffer, ndarray, placeholder  # noqa: F401
 from .codegen import Program, dtype_code, code_dtype
 from .promote import result_dtype, scalar_descr
 from .visitor import Visitor
-from .lowering import (TUNE, Lowered, broadcast_strides as _broadcast_strides, lower as _lower,
+from .lowering import (TUNE, broadcast_strides as _broadcast_strides, lower as _lower,
                        lower_axis_reduce as _lower_axis_reduce)
 
 hiprt.lib()  # fail at import when libdrhip.so has not been built
