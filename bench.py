@@ -383,7 +383,9 @@ def main():
             "kernel_us_warm": round(warm_med * 1e3, 2),
             "roofline_frac_warm": round(wl["nbytes"] / warm_med / 1e6 / HBM_PEAK_GBPS, 4),
             # what limits the kernel (rocprofv3 VALUBusy / traffic in profiles/)
-            "bound": {"bs64": "fp64 vector ALU and HBM", "bs32": "fp32 vector ALU and HBM",
+            "bound": {"bs64": "HBM (five float64 streams) and fp64 vector ALU",
+                      "bs32": "fp32 vector ALU and HBM", "rand": "vector ALU (64-bit multiplies)",
+                      "grid": "vector ALU and HBM", "stencil3d": "cache-line requests per compute unit",
                       "matmul32": "mfma", "matmul64": "mfma"}.get(name, "hbm"),
             **({"TFLOPs": round(wl["flops"] / kernel_ms / 1e9, 1),
                 "mfma_frac": round(wl["flops"] / kernel_ms / 1e9 / wl["mfma_peak"], 4),
