@@ -166,7 +166,7 @@ def main():
                             dr, S, K_, T, inp["r"], inp["sigma"])))) for S, K_, T in sets],
                         cpu=lambda: orc.black_scholes(inp["S"][:m], inp["K"][:m], inp["T"][:m],
                                                       inp["r"], inp["sigma"]), cpu_frac=0.25,
-                        cpu_code="oracle/numpy_oracle.py::black_scholes", inputs=inp)
+                        cpu_code="oracle/numpy_oracle.py::black_scholes", inputs=inp, sets=sets)
         if name == "jacobi":
             N = inp["u"].shape[0]
             nbytes = 4 * N * N + 4 * (N - 2) * (N - 2)
@@ -416,6 +416,27 @@ def main():
                 for which, r in rep.items()}
             res["parity"]["subsets"] = "k: options with |oracle price| >= 2^-k max(S, K)"
             del call, put, ocall, oput
+        if "sets" in wl and not args.no_parity:
+            # The stream mix alone: the same three loads and two stores per element with a
+            # body of two multiply-adds, launched as this workload's kernel is (the float64
+            # kernel keeps its blocks for several runs because of its tables in LDS).
+            def mix(S, K_, T):
+                return hip.run_multi([S * K_ + T, S - K_ * T])
+            res["stream_mix"] = {"body": "S*K+T, S-K*T (same operands and results)"}
+            for label, cap in (("one_run_per_block", 0), ("blocks_that_stay", hip.TUNE["table_blocks"])):
+                hip.set_tune(flat_cap=cap)
+                try:
+                    for S, K_, T in wl["sets"]:
+                        ring[0] = mix(S, K_, T)
+                    with hip.record() as cold_mix:
+                        for j, (S, K_, T) in enumerate(wl["sets"]):
+                            ring[j] = mix(S, K_, T)
+                    mix_ms = statistics.median(kernel_regions(cold_mix, R, max(1, K // R)))
+                    del cold_mix
+                finally:
+                    hip.set_tune(flat_cap=0)
+                res["stream_mix"][label] = {"kernel_us": round(mix_ms * 1e3, 2),
+                                            "frac": round(wl["nbytes"] / mix_ms / 1e6 / HBM_PEAK_GBPS, 4)}
         if not args.no_unfused:
             # one kernel per node: its temporaries are re-read by the next kernel, so this
             # leg gets the cache policy that suits it (streams stay cacheable up to the
