@@ -85,7 +85,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all",
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
-                         "dot | axis0 | axis1 | rows200 | rowbcast | transpose | interior | stencil3d | "
+                         "dot | axis0 | axis1 | rows200 | rowbcast | transpose | transpose3d | interior | stencil3d | "
                          "grid | rand | next (these ten: the operations either side of the five "
                          "configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
@@ -230,6 +230,16 @@ def main():
                         desc=f"a @ b {np.dtype(dt).name} 8192^3 (eager matrix product on the matrix cores)",
                         steps=[lambda: a.dot(b)._force()],
                         cpu=lambda: ha[:m, :m] @ hb[:m, :m], cpu_frac=(m / N) ** 2, cpu_code="numpy.matmul")
+        if name == "transpose3d":
+            shape = (512, 512, 1024)
+            hv = rs.standard_normal(shape).astype(np.float32)
+            nel = hv.size
+            vols = [dr.array(hv) for _ in range(sets_for(8 * nel))]
+            return dict(dtype="f32", n=nel, nbytes=8 * nel,
+                        desc="a.T * 2 f32 512x512x1024 (all three axes reversed)",
+                        steps=[(lambda v=v: hip.run(v.T * 2.0)) for v in vols],
+                        cpu=lambda: hv[:, :, :256].T * np.float32(2.0), cpu_frac=0.25,
+                        cpu_code="numpy.multiply")
         if name in ("axis0", "axis1", "rowbcast", "transpose", "interior", "rows200"):
             N = 16384
             ha = rs.standard_normal((N, N)).astype(np.float32)
@@ -482,7 +492,7 @@ def main():
         return res
 
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
-             "next": ["dot", "axis0", "axis1", "rows200", "rowbcast", "transpose", "interior",
+             "next": ["dot", "axis0", "axis1", "rows200", "rowbcast", "transpose", "transpose3d", "interior",
                       "stencil3d", "grid", "rand"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}

@@ -1765,7 +1765,7 @@ T_TILE = 64      # square tile edge: both the transposed read and the write coal
 
 
 def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_load=False,
-                        nt_store=False, unaligned=False, tile=(T_TILE, T_TILE)):
+                        nt_store=False, unaligned=False, tile=(T_TILE, T_TILE), nbatch=0):
     """2-D tiled kernel for expressions in which some operand is walked along the
     output's rows by its unit stride (a transposed view).
 
@@ -1778,16 +1778,22 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
                element size, 16-byte aligned rows and row strides: tiles that lie
                wholly inside the output then move 16 bytes per lane on both sides
                (the transposition itself happens in LDS, one word at a time)
+    nbatch     further output dimensions (every dimension but the two the tiles span): the
+               matrices of a batch are transposed one after the other, a block's matrix
+               comes from its index (`a.T` of a 3-D array is 1 batch dimension in the
+               middle).
     Parameters: leaf pointers, output pointers, scalars, H, W, tiles_x, then per 't'
     leaf its stride along output columns, per 'd' leaf its row stride, per output its
-    row stride."""
+    row stride, then per batch dimension its extent and the stride of every leaf and of
+    every output along it."""
     rs = "__restrict__ " if restrict else ""
     n_out = len(out_dtypes)
     TR, TC = tile
     per_thread = TR * TC // BLOCK
     src = [PREAMBLE, emit_body(prog, out_dtypes)]
-    params = [f"const {CTYPE[dt]}* {rs}a{i}" for i, dt in enumerate(prog.leaves)]
-    params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
+    sfx = "_" if nbatch else ""          # with a batch the kernel offsets the pointers first
+    params = [f"const {CTYPE[dt]}* {rs}a{i}{sfx}" for i, dt in enumerate(prog.leaves)]
+    params += [f"{CTYPE[dt]}* {rs}o{i}{sfx}" for i, dt in enumerate(out_dtypes)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += ["const int H", "const int W", "const int tiles_x"]
     for i, k in enumerate(leaf_kind):
@@ -1797,16 +1803,37 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
         if k[0] == "d":
             params.append(f"const long long rs{i}")
     params += [f"const long long ors{o}" for o in range(n_out)]
+    for d in range(nbatch):
+        params.append(f"const long long bd{d}")
+        params += [f"const long long bs{i}_{d}" for i in range(len(prog.leaves))]
+        params += [f"const long long bos{o}_{d}" for o in range(n_out)]
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{"]
     for i, k in enumerate(leaf_kind):
         if k[0] == "t":
             L.append(f"    __shared__ {CTYPE[prog.leaves[i]]} tt{i}[{TC * (TR + 1)}];")
+    blk = "blockIdx.x"
+    if nbatch:
+        L += [f"    const long long per_matrix = (long long)tiles_x * ((H + {TR - 1}) / {TR});",
+              "    long long rem_b = blockIdx.x / per_matrix;",
+              "    const int tile_id = (int)(blockIdx.x - rem_b * per_matrix);"]
+        for i in range(len(prog.leaves)):
+            L.append(f"    long long boff{i} = 0;")
+        for o in range(n_out):
+            L.append(f"    long long boo{o} = 0;")
+        for d in reversed(range(nbatch)):
+            L.append(f"    {{ const long long c = rem_b % bd{d}; rem_b /= bd{d};")
+            L += [f"      boff{i} += c * bs{i}_{d};" for i in range(len(prog.leaves))]
+            L += [f"      boo{o} += c * bos{o}_{d};" for o in range(n_out)]
+            L.append("    }")
+        L += [f"    const {CTYPE[dt]}* {rs}a{i} = a{i}_ + boff{i};" for i, dt in enumerate(prog.leaves)]
+        L += [f"    {CTYPE[dt]}* {rs}o{o} = o{o}_ + boo{o};" for o, dt in enumerate(out_dtypes)]
+        blk = "tile_id"
     # Diagonal order: blocks that run at the same time differ in both tile coordinates.
     # With row-major order they would share r0, and the transposed operand's tiles
     # (rows a power-of-two pitch apart) would all fall into the same few memory channels.
-    L += ["    const int band = blockIdx.x / tiles_x;",
-          "    const int tx = blockIdx.x - band * tiles_x;",
+    L += [f"    const int band = {blk} / tiles_x;",
+          f"    const int tx = {blk} - band * tiles_x;",
           f"    const int ty = (band + tx) % ((H + {TR - 1}) / {TR});",
           f"    const int r0 = ty * {TR};",
           f"    const int c0 = tx * {TC};"]

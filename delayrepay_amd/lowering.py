@@ -517,26 +517,45 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             low.srcs, low.scal, low.tail = srcs, scal_vals, tail_vals
             return low
 
-    # operands walked along the output's rows by their unit stride (transposed views)
-    transposed = (not reduce_op and ndim == 2 and all(s[1] == 1 for s in m_out)
-                  and all(s[1] == 1 or s == [0, 0] or (s[0] == 1 and s[1] != 1) for s in m_leaf)
-                  and any(s[0] == 1 and s[1] != 1 for s in m_leaf))
+    # operands walked along some other output dimension by their unit stride (transposed
+    # views): tiles span that dimension and the last one, every further dimension is a batch
+    last = ndim - 1
+    t_dims = set()
+    for st in m_leaf:
+        if any(st) and st[last] != 1:
+            ones = [d for d in range(last) if st[d] == 1]
+            t_dims.add(ones[0] if len(ones) == 1 else -1)
+    transposed = (not reduce_op and ndim >= 2 and all(st[last] == 1 for st in m_out)
+                  and len(t_dims) == 1 and -1 not in t_dims)
     if transposed:
-        kinds = tuple(("b",) if s == [0, 0] else ("d",) if s[1] == 1 else ("t",) for s in m_leaf)
+        tp = next(iter(t_dims))
+        batch = [d for d in range(last) if d != tp]
+        nbatch_blocks = 1
+        for d in batch:
+            nbatch_blocks *= mshape[d]
+        kinds = tuple(("b",) if not any(st) else ("d",) if st[last] == 1 else ("t",) for st in m_leaf)
         # Tile: 128 bytes of the transposed operand's rows by 1 KB of the output's rows.  What
         # is written contiguously counts for more than what is read contiguously; float32
         # 16384^2, percent of the HBM peak: 64 x 64 elements 66, 128 x 64: 67, 64 x 128: 68,
         # 32 x 256: 73, 16 x 512: 60, 32 x 384: 64.
+        # An operand whose columns lie a megabyte or more apart (the reversed axes of a 3-D
+        # array) puts every column of a tile on another page: fewer, longer columns then
+        # (512 x 512 x 1024 float32 reversed: 32 x 256: 59, 64 x 64: 64, 128 x 64: 67,
+        # 128 x 32: 66, 256 x 32: 65).
         widest = max(cg.ITEMSIZE[c] for c in list(prog.leaves) + list(out_codes))
-        t_r, t_c = TUNE["t_rows"] or 128 // widest, TUNE["t_cols"] or 1024 // widest
+        far = max(abs(st[last]) * cg.ITEMSIZE[c] for st, c, k in zip(m_leaf, prog.leaves, kinds)
+                  if k[0] == "t") >= 1 << 20
+        t_r = TUNE["t_rows"] or (512 if far else 128) // widest
+        t_c = TUNE["t_cols"] or (256 if far else 1024) // widest
         lds_bytes = sum((t_r + 1) * t_c * cg.ITEMSIZE[c]
                         for c, k in zip(prog.leaves, kinds) if k[0] == "t")
         if lds_bytes > 64 * 1024:
             t_r = t_c = cg.T_TILE
             lds_bytes = sum((t_r + 1) * t_c * cg.ITEMSIZE[c]
                             for c, k in zip(prog.leaves, kinds) if k[0] == "t")
-        if lds_bytes <= 64 * 1024:
-            H, W = mshape
+        if lds_bytes <= 64 * 1024 and (-(-mshape[tp] // t_r) * -(-mshape[last] // t_c)
+                                       * nbatch_blocks < 2 ** 31) and len(batch) <= 4:
+            H, W = mshape[tp], mshape[last]
             low.kind = "tile2dt"
             # 16 bytes per lane on both sides when every array has the same element
             # size and all rows (of the operands' own layouts) start 16-byte aligned
@@ -544,45 +563,49 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             vec = 16 // sizes.pop() if len(sizes) == 1 and sizes <= {4, 8} and TUNE["tvec"] else 0
             ua = False
             if vec and all(c in cg.VEC16 for c in list(prog.leaves) + list(out_codes)):
-                pitches = [(st[1] if k[0] == "t" else st[0], a.offset)
+                pitches = [(st[last] if k[0] == "t" else st[tp], a.offset)
                            for a, k, st in zip(leaves, kinds, m_leaf) if k[0] != "b"]
-                pitches += [(st[0], ptr // cg.ITEMSIZE[c]) for ptr, st, c in zip(out_ptrs, m_out, out_codes)
+                pitches += [(st[tp], ptr // cg.ITEMSIZE[c]) for ptr, st, c in zip(out_ptrs, m_out, out_codes)
                             if ptr % cg.ITEMSIZE[c] == 0]
                 if len(pitches) != len(out_ptrs) + sum(k[0] != "b" for k in kinds):
                     vec = 0
-                elif any(pitch % vec or first % vec for pitch, first in pitches):
+                elif any(pitch % vec or first % vec for pitch, first in pitches) or any(
+                        st[d] % vec for st in list(m_leaf) + list(m_out) for d in batch):
                     ua = True               # vectors at element alignment
                     vec = vec if TUNE["uvec"] else 0
             else:
                 vec = 0
-            out_bytes = sum(H * W * cg.ITEMSIZE[c] for c in out_codes)
-            in_bytes = sum(H * W * cg.ITEMSIZE[c] for c, k in zip(prog.leaves, kinds) if k[0] != "b")
+            out_bytes = sum(n * cg.ITEMSIZE[c] for c in out_codes)
+            in_bytes = sum(n * cg.ITEMSIZE[c] for c, k in zip(prog.leaves, kinds) if k[0] != "b")
             nts = bool(vec and TUNE["nts"]) and in_bytes + out_bytes > TUNE["cache_mib"] << 20
             ntl = bool(vec and TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
             ua = bool(ua and vec)
             low.key = ("tile2dt", prog.key(), kinds, tuple(out_codes), in_place, vec, ntl, nts, ua,
-                       t_r, t_c)
+                       t_r, t_c, len(batch))
 
             def emit():
                 return cg.emit_tile_transpose(prog, kinds, out_codes, restrict=not in_place,
                                               vec=vec, nt_load=ntl, nt_store=nts, unaligned=ua,
-                                              tile=(t_r, t_c))
+                                              tile=(t_r, t_c), nbatch=len(batch))
             low.emit = emit
             tiles_x = -(-W // t_c)
-            low.grid = tiles_x * -(-H // t_r)
+            low.grid = tiles_x * -(-H // t_r) * nbatch_blocks
             fmt = "@" + "P" * (len(leaves) + len(out_ptrs)) + scal_fmt + "iii"
             tail_vals = [H, W, tiles_x]
             for k, s in zip(kinds, m_leaf):
                 if k[0] == "t":
                     fmt += "q"
-                    tail_vals.append(s[1])
+                    tail_vals.append(s[last])
             for k, s in zip(kinds, m_leaf):
                 if k[0] == "d":
                     fmt += "q"
-                    tail_vals.append(s[0])
+                    tail_vals.append(s[tp])
             for s in m_out:
                 fmt += "q"
-                tail_vals.append(s[0])
+                tail_vals.append(s[tp])
+            for d in batch:
+                fmt += "q" * (1 + len(m_leaf) + len(m_out))
+                tail_vals += [mshape[d]] + [st[d] for st in m_leaf] + [st[d] for st in m_out]
             low.fmt = fmt
             low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
             low.scal, low.tail = scal_vals, tail_vals

@@ -1106,6 +1106,31 @@ def test_reductions_over_the_rows_of_wide_matrices_stream_whole_rows():
     assert np.allclose(v, h.astype(np.float64).var(axis=0), rtol=1e-4)
 
 
+def test_transposes_of_arrays_with_more_than_two_dimensions_go_through_the_lds_tile():
+    """Every permutation whose unit stride lands on another output dimension: the two
+    dimensions the tiles span are transposed through LDS, the others are a batch."""
+    import itertools
+    rs = np.random.RandomState(37)
+    for shape, dt in [((5, 70, 33), np.float32), ((3, 4, 130, 9), np.float64), ((40, 36, 64), np.float32),
+                      ((6, 50, 20), np.int8)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int8 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        for perm in itertools.permutations(range(len(shape))):
+            if perm[-1] == len(shape) - 1:
+                continue
+            ex = dr.transpose(a, perm) * 2
+            low = hip.lower_only(ex)[0]
+            assert low.kind == "tile2dt", (shape, perm, low.kind)
+            assert np.array_equal(ex.get(), h.transpose(perm) * 2), (shape, perm)
+    h = rs.uniform(-1, 1, (24, 40, 64)).astype(np.float32)
+    d = rs.uniform(-1, 1, (64, 40, 24)).astype(np.float32)
+    col = rs.uniform(-1, 1, (40, 1)).astype(np.float32)
+    got = (dr.array(h).T + dr.array(d) * 3.0 + dr.array(col)).get()      # reversed axes, a dense
+    assert np.array_equal(got, h.T + d * np.float32(3.0) + col)          # operand and a broadcast
+    big = rs.uniform(-1, 1, (64, 96, 128))
+    assert np.array_equal((dr.array(big).T * 2.0).get(), big.T * 2.0)
+
+
 def test_reduction_strategy_follows_the_operands_that_carry_the_traffic():
     """A column of weights beside a matrix (unit stride along the reduced axis) must not
     switch a sum over rows to the kernel for sums along rows."""
