@@ -55,9 +55,9 @@ CTYPE = {
     "b1": "unsigned char",
 }
 ITEMSIZE = {"f4": 4, "f8": 8, "i4": 4, "i8": 8, "u4": 4, "u1": 1, "b1": 1}
-# 16-byte vector type per dtype code (only 4- and 8-byte element types vectorise)
+# 16-byte vector type per dtype code (bytes only in flat kernels: masks and their users)
 VEC16 = {"f4": ("f4x4", 4), "f8": ("f8x2", 2), "i4": ("i4x4", 4), "i8": ("i8x2", 2),
-         "u4": ("u4x4", 4)}
+         "u4": ("u4x4", 4), "u1": ("u1x16", 16), "b1": ("u1x16", 16)}
 
 PREAMBLE = """\
 typedef float f4x4 __attribute__((ext_vector_type(4)));
@@ -70,6 +70,8 @@ typedef double f8x2u __attribute__((ext_vector_type(2), aligned(8)));
 typedef int i4x4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef long long i8x2u __attribute__((ext_vector_type(2), aligned(8)));
 typedef unsigned int u4x4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned char u1x16 __attribute__((ext_vector_type(16)));
+typedef unsigned char u1x16u __attribute__((ext_vector_type(16), aligned(1)));
 """
 # The `...u` types are the same vectors at element alignment: global memory takes 16-byte
 # accesses at any 4-byte address (measured on MI355X: 6.2-6.6 TB/s for a copy shifted by one

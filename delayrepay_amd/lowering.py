@@ -280,10 +280,12 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     if flat:
         leaf_class = tuple("b" if (s == [0] and n > 1) else "c" for s in m_leaf)
         ptrs = [a.ptr for a in leaves]
-        widths_ok = all(cg.ITEMSIZE[c] in (4, 8) for c, k in zip(prog.leaves, leaf_class) if k == "c")
+        # bytes (masks) move as vectors of sixteen; the wider operands beside them then take
+        # four or eight vectors per thread
+        widths_ok = all(c in cg.VEC16 for c, k in zip(prog.leaves, leaf_class) if k == "c")
         align_ok = all(p % 16 == 0 for p, k in zip(ptrs, leaf_class) if k == "c")
         if not reduce_op:
-            widths_ok = widths_ok and all(cg.ITEMSIZE[c] in (4, 8) for c in out_codes)
+            widths_ok = widths_ok and all(c in cg.VEC16 for c in out_codes)
             align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
         vec = widths_ok and n >= 64 and (align_ok or bool(TUNE["uvec"]))
         ua = vec and not align_ok      # vectors at element alignment
@@ -443,7 +445,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             kinds = tuple(("dv",) if d else k for d, k in zip(dv, kinds))
             gpr, rpt = TUNE["gpr"], TUNE["rpt"]
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
-            streams = all(any(st[:-1]) for st, k in zip(m_leaf, kinds) if k[0] in ("d", "dv"))
+            streams = all(all(st[:-1]) for st, k in zip(m_leaf, kinds) if k[0] in ("d", "dv"))
             if group is None and TUNE["row_gpr"] and streams:
                 # Nothing is shared between rows: a block takes one stretch of a row, as
                 # long as the row allows (up to 4 KB), like a chunk of a flat kernel, and
@@ -451,7 +453,8 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                 # 16384^2 float32, percent of the HBM peak: tiles of 8 rows x 256 columns
                 # 66, with non-temporal loads 69, 2 rows x 512: 76, 1 row x 1024: 80
                 # (a flat copy: 81); more rows per thread are slower (4: 70).  An operand that
-                # repeats from row to row keeps the taller tile, whose rows share it in L1.
+                # repeats along some outer dimension keeps the taller tile, whose rows share
+                # it in L1.
                 gpr = 16
                 while gpr < TUNE["row_gpr"] and gpr * vw < W + ph_o:
                     gpr *= 2

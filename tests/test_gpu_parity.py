@@ -1131,6 +1131,27 @@ def test_transposes_of_arrays_with_more_than_two_dimensions_go_through_the_lds_t
     assert np.array_equal((dr.array(big).T * 2.0).get(), big.T * 2.0)
 
 
+def test_masks_move_as_vectors_of_sixteen_bytes():
+    """Bool and uint8 operands and results in flat kernels: sixteen per lane and access, the
+    wider operands beside them four or eight vectors; lengths that are not multiples of
+    sixteen, views that start at odd bytes."""
+    rs = np.random.RandomState(47)
+    for n in (1 << 20, (1 << 20) + 13, 100, 65):
+        ha, hb = rs.uniform(-1, 1, n).astype(np.float32), rs.uniform(-1, 1, n)
+        hm = rs.uniform(-1, 1, n) > 0
+        hu = rs.randint(0, 200, n).astype(np.uint8)
+        a, b, m, u = dr.array(ha), dr.array(hb), dr.array(hm), dr.array(hu)
+        low, src = hip.lower_only(a > 0)
+        assert low.kind == "flat" and (n < 64 or "u1x16" in src)
+        assert np.array_equal((a > 0).get(), ha > 0)
+        assert np.array_equal(dr.where(m, a, b).get(), np.where(hm, ha, hb))
+        assert np.array_equal(np.logical_and(m, a > b).get(), np.logical_and(hm, ha > hb))
+        assert np.array_equal((u + np.uint8(3)).get(), hu + np.uint8(3))
+        assert np.array_equal(dr.where(m[1:], a[1:], 0.5).get(), np.where(hm[1:], ha[1:], np.float32(0.5)))
+        assert np.array_equal((u[3:] * a[3:]).get(), hu[3:] * ha[3:])
+        assert dr.sum(m) == hm.sum() and dr.sum(u) == hu.sum()
+
+
 def test_reduction_strategy_follows_the_operands_that_carry_the_traffic():
     """A column of weights beside a matrix (unit stride along the reduced axis) must not
     switch a sum over rows to the kernel for sums along rows."""
