@@ -72,7 +72,30 @@ typedef long long i8x2u __attribute__((ext_vector_type(2), aligned(8)));
 typedef unsigned int u4x4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef unsigned char u1x16 __attribute__((ext_vector_type(16)));
 typedef unsigned char u1x16u __attribute__((ext_vector_type(16), aligned(1)));
+typedef float f4x2 __attribute__((ext_vector_type(2)));
+typedef int i4x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u4x2 __attribute__((ext_vector_type(2)));
+typedef unsigned char u1x2 __attribute__((ext_vector_type(2)));
+typedef unsigned char u1x4 __attribute__((ext_vector_type(4)));
+typedef unsigned char u1x8 __attribute__((ext_vector_type(8)));
+typedef float f4x2u __attribute__((ext_vector_type(2), aligned(4)));
+typedef int i4x2u __attribute__((ext_vector_type(2), aligned(4)));
+typedef unsigned int u4x2u __attribute__((ext_vector_type(2), aligned(4)));
+typedef unsigned char u1x2u __attribute__((ext_vector_type(2), aligned(1)));
+typedef unsigned char u1x4u __attribute__((ext_vector_type(4), aligned(1)));
+typedef unsigned char u1x8u __attribute__((ext_vector_type(8), aligned(1)));
 """
+
+
+def flat_vec(dt, E):
+    """(vector type, elements per vector, vectors per thread) a flat kernel uses for a
+    stream of type `dt` when a thread handles E elements per step: the whole 16-byte
+    vector, several of them (only when E exceeds it), or a shorter vector of E elements,
+    so that the lanes of a wave always read one contiguous stretch."""
+    vt, per = VEC16[dt]
+    if E >= per:
+        return vt, per, E // per
+    return f"{vt.split('x')[0]}x{E}", E, 1
 # The `...u` types are the same vectors at element alignment: global memory takes 16-byte
 # accesses at any 4-byte address (measured on MI355X: 6.2-6.6 TB/s for a copy shifted by one
 # to three floats against 6.7 TB/s aligned, and 3.5 TB/s with one element per lane), so
@@ -251,15 +274,20 @@ def _philox_value(name, raw):
 
 
 def flat_elements(prog, leaf_class, out_dtypes, reduce_op):
-    """Elements one thread handles per vector step of the flat kernel: enough to fill a
-    16-byte vector of the narrowest streamed type; four when the program draws Philox
-    numbers, whose blocks hold four outputs (a thread then makes each block once)."""
+    """Elements one thread handles per vector step of the flat kernel: a 16-byte vector of
+    the widest streamed type (narrower streams move shorter vectors, see `flat_vec`: with
+    several vectors of the wider type per lane a wave's load would touch every cache line
+    of its stretch once per vector: float32 x float64 68 % of the HBM peak, a mask beside
+    two float32 operands 31 %); four when the program draws Philox numbers, whose blocks
+    hold four outputs (a thread then makes each block once)."""
     widths = [ITEMSIZE[dt] for dt, c in zip(prog.leaves, leaf_class) if c == "c"]
     if not reduce_op:
         widths += [ITEMSIZE[dt] for dt in out_dtypes]
     if any(name.startswith("philox") for name, _, _, _ in prog.ops):
         widths.append(4)
-    return 16 // min(widths) if widths else 4
+    if any(name.startswith("philox") for name, _, _, _ in prog.ops):
+        return 16 // min(widths)
+    return 16 // max(widths) if widths else 4
 
 
 class Program:
@@ -558,9 +586,8 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
             if c != "c":
                 continue
             if vec:
-                vt, per = VEC16[dt]
+                vt, per, chunks = flat_vec(dt, E)
                 vt += ua
-                chunks = E // per
                 for ch in range(chunks):
                     ptr = f"(const {vt}*)a{i} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
                         else f"(const {vt}*)a{i} + ({idx})"
@@ -570,8 +597,8 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                              f"{_ld(nt_load, f'a{i} + ({idx})')};")
         if vec and not reduce_op:
             for o, dt in enumerate(out_dtypes):
-                vt, per = VEC16[dt]
-                for ch in range(E // per):
+                vt, per, chunks = flat_vec(dt, E)
+                for ch in range(chunks):
                     work.append(f"{pad}{vt} R{o}_{ch}{tag};")
         for e in range(E):
             args = []
@@ -579,7 +606,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                 if c == "b":
                     args.append(f"b{i}")
                 elif vec:
-                    per = VEC16[dt][1]
+                    per = flat_vec(dt, E)[1]
                     args.append(f"L{i}_{e // per}{tag}[{e % per}]")
                 else:
                     args.append(f"L{i}{tag}")
@@ -590,16 +617,15 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
             if reduce_op:
                 tail = f"acc{e} = {_combine(reduce_op, f'acc{e}', 't0')};"
             elif vec:
-                tail = " ".join(f"R{o}_{e // VEC16[dt][1]}{tag}[{e % VEC16[dt][1]}] = t{o};"
+                tail = " ".join(f"R{o}_{e // flat_vec(dt, E)[1]}{tag}[{e % flat_vec(dt, E)[1]}] = t{o};"
                                 for o, dt in enumerate(out_dtypes))
             else:
                 tail = " ".join(_st(nt_store, f"t{o}", f"o{o} + ({idx})") for o in range(n_out))
             work.append(f"{pad}{{ {decl} {call} {tail} }}")
         if vec and not reduce_op:
             for o, dt in enumerate(out_dtypes):
-                vt, per = VEC16[dt]
+                vt, per, chunks = flat_vec(dt, E)
                 vt += ua
-                chunks = E // per
                 for ch in range(chunks):
                     ptr = f"({vt}*)o{o} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
                         else f"({vt}*)o{o} + ({idx})"
@@ -635,7 +661,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
             if c == "b":
                 args.append(f"b{i}")
                 continue
-            per = VEC16[dt][1]
+            per = flat_vec(dt, E)[1]
             items = ", ".join(f"L{i}_{e // per}_u{u}[{e % per}]" for u in range(unroll)
                               for e in range(E))
             all_work.append(f"{pad}const {CTYPE[dt]} P{i}[{P}] = {{{items}}};")
@@ -650,8 +676,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                     all_work.append(f"{pad}acc{e} = {_combine(reduce_op, f'acc{e}', f'T0[{u * E + e}]')};")
                 continue
             for o, dt in enumerate(out_dtypes):
-                vt, per = VEC16[dt]
-                chunks = E // per
+                vt, per, chunks = flat_vec(dt, E)
                 for ch in range(chunks):
                     items = ", ".join(f"T{o}[{u * E + ch * per + k}]" for k in range(per))
                     idx = f"v + {u * BLOCK}" if u else "v"
