@@ -304,8 +304,15 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                               ("divide", "true_divide", "reciprocal")) and name not in cheap else 1
                        for name, _, _, _ in prog.ops)
             light = cost <= 4 * n_in + 4
-            unroll = unroll or (max(1, min(8, 8 // n_in)) if light else 4)
-            red_cap = red_cap or (grid_cap() // TUNE["bpc"] if light else 4096)
+            # one operand: 6 vectors in flight 89.9, 8: 87.1, 4: 75.3.  Maxima and minima (NaN
+            # checks per element) want two blocks per compute unit with half as many vectors
+            # each: 87.9 against 75.7.
+            per_lane = {1: 6, 2: 4, 3: 2, 4: 2}.get(n_in, 1)
+            cus = grid_cap() // TUNE["bpc"]
+            if light and reduce_op != "add":
+                per_lane, cus = max(1, per_lane // 2 + per_lane % 2), 2 * cus
+            unroll = unroll or (per_lane if light else 4)
+            red_cap = red_cap or (cus if light else 4096)
         packed = bool(cg.packs(prog, vec) and TUNE["pack"])
         if not unroll and packed:
             unroll = 1          # the pack below decides
