@@ -1718,7 +1718,7 @@ def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8):
     return "\n".join(src) + "\n"
 
 
-def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4):
+def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False):
     """Reduction over a long unit-stride last dimension: a block per (row, slice) streams
     its stretch of the row like a flat reduction (256 lanes x 16 bytes x `unroll` per step,
     one accumulator per vector element), combines through `dr_block_reduce` and writes one
@@ -1727,8 +1727,12 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4):
     flat reduction).
 
     leaf_kind  per leaf 'v' (unit stride along the row) or 'k' (constant along it)
+    outer      a second, outer reduced dimension (sum over the first and last axis of a
+               3-D array): a block then takes whole rows, a slice of the outer range
     Parameters: leaf pointers, output pointer, scalars, K, R, S, RS, then per leaf the
-    stride between rows (elements).  Output layout [row][slice]."""
+    stride between rows (elements); with `outer` R is the row length, S and RS cut the
+    outer extent RO, and RO and every leaf's outer stride follow.  Output layout
+    [row][slice]."""
     ct = CTYPE[acc_dt]
     nl = len(prog.leaves)
     widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "v"}
@@ -1739,6 +1743,9 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4):
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += ["const long long K", "const long long R", "const long long S", "const long long RS"]
     params += [f"const long long sk{i}" for i in range(nl)]
+    if outer:
+        params.append("const long long RO")
+        params += [f"const long long so{i}" for i in range(nl)]
     call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
     ident = _identity(op, acc_dt)
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
@@ -1746,34 +1753,48 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4):
          "    for (long long o = blockIdx.x; o < K * S; o += gridDim.x) {",
          "        const long long k = o / S;",
          "        const long long sl = o - k * S;",
-         "        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;"]
+         f"        {ct} acc[{V}];",
+         "#pragma unroll",
+         f"        for (int e = 0; e < {V}; ++e) acc[e] = {ident};"]
+    if outer:
+        L += ["        const long long q_end = (sl + 1) * RS < RO ? (sl + 1) * RS : RO;",
+              "        const long long r_end = R;",
+              f"#pragma unroll {unroll}",
+              "        for (long long q = sl * RS; q < q_end; ++q) {"]
+        base = lambda i: f"a{i} + k * sk{i} + q * so{i}"
+        const = lambda i: f"a{i}[k * sk{i} + q * so{i}]"
+        first, pad = f"(long long)threadIdx.x * {V}", "    "
+    else:
+        L.append("        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;")
+        base = lambda i: f"a{i} + k * sk{i}"
+        const = lambda i: f"a{i}[k * sk{i}]"
+        first, pad = f"sl * RS + (long long)threadIdx.x * {V}", ""
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
-            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+            L.append(f"{pad}        const {CTYPE[dt]}* row{i} = {base(i)};")
         else:
-            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
-    L += [f"        {ct} acc[{V}];",
-          "#pragma unroll",
-          f"        for (int e = 0; e < {V}; ++e) acc[e] = {ident};",
-          f"        long long r = sl * RS + (long long)threadIdx.x * {V};",
-          f"#pragma unroll {unroll}",
-          f"        for (; r + {V} <= r_end; r += {BLOCK * V}) {{"]
+            L.append(f"{pad}        const {CTYPE[dt]} c{i} = {const(i)};")
+    L += [f"{pad}        long long r = {first};",
+          f"#pragma unroll {1 if outer else unroll}",
+          f"{pad}        for (; r + {V} <= r_end; r += {BLOCK * V}) {{"]
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
             vt = VEC16[dt][0] + "u"
-            L.append(f"            const {vt} X{i} = __builtin_nontemporal_load((const {vt}*)(row{i} + r));")
+            L.append(f"{pad}            const {vt} X{i} = __builtin_nontemporal_load((const {vt}*)(row{i} + r));")
     for e in range(V):
         vargs = [f"X{i}[{e}]" if kind == "v" else f"c{i}" for i, kind in enumerate(leaf_kind)]
-        L.append(f"            {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
+        L.append(f"{pad}            {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
                  f"acc[{e}] = {_combine(op, f'acc[{e}]', 't0')}; }}")
-    L.append("        }")
+    L.append(f"{pad}        }}")
     # exactly one thread is left with r < r_end: the one whose next vector would straddle
     # the end of the stretch; it takes those elements one by one
     sargs = [f"row{i}[r]" if kind == "v" else f"c{i}" for i, kind in enumerate(leaf_kind)]
-    L += ["        for (; r < r_end; ++r) {",
-          f"            {ct} t0; dr_body({', '.join(sargs + call_tail)});",
-          f"            acc[0] = {_combine(op, 'acc[0]', 't0')};",
-          "        }"]
+    L += [f"{pad}        for (; r < r_end; ++r) {{",
+          f"{pad}            {ct} t0; dr_body({', '.join(sargs + call_tail)});",
+          f"{pad}            acc[0] = {_combine(op, 'acc[0]', 't0')};",
+          f"{pad}        }}"]
+    if outer:
+        L.append("        }")
     accs = [f"acc[{e}]" for e in range(V)]
     while len(accs) > 1:
         accs = [f"({_combine(op, accs[i], accs[i + 1])})" if i + 1 < len(accs) else accs[i]

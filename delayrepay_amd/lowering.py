@@ -803,6 +803,35 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
                 low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
                 low.scal, low.tail = list(scalars), [K, R, S, RS] + [r[0] for r in rsets]
                 return low, S, K, "col"
+    if (strategy == "row" and slices is None and len(rmerged) == 2 and len(kmerged) == 1
+            and rmerged[1] >= 1024 and TUNE["ax_block"] > 0 and TUNE["uvec"]
+            and all(r[1] in (0, 1) for r in rsets)):
+        widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[1] == 1}
+        if len(widths) == 1 and widths <= {4, 8} and all(
+                c in cg.VEC16 for c, r in zip(prog.leaves, rsets) if r[1] == 1):
+            # the first and the last axis of a 3-D array reduced (per-channel statistics): a
+            # block takes whole rows of the last axis over a slice of the first
+            RO, RI = rmerged
+            S = max(1, min(-(-TUNE["ax_blocks"] // K), RO // 4, TUNE["ax_slices"]))
+            QS = -(-RO // S)
+            S = -(-RO // QS)
+            kinds = tuple("v" if r[1] == 1 else "k" for r in rsets)
+            low = Lowered()
+            low.lds = 0
+            low.fin_count = 0
+            low.kind = "axis_block"
+            low.key = ("axis_block", prog.key(), kinds, acc, reduce_op, "outer")
+
+            def emit_block2():
+                return cg.emit_block_rows(prog, kinds, acc, reduce_op, outer=True)
+            low.emit = emit_block2
+            low.grid = max(1, min(K * S, 1 << 20))
+            low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+                       + "qqqq" + "q" * len(leaves) + "q" + "q" * len(leaves))
+            low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+            low.scal = list(scalars)
+            low.tail = [K, RI, S, QS] + [k[0] for k in ksets] + [RO] + [r[0] for r in rsets]
+            return low, S, K, "row"
     if (strategy == "row" and slices is None and len(rmerged) == 1 and len(kmerged) == 1
             and R >= TUNE["ax_block"] > 0 and TUNE["uvec"] and all(r[0] in (0, 1) for r in rsets)):
         widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == 1}

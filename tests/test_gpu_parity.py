@@ -1081,6 +1081,27 @@ def test_reductions_over_long_rows_take_a_block_per_row_slice():
     assert np.allclose(m, h.mean(axis=1, dtype=np.float64), rtol=2e-5)
 
 
+def test_reductions_over_the_first_and_last_axis_of_a_three_dimensional_array():
+    """Per-channel statistics: (N, C, L) reduced over N and L; rows of the last axis that
+    are not multiples of the vector, an operand constant along the last axis."""
+    rs = np.random.RandomState(33)
+    for shape, dt in [((9, 5, 1024), np.float32), ((33, 7, 1500), np.float64), ((4, 3, 2049), np.int32)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (0, 2)))[0]
+        assert low.kind == "axis_block" and low.key[-1] == "outer", (shape, low.kind)
+        tol = dict(rtol=2e-5, atol=1e-4) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
+        assert np.allclose(dr.sum(a * a, axis=(0, 2)).get(), (h.astype(np.float64) ** 2).sum(axis=(0, 2)), **tol)
+        assert np.array_equal(dr.max(a, axis=(0, 2)).get(), h.max(axis=(0, 2)))
+        assert np.array_equal(dr.min(a[1:, :, 3:-2], axis=(0, 2)).get(), h[1:, :, 3:-2].min(axis=(0, 2)))
+    h = rs.uniform(0, 1, (40, 6, 1100)).astype(np.float32)
+    w = rs.uniform(0, 1, (40, 6, 1)).astype(np.float32)
+    got = dr.sum(dr.array(h) * dr.array(w), axis=(0, 2)).get()
+    assert np.allclose(got, (h.astype(np.float64) * w).sum(axis=(0, 2)), rtol=2e-5)
+    m = dr.mean(dr.array(h), axis=(0, 2)).get()
+    assert np.allclose(m, h.mean(axis=(0, 2), dtype=np.float64), rtol=2e-5)
+
+
 def test_reductions_over_the_rows_of_wide_matrices_stream_whole_rows():
     """Kept rows of 256 vectors or more: a block owns 256 lanes x one vector of columns and
     walks a slice of rows; widths that are not multiples of the vector, views that start off
