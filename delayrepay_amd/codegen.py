@@ -141,8 +141,13 @@ _BOOL_ARITH = {"add": "|", "maximum": "|", "fmax": "|", "multiply": "&", "minimu
 _PREDICATES = {"isnan", "isinf", "isfinite", "logical_not", "logical_and", "logical_or",
                "logical_xor"}
 
+# integer and bool operands only (NumPy has no loop for floats: the type probe raises its
+# TypeError); on bool they are the logical operations
+_BITWISE = {"bitwise_and": "&", "bitwise_or": "|", "bitwise_xor": "^"}
+_SHIFTS = {"left_shift": "<<", "right_shift": ">>"}
+
 SUPPORTED_UFUNCS = (set(_FLOAT_FUNCS1) | set(_FLOAT_FUNCS2) | set(_INFIX) | set(_COMPARE)
-                    | _PREDICATES
+                    | _PREDICATES | set(_BITWISE) | set(_SHIFTS) | {"invert"}
                     | {"negative", "positive", "absolute", "fabs", "reciprocal", "maximum",
                        "minimum", "square", "sign"})
 
@@ -164,6 +169,26 @@ def op_expr(name, dt, args):
             raise TypeError(f"numpy boolean {name} is not supported, as in NumPy "
                             "(use bitwise or logical operations instead)")
         return f"(unsigned char)({args[0]} {op} {args[1]})"
+    if name in _BITWISE:
+        if is_float:
+            raise TypeError(f"ufunc {name!r} not supported for float operands")
+        return f"({CTYPE[dt]})({args[0]} {_BITWISE[name]} {args[1]})"
+    if name == "invert":
+        if is_float:
+            raise TypeError("ufunc 'invert' not supported for float operands")
+        return f"(unsigned char)({args[0]} == 0)" if dt == "b1" else f"({CTYPE[dt]})(~{args[0]})"
+    if name in _SHIFTS:
+        if is_float or dt == "b1":
+            raise TypeError(f"ufunc {name!r} not supported for these operands")
+        # counts of the type's width or more shift everything out, as in NumPy (the
+        # hardware would use the count modulo the width)
+        bits = 8 * ITEMSIZE[dt]
+        a, b = args
+        uns = "unsigned " + CTYPE[dt] if dt[0] == "i" else CTYPE[dt]
+        if name == "left_shift":
+            return f"(({uns}){b} >= {bits} ? ({CTYPE[dt]})0 : ({CTYPE[dt]})(({uns}){a} << {b}))"
+        fill = f"({CTYPE[dt]})({a} < 0 ? -1 : 0)" if dt[0] == "i" else f"({CTYPE[dt]})0"
+        return f"(({uns}){b} >= {bits} ? {fill} : ({CTYPE[dt]})({a} >> {b}))"
     if name in _INFIX:
         if name in ("divide", "true_divide") and not is_float:
             raise NotImplementedError("integer division has no float result type here")
@@ -1650,7 +1675,7 @@ def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
     return "\n".join(src) + "\n"
 
 
-def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8):
+def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8, outer=False, stagger=True):
     """Reduction over the rows of a matrix whose kept dimension has unit stride: a block owns
     256 x V adjacent columns (V the elements of a 16-byte vector: 4 KB of every row) and a
     slice of rows, and walks the rows with `unroll` loads in flight per lane; every lane
@@ -1658,8 +1683,15 @@ def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8):
     column tiles are adjacent in launch order: together they read whole rows.
 
     leaf_kind  per leaf 'v' (unit stride along the kept dimension) or 'k' (constant along it)
+    stagger    every block starts its walk at a different row of its slice and wraps round:
+               slices whose first rows lie a power of two apart (8 x 8192 x 2048 float32
+               summed over the middle axis) otherwise march over the same memory channels
+               in step (measured 60 % of the HBM peak in step, 82 % staggered)
+    outer      a second, outer kept dimension (the middle axis of a 3-D array reduced): its
+               index is part of the block number, column tiles stay inside one row
     Parameters: leaf pointers, output pointer, scalars, K, R, S, RS, then per leaf the
-    stride between rows (elements).  Output layout [slice][column]."""
+    stride between rows (elements); with `outer` its extent KO and every leaf's stride
+    along it follow.  Output layout [slice][outer][column]."""
     ct = CTYPE[acc_dt]
     nl = len(prog.leaves)
     widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "v"}
@@ -1671,34 +1703,52 @@ def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8):
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += ["const long long K", "const long long R", "const long long S", "const long long RS"]
     params += [f"const long long sr{i}" for i in range(nl)]
+    if outer:
+        params.append("const long long KO")
+        params += [f"const long long sko{i}" for i in range(nl)]
     call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
     ident = _identity(op, acc_dt)
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{",
-         f"    const long long ktiles = (K + {TK - 1}) / {TK};",
-         "    for (long long b = blockIdx.x; b < ktiles * S; b += gridDim.x) {",
-         "        const long long sl = b / ktiles;",
-         f"        const long long g = (b - sl * ktiles) * {TK} + (long long)threadIdx.x * {V};",
+         f"    const long long ktiles = (K + {TK - 1}) / {TK};"]
+    if outer:
+        L += ["    for (long long b = blockIdx.x; b < ktiles * KO * S; b += gridDim.x) {",
+              "        const long long sl = b / (ktiles * KO);",
+              "        const long long ko = (b - sl * ktiles * KO) / ktiles;",
+              "        const long long kt = b - (sl * KO + ko) * ktiles;"]
+        L += [f"        const {CTYPE[dt]}* A{i} = a{i} + ko * sko{i};" for i, dt in enumerate(prog.leaves)]
+        L.append(f"        {ct}* O = out + (sl * KO + ko) * K;")
+    else:
+        L += ["    for (long long b = blockIdx.x; b < ktiles * S; b += gridDim.x) {",
+              "        const long long sl = b / ktiles;",
+              "        const long long kt = b - sl * ktiles;"]
+        L += [f"        const {CTYPE[dt]}* A{i} = a{i};" for i, dt in enumerate(prog.leaves)]
+        L.append(f"        {ct}* O = out + sl * K;")
+    L += [f"        const long long g = kt * {TK} + (long long)threadIdx.x * {V};",
          "        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;",
+         f"        const long long r_mid = sl * RS + {'(b * 37) % (r_end - sl * RS)' if stagger else '0'};",
          f"        {ct} acc[{V}];",
          "#pragma unroll",
          f"        for (int e = 0; e < {V}; ++e) acc[e] = {ident};",
          f"        if (g + {V} <= K) {{",
+         "          for (int half = 0; half < 2; ++half) {",
+         "            const long long ra = half ? sl * RS : r_mid, rb = half ? r_mid : r_end;",
          f"#pragma unroll {unroll}",
-         "            for (long long r = sl * RS; r < r_end; ++r) {"]
+         "            for (long long r = ra; r < rb; ++r) {"]
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
             vt = VEC16[dt][0] + "u"
-            L.append(f"                const {vt} X{i} = __builtin_nontemporal_load((const {vt}*)(a{i} + g + r * sr{i}));")
+            L.append(f"                const {vt} X{i} = __builtin_nontemporal_load((const {vt}*)(A{i} + g + r * sr{i}));")
         else:
-            L.append(f"                const {CTYPE[dt]} c{i} = a{i}[r * sr{i}];")
+            L.append(f"                const {CTYPE[dt]} c{i} = A{i}[r * sr{i}];")
     for e in range(V):
         vargs = [f"X{i}[{e}]" if kind == "v" else f"c{i}" for i, kind in enumerate(leaf_kind)]
         L.append(f"                {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
                  f"acc[{e}] = {_combine(op, f'acc[{e}]', 't0')}; }}")
-    sargs = [f"a{i}[g + e + r * sr{i}]" if kind == "v" else f"a{i}[r * sr{i}]"
+    sargs = [f"A{i}[g + e + r * sr{i}]" if kind == "v" else f"A{i}[r * sr{i}]"
              for i, kind in enumerate(leaf_kind)]
     L += ["            }",
+          "          }",
           "        } else if (g < K) {          // the vector that straddles the last column",
           "            for (long long r = sl * RS; r < r_end; ++r) {",
           "#pragma unroll",
@@ -1712,7 +1762,7 @@ def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8):
           "        }",
           "#pragma unroll",
           f"        for (int e = 0; e < {V}; ++e)",
-          "            if (g + e < K) out[sl * K + g + e] = acc[e];",
+          "            if (g + e < K) O[g + e] = acc[e];",
           "    }", "}"]
     src.append("\n".join(L))
     return "\n".join(src) + "\n"

@@ -35,6 +35,7 @@ TUNE = {
     "ax_stream": 256,    # kept unit-stride extents of 256 vectors or more: blocks to aim for, one
                          # per compute unit (0: off)
     "ax_stream_unroll": 8,   # ... and rows in flight per lane
+    "ax_stream_stagger": 1,  # ... and blocks start at different rows of their slices
     "ntl": 1,         # allow non-temporal loads  } see the cache policy in `lower`
     "nts": 1,         # allow non-temporal stores }
     "cache_mib": 32,  # working sets up to this size (the eight L2s together) stay cacheable
@@ -792,16 +793,50 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
                 low.fin_count = 0
                 low.kind = "axis_stream"
                 unroll = TUNE["ax_stream_unroll"]
-                low.key = ("axis_stream", prog.key(), kinds, acc, reduce_op, unroll)
+                stagger = bool(TUNE["ax_stream_stagger"])
+                low.key = ("axis_stream", prog.key(), kinds, acc, reduce_op, unroll, stagger)
 
                 def emit_stream():
-                    return cg.emit_col_stream(prog, kinds, acc, reduce_op, unroll)
+                    return cg.emit_col_stream(prog, kinds, acc, reduce_op, unroll, stagger=stagger)
                 low.emit = emit_stream
                 low.grid = max(1, min(ktiles * S, 1 << 20))
                 low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
                            + "qqqq" + "q" * len(leaves))
                 low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
                 low.scal, low.tail = list(scalars), [K, R, S, RS] + [r[0] for r in rsets]
+                return low, S, K, "col"
+    if (strategy == "col" and slices is None and len(rmerged) == 1 and len(kmerged) == 2
+            and TUNE["ax_stream"] > 0 and TUNE["uvec"] and all(k[1] in (0, 1) for k in ksets)):
+        widths = {cg.ITEMSIZE[c] for c, k in zip(prog.leaves, ksets) if k[1] == 1}
+        if len(widths) == 1 and widths <= {4, 8} and all(
+                c in cg.VEC16 for c, k in zip(prog.leaves, ksets) if k[1] == 1):
+            V = 16 // next(iter(widths))
+            KO, KI = kmerged
+            ktiles = -(-KI // (cg.BLOCK * V))
+            if KI >= cg.BLOCK * V and R >= 64:
+                # the middle axis of a 3-D array reduced: the same walk down the rows, once per
+                # index of the first axis
+                S = max(1, min(-(-TUNE["ax_stream"] // (ktiles * KO)), R // 32, TUNE["ax_slices"]))
+                RS = -(-R // S)
+                S = -(-R // RS)
+                kinds = tuple("v" if k[1] == 1 else "k" for k in ksets)
+                low = Lowered()
+                low.lds = 0
+                low.fin_count = 0
+                low.kind = "axis_stream"
+                unroll = TUNE["ax_stream_unroll"]
+                stagger = bool(TUNE["ax_stream_stagger"])
+                low.key = ("axis_stream", prog.key(), kinds, acc, reduce_op, unroll, stagger, "outer")
+
+                def emit_stream2():
+                    return cg.emit_col_stream(prog, kinds, acc, reduce_op, unroll, outer=True, stagger=stagger)
+                low.emit = emit_stream2
+                low.grid = max(1, min(ktiles * KO * S, 1 << 20))
+                low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+                           + "qqqq" + "q" * len(leaves) + "q" + "q" * len(leaves))
+                low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+                low.scal = list(scalars)
+                low.tail = [KI, R, S, RS] + [r[0] for r in rsets] + [KO] + [k[0] for k in ksets]
                 return low, S, K, "col"
     if (strategy == "row" and slices is None and len(rmerged) == 2 and len(kmerged) == 1
             and rmerged[1] >= 1024 and TUNE["ax_block"] > 0 and TUNE["uvec"]

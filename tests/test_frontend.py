@@ -305,6 +305,26 @@ def test_views_without_shared_rows_stream_row_by_row():
     assert low.key[0] == "tile2dv" and low.key[8:10] == (64, 2)
 
 
+def test_bitwise_operations_lower_with_numpy_result_types():
+    """`&`, `|`, `^`, `~` and shifts fuse for masks and integers; their result types are
+    NumPy's, and float operands get NumPy's TypeError when the expression is traced."""
+    P = lambda dt: NPArray(hip.placeholder((5003,), dt))
+    a, b = P(np.float32), P(np.float32)
+    for dt in (np.int32, np.int64, np.uint32, np.uint8):
+        x, y = P(dt), P(dt)
+        for e, want in [((a > b) & (a < 1.0), np.bool_), ((a > b) | ~(b < 0.5), np.bool_), (x & y, dt),
+                        (~x, dt), (x ^ 15, dt), (x << 3, dt), (np.right_shift(x, y), dt),
+                        (x & (a > 0), dt)]:
+            assert e.dtype == np.dtype(want)
+            low, src = hip.lower_only(e)
+            assert low.kind == "flat" and len(hip.compile_source(src)) > 0
+    assert "(unsigned int)" in hip.lower_only(P(np.int32) << P(np.int32))[1]
+    with pytest.raises(TypeError):
+        hip.lower_only(a & b)
+    with pytest.raises(TypeError):
+        hip.lower_only(~a)
+
+
 def test_shifted_views_lower_to_lds_stencil():
     n = 512
     u = NPArray(hip.placeholder((n, n), np.float32))
@@ -358,7 +378,10 @@ def test_two_roots_share_one_kernel():
     hip.compile_source(src)
 
 
-@pytest.mark.parametrize("name", sorted(cg.SUPPORTED_UFUNCS - {"square"}))
+_INTEGER_ONLY = set(cg._BITWISE) | set(cg._SHIFTS) | {"invert"}
+
+
+@pytest.mark.parametrize("name", sorted(cg.SUPPORTED_UFUNCS - {"square"} - _INTEGER_ONLY))
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_every_supported_ufunc_generates_compilable_source(name, dtype):
     fn = getattr(np, name, None)

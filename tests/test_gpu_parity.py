@@ -707,6 +707,38 @@ def test_where_clip_sign_and_predicates():
     assert np.array_equal(np.where(dr.array(i0) > 0, dr.array(i0), -1).get(), np.where(i0 > 0, i0, -1))
 
 
+def test_bitwise_operations_and_shifts_follow_numpy():
+    """`&`, `|`, `^`, `~` on masks and integers, shifts with counts up to and beyond the
+    type's width (NumPy shifts everything out), mixed bool / integer operands, float
+    operands refused with NumPy's TypeError."""
+    rs = np.random.RandomState(41)
+    n = 5003
+    a0, b0 = rs.standard_normal(n).astype(np.float32), rs.standard_normal(n).astype(np.float32)
+    a, b = dr.array(a0), dr.array(b0)
+    assert np.array_equal(((a > b) & (a < 1.0)).get(), (a0 > b0) & (a0 < 1.0))
+    assert np.array_equal(((a > b) | ~(b < 0.5)).get(), (a0 > b0) | ~(b0 < 0.5))
+    assert np.array_equal(((a > 0) ^ (b > 0)).get(), (a0 > 0) ^ (b0 > 0))
+    assert bits_equal(np.where((a > b) & (b > 0), a, b).get(), np.where((a0 > b0) & (b0 > 0), a0, b0))
+    assert int(dr.sum((a > 0) & (b > 0))) == int(np.sum((a0 > 0) & (b0 > 0)))
+    for dt in (np.int32, np.int64, np.uint32, np.uint8):
+        info = np.iinfo(dt)
+        x0 = rs.randint(info.min, info.max, n, dtype=dt)
+        y0 = rs.randint(info.min, info.max, n, dtype=dt)
+        k0 = rs.randint(0, 8 * np.dtype(dt).itemsize + 3, n).astype(dt)
+        x, y, k = dr.array(x0), dr.array(y0), dr.array(k0)
+        for got, want in [((x & y), x0 & y0), ((x | y), x0 | y0), ((x ^ y), x0 ^ y0), (~x, ~x0),
+                          ((x & 15), x0 & 15), ((x << 3), x0 << 3), ((x >> 2), x0 >> 2),
+                          (np.left_shift(x, k), np.left_shift(x0, k0)),
+                          (np.right_shift(x, k), np.right_shift(x0, k0)),
+                          ((x & (a > 0)), x0 & (a0 > 0))]:
+            got = got.get()
+            assert got.dtype == want.dtype and np.array_equal(got, want), dt
+    with pytest.raises(TypeError):
+        (a & b).get()
+    with pytest.raises(TypeError):
+        (~a).get()
+
+
 def test_transposed_operands_go_through_lds_and_match():
     rs = np.random.RandomState(15)
     for shape in [(64, 64), (100, 200), (257, 63), (1, 300), (1000, 3)]:
@@ -1100,6 +1132,28 @@ def test_reductions_over_the_first_and_last_axis_of_a_three_dimensional_array():
     assert np.allclose(got, (h.astype(np.float64) * w).sum(axis=(0, 2)), rtol=2e-5)
     m = dr.mean(dr.array(h), axis=(0, 2)).get()
     assert np.allclose(m, h.mean(axis=(0, 2), dtype=np.float64), rtol=2e-5)
+
+
+def test_reductions_over_the_middle_axis_of_a_three_dimensional_array():
+    """(N, R, L) reduced over R with long rows L: the row-streaming kernel once per index of
+    the first axis; ragged rows, views off 16 bytes, slices of R, an operand constant along L."""
+    rs = np.random.RandomState(35)
+    for shape, dt in [((3, 700, 1024), np.float32), ((5, 64, 1500), np.float64), ((2, 3000, 2049), np.int32)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int32 else rs.randint(-9, 9, shape)).astype(dt)
+        a = dr.array(h)
+        low = hip.lower_only(ReduceEx(np.add, a * a, (1,)))[0]
+        assert low.kind == "axis_stream" and low.key[-1] == "outer", (shape, low.kind)
+        tol = dict(rtol=2e-5, atol=1e-4) if dt == np.float32 else dict(rtol=1e-13, atol=1e-13)
+        assert np.allclose(dr.sum(a * a, axis=1).get(), (h.astype(np.float64) ** 2).sum(axis=1), **tol)
+        assert np.array_equal(dr.max(a, axis=1).get(), h.max(axis=1))
+        assert np.array_equal(dr.min(a[1:, 2:-1, 3:-2], axis=1).get(), h[1:, 2:-1, 3:-2].min(axis=1))
+    h = rs.uniform(0, 1, (6, 90, 1100)).astype(np.float32)
+    w = rs.uniform(0, 1, (6, 90, 1)).astype(np.float32)
+    got = dr.sum(dr.array(h) * dr.array(w), axis=1).get()
+    assert np.allclose(got, (h.astype(np.float64) * w).sum(axis=1), rtol=2e-5)
+    v = rs.uniform(0, 1, (1, 90, 1100)).astype(np.float32)
+    got = dr.sum(dr.array(h) * dr.array(v), axis=1).get()
+    assert np.allclose(got, (h.astype(np.float64) * v).sum(axis=1), rtol=2e-5)
 
 
 def test_reductions_over_the_rows_of_wide_matrices_stream_whole_rows():
