@@ -44,6 +44,7 @@ TUNE = {
     "th": 16,         # stencil tile height (rows)
     "lds": 1,         # stage shifted views through LDS (0: read them directly)
     "svec": 1,        # aligned stencils: 16-byte loads into LDS and 16-byte stores
+    "row1d": 1,       # shifted views of one vector: tiled as a matrix of one row
     "gpr": 64,        # vectorised stencil: 16-byte column groups per tile row
     "rpt": 2,         # vectorised stencil: consecutive rows per thread
     "row_gpr": 256,   # vector tiles without a halo group: most column groups per block (0: as
@@ -278,6 +279,24 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
 
     flat = ndim <= 1 and all(s == [1] or s == [0] or s == [] for s in m_leaf) \
         and all(s == [1] or s == [] for s in m_out)
+    if flat and ndim == 1 and not reduce_op and TUNE["lds"] and TUNE["svec"] and TUNE["row1d"] \
+            and 4096 <= n < 2 ** 31 - 4096:
+        # Shifted views of one vector (differences, 1-D stencils): every view would fetch the
+        # same cache lines again through L1.  As a matrix of one row the vector goes through
+        # the tiled kernel's LDS window once.  Second difference of 2^27 float32: 65 % of the
+        # HBM peak as a flat kernel.
+        same = {}
+        for a, st, c in zip(leaves, m_leaf, prog.leaves):
+            if st == [1]:
+                same.setdefault((id(a.buf), c), set()).add(a.offset)
+        offs = max(same.values(), key=len) if same else set()
+        if len(offs) >= 2 and max(offs) - min(offs) <= 32:
+            flat = False
+            ndim = 2
+            far = 1 << 40               # the pitch of the one row: never multiplied by a row > 0
+            mshape = [1] + list(mshape)
+            m_leaf = [[far if st == [1] else 0] + list(st) for st in m_leaf]
+            m_out = [[far] + list(st) for st in m_out]
     if flat:
         leaf_class = tuple("b" if (s == [0] and n > 1) else "c" for s in m_leaf)
         ptrs = [a.ptr for a in leaves]
@@ -441,9 +460,12 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                 ph_o = (out_ptrs[0] // gsize) % vw
                 dv = [d and row_aligned(i, ph_o) for i, d in enumerate(sized)]
                 missed = dv != sized        # some operand would fall back to element loads
-            if group is None and same_size and TUNE["uvec"] and W >= 4 * vw and missed:
-                # without a halo group nothing ties the tiles to 16-byte boundaries: rows of
-                # any pitch and phase move as vectors at element alignment
+            if ((group is None or g_args[0] % vw == 0) and same_size and TUNE["uvec"]
+                    and W >= 4 * vw and missed):
+                # rows of any pitch and phase move as vectors at element alignment; only a
+                # halo group ties the tiles to 16-byte boundaries, those of its own buffer
+                # (a stencil over a padded array written to a fresh one, whose rows are a
+                # few elements shorter)
                 vec_ok = ua = True
                 ph_o = 0
                 dv = sized
@@ -452,6 +474,8 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             # direct operands whose rows share the outputs' alignment load as vectors
             kinds = tuple(("dv",) if d else k for d, k in zip(dv, kinds))
             gpr, rpt = TUNE["gpr"], TUNE["rpt"]
+            if H == 1:                   # one long row: the whole block side by side
+                gpr, rpt = cg.BLOCK, 1
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
             streams = all(all(st[:-1]) for st, k in zip(m_leaf, kinds) if k[0] in ("d", "dv"))
             if group is None and TUNE["row_gpr"] and streams:

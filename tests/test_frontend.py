@@ -329,11 +329,18 @@ def test_shifted_views_lower_to_lds_stencil():
     n = 512
     u = NPArray(hip.placeholder((n, n), np.float32))
     rhs = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+    # a fresh output has rows of 510: the tiles follow the 16-byte boundaries of the grid's
+    # buffer and the stores are vectors at element alignment
     low, src = hip.lower_only(rhs)
-    assert low.kind == "tile2d"
-    assert "__shared__ float tile[" in src and "__syncthreads" in src      # fresh output: rows
-    kinds = low.key[2]                                                    # of 510 are unaligned
+    assert low.kind == "tile2d" and low.key[0] == "tile2dv" and low.key[-1] is True
+    assert "__shared__ f4x4 tile[" in src and "(f4x4u*)(o0 +" in src and "(const f4x4*)(gp + lin)" in src
+    kinds = low.key[2]
     assert sorted(k[1:] for k in kinds) == [(0, 0), (1, -1), (1, 1), (2, 0)]
+    hip.compile_source(src)
+    # a grid whose own rows are not 16-byte periodic: element loads into LDS
+    odd = NPArray(hip.placeholder((n - 1, n - 1), np.float32))
+    low, src = hip.lower_only(0.25 * (odd[:-2, 1:-1] + odd[2:, 1:-1] + odd[1:-1, :-2] + odd[1:-1, 2:]))
+    assert low.key[0] == "tile2d" and "__shared__ float tile[" in src and "__syncthreads" in src
     hip.compile_source(src)
     # written back into the grid's interior, rows stay 16-byte periodic: vector variant
     dst = hip.placeholder((n - 2, n - 2), np.float32, strides=(n, 1), offset=n + 1)

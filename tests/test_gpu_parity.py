@@ -409,6 +409,53 @@ def test_wide_and_asymmetric_stencils(dtype):
         assert bits_equal(fn(dr.array(a0)).get(), fn(OracleArray(a0)).get()), fn.__name__
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_stencils_written_to_fresh_arrays_store_vectors_at_element_alignment(dtype):
+    """The grid's rows are 16-byte periodic, the fresh result's rows (a few elements shorter)
+    are not: LDS window along the grid's boundaries, stores at element alignment; another
+    operand beside the window, a grid that starts off 16 bytes."""
+    rs = np.random.RandomState(43)
+    for shape in [(67, 200), (130, 1032), (9, 4100)]:
+        a0 = rs.uniform(-1, 1, shape).astype(dtype)
+        w0 = rs.uniform(-1, 1, (shape[0] - 2, shape[1] - 2)).astype(dtype)
+
+        def nine(a, w):
+            return (a[:-2, :-2] + a[:-2, 1:-1] + a[:-2, 2:] + a[1:-1, :-2] + a[1:-1, 1:-1]
+                    + a[1:-1, 2:] + a[2:, :-2] + a[2:, 1:-1] + a[2:, 2:]) * w
+        a, w = dr.array(a0), dr.array(w0)
+        low = hip.lower_only(nine(a, w))[0]
+        vw = 16 // np.dtype(dtype).itemsize
+        assert low.key[0] == "tile2dv" and low.key[-1] is ((shape[1] - 2) % vw != 0), shape
+        assert bits_equal(nine(a, w).get(), nine(OracleArray(a0), OracleArray(w0)).get()), shape
+        sub, osub = a[1:, 4:], OracleArray(a0)[1:, 4:]        # still 16-byte periodic rows
+        assert bits_equal(nine(sub, w[1:, 4:]).get(), nine(osub, OracleArray(w0)[1:, 4:]).get()), shape
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_shifted_views_of_a_vector_go_through_the_lds_window(dtype):
+    """Differences and 1-D stencils: the vector is tiled as a matrix of one row; lengths
+    around the tile width, views that start off 16 bytes, an operand beside the window,
+    results written back into the vector."""
+    rs = np.random.RandomState(44)
+    for n in (4099, 5120, 100003, (1 << 20) + 5):
+        a0 = rs.uniform(-1, 1, n).astype(dtype)
+        b0 = rs.uniform(-1, 1, n).astype(dtype)
+        a, b, oa, ob = dr.array(a0), dr.array(b0), OracleArray(a0), OracleArray(b0)
+        low = hip.lower_only(a[2:] + a[:-2] - 2.0 * a[1:-1])[0]
+        assert low.key[0] == "tile2dv" and low.tail[0] == 1, n
+        assert bits_equal((a[1:] - a[:-1]).get(), (oa[1:] - oa[:-1]).get()), n
+        assert bits_equal((a[2:] + a[:-2] - 2.0 * a[1:-1]).get(), (oa[2:] + oa[:-2] - 2.0 * oa[1:-1]).get()), n
+        assert bits_equal(((a[5:] - a[:-5]) * b[3:-2]).get(), ((oa[5:] - oa[:-5]) * ob[3:-2]).get()), n
+        s, os_ = a[3:-1], oa[3:-1]
+        assert bits_equal((s[1:] * s[:-1]).get(), (os_[1:] * os_[:-1]).get()), n
+    u0 = rs.uniform(0, 1, 50001).astype(dtype)
+    u, ou = dr.array(u0), OracleArray(u0.copy())
+    for _ in range(3):
+        for arr in (u, ou):
+            arr[1:-1] = 0.5 * (arr[:-2] + arr[2:])
+    assert bits_equal(u.get(), ou.get())
+
+
 def test_boundary_change_between_sweeps_is_seen():
     """The ping-pong copy is refreshed when something else writes the buffer."""
     u0 = np.zeros((20, 24), np.float32)
