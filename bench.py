@@ -85,9 +85,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all",
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
-                         "dot | axis0 | axis1 | rows200 | rowbcast | transpose | transpose3d | interior | stencil3d | "
-                         "grid | rand | next (these ten: the operations either side of the five "
-                         "configurations); "
+                         "dot | axis0 | axis1 | axis1_3d | matvec | rows200 | rowbcast | transpose | "
+                         "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | next (all "
+                         "of these: the operations either side of the five configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before each timed region (clock ramp-up)")
@@ -230,6 +230,46 @@ def main():
                         desc=f"a @ b {np.dtype(dt).name} 8192^3 (eager matrix product on the matrix cores)",
                         steps=[lambda: a.dot(b)._force()],
                         cpu=lambda: ha[:m, :m] @ hb[:m, :m], cpu_frac=(m / N) ** 2, cpu_code="numpy.matmul")
+        if name == "axis1_3d":
+            shape = (256, 512, 1024)
+            hv = rs.standard_normal(shape).astype(np.float32)
+            vols = [dr.array(hv) for _ in range(sets_for(4 * hv.size))]
+            return dict(dtype="f32", n=hv.size, nbytes=4 * hv.size + 4 * shape[0] * shape[2],
+                        desc="sum(a, axis=1) f32 256x512x1024 (the middle axis)",
+                        steps=[(lambda v=v: hip.run(ReduceEx(np.add, v, (1,)))) for v in vols],
+                        cpu=lambda: hv[:64].sum(axis=1), cpu_frac=0.25, cpu_code="numpy.sum")
+        if name == "matvec":
+            N = 16384
+            ha, hx = rs.standard_normal((N, N)).astype(np.float32), rs.standard_normal(N).astype(np.float32)
+            x = dr.array(hx)
+            mats = [dr.array(ha) for _ in range(sets_for(4 * N * N))]
+            return dict(dtype="f32", n=N * N, nbytes=4 * N * N + 8 * N,
+                        desc="a @ x f32 16384x16384 (the fused row reduction `@` builds)",
+                        steps=[(lambda a=a: hip.run(ReduceEx(np.add, a * x, (1,)))) for a in mats],
+                        cpu=lambda: ha[:N // 4] @ hx, cpu_frac=0.25, cpu_code="numpy.matmul")
+        if name == "diff2":
+            n = 1 << 27
+            hx = rs.standard_normal(n).astype(np.float32)
+            vecs = [dr.array(hx) for _ in range(sets_for(8 * n))]
+            return dict(dtype="f32", n=n - 2, nbytes=8 * n - 8,
+                        desc="x[2:] + x[:-2] - 2 x[1:-1] f32 n=2^27 (three shifted views of one vector)",
+                        steps=[(lambda v=v: hip.run(v[2:] + v[:-2] - 2.0 * v[1:-1])) for v in vecs],
+                        cpu=lambda: hx[2:n // 4] + hx[:n // 4 - 2] - np.float32(2.0) * hx[1:n // 4 - 1],
+                        cpu_frac=0.25, cpu_code="numpy.add, numpy.subtract, numpy.multiply")
+        if name == "stencil9":
+            N = 8192
+            hu = rs.uniform(0, 1, (N, N)).astype(np.float32)
+            M = N - 2
+            grids = [dr.array(hu) for _ in range(sets_for(4 * N * N + 4 * M * M))]
+
+            def nine(u):
+                return (u[:-2, :-2] + u[:-2, 1:-1] + u[:-2, 2:] + u[1:-1, :-2] + u[1:-1, 1:-1]
+                        + u[1:-1, 2:] + u[2:, :-2] + u[2:, 1:-1] + u[2:, 2:]) * (1.0 / 9.0)
+            return dict(dtype="f32", n=M * M, nbytes=4 * N * N + 4 * M * M,
+                        desc="9-point stencil f32 8192^2 into a fresh 8190^2 array (rows not 16-byte periodic)",
+                        steps=[(lambda u=u: hip.run(nine(u))) for u in grids],
+                        cpu=lambda: hu[1:N // 8, 1:-1] + hu[:N // 8 - 1, 1:-1], cpu_frac=1 / 8,
+                        cpu_code="numpy.add (two of the nine views)")
         if name == "transpose3d":
             shape = (512, 512, 1024)
             hv = rs.standard_normal(shape).astype(np.float32)
@@ -492,8 +532,8 @@ def main():
         return res
 
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
-             "next": ["dot", "axis0", "axis1", "rows200", "rowbcast", "transpose", "transpose3d", "interior",
-                      "stencil3d", "grid", "rand"]}.get(args.workload, [args.workload])
+             "next": ["dot", "axis0", "axis1", "axis1_3d", "matvec", "rows200", "rowbcast", "transpose",
+                      "transpose3d", "interior", "diff2", "stencil9", "stencil3d", "grid", "rand"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:

@@ -124,6 +124,10 @@ class _Fallback:
         b = _Fallback.ascontiguousarray(b, dt)
         if a.ndim == 1 and b.ndim == 1:
             return run_reduce_product(a, b)
+        if (a.ndim, b.ndim) in ((2, 1), (1, 2)):
+            # one pass over the matrix as a fused reduction
+            from . import delayarray as fe
+            return fe.NPArray(a)._dot([fe.NPArray(a), fe.NPArray(b)], {})._force()
         a2 = a.reshape(1, -1) if a.ndim == 1 else a
         b2 = b.reshape(-1, 1) if b.ndim == 1 else b
         if a2.ndim != 2 or b2.ndim != 2 or a2.shape[1] != b2.shape[0]:

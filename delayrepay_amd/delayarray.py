@@ -148,6 +148,17 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         if len(left.shape) == 1 and len(right.shape) == 1:
             # vector . vector: fused multiply + reduction
             return _reduce(np.add, left * right)
+        floats = left.dtype.kind == "f" and right.dtype.kind == "f"
+        if floats and len(left.shape) == 2 and len(right.shape) == 1:
+            # matrix . vector reads the matrix once: a fused row reduction streams it at
+            # HBM speed, a matrix-matrix kernel with one output column does not
+            if left.shape[1] != right.shape[0]:
+                raise ValueError(f"shapes {left.shape} and {right.shape} not aligned")
+            return _reduce(np.add, left * right, axis=1)
+        if floats and len(left.shape) == 1 and len(right.shape) == 2:
+            if left.shape[0] != right.shape[0]:
+                raise ValueError(f"shapes {left.shape} and {right.shape} not aligned")
+            return _reduce(np.add, left.reshape(left.shape[0], 1) * right, axis=0)
         return cast(_backend.fallback.dot)(left._force(), right._force())
 
     def dot(self, other, out=None):

@@ -324,12 +324,19 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                               ("divide", "true_divide", "reciprocal")) and name not in cheap else 1
                        for name, _, _, _ in prog.ops)
             light = cost <= 4 * n_in + 4
-            # one operand: 6 vectors in flight 89.9, 8: 87.1, 4: 75.3.  Maxima and minima (NaN
-            # checks per element) want two blocks per compute unit with half as many vectors
-            # each: 87.9 against 75.7.
+            # one operand: 6 vectors in flight 89.9, 8: 87.1, 4: 75.3.  That holds for float
+            # sums of at most one operation per operand.  With one wave per SIMD nothing hides
+            # the arithmetic between two batches of loads, so maxima and minima (NaN checks
+            # per element), counts of masks (64-bit integer sums) and longer bodies want two
+            # blocks per compute unit with half as many vectors each.  One float32 operand,
+            # 2^27, 256 x 6 against 512 x 3: max 75.7 / 87.9, count(a > c) 64.9 / 87.4,
+            # count((a > c) & (a < d)) 46.5 / 86.1, sum(a*a*a + a) 83.6 / 88.2,
+            # sum(where(a > c, a, 0)) 81.5 / 88.4, sum(abs(a)) 86.6 / 87.6.
             per_lane = {1: 6, 2: 4, 3: 2, 4: 2}.get(n_in, 1)
             cus = grid_cap() // TUNE["bpc"]
-            if light and reduce_op != "add":
+            bare = (reduce_op == "add" and len(prog.ops) <= n_in
+                    and all(c in ("f4", "f8") for c in out_codes))
+            if light and not bare:
                 per_lane, cus = max(1, per_lane // 2 + per_lane % 2), 2 * cus
             unroll = unroll or (per_lane if light else 4)
             red_cap = red_cap or (cus if light else 4096)

@@ -754,6 +754,38 @@ def test_where_clip_sign_and_predicates():
     assert np.array_equal(np.where(dr.array(i0) > 0, dr.array(i0), -1).get(), np.where(i0 > 0, i0, -1))
 
 
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 2e-5), (np.float64, 1e-13)])
+def test_matrix_vector_products_are_fused_reductions(dtype, tol):
+    """`A @ x` and `x @ A` read the matrix once as a reduction along / over its rows, fused
+    with the expressions that make their operands; transposed and lazy operands, `np.dot`,
+    mismatched shapes."""
+    rs = np.random.RandomState(45)
+    for m, k in [(600, 777), (33, 5000), (3000, 64), (1, 300), (257, 1)]:
+        a0, x0, y0 = (rs.standard_normal(s).astype(dtype) for s in ((m, k), (k,), (m,)))
+        a, x, y = dr.array(a0), dr.array(x0), dr.array(y0)
+        ref = a0.astype(np.float64) @ x0.astype(np.float64)
+        scale = np.abs(a0.astype(np.float64)) @ np.abs(x0.astype(np.float64))
+        for got in (a @ x, np.dot(a, x), a.dot(x)):
+            got = got.get()
+            assert got.shape == (m,) and got.dtype == dtype
+            assert np.all(np.abs(got - ref) <= tol * scale), (m, k)
+        refl = y0.astype(np.float64) @ a0.astype(np.float64)
+        scalel = np.abs(y0.astype(np.float64)) @ np.abs(a0.astype(np.float64))
+        got = (y @ a).get()
+        assert got.shape == (k,) and got.dtype == dtype and np.all(np.abs(got - refl) <= tol * scalel), (m, k)
+        got = (a.T @ y).get()
+        assert np.all(np.abs(got - refl) <= tol * scalel), (m, k)
+        got = ((a * 2.0) @ (x + 1.0) - y).get()                   # fuses on both sides
+        ref2 = (a0.astype(np.float64) * 2.0) @ (x0.astype(np.float64) + 1.0) - y0
+        assert np.all(np.abs(got - ref2) <= tol * (2 * scale + 2 * np.abs(a0).sum(axis=1) + 1)), (m, k)
+    with pytest.raises(ValueError):
+        dr.array(np.zeros((4, 5), dtype)) @ dr.array(np.zeros(4, dtype))
+    with pytest.raises(ValueError):
+        dr.array(np.zeros(5, dtype)) @ dr.array(np.zeros((4, 5), dtype))
+    i = dr.array(np.arange(12).reshape(3, 4)) @ dr.array(np.arange(4))     # integers: as before
+    assert np.array_equal(np.asarray(i.get(), dtype=np.int64), np.arange(12).reshape(3, 4) @ np.arange(4))
+
+
 def test_bitwise_operations_and_shifts_follow_numpy():
     """`&`, `|`, `^`, `~` on masks and integers, shifts with counts up to and beyond the
     type's width (NumPy shifts everything out), mixed bool / integer operands, float
