@@ -836,7 +836,7 @@ def _outer_params(leaf_kind, n_out, nouter):
     outer strides of every directly read operand, then of every output."""
     params = [f"const long long od{d}" for d in range(1, nouter)]
     for i, k in enumerate(leaf_kind):
-        if k[0] in ("d", "dv", "r"):
+        if k[0] in ("d", "dv", "dr", "r"):
             params += [f"const long long os{i}_{d}" for d in range(nouter)]
     for o in range(n_out):
         params += [f"const long long oos{o}_{d}" for d in range(nouter)]
@@ -844,7 +844,8 @@ def _outer_params(leaf_kind, n_out, nouter):
 
 
 def _base_names(leaf_kind, n_out):
-    names = [(f"base{i}", f"os{i}") for i, k in enumerate(leaf_kind) if k[0] in ("d", "dv", "r")]
+    names = [(f"base{i}", f"os{i}") for i, k in enumerate(leaf_kind)
+             if k[0] in ("d", "dv", "dr", "r")]
     return names + [(f"obase{o}", f"oos{o}") for o in range(n_out)]
 
 
@@ -953,7 +954,10 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
                ('dv',) 2-D operand whose rows have the outputs' phase and a stride
                that is a multiple of VW: read with 16-byte loads;
                ('d',) other operand with unit stride along the last dimension: element
-               loads; ('r',) operand constant along the last dimension;
+               loads; ('dr',) operand walked backwards along the last dimension (stride
+               -1, a flipped view): one 16-byte load at element alignment from the
+               mirrored place, its elements reversed in registers;
+               ('r',) operand constant along the last dimension;
                ('b',) single element broadcast
     group      None, or (dtype code, dy_max, dx_min, dx_max) with the group's row
                stride a multiple of VW and `phase_group` its reference element's phase
@@ -1041,7 +1045,7 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
         if k[0] == "g":
             _, dy, dx = k
             return f"ts[(lr + {dy}) * {LW} + g * {VW} + {e + dx - dx_min + ph}]"
-        if k[0] in ("d", "dv"):
+        if k[0] in ("d", "dv", "dr"):
             return f"D{i}[{e}]"
         if k[0] == "r":
             return f"a{i}[base{i}]"
@@ -1063,6 +1067,17 @@ def emit_stencil_vec(prog, leaf_kind, group, out_dtypes, groups_per_row, rows_pe
                   f"            D{i} = {_ld(nt_load, ptr)};",
                   "        } else {"]
             L += [f"            D{i}[{e}] = (jf + {e} >= 0 && jf + {e} < W) ? a{i}[base{i} + jf + {e}] "
+                  f": ({CTYPE[prog.leaves[i]]})0;" for e in range(VW)]
+            L.append("        }")
+        elif k[0] == "dr":
+            lvt = VEC16[prog.leaves[i]][0]
+            ptr = f"(const {lvt}u*)(a{i} + base{i} - jf - {VW - 1})"
+            L += [f"        {lvt} D{i};",
+                  "        if (inner) {",
+                  f"            const {lvt}u T{i} = {_ld(nt_load, ptr)};",
+                  "            " + " ".join(f"D{i}[{e}] = T{i}[{VW - 1 - e}];" for e in range(VW)),
+                  "        } else {"]
+            L += [f"            D{i}[{e}] = (jf + {e} >= 0 && jf + {e} < W) ? a{i}[base{i} - jf - {e}] "
                   f": ({CTYPE[prog.leaves[i]]})0;" for e in range(VW)]
             L.append("        }")
         elif k[0] == "d":

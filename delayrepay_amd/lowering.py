@@ -297,6 +297,15 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             mshape = [1] + list(mshape)
             m_leaf = [[far if st == [1] else 0] + list(st) for st in m_leaf]
             m_out = [[far] + list(st) for st in m_out]
+    if ndim == 1 and not reduce_op and any(s == [-1] for s in m_leaf) \
+            and all(s in ([1], [0], [-1]) for s in m_leaf) and all(s == [1] for s in m_out) \
+            and n < 2 ** 31 - 4096:
+        # a flipped vector: as a matrix of one row it takes the tiled kernel's reversed loads
+        ndim = 2
+        far = 1 << 40
+        mshape = [1] + list(mshape)
+        m_leaf = [[0 if st == [0] else far] + list(st) for st in m_leaf]
+        m_out = [[far] + list(st) for st in m_out]
     if flat:
         leaf_class = tuple("b" if (s == [0] and n > 1) else "c" for s in m_leaf)
         ptrs = [a.ptr for a in leaves]
@@ -399,11 +408,20 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     # kernel's "rows" (decomposed per row when there are several).
     nouter = ndim - 1
     tiled = (not reduce_op and ndim >= 2 and all(s[-1] == 1 for s in m_out)
-             and all(s[-1] in (0, 1) for s in m_leaf))
+             and all(s[-1] in (0, 1, -1) for s in m_leaf))
+    # operands walked backwards along the last dimension (flipped views) are read as vectors
+    # at element alignment and reversed in registers: only the vector kernel does that
+    rev = [i for i, s in enumerate(m_leaf) if s[-1] == -1] if tiled else []
+    if rev:
+        g0 = cg.ITEMSIZE[out_codes[0]]
+        tiled = bool(TUNE["svec"] and TUNE["uvec"] and g0 in (4, 8)
+                     and all(cg.ITEMSIZE[c] == g0 for c in out_codes)
+                     and all(cg.ITEMSIZE[prog.leaves[i]] == g0 for i in rev)
+                     and mshape[-1] >= 4 * (16 // g0))
     rows = 1
     for d in mshape[:-1]:
         rows *= d
-    if tiled and ndim == 3 and TUNE["lds"] and TUNE["svec"] and TUNE["s3"]:
+    if tiled and ndim == 3 and TUNE["lds"] and TUNE["svec"] and TUNE["s3"] and not rev:
         low3 = _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_ptrs,
                                 scal_fmt, scal_vals, in_place)
         if low3 is not None:
@@ -415,7 +433,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         group = None
         # halo group (2-D only): >= 2 leaves that are shifted views of one buffer
         groups = {}
-        if ndim == 2:
+        if ndim == 2 and not rev:
             for i, (a, s) in enumerate(zip(leaves, m_leaf)):
                 if s[1] == 1 and s[0] > 0:
                     groups.setdefault((id(a.buf), s[0], prog.leaves[i]), []).append(i)
@@ -445,7 +463,8 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                 g_args = [rs, -ref_off, g_buf.nbytes // itemsize - ref_off]
         for i, s in enumerate(m_leaf):
             if kinds[i] is None:
-                kinds[i] = ("b",) if not any(s) else ("d",) if s[-1] == 1 else ("r",)
+                kinds[i] = (("b",) if not any(s) else ("d",) if s[-1] == 1 else
+                            ("dr",) if s[-1] == -1 else ("r",))
         kinds = tuple(kinds)
         low.kind = "tile2d"
         vec_ok = ua = False
@@ -484,7 +503,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             if H == 1:                   # one long row: the whole block side by side
                 gpr, rpt = cg.BLOCK, 1
             sntl, snts = bool(TUNE["sntl"]), bool(TUNE["snts"])
-            streams = all(all(st[:-1]) for st, k in zip(m_leaf, kinds) if k[0] in ("d", "dv"))
+            streams = all(all(st[:-1]) for st, k in zip(m_leaf, kinds) if k[0] in ("d", "dv", "dr"))
             if group is None and TUNE["row_gpr"] and streams:
                 # Nothing is shared between rows: a block takes one stretch of a row, as
                 # long as the row allows (up to 4 KB), like a chunk of a flat kernel, and
@@ -498,7 +517,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                 while gpr < TUNE["row_gpr"] and gpr * vw < W + ph_o:
                     gpr *= 2
                 rpt = 1
-                in_bytes = sum(a.nbytes for a, k in zip(leaves, kinds) if k[0] in ("d", "dv"))
+                in_bytes = sum(a.nbytes for a, k in zip(leaves, kinds) if k[0] in ("d", "dv", "dr"))
                 out_bytes = sum(n * cg.ITEMSIZE[c] for c in out_codes)
                 snts = bool(TUNE["nts"]) and in_bytes + out_bytes > TUNE["cache_mib"] << 20
                 sntl = bool(TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
@@ -545,7 +564,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             fmt += "q" * (nouter - 1)
             tail_vals += list(mshape[1:-1])
             for k, s in zip(kinds, m_leaf):
-                if k[0] in ("d", "dv", "r"):
+                if k[0] in ("d", "dv", "dr", "r"):
                     fmt += "q" * nouter
                     tail_vals += list(s[:-1])
             for s in m_out:

@@ -456,6 +456,46 @@ def test_shifted_views_of_a_vector_go_through_the_lds_window(dtype):
     assert bits_equal(u.get(), ou.get())
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32])
+def test_flipped_views_are_read_as_reversed_vectors(dtype):
+    """`a[::-1]`, `m[:, ::-1]`, `m[::-1, ::-1]`: 16-byte loads from the mirrored place,
+    reversed in registers; widths around the vector and tile sizes, a flipped operand beside
+    a straight one, flips of interior views, a flipped 3-D array; narrow and mixed-width
+    cases keep the element-wise kernel."""
+    rs = np.random.RandomState(46)
+    mk = (lambda s: rs.randint(-99, 99, s).astype(dtype)) if dtype == np.int32 else \
+        (lambda s: rs.uniform(-1, 1, s).astype(dtype))
+    for n in (17, 1000, 4099, 100003):
+        a0, b0 = mk(n), mk(n)
+        a, b = dr.array(a0), dr.array(b0)
+        assert hip.lower_only(a[::-1] * 2)[0].key[0] == "tile2dv", n
+        assert np.array_equal((a[::-1] * 2).get(), a0[::-1] * 2), n
+        assert np.array_equal((a[::-1] + b).get(), a0[::-1] + b0), n
+        assert np.array_equal((a[3:-2][::-1] - b[:-5]).get(), a0[3:-2][::-1] - b0[:-5]), n
+    for shape in [(5, 16), (33, 1030), (257, 4100)]:
+        m0, k0 = mk(shape), mk(shape)
+        m, k = dr.array(m0), dr.array(k0)
+        low = hip.lower_only(m[:, ::-1] * 2)[0]
+        assert low.key[0] == "tile2dv" and ("dr",) in low.key[2], shape
+        assert np.array_equal((m[:, ::-1] * 2).get(), m0[:, ::-1] * 2), shape
+        assert np.array_equal((m[:, ::-1] + k).get(), m0[:, ::-1] + k0), shape
+        assert np.array_equal((m[::-1, ::-1] - k).get(), m0[::-1, ::-1] - k0), shape
+        assert np.array_equal((m[::-1, ::-1] + m[:, ::-1] + m[::-1]).get(),
+                              m0[::-1, ::-1] + m0[:, ::-1] + m0[::-1]), shape
+        assert np.array_equal((m[1:-1, 2:-1][:, ::-1] * k[1:-1, :-3]).get(),
+                              m0[1:-1, 2:-1][:, ::-1] * k0[1:-1, :-3]), shape
+        row0 = mk(shape[1])
+        assert np.array_equal((m[:, ::-1] + dr.array(row0)).get(), m0[:, ::-1] + row0), shape
+    v0 = mk((6, 7, 300))
+    assert np.array_equal((dr.array(v0)[:, :, ::-1] * 3).get(), v0[:, :, ::-1] * 3)
+    assert np.array_equal((dr.array(v0)[::-1, ::-1, ::-1] * 3).get(), v0[::-1, ::-1, ::-1] * 3)
+    n0 = mk((40, 3))                                            # rows shorter than four vectors
+    assert np.array_equal((dr.array(n0)[:, ::-1] * 2).get(), n0[:, ::-1] * 2)
+    d0 = rs.uniform(-1, 1, (9, 200))                            # float64 beside the flipped operand
+    m0 = mk((9, 200))
+    assert np.array_equal((dr.array(m0)[:, ::-1] * dr.array(d0)).get(), m0[:, ::-1] * d0)
+
+
 def test_boundary_change_between_sweeps_is_seen():
     """The ping-pong copy is refreshed when something else writes the buffer."""
     u0 = np.zeros((20, 24), np.float32)
