@@ -245,3 +245,71 @@ def test_random_geometry_matches_numpy(seed):
             dst_h[key] = h
             got, ref = dst_d.get(), dst_h
     assert got.dtype == np.asarray(ref).dtype and bits_equal(got, np.asarray(ref)), (seed, shape, mode)
+
+
+# ---- the same with flipped axes and combined masks ------------------------------------------------
+
+def flip_leaf(rs, shape, dtype):
+    d, h = geo_leaf(rs, shape, dtype)
+    how = rs.randint(4)
+    if how == 0 or d.shape != tuple(shape):          # (lower-rank leaves flip along their own axes)
+        return d, h
+    if how == 1:
+        key = (Ellipsis, slice(None, None, -1))
+    elif how == 2:
+        key = (slice(None, None, -1),)
+    else:
+        key = tuple(slice(None, None, -1) for _ in shape)
+    return d[key], h[key]
+
+
+def flip_expr(rs, shape, depth):
+    if depth == 0:
+        return flip_leaf(rs, shape, GEO_DTYPES[rs.randint(len(GEO_DTYPES))])
+    op = rs.randint(7)
+    d, h = flip_expr(rs, shape, depth - 1)
+    if op == 0:
+        return d * 2.5, h * 2.5
+    if op == 1:
+        return dr.where((d > 0) & (d < 50), d, 1), np.where((h > 0) & (h < 50), h, 1)
+    if op == 2:
+        return (d + 0).astype(np.float32), (h + 0).astype(np.float32)
+    d2, h2 = flip_expr(rs, shape, depth - 1)
+    if op == 3:
+        return d + d2, h + h2
+    if op == 4:
+        return dr.where((d > d2) | ~(d2 > 0), d, d2), np.where((h > h2) | ~(h2 > 0), h, h2)
+    if op == 5:
+        return np.minimum(d, d2), np.minimum(h, h2)
+    return d - d2, h - h2
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_geometry_with_flips_and_masks(seed):
+    rs = np.random.RandomState(12000 + seed)
+    nd = int(rs.randint(1, 4))
+    shape = tuple(int(rs.choice([1, 3, 16, 33, 64, 130, 1030])) for _ in range(nd))
+    if np.prod(shape) > 1 << 21:
+        shape = shape[:2]
+    with np.errstate(all="ignore"):
+        d, h = flip_expr(rs, shape, int(rs.randint(0, 4)))
+        anchor = make_host(rs, shape, np.float32)
+        if rs.randint(2):
+            d, h = d + dr.array(anchor)[..., ::-1], h + anchor[..., ::-1]
+        else:
+            d, h = d + dr.array(anchor), h + anchor
+        mode = rs.randint(3)
+        if mode == 0 or len(shape) < 2:
+            got, ref = d.get(), h
+        elif mode == 1:
+            axis = int(rs.randint(len(shape)))
+            got, ref = dr.max(d, axis=axis).get(), np.max(h, axis=axis)
+        else:
+            pad = tuple(s + 2 for s in shape)
+            host = make_host(rs, pad, np.float64)
+            dst_d, dst_h = dr.array(host), host.copy()
+            key = tuple(slice(1, 1 + s) for s in shape)
+            dst_d[key] = d
+            dst_h[key] = h
+            got, ref = dst_d.get(), dst_h
+    assert got.dtype == np.asarray(ref).dtype and bits_equal(got, np.asarray(ref)), (seed, shape, mode)
