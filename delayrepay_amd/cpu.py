@@ -26,6 +26,10 @@ class CpuVisitor(Visitor):
         return node.val
 
     def _apply(self, node):
+        if node.__dict__.get("_cut"):
+            # where the front end evaluated an operand of a very deep expression the walk
+            # ends (every other evaluated node is computed again, as in the reference)
+            return node.array
         return node.func(*[self.visit(child) for child in node.children])
 
     visit_UnaryFuncEx = _apply

@@ -81,6 +81,7 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
                 return arr
             del self.array  # a leaf was written to since: recompute
         self.array = _backend.run(self)
+        self._depth = 0     # a leaf of whatever is built on it from now on
         return self.array
 
     def __array__(self, dtype=None, copy=None):
@@ -474,14 +475,49 @@ def reset():
         forget()
 
 
+# An expression this many operations deep has its deepest operand evaluated before it
+# grows further (`x = f(x)` in a loop that never asks for a value): the walkers over
+# the DAG recurse, and nobody wants a kernel of thousands of operations.
+MAX_DEPTH = 128
+
 class NumpyEx(DelayArray, metaclass=Memoiser):
     """Interior or leaf node of the expression DAG."""
 
     children = ()
+    _depth = 0
 
     def __init__(self, children=()):
         super().__init__()
-        self.children = list(children)
+        self.children = children = list(children)
+        if children:
+            depth = 0
+            for c in children:
+                if c._depth > depth:
+                    depth = c._depth
+            if depth >= MAX_DEPTH:
+                depth = 0
+                for c in children:
+                    if c._depth >= MAX_DEPTH:
+                        c._force()
+                        c._cut = True       # backends that re-walk evaluated nodes stop here
+                    if c._depth > depth:
+                        depth = c._depth
+            self._depth = depth + 1
+
+    def _seal(self):
+        """Turn this evaluated node into a plain holder of its array: it forgets what it
+        was computed from (and lets go of it), is never recomputed, and building the
+        same expression again makes a new node."""
+        d = self.__dict__
+        d.pop("_deps", None)
+        d.pop("_plan", None)
+        d.pop("_multi", None)
+        d.pop("_gen", None)
+        key = d.get("_key")
+        if key is not None and Memoiser._cache.get(key) is self:
+            Memoiser._cache.pop(key)
+        self.children = []
+        self._depth = 0
 
     @classmethod
     def _memo_key(cls, func, *children):

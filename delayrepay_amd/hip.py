@@ -184,6 +184,14 @@ class Tracer(Visitor):
                 deps = node.__dict__.get("_deps")
                 if deps is not None and any(buf.version != ver for buf, ver in deps):
                     arr = None  # stale: recompute inside this kernel
+                elif node.__dict__.get("_gen", 0) >= MAX_GENERATIONS:
+                    # the end of a long chain of results computed from results (`x = f(x)`
+                    # in a loop): from here on this one is an array in its own right, and
+                    # what it was computed from can be freed (a front end without `_seal`
+                    # keeps its chain)
+                    seal = getattr(node, "_seal", None)
+                    if seal is not None:
+                        seal()
         if arr is not None:
             res = self.leaf(arr)
             self.leaf_nodes.append((node, arr, node.__dict__.get("_deps")))
@@ -483,6 +491,11 @@ class record:
         return False
 
 
+# A result computed from results computed from results ...: past this many levels the
+# older result is asked to become an array in its own right (`node._seal()`), so a loop of
+# `x = f(x)` holds a bounded number of earlier iterates, and of their dependencies, alive.
+MAX_GENERATIONS = 4
+
 _STAMP = 0            # bumped whenever tunables or the fusion mode change
 _RECENT = collections.deque(maxlen=int(os.environ.get("DELAYREPAY_KEEP", "16")))
 _RECENT_BYTES = int(os.environ.get("DELAYREPAY_KEEP_BYTES", str(8 << 30)))
@@ -532,6 +545,15 @@ class Plan:
                     if buf.version != ver:
                         return False
         return True
+
+    def generation(self):
+        """1 + the longest chain of cached results below this one."""
+        gen = 0
+        for node, _, _ in self.checks:
+            g = node.__dict__.get("_gen", 0)
+            if g > gen:
+                gen = g
+        return gen + 1
 
     def deps(self):
         """What the result just computed depends on, as (buffer, version) pairs: the
@@ -809,6 +831,7 @@ def run(ex):
         STATS["plan_hits"] += 1
     out = _launch_fresh(plan)[0]
     d["_deps"] = plan.deps()
+    d["_gen"] = plan.generation()
     return out
 
 
@@ -836,11 +859,13 @@ def run_multi(exs):
             _remember(exs[idxs[0]])
         outs = _launch_fresh(plan)
         deps = plan.deps()
+        gen = plan.generation()
         for i, out in zip(idxs, outs):
             if out.shape != shape:   # every leaf of this root was a broadcast scalar
                 out = materialise(out, shape=shape)
             results[i] = out
             exs[i].__dict__["_deps"] = deps
+            exs[i].__dict__["_gen"] = gen
     return results
 
 

@@ -122,6 +122,13 @@ SCRIPT = textwrap.dedent("""
     for _ in range(60):
         big = big + 1.0
     assert isinstance(big[1:3], NPArray) and "array" in big.__dict__       # too large: evaluated once
+    # a loop of x = f(x) that never asks for a value: the expression stops growing at
+    # MAX_DEPTH operations (its deepest operand is evaluated), so nothing recurses too far
+    x, hx = array(np.full(32, 1.0)), np.full(32, 1.0)
+    for _ in range(3000):
+        x, hx = x * 0.999 + 0.5, hx * 0.999 + 0.5
+        assert x._depth <= dnp.delayarray.MAX_DEPTH
+    assert "array" not in x.__dict__ and np.array_equal(x.get(), hx)
     print("cpu-backend-ok")
 """)
 

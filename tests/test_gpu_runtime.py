@@ -291,3 +291,55 @@ def test_matrix_product_on_the_matrix_cores(dtype, tol):
     a = rs.standard_normal((600, 777)).astype(dtype)
     assert np.allclose((dr.array(a) @ dr.array(v)).get(), a @ v, rtol=1e-4 if dtype == np.float32 else 1e-12,
                        atol=1e-4 if dtype == np.float32 else 1e-12)
+
+
+def test_a_loop_of_functional_updates_holds_a_bounded_history():
+    """`x = f(x)` evaluated every pass: results computed from results are a chain; past
+    `hip.MAX_GENERATIONS` links the older result becomes an array in its own right, so the
+    chain, its dependency lists and the device memory of earlier iterates stay bounded."""
+    import gc
+    import delayrepay_amd as dr
+    from delayrepay_amd import hip
+    n = 1 << 18
+    hx, hy = np.full(n, 1.0, np.float32), np.full(n, 0.25, np.float32)
+    y = dr.array(hy)
+    x = dr.array(hx)
+    gc.collect()
+    base = hiprt.pool_stats()["bytes_in_use"]
+    longest = 0
+    hist = [hx]
+    for k in range(300):
+        x = x * 0.5 + y
+        x.run()
+        hx = hx * np.float32(0.5) + hy
+        hist.append(hx)
+        longest = max(longest, len(x.__dict__["_deps"]))
+        assert x.__dict__["_gen"] <= hip.MAX_GENERATIONS
+    assert longest <= 2 * (hip.MAX_GENERATIONS + 1)
+    assert np.array_equal(x.get(), hx)
+    gc.collect()
+    held = hiprt.pool_stats()["bytes_in_use"] - base
+    # the chain itself, and the last evaluated roots that are kept for plan reuse
+    assert held <= (hip.MAX_GENERATIONS + 2 + hip._RECENT.maxlen) * 4 * n, held
+    # the links above the last iterate that became an array in its own right still follow
+    # their inputs: y changes, and x is computed afresh from that iterate
+    links = x.__dict__["_gen"]
+    y[:] = 1.0
+    want = hist[-1 - links]
+    for _ in range(links):
+        want = want * np.float32(0.5) + np.float32(1.0)
+    assert np.array_equal(x.get(), want)
+
+
+def test_an_expression_never_asked_for_stops_growing():
+    import delayrepay_amd as dr
+    from delayrepay_amd import delayarray
+    n = 4096
+    hx, hy = np.full(n, 1.0), np.linspace(0, 1, n)
+    x, y = dr.array(hx), dr.array(hy)
+    for _ in range(700):
+        x = x * 0.999 + y
+        hx = hx * 0.999 + hy
+        assert x._depth <= delayarray.MAX_DEPTH
+    assert abs(float(dr.sum(x)) - hx.sum()) <= 1e-9 * hx.sum()
+    assert np.allclose(x.get(), hx, rtol=1e-12)
