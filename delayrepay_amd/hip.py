@@ -18,6 +18,7 @@ Nothing is computed on the host, and there is no fall-back to NumPy: a missing
 library or GPU raises.
 """
 import collections
+import copy
 import hashlib
 import os
 import struct
@@ -44,7 +45,7 @@ COMPILE_OPTS = [
 
 _FUSED = "DELAY_UNFUSED" not in os.environ
 STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0,
-         "disk_write_failures": 0}
+         "lowering_hits": 0, "disk_write_failures": 0}
 
 _COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal") \
     + tuple(cg._PREDICATES)
@@ -501,24 +502,36 @@ _RECENT = collections.deque(maxlen=int(os.environ.get("DELAYREPAY_KEEP", "16")))
 _RECENT_BYTES = int(os.environ.get("DELAYREPAY_KEEP_BYTES", str(8 << 30)))
 
 
+_RECENT_SIZES = collections.deque()
+_recent_held = 0
+
+
 def _remember(node):
     """Keep `node` alive so that the same expression, built again, finds its nodes in
     the hash-cons table and its plan on the root.  A kept root also keeps its cached
     result, so the memory held this way is bounded as well as the count."""
+    global _recent_held
+    if not _RECENT.maxlen:
+        return
+    nbytes = numpy.dtype(node.dtype).itemsize
+    for d in node.shape:
+        nbytes *= d
+    if len(_RECENT) == _RECENT.maxlen:
+        _recent_held -= _RECENT_SIZES.popleft()
     _RECENT.append(node)
-    held = 0
-    for k in range(len(_RECENT) - 1, -1, -1):       # newest first
-        arr = _RECENT[k].__dict__.get("array")
-        held += getattr(arr, "nbytes", 0)
-        if held > _RECENT_BYTES and k < len(_RECENT) - 1:
-            for _ in range(k + 1):
-                _RECENT.popleft()
-            break
+    _RECENT_SIZES.append(nbytes)
+    _recent_held += nbytes
+    while _recent_held > _RECENT_BYTES and len(_RECENT) > 1:
+        _RECENT.popleft()
+        _recent_held -= _RECENT_SIZES.popleft()
 
 
 def forget():
     """Drop the recently evaluated roots kept alive for plan reuse."""
+    global _recent_held
     _RECENT.clear()
+    _RECENT_SIZES.clear()
+    _recent_held = 0
 
 
 class Plan:
@@ -650,6 +663,50 @@ def _fire(plan, out_ptrs, reduce_out=None):
 # evaluation entry points
 # ---------------------------------------------------------------------------
 
+_LOWERED = {}          # structure and geometry of an evaluation -> (Lowered, where its sources come from)
+_LOWERED_MAX = 4096
+
+
+def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, reduce_op,
+                in_place=False):
+    """`lowering.lower`, remembered by everything it looks at: the program, every operand's
+    geometry, alignment, buffer size and which operands share a buffer, the destinations and
+    the tunables.  The same expression over fresh arrays of the same layout (`x = f(x)` in a
+    loop) then only has its buffers and scalar values filled in."""
+    bufs = {}
+    geo = []
+    for a in leaves:
+        buf = a.buf
+        geo.append((a.shape, a._strides, a.offset, a.dtype.str, bufs.setdefault(id(buf), len(bufs)),
+                    buf.nbytes, buf.ptr & 255))
+    key = (prog.key(), tuple(geo), tuple(shape), tuple(out_codes), tuple(out_ptrs),
+           tuple(tuple(st) for st in out_strides), reduce_op, in_place, tuple(TUNE.values()))
+    hit = _LOWERED.get(key)
+    if hit is not None:
+        template, recipe = hit
+        low = copy.copy(template)
+        low.srcs = [(leaves[i].buf, off) for i, off in recipe]
+        low.scal = list(scalars)
+        STATS["lowering_hits"] += 1
+        return low
+    low = _lower(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, reduce_op, in_place)
+    recipe = []
+    for buf, off in low.srcs:
+        for i, a in enumerate(leaves):
+            if a.buf is buf and a.offset * a.dtype.itemsize == off:
+                recipe.append((i, off))
+                break
+        else:
+            return low          # a source that is no operand's own view: not remembered
+    if low.scal == list(scalars):
+        if len(_LOWERED) >= _LOWERED_MAX:
+            _LOWERED.clear()
+        template = copy.copy(low)
+        template.srcs = template.scal = None      # holds no buffer alive
+        _LOWERED[key] = (template, recipe)
+    return low
+
+
 def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
     """Lower traced `roots` (list of (ref, code)) into a Plan.  `dst`: existing
     destination view (single root); `reduce_op`/`axes`: reduce the single root with
@@ -712,7 +769,7 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
             plan.empty = True
             plan.low = None
             return plan
-        plan.low = _lower(prog, leaves, tracer.scalars, shape, [plan.acc], [], [], reduce_op)
+        plan.low = _lower_memo(prog, leaves, tracer.scalars, shape, [plan.acc], [], [], reduce_op)
         if tracer.iotas and plan.low.kind != "flat":
             tracer.materialise_indices()
             return _make_plan(tracer, roots, None, reduce_op)
@@ -739,7 +796,7 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
         plan.empty = True
         plan.low = None
         return plan
-    plan.low = _lower(prog, leaves, tracer.scalars, shape, out_codes, out_ptrs, out_strides, None,
+    plan.low = _lower_memo(prog, leaves, tracer.scalars, shape, out_codes, out_ptrs, out_strides, None,
                       in_place)
     if tracer.iotas and plan.low.kind != "flat":
         tracer.materialise_indices()

@@ -275,7 +275,6 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     low.fin_count = 0
     scal_fmt = "".join(_SCALAR_FMT[c] for c in prog.scalars)
     scal_vals = list(scalars)
-    tune = tuple(sorted(TUNE.items()))
 
     flat = ndim <= 1 and all(s == [1] or s == [0] or s == [] for s in m_leaf) \
         and all(s == [1] or s == [] for s in m_out)
@@ -536,7 +535,8 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                                            xcd_bands=bands, nouter=nouter, unaligned=ua)[0]
             tiles_x = -(-(W + ph_o) // tw)     # tiles start `ph_o` columns left of the view
         else:
-            low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place, tune, nouter)
+            low.key = ("tile2d", prog.key(), kinds, group, tuple(out_codes), in_place,
+                       tuple(sorted(TUNE.items())), nouter)
 
             def emit():
                 return cg.emit_stencil(prog, kinds, group, out_codes, tw, th,
@@ -677,7 +677,8 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         mshape, m_leaf, m_out, ndim = [1], [[0] for _ in m_leaf], [[0] for _ in m_out], 1
     index32 = n < 2 ** 31
     low.kind = "nd"
-    low.key = ("nd", prog.key(), ndim, tuple(out_codes), index32, reduce_op, tune)
+    low.key = ("nd", prog.key(), ndim, tuple(out_codes), index32, reduce_op,
+               tuple(sorted(TUNE.items())))
 
     def emit():
         return cg.emit_nd(prog, ndim, out_codes, index32, reduce_op)

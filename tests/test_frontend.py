@@ -13,7 +13,7 @@ import pytest
 
 import delayrepay_amd as dr
 from delayrepay_amd import codegen as cg
-from delayrepay_amd import hip, hiprt, mathlib, mathlib32
+from delayrepay_amd import hip, hiprt, lowering, mathlib, mathlib32
 from delayrepay_amd.delayarray import (BinaryFuncEx, BinaryNumpyEx, CastEx, FullEx, IotaEx, NPArray,
                                        ReduceEx, Scalar, UnaryFuncEx, Memoiser)
 
@@ -303,6 +303,37 @@ def test_views_without_shared_rows_stream_row_by_row():
     row = NPArray(hip.placeholder((n,), np.float32))             # repeats from row to row:
     low, src = hip.lower_only(m + row)                            # the taller tile shares it
     assert low.key[0] == "tile2dv" and low.key[8:10] == (64, 2)
+
+
+def test_lowering_is_remembered_by_structure_and_geometry():
+    """The same expression over fresh arrays of the same layout reuses the kernel choice,
+    with the new buffers and scalar values filled in; another layout, alignment, buffer
+    size, sharing of buffers or tunable is another entry."""
+    def build(c, **kw):
+        x, y = leaf((300, 1000), **kw), leaf((300, 1000))
+        return hip.lower_only(x * c + y)[0], x, y
+    first, x1, y1 = build(2.0)
+    hits = hip.STATS["lowering_hits"]
+    again, x2, y2 = build(-7.5)
+    assert hip.STATS["lowering_hits"] == hits + 1
+    assert again is not first and again.key == first.key and again.tail == first.tail
+    assert [b for b, _ in again.srcs] == [x2.array.buf, y2.array.buf] and again.scal == [np.float32(-7.5)]
+    assert [b for b, _ in first.srcs] == [x1.array.buf, y1.array.buf] and first.scal == [np.float32(2.0)]
+    shifted, _, _ = build(2.0, offset=3)                       # another alignment
+    assert hip.STATS["lowering_hits"] == hits + 1 and shifted.key != first.key
+    a = leaf((64, 64))
+    hip.lower_only(a[1:, :-1] + a[:-1, 1:])                     # two views of one buffer ...
+    hits = hip.STATS["lowering_hits"]
+    b, c = leaf((64, 64)), leaf((64, 64))
+    low = hip.lower_only(b[1:, :-1] + c[:-1, 1:])[0]            # ... are not two buffers
+    assert hip.STATS["lowering_hits"] == hits and all(k[0] != "g" for k in low.key[2])
+    old = lowering.TUNE["unroll"]
+    try:
+        lowering.TUNE["unroll"] = 4
+        tuned, _, _ = build(2.0)
+        assert tuned.key != first.key
+    finally:
+        lowering.TUNE["unroll"] = old
 
 
 def test_bitwise_operations_lower_with_numpy_result_types():
