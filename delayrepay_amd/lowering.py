@@ -1,7 +1,8 @@
 """Layout analysis and kernel choice of the HIP backend.
 
 Given a traced `Program` and the geometry of its operands, decide which kernel
-shape evaluates it (`flat`, `tile2d`/`tile2dv`, `nd`, `axis`), build the cache key
+shape evaluates it (`flat`, `tile2d`/`tile2dv`, `tile3d`, `tile2dt`, `nd`, the `axis_*`
+family), build the cache key
 (program + layout classes + dtypes + the tunables that shape the source), and
 prepare the launch recipe: grid, argument-block format, pointer sources and the
 constant tail of the argument block.  The reference has no counterpart: CuPy's
