@@ -1783,7 +1783,7 @@ def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8, outer=False, stagger=
     return "\n".join(src) + "\n"
 
 
-def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False):
+def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False, shared=()):
     """Reduction over a long unit-stride last dimension: a block per (row, slice) streams
     its stretch of the row like a flat reduction (256 lanes x 16 bytes x `unroll` per step,
     one accumulator per vector element), combines through `dr_block_reduce` and writes one
@@ -1794,6 +1794,9 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False):
     leaf_kind  per leaf 'v' (unit stride along the row) or 'k' (constant along it)
     outer      a second, outer reduced dimension (sum over the first and last axis of a
                3-D array): a block then takes whole rows, a slice of the outer range
+    shared     indices of 'v' leaves that every row reads again (the vector of a
+               matrix-vector product): cached loads; the others are read once and
+               non-temporal
     Parameters: leaf pointers, output pointer, scalars, K, R, S, RS, then per leaf the
     stride between rows (elements); with `outer` R is the row length, S and RS cut the
     outer extent RO, and RO and every leaf's outer stride follow.  Output layout
@@ -1845,7 +1848,8 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False):
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
             vt = VEC16[dt][0] + "u"
-            L.append(f"{pad}            const {vt} X{i} = __builtin_nontemporal_load((const {vt}*)(row{i} + r));")
+            ptr = f"(const {vt}*)(row{i} + r)"
+            L.append(f"{pad}            const {vt} X{i} = {_ld(i not in shared, ptr)};")
     for e in range(V):
         vargs = [f"X{i}[{e}]" if kind == "v" else f"c{i}" for i, kind in enumerate(leaf_kind)]
         L.append(f"{pad}            {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
@@ -1868,6 +1872,94 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False):
           "        if (threadIdx.x == 0) out[o] = total;",
           "        __syncthreads();          // the block reduction's LDS words are reused",
           "    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"
+
+
+def emit_block_rows_shared(prog, leaf_kind, acc_dt, op, shared, rows=4, unroll=2):
+    """`emit_block_rows` for reductions in which some operand is the same for every row (the
+    vector of a matrix-vector product): a block takes `rows` adjacent rows at once, loads
+    the shared operands' vectors once per step and uses them for all of them, so a step
+    issues rows + 1 loads for rows x V elements instead of 2 x rows.  Every row is summed
+    in the order `emit_block_rows` uses, so the results are the same to the bit.
+
+    leaf_kind  per leaf 'v' (unit stride along the row) or 'k' (constant along it)
+    shared     indices of the 'v' leaves every row reads again (cached loads; the others
+               are read once and non-temporal)
+    Parameters: leaf pointers, output pointer, scalars, K (rows), R (row length), then per
+    leaf the stride between rows (elements).  One output per row."""
+    ct = CTYPE[acc_dt]
+    nl = len(prog.leaves)
+    widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "v"}
+    V = 16 // widths.pop()
+    src = [PREAMBLE, emit_body(prog, [acc_dt]), emit_block_reduce(op, acc_dt)]
+    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
+    params.append(f"{ct}* __restrict__ out")
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += ["const long long K", "const long long R"]
+    params += [f"const long long sk{i}" for i in range(nl)]
+    call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
+    ident = _identity(op, acc_dt)
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{",
+         f"    for (long long k0 = (long long)blockIdx.x * {rows}; k0 < K; k0 += (long long)gridDim.x * {rows}) {{",
+         f"        {ct} acc[{rows}][{V}];",
+         "#pragma unroll",
+         f"        for (int j = 0; j < {rows}; ++j)",
+         "#pragma unroll",
+         f"            for (int e = 0; e < {V}; ++e) acc[j][e] = {ident};"]
+    for j in range(rows):
+        L.append(f"        const long long kr{j} = k0 + {j} < K ? k0 + {j} : K - 1;   // past the end: the last row again, not stored")
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind == "v" and i in shared:
+            continue
+        for j in range(rows):
+            if kind == "v":
+                L.append(f"        const {CTYPE[dt]}* row{i}_{j} = a{i} + kr{j} * sk{i};")
+            else:
+                L.append(f"        const {CTYPE[dt]} c{i}_{j} = a{i}[kr{j} * sk{i}];")
+    L += [f"        long long r = (long long)threadIdx.x * {V};",
+          f"#pragma unroll {unroll}",
+          f"        for (; r + {V} <= R; r += {BLOCK * V}) {{"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind != "v":
+            continue
+        vt = VEC16[dt][0] + "u"
+        if i in shared:
+            L.append(f"            const {vt} X{i} = *((const {vt}*)(a{i} + r));")
+        else:
+            for j in range(rows):
+                L.append(f"            const {vt} X{i}_{j} = __builtin_nontemporal_load((const {vt}*)(row{i}_{j} + r));")
+
+    def arg(i, kind, j, e):
+        if kind == "v":
+            return f"X{i}[{e}]" if i in shared else f"X{i}_{j}[{e}]"
+        return f"c{i}_{j}"
+
+    for j in range(rows):
+        for e in range(V):
+            vargs = [arg(i, kind, j, e) for i, kind in enumerate(leaf_kind)]
+            L.append(f"            {{ {ct} t0; dr_body({', '.join(vargs + call_tail)}); "
+                     f"acc[{j}][{e}] = {_combine(op, f'acc[{j}][{e}]', 't0')}; }}")
+    L.append("        }")
+    # the one thread whose next vector would straddle the end of the row takes the rest of
+    # it element by element
+    L.append("        for (; r < R; ++r) {")
+    for j in range(rows):
+        sargs = [(f"a{i}[r]" if i in shared else f"row{i}_{j}[r]") if kind == "v" else f"c{i}_{j}"
+                 for i, kind in enumerate(leaf_kind)]
+        L.append(f"            {{ {ct} t0; dr_body({', '.join(sargs + call_tail)}); "
+                 f"acc[{j}][0] = {_combine(op, f'acc[{j}][0]', 't0')}; }}")
+    L.append("        }")
+    for j in range(rows):
+        accs = [f"acc[{j}][{e}]" for e in range(V)]
+        while len(accs) > 1:
+            accs = [f"({_combine(op, accs[i], accs[i + 1])})" if i + 1 < len(accs) else accs[i]
+                    for i in range(0, len(accs), 2)]
+        L += [f"        {{ const {ct} total = dr_block_reduce({accs[0]});",
+              f"          if (threadIdx.x == 0 && k0 + {j} < K) out[k0 + {j}] = total;",
+              "          __syncthreads(); }"]
+    L += ["    }", "}"]
     src.append("\n".join(L))
     return "\n".join(src) + "\n"
 

@@ -33,6 +33,8 @@ TUNE = {
     "ax_group_steps": 8,  # most 16-byte units a lane of such a group takes from its row
     "ax_slices": 512,    # most slices (the second pass walks them serially per output)
     "ax_block": 4096,    # reduced unit-stride extents from this length: a block per row slice
+    "ax_block_rows": 2,  # ... and this many rows per block when an operand is the same for all
+    "ax_block_rows_unroll": 2,   # ... with this many steps in flight
     "ax_stream": 256,    # kept unit-stride extents of 256 vectors or more: blocks to aim for, one
                          # per compute unit (0: off)
     "ax_stream_unroll": 8,   # ... and rows in flight per lane
@@ -931,14 +933,33 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
             RS = -(-R // S)
             S = -(-R // RS)
             kinds = tuple("v" if r[0] == 1 else "k" for r in rsets)
+            # an operand that is the same for every row (the vector of a matrix-vector
+            # product) stays in the caches; `a @ x` on 16384^2 float32: 76.8 % of the HBM
+            # peak with every load non-temporal
+            shared = tuple(i for i, (k, r) in enumerate(zip(ksets, rsets)) if r[0] == 1 and k[0] == 0)
             low = Lowered()
             low.lds = 0
             low.fin_count = 0
             low.kind = "axis_block"
-            low.key = ("axis_block", prog.key(), kinds, acc, reduce_op)
+            low.key = ("axis_block", prog.key(), kinds, acc, reduce_op, shared)
+            rows = TUNE["ax_block_rows"]
+            if shared and S == 1 and rows > 1 and K >= 1024 * rows:
+                # several rows per block: the shared operand is loaded once for all of them
+                unroll = TUNE["ax_block_rows_unroll"]
+                low.key = ("axis_block", prog.key(), kinds, acc, reduce_op, shared, unroll, rows)
+
+                def emit_rows():
+                    return cg.emit_block_rows_shared(prog, kinds, acc, reduce_op, shared, rows, unroll)
+                low.emit = emit_rows
+                low.grid = max(1, min(-(-K // rows), 1 << 20))
+                low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
+                           + "qq" + "q" * len(leaves))
+                low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+                low.scal, low.tail = list(scalars), [K, R] + [k[0] for k in ksets]
+                return low, 1, K, "row"
 
             def emit_block():
-                return cg.emit_block_rows(prog, kinds, acc, reduce_op)
+                return cg.emit_block_rows(prog, kinds, acc, reduce_op, shared=shared)
             low.emit = emit_block
             low.grid = max(1, min(K * S, 1 << 20))
             low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)

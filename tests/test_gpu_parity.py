@@ -26,7 +26,7 @@ import numpy as np
 import pytest
 
 import delayrepay_amd as dr
-from delayrepay_amd import hip
+from delayrepay_amd import hip, lowering
 from delayrepay_amd.delayarray import ReduceEx
 from oracle import numpy_oracle as orc
 from oracle.numpy_oracle import OracleArray
@@ -824,6 +824,36 @@ def test_matrix_vector_products_are_fused_reductions(dtype, tol):
         dr.array(np.zeros(5, dtype)) @ dr.array(np.zeros((4, 5), dtype))
     i = dr.array(np.arange(12).reshape(3, 4)) @ dr.array(np.arange(4))     # integers: as before
     assert np.array_equal(np.asarray(i.get(), dtype=np.int64), np.arange(12).reshape(3, 4) @ np.arange(4))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_rows_that_share_an_operand_take_several_rows_per_block(dtype):
+    """Row reductions with an operand that is the same for every row (`A @ x`): several rows
+    per block, the shared vectors loaded once; the same sums to the bit as a block per row,
+    row counts that are not multiples of the group, ragged row lengths, a per-row weight."""
+    rs = np.random.RandomState(47)
+    for m, k in [(4096, 4096), (4099, 5001), (5000, 4100)]:
+        a0, x0, w0 = (rs.standard_normal(s).astype(dtype) for s in ((m, k), (k,), (m, 1)))
+        a, x, w = dr.array(a0), dr.array(x0), dr.array(w0)
+        results = {}
+        default = lowering.TUNE["ax_block_rows"]
+        for rows in (2, 3, 4, 1):
+            hip.set_tune(ax_block_rows=rows)
+            try:
+                low = hip.lower_only(ReduceEx(np.add, a * x, (1,)))[0]
+                assert low.kind == "axis_block" and (low.key[-1] == rows) == (rows > 1), (m, k, rows)
+                results[rows] = (hip.run(ReduceEx(np.add, a * x, (1,))).get(),
+                                 hip.run(ReduceEx(np.maximum, a * x * w, (1,))).get())
+            finally:
+                hip.set_tune(ax_block_rows=default)
+        for rows in (2, 3, 4):
+            assert bits_equal(results[rows][0], results[1][0]), (m, k, rows)
+            assert bits_equal(results[rows][1], results[1][1]), (m, k, rows)
+        ref = a0.astype(np.float64) @ x0.astype(np.float64)
+        scale = np.abs(a0.astype(np.float64)) @ np.abs(x0.astype(np.float64))
+        tol = 2e-5 if dtype == np.float32 else 1e-13
+        assert np.all(np.abs(results[4][0] - ref) <= tol * scale)
+        assert np.array_equal(results[4][1], (a0 * x0 * w0).max(axis=1))
 
 
 def test_bitwise_operations_and_shifts_follow_numpy():
