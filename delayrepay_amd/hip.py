@@ -18,7 +18,6 @@ Nothing is computed on the host, and there is no fall-back to NumPy: a missing
 library or GPU raises.
 """
 import collections
-import copy
 import hashlib
 import os
 import struct
@@ -32,7 +31,8 @@ from .devarray import Buffer, ndarray, placeholder  # noqa: F401
 from .codegen import Program, dtype_code, code_dtype
 from .promote import result_dtype, scalar_descr
 from .visitor import Visitor
-from .lowering import (TUNE, broadcast_strides as _broadcast_strides, lower as _lower,
+from .lowering import (TUNE, Lowered as _Lowered, broadcast_strides as _broadcast_strides,
+                       lower as _lower,
                        lower_axis_reduce as _lower_axis_reduce)
 
 hiprt.lib()  # fail at import when libdrhip.so has not been built
@@ -684,7 +684,9 @@ def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, 
     hit = _LOWERED.get(key)
     if hit is not None:
         template, recipe = hit
-        low = copy.copy(template)
+        low = _Lowered()
+        low.key, low.kind, low.emit, low.fmt = template.key, template.kind, template.emit, template.fmt
+        low.tail, low.grid, low.fin_count, low.lds = template.tail, template.grid, template.fin_count, template.lds
         low.srcs = [(leaves[i].buf, off) for i, off in recipe]
         low.scal = list(scalars)
         STATS["lowering_hits"] += 1
@@ -701,10 +703,24 @@ def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, 
     if low.scal == list(scalars):
         if len(_LOWERED) >= _LOWERED_MAX:
             _LOWERED.clear()
-        template = copy.copy(low)
-        template.srcs = template.scal = None      # holds no buffer alive
+        template = _Lowered()                     # holds no buffer alive
+        template.key, template.kind, template.emit, template.fmt = low.key, low.kind, low.emit, low.fmt
+        template.tail, template.grid, template.fin_count, template.lds = (low.tail, low.grid,
+                                                                          low.fin_count, low.lds)
         _LOWERED[key] = (template, recipe)
     return low
+
+
+def _common_shape(leaves, gen_shapes):
+    """Broadcast shape of the operands (most often they all have the same one)."""
+    if leaves and not gen_shapes:
+        first = leaves[0].shape
+        for a in leaves:
+            if a.shape != first:
+                break
+        else:
+            return first
+    return tuple(numpy.broadcast_shapes(*[a.shape for a in leaves], *gen_shapes))
 
 
 def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
@@ -734,7 +750,7 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
     plan.kern2 = None
     plan.scratch = 0
     if reduce_op:
-        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves], *tracer.gen_shapes))
+        shape = _common_shape(leaves, tracer.gen_shapes)
         code = roots[0][1]
         plan.acc = "i8" if (reduce_op == "add" and code in ("i4", "u4", "u1", "b1")) else code
         plan.out_dtypes = [code_dtype(plan.acc)]
@@ -775,7 +791,7 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
             return _make_plan(tracer, roots, None, reduce_op)
         return plan
     if dst is None:
-        shape = tuple(numpy.broadcast_shapes(*[a.shape for a in leaves], *tracer.gen_shapes))
+        shape = _common_shape(leaves, tracer.gen_shapes)
         plan.out_dtypes = [code_dtype(code) for _, code in roots]
         out_codes = [code for _, code in roots]
         out_ptrs = [0] * len(roots)          # pool blocks are 256-byte aligned
