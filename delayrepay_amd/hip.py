@@ -126,8 +126,9 @@ class Tracer(Visitor):
     (delayrepay/delayarray.py:434-452,462-467), gets NumPy's result all the same.
     Each handler returns (operand reference, dtype code)."""
 
-    def __init__(self, evaluated=None):
+    def __init__(self, evaluated=None, reuse=False):
         super().__init__()
+        self._reuse = reuse       # evaluate deep operands met in an earlier evaluation first
         self.leaves = []
         self.leaf_codes = []
         self._leaf_index = {}
@@ -210,10 +211,22 @@ class Tracer(Visitor):
         """[(child, reference-or-None, descriptor)]: array-valued children are traced,
         numbers are left for the consumer (a weak scalar takes the consumer's type)."""
         out = []
+        reuse = self._reuse
         for child in children:
             if _kind(child) == "Scalar":
                 out.append((child, None, scalar_descr(child.val)))
             else:
+                if reuse:
+                    d = child.__dict__
+                    if "array" not in d and getattr(child, "_depth", 0) >= REUSE_DEPTH:
+                        if "_seen" not in d:
+                            d["_seen"] = True
+                        elif id(child) not in self._memo:
+                            # A deep operand that an earlier evaluation already computed
+                            # inline (`x = f(x)` carried through a loop that only ever asks
+                            # for `sum(g(x))`): computed once on its own now, it is a leaf
+                            # here and in everything built on it later.
+                            child._force()
                 ref, code = self.visit(child)
                 out.append((child, ref, ("a", code)))
         return out
@@ -496,6 +509,10 @@ class record:
 # older result is asked to become an array in its own right (`node._seal()`), so a loop of
 # `x = f(x)` holds a bounded number of earlier iterates, and of their dependencies, alive.
 MAX_GENERATIONS = 4
+# An unevaluated operand at least this many operations deep that an earlier evaluation has
+# already walked through is evaluated on its own when it is met again (shallower ones are
+# cheaper to compute again than to write and read back).
+REUSE_DEPTH = 8
 
 _STAMP = 0            # bumped whenever tunables or the fusion mode change
 _RECENT = collections.deque(maxlen=int(os.environ.get("DELAYREPAY_KEEP", "16")))
@@ -890,7 +907,7 @@ def run(ex):
     d = ex.__dict__
     plan = d.get("_plan")
     if plan is None or not plan.valid():
-        tracer = Tracer()
+        tracer = Tracer(reuse=True)
         if _kind(ex) == "ReduceEx":
             root = tracer.visit(ex.children[0])
             plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__,
@@ -925,7 +942,7 @@ def run_multi(exs):
             plan = cached[1]
             STATS["plan_hits"] += 1
         else:
-            tracer = Tracer()
+            tracer = Tracer(reuse=True)
             roots = [_trace_root(tracer, exs[i]) for i in idxs]
             plan = _make_plan(tracer, roots)
             first["_multi"] = (key, plan, [exs[i] for i in idxs])
@@ -1043,7 +1060,7 @@ def run_into(ex, dst):
         plan = cached[1]
         STATS["plan_hits"] += 1
     else:
-        tracer = Tracer()
+        tracer = Tracer(reuse=True)
         root = _trace_root(tracer, ex)
         plan = _plan_write(tracer, root, dst)
         d["_into"] = (key, plan, dst.buf)     # holding the buffer keeps its id unique

@@ -343,3 +343,34 @@ def test_an_expression_never_asked_for_stops_growing():
         assert x._depth <= delayarray.MAX_DEPTH
     assert abs(float(dr.sum(x)) - hx.sum()) <= 1e-9 * hx.sum()
     assert np.allclose(x.get(), hx, rtol=1e-12)
+
+
+def test_a_carried_expression_that_is_only_ever_reduced_is_evaluated_on_second_sight():
+    """`x = f(x)` carried through a loop that only asks for `sum(g(x))`: the reduction walks
+    through x's whole expression.  Once that expression is `hip.REUSE_DEPTH` operations deep
+    and is met in a second evaluation, it is computed once on its own and is a leaf from then
+    on, so the work per pass and the number of kernel structures stay bounded."""
+    import delayrepay_amd as dr
+    n = 1 << 14
+    hx, hy = np.linspace(0.0, 1.0, n), np.linspace(1.0, 2.0, n)
+    x, y = dr.array(hx), dr.array(hy)
+    structures = set()
+    before = len(hip._KERNELS)
+    carried = []
+    for k in range(60):
+        x = x * 0.5 + y
+        hx = hx * 0.5 + hy
+        got = float(dr.sum(x * x))
+        want = float(np.sum(hx * hx))
+        assert abs(got - want) <= 1e-12 * want, k
+        carried.append(x)
+    assert len(hip._KERNELS) - before <= 12                  # not one structure per pass
+    evaluated = sum("array" in node.__dict__ for node in carried)
+    assert evaluated >= 40                                    # most iterates became leaves
+    assert np.allclose(x.get(), hx, rtol=1e-14)
+    # shallow shared operands are computed again rather than written and read back
+    a, b = dr.array(hx), dr.array(hy)
+    d = a - b
+    r1, r2 = float(dr.sum(d * d)), float(dr.sum(abs(d)))
+    assert "array" not in d.__dict__
+    assert abs(r1 - np.sum((hx - hy) ** 2)) <= 1e-12 * r1 and abs(r2 - np.sum(np.abs(hx - hy))) <= 1e-12 * r2
