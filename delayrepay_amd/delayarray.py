@@ -120,10 +120,15 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
             return _reduce(ufunc, inputs[0], **kwargs)
         if method != "__call__":
             return NotImplemented
+        target = None
         if kwargs:
             out = kwargs.get("out")
             if isinstance(out, tuple) and len(out) == 1 and out[0] is inputs[0]:
                 # `x += y`: like the reference, build a new node and let Python rebind x
+                kwargs = {k: v for k, v in kwargs.items() if k != "out"}
+            elif isinstance(out, tuple) and len(out) == 1 and isinstance(out[0], DelayArray):
+                # `np.multiply(a, b, out=c)`: the fused kernel writes straight into c
+                target = out[0]
                 kwargs = {k: v for k, v in kwargs.items() if k != "out"}
             bad = [k for k, v in kwargs.items() if v is not None]
             if bad:
@@ -131,7 +136,17 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         if ufunc.__name__ == "matmul":
             return self._dot(inputs, {})
         args = [arg_to_numpy_ex(arg) for arg in inputs]
-        return create_ex(ufunc, args)
+        node = create_ex(ufunc, args)
+        if target is not None:
+            if tuple(node.shape) != tuple(target.shape):
+                raise ValueError(f"non-broadcastable output operand with shape {tuple(target.shape)} "
+                                 f"doesn't match the broadcast shape {tuple(node.shape)}")
+            if not np.can_cast(node.dtype, target.dtype, casting="same_kind"):
+                raise TypeError(f"Cannot cast ufunc '{ufunc.__name__}' output from {node.dtype} to "
+                                f"{target.dtype} with casting rule 'same_kind'")
+            target[...] = node
+            return target
+        return node
 
     def __array_function__(self, func, types, args, kwargs):
         if func.__name__ == "dot":

@@ -122,6 +122,17 @@ SCRIPT = textwrap.dedent("""
     for _ in range(60):
         big = big + 1.0
     assert isinstance(big[1:3], NPArray) and "array" in big.__dict__       # too large: evaluated once
+    # out= on a ufunc writes into the destination and returns it (tests/test.py has no such case;
+    # the reference ignores the keyword, delayarray.py:46-61)
+    dst, src = array(np.zeros(64)), array(np.arange(64.0))
+    back = np.multiply(src, 3.0, out=dst)
+    assert back is dst and np.array_equal(dst.get(), np.arange(64.0) * 3.0)
+    assert np.sqrt(src, out=dst) is dst and np.array_equal(dst.get(), np.sqrt(np.arange(64.0)))
+    try:
+        np.add(src, 1.0, out=array(np.zeros(64, dtype=np.int32)))
+        raise SystemExit("a float result must not be cast into an integer destination")
+    except TypeError:
+        pass
     # a loop of x = f(x) that never asks for a value: the expression stops growing at
     # MAX_DEPTH operations (its deepest operand is evaluated), so nothing recurses too far
     x, hx = array(np.full(32, 1.0)), np.full(32, 1.0)

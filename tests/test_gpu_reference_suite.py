@@ -8,6 +8,7 @@ import numpy.testing as npt
 import pytest
 
 import delayrepay as dnp
+from delayrepay_amd import hip
 from delayrepay import NPArray, array, full, ones, sum  # noqa: A004
 
 from .helpers import bits_equal, ulp_distance
@@ -216,6 +217,34 @@ class TestSurface:
         assert np.all(c.get() == 12)       # through b, although b's buffer was never written
         assert np.all(b.get() == 11)
         assert np.all(p.get() == 22) and np.all(q.get() == 10)
+
+    def test_out_keyword_writes_into_the_destination(self):
+        """`np.multiply(a, b, out=c)`: one fused kernel writes c (also a view, also with a
+        conversion NumPy allows); the call returns c; shapes and unsafe casts are refused
+        as NumPy refuses them."""
+        a0, b0 = np.arange(40.0).reshape(5, 8), np.linspace(1, 2, 40).reshape(5, 8)
+        a, b = array(a0), array(b0)
+        c = array(np.zeros((5, 8)))
+        launches = hip.STATS["launches"]
+        assert np.multiply(a + 1, b, out=c) is c
+        assert hip.STATS["launches"] == launches + 1
+        assert np.array_equal(c.get(), (a0 + 1) * b0)
+        big = array(np.zeros((7, 10)))
+        view = big[1:6, 1:9]
+        np.subtract(a, b, out=view)
+        want = np.zeros((7, 10))
+        want[1:6, 1:9] = a0 - b0
+        assert np.array_equal(big.get(), want)
+        f32 = array(np.zeros((5, 8), dtype=np.float32))
+        np.add(a, b, out=f32)
+        assert np.array_equal(f32.get(), (a0 + b0).astype(np.float32))
+        with pytest.raises(TypeError):
+            np.add(a, b, out=array(np.zeros((5, 8), dtype=np.int64)))
+        with pytest.raises(ValueError):
+            np.add(a, b, out=array(np.zeros((5, 9))))
+        x = array(a0.copy())
+        y = np.add(x, 1.0, out=x)                  # the destination is an operand: a new node,
+        assert y is not x and np.array_equal(y.get(), a0 + 1)    # as for `x += 1` (delayarray.py:46-61)
 
     def test_a_write_into_an_evaluated_expression_survives(self):
         x0 = np.arange(8.0)
