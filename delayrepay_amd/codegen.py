@@ -148,6 +148,7 @@ _SHIFTS = {"left_shift": "<<", "right_shift": ">>"}
 
 SUPPORTED_UFUNCS = (set(_FLOAT_FUNCS1) | set(_FLOAT_FUNCS2) | set(_INFIX) | set(_COMPARE)
                     | _PREDICATES | set(_BITWISE) | set(_SHIFTS) | {"invert"}
+                    | {"floor_divide", "remainder"}
                     | {"negative", "positive", "absolute", "fabs", "reciprocal", "maximum",
                        "minimum", "square", "sign"})
 
@@ -155,6 +156,41 @@ SUPPORTED_UFUNCS = (set(_FLOAT_FUNCS1) | set(_FLOAT_FUNCS2) | set(_INFIX) | set(
 def _fn(name, dt):
     """C math function for a float dtype: `sinf` for f4, `sin` for f8."""
     return name + ("f" if dt == "f4" else "")
+
+
+def _divmod_expr(name, dt, args):
+    """`//` and `%` as NumPy computes them (numpy/_core/src/npymath/npy_math_internal.h.src,
+    `npy_divmod`; loops.c.src for the integer rules): the quotient is floored, the
+    remainder takes the divisor's sign; floats go through an exact `fmod`, the quotient
+    is snapped to the nearest integer, zeros keep the sign NumPy gives them, a zero
+    divisor gives a / b (quotient) and NaN (remainder); integer division by zero gives 0,
+    and the most negative integer divided by -1 stays itself (remainder 0)."""
+    ct = CTYPE[dt]
+    a, b = args
+    want_div = name == "floor_divide"
+    if dt in ("f4", "f8"):
+        fmod, floor, copysign = _fn("fmod", dt), _fn("floor", dt), _fn("copysign", dt)
+        body = (f"const {ct} a_ = {a}, b_ = {b}; {ct} m_ = {fmod}(a_, b_); {ct} d_; "
+                f"if (b_ == 0) {{ d_ = a_ / b_; }} else {{ "
+                f"d_ = (a_ - m_) / b_; "
+                f"if (m_ != 0) {{ if ((b_ < 0) != (m_ < 0)) {{ m_ += b_; d_ -= ({ct})1; }} }} "
+                f"else {{ m_ = {copysign}(({ct})0, b_); }} "
+                f"if (d_ != 0) {{ {ct} f_ = {floor}(d_); if (d_ - f_ > ({ct})0.5) f_ += ({ct})1; d_ = f_; }} "
+                f"else {{ d_ = {copysign}(({ct})0, a_ / b_); }} }} ")
+        return "({ " + body + ("d_" if want_div else "m_") + "; })"
+    if dt == "b1":
+        raise TypeError(f"ufunc {name!r} is not fused for boolean operands")
+    if dt[0] == "u":
+        op = "/" if want_div else "%"
+        return f"({b} == 0 ? ({ct})0 : ({ct})({a} {op} {b}))"
+    lowest = {"i4": "(-2147483647 - 1)", "i8": "(-9223372036854775807LL - 1)"}[dt]
+    if want_div:
+        return ("({ " + f"const {ct} a_ = {a}, b_ = {b}; {ct} q_; "
+                f"if (b_ == 0) q_ = 0; else if (a_ == {lowest} && b_ == -1) q_ = a_; "
+                f"else {{ q_ = a_ / b_; if (((a_ > 0) != (b_ > 0)) && q_ * b_ != a_) --q_; }} q_; " + "})")
+    return ("({ " + f"const {ct} a_ = {a}, b_ = {b}; {ct} r_; "
+            f"if (b_ == 0 || (a_ == {lowest} && b_ == -1)) r_ = 0; "
+            f"else {{ r_ = a_ % b_; if (r_ != 0 && ((a_ > 0) != (b_ > 0))) r_ += b_; }} r_; " + "})")
 
 
 def op_expr(name, dt, args):
@@ -189,6 +225,8 @@ def op_expr(name, dt, args):
             return f"(({uns}){b} >= {bits} ? ({CTYPE[dt]})0 : ({CTYPE[dt]})(({uns}){a} << {b}))"
         fill = f"({CTYPE[dt]})({a} < 0 ? -1 : 0)" if dt[0] == "i" else f"({CTYPE[dt]})0"
         return f"(({uns}){b} >= {bits} ? {fill} : ({CTYPE[dt]})({a} >> {b}))"
+    if name in ("floor_divide", "remainder"):
+        return _divmod_expr(name, dt, args)
     if name in _INFIX:
         if name in ("divide", "true_divide") and not is_float:
             raise NotImplementedError("integer division has no float result type here")

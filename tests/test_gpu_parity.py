@@ -856,6 +856,47 @@ def test_rows_that_share_an_operand_take_several_rows_per_block(dtype):
         assert np.array_equal(results[4][1], (a0 * x0 * w0).max(axis=1))
 
 
+def test_floor_division_and_remainder_follow_numpy():
+    """`//` and `%`: floored quotient, remainder with the divisor's sign, to the bit; zero
+    divisors, infinities, NaN, signed zeros, exact multiples, quotients just below an integer;
+    integers with zero divisors and the most negative value divided by -1; mixed operands."""
+    rs = np.random.RandomState(48)
+    n = 6001
+    for dt in (np.float32, np.float64):
+        a0 = (rs.standard_normal(n) * 50).astype(dt)
+        b0 = (rs.standard_normal(n) * 3).astype(dt)
+        special = np.array([0.0, -0.0, 1.0, -1.0, 3.0, -3.0, 0.5, -0.5, np.inf, -np.inf, np.nan, 1e30, -1e-30,
+                            7.0, -7.0, 0.1, 0.3], dt)
+        a0[:special.size ** 2] = np.repeat(special, special.size)
+        b0[:special.size ** 2] = np.tile(special, special.size)
+        a0[400:800] = np.round(a0[400:800])                       # exact multiples
+        b0[400:800] = np.round(b0[400:800]) + (np.round(b0[400:800]) == 0)
+        a, b = dr.array(a0), dr.array(b0)
+        with np.errstate(all="ignore"):
+            assert bits_equal((a // b).get(), a0 // b0), dt
+            assert bits_equal((a % b).get(), a0 % b0), dt
+            assert bits_equal((a // 3).get(), a0 // dt(3)) and bits_equal((a % -0.7).get(), a0 % dt(-0.7)), dt
+            assert bits_equal(np.remainder(a, b).get(), np.remainder(a0, b0)), dt
+            assert bits_equal(((a // b) * b + a % b).get(), (a0 // b0) * b0 + a0 % b0), dt
+    for dt in (np.int32, np.int64, np.uint32, np.uint8):
+        info = np.iinfo(dt)
+        x0 = rs.randint(max(info.min, -10 ** 9), min(info.max, 10 ** 9), n).astype(dt)
+        y0 = rs.randint(max(info.min, -40), min(info.max, 40) if dt != np.uint8 else 40, n).astype(dt)
+        x0[:6] = [info.min, info.min, info.max, 0, info.min, 7]
+        y0[:6] = [info.max if info.min == 0 else -1, 1, 1 if info.min == 0 else -1, 0, 0, 0]
+        x, y = dr.array(x0), dr.array(y0)
+        with np.errstate(all="ignore"):
+            for got, want in [(x // y, x0 // y0), (x % y, x0 % y0), (x // 7, x0 // 7), (x % 7, x0 % 7),
+                              ((x % 2 == 0), (x0 % 2 == 0))]:
+                got = got.get()
+                assert got.dtype == want.dtype and np.array_equal(got, want), dt
+    i0 = rs.randint(-99, 99, n)
+    f0 = rs.standard_normal(n)
+    with np.errstate(all="ignore"):
+        assert bits_equal((dr.array(i0) % dr.array(f0)).get(), i0 % f0)
+        assert bits_equal((dr.array(f0) // dr.array(i0)).get(), f0 // i0)
+
+
 def test_bitwise_operations_and_shifts_follow_numpy():
     """`&`, `|`, `^`, `~` on masks and integers, shifts with counts up to and beyond the
     type's width (NumPy shifts everything out), mixed bool / integer operands, float
