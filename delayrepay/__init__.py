@@ -7,7 +7,8 @@ import sys as _sys
 import delayrepay_amd as _impl
 from delayrepay_amd import *  # noqa: F401,F403
 from delayrepay_amd import (sum, max, min, abs, mean, var, average, evaluate,  # noqa: F401
-                            synchronize, reset, pi, backend, random)
+                            synchronize, reset, pi, backend, random, std, count_nonzero, isclose,
+                            allclose, norm, any, all)  # noqa: A004
 
 for _name in ("backend", "delayarray", "visitor", "random", "cpu", "hip", "codegen", "devarray",
               "hiprt"):

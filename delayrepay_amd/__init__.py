@@ -9,7 +9,9 @@ from . import backend as _be
 from .delayarray import *  # noqa: F401,F403
 from .delayarray import (DelayArray, NPArray, Scalar, NumpyEx, BinaryNumpyEx, BinaryFuncEx,  # noqa: F401
                          UnaryFuncEx, ReduceEx, CastEx, Memoiser, reset, evaluate, synchronize,
-                         sum, max, min, abs, mean, var, average, where, clip, WhereEx)
+                         sum, max, min, abs, mean, var, average, where, clip, WhereEx,
+                         std, count_nonzero, isclose, allclose, norm)
+from .delayarray import any_ as any, all_ as all  # noqa: F401,A004
 from . import random  # noqa: F401
 
 backend = _be.backend

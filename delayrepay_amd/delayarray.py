@@ -1098,6 +1098,66 @@ _eager_transpose = cast(_eager("transpose"))
 _eager_roll = cast(_eager("roll"))
 
 
+@implements(np.std)
+def std(arr, axis=None, ddof=0, keepdims=False, **kwargs):
+    return np.sqrt(var(arr, axis=axis, ddof=ddof, keepdims=keepdims, **kwargs))
+
+
+def _truth(arr):
+    arr = arg_to_numpy_ex(arr)
+    return arr if arr.dtype == np.bool_ else np.not_equal(arr, 0)
+
+
+@implements(np.any)
+def any_(arr, axis=None, keepdims=False, **kwargs):
+    """True where some element along `axis` is non-zero: the fused maximum of a mask."""
+    return _reduce(np.maximum, _truth(arr), axis=axis, keepdims=keepdims, **kwargs)
+
+
+@implements(np.all)
+def all_(arr, axis=None, keepdims=False, **kwargs):
+    return _reduce(np.minimum, _truth(arr), axis=axis, keepdims=keepdims, **kwargs)
+
+
+@implements(np.count_nonzero)
+def count_nonzero(arr, axis=None, keepdims=False):
+    return _reduce(np.add, _truth(arr), axis=axis, keepdims=keepdims)
+
+
+@implements(np.isclose)
+def isclose(a, b, rtol=1e-05, atol=1e-08, equal_nan=False):
+    """`numpy.isclose`, one fused mask: |a - b| <= atol + rtol |b| where b is finite, or a == b
+    (equal infinities), or both NaN when asked for."""
+    a, b = arg_to_numpy_ex(a), arg_to_numpy_ex(b)
+    near = np.less_equal(np.absolute(a - b), atol + rtol * np.absolute(b))
+    close = (near & np.isfinite(b)) | np.equal(a, b)
+    if equal_nan:
+        close = close | (np.isnan(a) & np.isnan(b))
+    return close
+
+
+@implements(np.allclose)
+def allclose(a, b, rtol=1e-05, atol=1e-08, equal_nan=False):
+    """`numpy.allclose`: the mask of `isclose` fused with its reduction; a Python bool."""
+    return bool(all_(isclose(a, b, rtol=rtol, atol=atol, equal_nan=equal_nan)))
+
+
+@implements(np.linalg.norm)
+def norm(x, ord=None, axis=None, keepdims=False):           # noqa: A002
+    """`numpy.linalg.norm` for the 2-norm of vectors and the Frobenius norm (the defaults):
+    the square root of a fused sum of squares."""
+    x = arg_to_numpy_ex(x)
+    flat = axis is None or isinstance(axis, (int, np.integer)) or len(axis) == 1
+    if not (ord is None or (ord == 2 and flat and (axis is not None or x.ndim == 1))
+            or (ord == "fro" and (x.ndim == 2 or (axis is not None and not flat)))):
+        raise NotImplementedError(f"norm(ord={ord!r}, axis={axis!r}) is not supported on lazy arrays")
+    if x.dtype.kind in "iub":
+        x = x.astype(np.float64)
+    total = _reduce(np.add, x * x, axis=axis, keepdims=keepdims)
+    total = total if isinstance(total, DelayArray) else NPArray(total)
+    return np.sqrt(total)
+
+
 @implements(np.transpose)
 def transpose(arr, axes=None):
     """View of the evaluated array with permuted axes (delayarray.py:521-524); a small

@@ -133,6 +133,19 @@ SCRIPT = textwrap.dedent("""
         raise SystemExit("a float result must not be cast into an integer destination")
     except TypeError:
         pass
+    # any / all / count_nonzero / std / isclose / allclose / linalg.norm: compositions of the
+    # fused reductions (none is registered by the reference, delayarray.py:485-615)
+    h0 = np.random.RandomState(3).standard_normal((50, 70))
+    h1 = h0 + 1e-9
+    d0, d1 = array(h0), array(h1)
+    assert bool(np.any(d0 > 3)) == (h0 > 3).any() and bool(np.all(d0 > -5)) == (h0 > -5).all()
+    assert np.array_equal(np.any(d0 > 2, axis=1).get(), (h0 > 2).any(axis=1))
+    assert np.array_equal(np.all(d0 > -2, axis=0).get(), (h0 > -2).all(axis=0))
+    assert np.allclose(d0, d1) is True and np.allclose(d0, d1 + 1) is False
+    assert np.array_equal(np.isclose(d0, d1, rtol=0, atol=5e-10).get(), np.isclose(h0, h1, rtol=0, atol=5e-10))
+    assert abs(float(np.linalg.norm(d0)) - np.linalg.norm(h0)) < 1e-12
+    assert np.allclose(np.linalg.norm(d0, axis=1).get(), np.linalg.norm(h0, axis=1), rtol=1e-14)
+    assert abs(float(np.std(d0)) - h0.std()) < 1e-14 and int(np.count_nonzero(d0 > 0)) == np.count_nonzero(h0 > 0)
     # a loop of x = f(x) that never asks for a value: the expression stops growing at
     # MAX_DEPTH operations (its deepest operand is evaluated), so nothing recurses too far
     x, hx = array(np.full(32, 1.0)), np.full(32, 1.0)

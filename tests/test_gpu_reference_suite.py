@@ -218,6 +218,45 @@ class TestSurface:
         assert np.all(b.get() == 11)
         assert np.all(p.get() == 22) and np.all(q.get() == 10)
 
+    def test_truth_tests_norms_and_closeness(self):
+        """`any`, `all`, `count_nonzero`, `std`, `isclose`, `allclose`, `linalg.norm`: masks
+        and squares fused with their reductions; NaN and infinities in `isclose` as NumPy
+        treats them; the convergence test of an iteration as one would write it."""
+        rs = np.random.RandomState(9)
+        h0 = rs.standard_normal((300, 1100)).astype(np.float32)
+        h1 = h0 + rs.uniform(-1e-6, 1e-6, h0.shape).astype(np.float32)
+        h0[3, 4], h1[3, 4] = np.inf, np.inf
+        h0[5, 6], h1[5, 6] = np.nan, np.nan
+        h0[7, 8], h1[7, 8] = np.inf, -np.inf
+        a, b = array(h0), array(h1)
+        with np.errstate(all="ignore"):
+            assert np.array_equal(np.isclose(a, b).get(), np.isclose(h0, h1))
+            assert np.array_equal(np.isclose(a, b, equal_nan=True).get(), np.isclose(h0, h1, equal_nan=True))
+            assert np.allclose(a, b) is False and np.allclose(a[10:], b[10:], atol=1e-5) is True
+        g0 = np.where(np.isfinite(h0), h0, 0).astype(np.float32)
+        g = array(g0)
+        assert bool(np.any(g > 4)) == bool((g0 > 4).any()) and bool(np.all(g > -6)) == bool((g0 > -6).all())
+        assert np.array_equal(np.any(g > 3, axis=0).get(), (g0 > 3).any(axis=0))
+        assert np.array_equal(np.all(g > -3, axis=1).get(), (g0 > -3).all(axis=1))
+        assert np.array_equal(np.any(g, axis=1).get(), g0.any(axis=1))
+        assert int(np.count_nonzero(g > 0)) == np.count_nonzero(g0 > 0)
+        assert np.array_equal(np.count_nonzero(g > 1, axis=1).get(), np.count_nonzero(g0 > 1, axis=1))
+        ref = np.linalg.norm(g0.astype(np.float64))
+        assert abs(float(np.linalg.norm(g)) - ref) <= 2e-6 * ref
+        npt.assert_allclose(np.linalg.norm(g, axis=1).get(), np.linalg.norm(g0.astype(np.float64), axis=1), rtol=2e-6)
+        npt.assert_allclose(float(np.linalg.norm(g[0], 2)), np.linalg.norm(g0[0].astype(np.float64)), rtol=2e-6)
+        npt.assert_allclose(float(np.std(g)), g0.astype(np.float64).std(), rtol=2e-6)
+        npt.assert_allclose(np.std(g, axis=0, ddof=1).get(), g0.astype(np.float64).std(axis=0, ddof=1), rtol=2e-5)
+        with pytest.raises(NotImplementedError):
+            np.linalg.norm(g, 1)
+        x = array(np.full(4096, 8.0))
+        steps = 0
+        while not np.allclose(x, 1.0, rtol=0, atol=1e-6) and steps < 100:
+            x = 0.5 * (x + 1.0)
+            x.run()
+            steps += 1
+        assert 20 <= steps <= 30 and float(np.linalg.norm(x - 1.0)) < 1e-3
+
     def test_out_keyword_writes_into_the_destination(self):
         """`np.multiply(a, b, out=c)`: one fused kernel writes c (also a view, also with a
         conversion NumPy allows); the call returns c; shapes and unsafe casts are refused
