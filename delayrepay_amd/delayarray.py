@@ -26,6 +26,7 @@ or bounded memory:
   * `dst[key] = lazy_expression` is handed to the backend as one fused write;
   * `evaluate(a, b, ...)` computes several roots in one kernel.
 """
+import builtins
 import math
 import numbers
 import weakref
@@ -1156,6 +1157,178 @@ def norm(x, ord=None, axis=None, keepdims=False):           # noqa: A002
     total = _reduce(np.add, x * x, axis=axis, keepdims=keepdims)
     total = total if isinstance(total, DelayArray) else NPArray(total)
     return np.sqrt(total)
+
+
+# ---- views and compositions NumPy code reaches for (none is registered by the reference;
+#      each is indexing, arithmetic or a fused write that the backend already has) -----------
+
+def _axis(axis, ndim):
+    axis = int(axis)
+    if not -ndim <= axis < ndim:
+        raise np.exceptions.AxisError(axis, ndim)
+    return axis % ndim
+
+
+@implements(np.flip)
+def flip(m, axis=None):
+    """Reversed along `axis` (all axes when None): a view with negative strides, read as
+    reversed vectors by the tiled kernel."""
+    m = arg_to_numpy_ex(m)
+    axes = range(m.ndim) if axis is None else \
+        [_axis(a, m.ndim) for a in ((axis,) if isinstance(axis, (int, np.integer)) else axis)]
+    key = [slice(None)] * m.ndim
+    for a in axes:
+        key[a] = slice(None, None, -1)
+    return m[tuple(key)]
+
+
+@implements(np.flipud)
+def flipud(m):
+    return flip(m, 0)
+
+
+@implements(np.fliplr)
+def fliplr(m):
+    if arg_to_numpy_ex(m).ndim < 2:
+        raise ValueError("Input must be >= 2-d.")
+    return flip(m, 1)
+
+
+@implements(np.diff)
+def diff(a, n=1, axis=-1, **kwargs):
+    """n-th difference along `axis`: shifted views of one expression, one stencil kernel."""
+    if kwargs:
+        raise NotImplementedError(f"diff keyword(s) {sorted(kwargs)} are not supported on lazy arrays")
+    a = arg_to_numpy_ex(a)
+    axis = _axis(axis, a.ndim)
+    hi, lo = [slice(None)] * a.ndim, [slice(None)] * a.ndim
+    hi[axis], lo[axis] = slice(1, None), slice(None, -1)
+    for _ in range(int(n)):
+        a = a[tuple(hi)] ^ a[tuple(lo)] if a.dtype == np.bool_ else a[tuple(hi)] - a[tuple(lo)]
+    return a
+
+
+@implements(np.outer)
+def outer(a, b):
+    a, b = arg_to_numpy_ex(a), arg_to_numpy_ex(b)
+    return a.reshape(a.size, 1) * b.reshape(1, b.size)
+
+
+@implements(np.ptp)
+def ptp(a, axis=None, keepdims=False):
+    return max(a, axis=axis, keepdims=keepdims) - min(a, axis=axis, keepdims=keepdims)
+
+
+@implements(np.expand_dims)
+def expand_dims(a, axis):
+    a = arg_to_numpy_ex(a)
+    axes = (axis,) if isinstance(axis, (int, np.integer)) else tuple(axis)
+    ndim = a.ndim + len(axes)
+    axes = sorted(_axis(x, ndim) for x in axes)
+    key = [slice(None)] * ndim
+    for x in axes:
+        key[x] = None
+    return a[tuple(key)]
+
+
+@implements(np.squeeze)
+def squeeze(a, axis=None):
+    a = arg_to_numpy_ex(a)
+    if axis is None:
+        drop = [k for k, d in enumerate(a.shape) if d == 1]
+    else:
+        drop = [_axis(x, a.ndim) for x in ((axis,) if isinstance(axis, (int, np.integer)) else axis)]
+        if builtins.any(a.shape[k] != 1 for k in drop):
+            raise ValueError("cannot select an axis to squeeze out which has size not equal to one")
+    return a[tuple(0 if k in drop else slice(None) for k in range(a.ndim))]
+
+
+@implements(np.swapaxes)
+def swapaxes(a, axis1, axis2):
+    a = arg_to_numpy_ex(a)
+    order = list(range(a.ndim))
+    i, j = _axis(axis1, a.ndim), _axis(axis2, a.ndim)
+    order[i], order[j] = order[j], order[i]
+    return transpose(a, order)
+
+
+@implements(np.moveaxis)
+def moveaxis(a, source, destination):
+    a = arg_to_numpy_ex(a)
+    src = [_axis(x, a.ndim) for x in ((source,) if isinstance(source, (int, np.integer)) else source)]
+    dst = [_axis(x, a.ndim) for x in ((destination,) if isinstance(destination, (int, np.integer))
+                                      else destination)]
+    if len(src) != len(dst):
+        raise ValueError("`source` and `destination` arguments must have the same number of elements")
+    order = [k for k in range(a.ndim) if k not in src]
+    for d, sx in sorted(zip(dst, src)):
+        order.insert(d, sx)
+    return transpose(a, order)
+
+
+@implements(np.reshape)
+def reshape(a, *args, **kwargs):
+    return arg_to_numpy_ex(a).reshape(*args, **kwargs)
+
+
+@implements(np.ravel)
+def ravel(a):
+    return arg_to_numpy_ex(a).ravel()
+
+
+@implements(np.concatenate)
+def concatenate(arrays, axis=0, **kwargs):
+    """Every part is written straight into its slice of the result by its own fused kernel:
+    lazy parts are never materialised on their own."""
+    if kwargs:
+        raise NotImplementedError(f"concatenate keyword(s) {sorted(kwargs)} are not supported on lazy arrays")
+    parts = [arg_to_numpy_ex(a) for a in arrays]
+    if not parts:
+        raise ValueError("need at least one array to concatenate")
+    if axis is None:
+        parts, axis = [p.ravel() for p in parts], 0
+    ndim = parts[0].ndim
+    if ndim == 0:
+        raise ValueError("zero-dimensional arrays cannot be concatenated")
+    axis = _axis(axis, ndim)
+    for p in parts:
+        if p.ndim != ndim or builtins.any(p.shape[k] != parts[0].shape[k] for k in range(ndim) if k != axis):
+            raise ValueError("all the input array dimensions except for the concatenation axis must match exactly")
+    shape = list(parts[0].shape)
+    shape[axis] = builtins.sum(p.shape[axis] for p in parts)
+    dtype = np.result_type(*[p.dtype for p in parts])
+    out = NPArray(_backend.fallback.empty(tuple(shape), dtype=dtype))
+    at = 0
+    for p in parts:
+        key = [slice(None)] * ndim
+        key[axis] = slice(at, at + p.shape[axis])
+        if p.shape[axis]:
+            out[tuple(key)] = p
+        at += p.shape[axis]
+    return out
+
+
+@implements(np.stack)
+def stack(arrays, axis=0, **kwargs):
+    parts = [arg_to_numpy_ex(a) for a in arrays]
+    if not parts:
+        raise ValueError("need at least one array to stack")
+    if builtins.any(p.shape != parts[0].shape for p in parts):
+        raise ValueError("all input arrays must have the same shape")
+    axis = _axis(axis, parts[0].ndim + 1)
+    return concatenate([expand_dims(p, axis) for p in parts], axis=axis, **kwargs)
+
+
+@implements(np.vstack)
+def vstack(tup):
+    parts = [arg_to_numpy_ex(a) for a in tup]
+    return concatenate([p.reshape(1, -1) if p.ndim < 2 else p for p in parts], axis=0)
+
+
+@implements(np.hstack)
+def hstack(tup):
+    parts = [arg_to_numpy_ex(a) for a in tup]
+    return concatenate(parts, axis=0 if parts and parts[0].ndim == 1 else 1)
 
 
 @implements(np.transpose)

@@ -146,6 +146,28 @@ SCRIPT = textwrap.dedent("""
     assert abs(float(np.linalg.norm(d0)) - np.linalg.norm(h0)) < 1e-12
     assert np.allclose(np.linalg.norm(d0, axis=1).get(), np.linalg.norm(h0, axis=1), rtol=1e-14)
     assert abs(float(np.std(d0)) - h0.std()) < 1e-14 and int(np.count_nonzero(d0 > 0)) == np.count_nonzero(h0 > 0)
+    # flips, differences, axis manipulation, concatenation: indexing, arithmetic and fused writes
+    rs_ = np.random.RandomState(0)
+    h, g = rs_.standard_normal((4, 5, 6)), rs_.standard_normal((4, 5, 6))
+    a, b = array(h), array(g)
+    eq = lambda x, y: np.array_equal(x.get(), y)
+    assert eq(np.flip(a), np.flip(h)) and eq(np.flip(a + 1, (0, 2)), np.flip(h + 1, (0, 2)))
+    assert eq(np.flipud(a), np.flipud(h)) and eq(np.fliplr(a), np.fliplr(h))
+    assert eq(np.diff(a), np.diff(h)) and eq(np.diff(a * 2, n=2, axis=0), np.diff(h * 2, n=2, axis=0))
+    assert eq(np.diff(a > 0, axis=1), np.diff(h > 0, axis=1))
+    assert eq(np.outer(a[0, 0], b[1, 1]), np.outer(h[0, 0], g[1, 1])) and eq(np.ptp(a, axis=1), np.ptp(h, axis=1))
+    assert eq(np.expand_dims(a + b, (0, -1)), np.expand_dims(h + g, (0, -1)))
+    assert eq(np.squeeze(np.expand_dims(a, 2)), h) and eq(np.squeeze(a[:1] * 2, axis=0), h[0] * 2)
+    assert eq(np.swapaxes(a, 0, 2), np.swapaxes(h, 0, 2))
+    assert eq(np.moveaxis(a + 1, (0, 1), (2, 0)), np.moveaxis(h + 1, (0, 1), (2, 0)))
+    assert eq(np.reshape(a, (20, 6)), h.reshape(20, 6)) and eq(np.ravel(a * b), (h * g).ravel())
+    assert eq(np.concatenate([a, b * 2, a + b], axis=1), np.concatenate([h, g * 2, h + g], axis=1))
+    assert eq(np.concatenate([a, b], axis=None), np.concatenate([h, g], axis=None))
+    mixed = np.concatenate([a, b.astype(np.float32)], axis=-1)
+    assert mixed.dtype == np.float64 and eq(mixed, np.concatenate([h, g.astype(np.float32)], axis=-1))
+    assert eq(np.stack([a, b + 1], axis=2), np.stack([h, g + 1], axis=2))
+    assert eq(np.vstack([a[0, 0], b[0, 0]]), np.vstack([h[0, 0], g[0, 0]]))
+    assert eq(np.hstack([a[0], b[0]]), np.hstack([h[0], g[0]]))
     # a loop of x = f(x) that never asks for a value: the expression stops growing at
     # MAX_DEPTH operations (its deepest operand is evaluated), so nothing recurses too far
     x, hx = array(np.full(32, 1.0)), np.full(32, 1.0)

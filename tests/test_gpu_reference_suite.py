@@ -257,6 +257,41 @@ class TestSurface:
             steps += 1
         assert 20 <= steps <= 30 and float(np.linalg.norm(x - 1.0)) < 1e-3
 
+    def test_views_differences_and_concatenation(self):
+        """`flip`, `diff`, `outer`, `ptp`, `expand_dims`, `squeeze`, `swapaxes`, `moveaxis`,
+        `reshape`, `ravel`, `concatenate`, `stack`, `vstack`, `hstack` against NumPy; the
+        parts of a concatenation are written into place by one fused kernel each."""
+        rs_ = np.random.RandomState(0)
+        h, g = rs_.standard_normal((4, 5, 6)), rs_.standard_normal((4, 5, 6))
+        a, b = array(h), array(g)
+        eq = lambda x, y: np.array_equal(x.get(), y)
+        assert eq(np.flip(a), np.flip(h)) and eq(np.flip(a + 1, (0, 2)), np.flip(h + 1, (0, 2)))
+        assert eq(np.flipud(a), np.flipud(h)) and eq(np.fliplr(a), np.fliplr(h))
+        assert eq(np.diff(a), np.diff(h)) and eq(np.diff(a * 2, n=2, axis=0), np.diff(h * 2, n=2, axis=0))
+        assert eq(np.diff(a > 0, axis=1), np.diff(h > 0, axis=1))
+        assert eq(np.outer(a[0, 0], b[1, 1]), np.outer(h[0, 0], g[1, 1])) and eq(np.ptp(a, axis=1), np.ptp(h, axis=1))
+        assert eq(np.expand_dims(a + b, (0, -1)), np.expand_dims(h + g, (0, -1)))
+        assert eq(np.squeeze(np.expand_dims(a, 2)), h) and eq(np.squeeze(a[:1] * 2, axis=0), h[0] * 2)
+        assert eq(np.swapaxes(a, 0, 2), np.swapaxes(h, 0, 2))
+        assert eq(np.moveaxis(a + 1, (0, 1), (2, 0)), np.moveaxis(h + 1, (0, 1), (2, 0)))
+        assert eq(np.reshape(a, (20, 6)), h.reshape(20, 6)) and eq(np.ravel(a * b), (h * g).ravel())
+        assert eq(np.concatenate([a, b * 2, a + b], axis=1), np.concatenate([h, g * 2, h + g], axis=1))
+        assert eq(np.concatenate([a, b], axis=None), np.concatenate([h, g], axis=None))
+        mixed = np.concatenate([a, b.astype(np.float32)], axis=-1)
+        assert mixed.dtype == np.float64 and eq(mixed, np.concatenate([h, g.astype(np.float32)], axis=-1))
+        assert eq(np.stack([a, b + 1], axis=2), np.stack([h, g + 1], axis=2))
+        assert eq(np.vstack([a[0, 0], b[0, 0]]), np.vstack([h[0, 0], g[0, 0]]))
+        assert eq(np.hstack([a[0], b[0]]), np.hstack([h[0], g[0]]))
+        big = array(np.arange(200000.0))
+        launches = hip.STATS["launches"]
+        both = np.concatenate([big * 2, np.sqrt(big), big[::-1]])
+        assert hip.STATS["launches"] == launches + 3
+        ref = np.arange(200000.0)
+        assert np.array_equal(both.get(), np.concatenate([ref * 2, np.sqrt(ref), ref[::-1]]))
+        assert np.array_equal(np.diff(big * big, n=2).get(), np.diff(ref * ref, n=2))
+        with pytest.raises(ValueError):
+            np.concatenate([a, b[:, :4]], axis=0)
+
     def test_out_keyword_writes_into_the_destination(self):
         """`np.multiply(a, b, out=c)`: one fused kernel writes c (also a view, also with a
         conversion NumPy allows); the call returns c; shapes and unsafe casts are refused
