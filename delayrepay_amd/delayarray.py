@@ -1331,6 +1331,34 @@ def hstack(tup):
     return concatenate(parts, axis=0 if parts and parts[0].ndim == 1 else 1)
 
 
+@implements(np.broadcast_to)
+def broadcast_to(a, shape, **kwargs):
+    """Stretched view (no copy) of the evaluated array, as a leaf."""
+    return NPArray(_backend.fallback.broadcast_to(arg_to_numpy_ex(a)._force(), _shape_of(shape)))
+
+
+@implements(np.trace)
+def trace(a, offset=0, axis1=0, axis2=1, **kwargs):
+    a = arg_to_numpy_ex(a)
+    if a.ndim != 2 or (axis1, axis2) != (0, 1) or kwargs:
+        raise NotImplementedError("trace is supported for matrices (axis1=0, axis2=1) only")
+    return _reduce(np.add, diag(a, offset))
+
+
+@implements(np.inner)
+def inner(a, b):
+    a, b = arg_to_numpy_ex(a), arg_to_numpy_ex(b)
+    if a.ndim != 1 or b.ndim != 1:
+        raise NotImplementedError("inner is supported for vectors only")
+    return a._dot([a, b], {})
+
+
+@implements(np.vdot)
+def vdot(a, b):
+    a, b = arg_to_numpy_ex(a), arg_to_numpy_ex(b)
+    return inner(a.ravel(), b.ravel())
+
+
 @implements(np.transpose)
 def transpose(arr, axes=None):
     """View of the evaluated array with permuted axes (delayarray.py:521-524); a small

@@ -291,6 +291,13 @@ class TestSurface:
         assert np.array_equal(np.diff(big * big, n=2).get(), np.diff(ref * ref, n=2))
         with pytest.raises(ValueError):
             np.concatenate([a, b[:, :4]], axis=0)
+        m0, v0 = rs_.standard_normal((60, 60)), rs_.standard_normal(60)
+        m, v = array(m0), array(v0)
+        npt.assert_allclose(float(np.trace(m)), np.trace(m0), rtol=1e-13)
+        npt.assert_allclose(float(np.trace(m, 2)), np.trace(m0, 2), rtol=1e-13)
+        npt.assert_allclose(float(np.inner(v, v)), np.inner(v0, v0), rtol=1e-13)
+        npt.assert_allclose(float(np.vdot(m, m)), np.vdot(m0, m0), rtol=1e-13)
+        assert np.array_equal((np.broadcast_to(v, (60, 60)) + m).get(), v0 + m0)
 
     def test_out_keyword_writes_into_the_destination(self):
         """`np.multiply(a, b, out=c)`: one fused kernel writes c (also a view, also with a
