@@ -321,6 +321,51 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
     def var(self, *args, **kwargs):
         return np.var(self, *args, **kwargs)
 
+    def std(self, *args, **kwargs):
+        return np.std(self, *args, **kwargs)
+
+    def any(self, *args, **kwargs):
+        return np.any(self, *args, **kwargs)
+
+    def all(self, *args, **kwargs):
+        return np.all(self, *args, **kwargs)
+
+    def ptp(self, *args, **kwargs):
+        return np.ptp(self, *args, **kwargs)
+
+    def clip(self, a_min=None, a_max=None, **kwargs):
+        return np.clip(self, a_min, a_max, **kwargs)
+
+    def cumsum(self, *args, **kwargs):
+        return np.cumsum(self, *args, **kwargs)
+
+    def squeeze(self, axis=None):
+        return np.squeeze(self, axis)
+
+    def swapaxes(self, axis1, axis2):
+        return np.swapaxes(self, axis1, axis2)
+
+    def trace(self, *args, **kwargs):
+        return np.trace(self, *args, **kwargs)
+
+    def item(self, *args):
+        """The element as a Python number (of a one-element array when no index is given)."""
+        return self.get().item(*args)
+
+    def tolist(self):
+        return self.get().tolist()
+
+    def fill(self, value):
+        self[...] = value
+
+    @property
+    def itemsize(self):
+        return np.dtype(self.dtype).itemsize
+
+    @property
+    def nbytes(self):
+        return self.size * self.itemsize
+
     def repeat(self, *args, **kwargs):
         return repeat(self, *args, **kwargs)
 

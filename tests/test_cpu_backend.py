@@ -168,6 +168,16 @@ SCRIPT = textwrap.dedent("""
     assert eq(np.stack([a, b + 1], axis=2), np.stack([h, g + 1], axis=2))
     assert eq(np.vstack([a[0, 0], b[0, 0]]), np.vstack([h[0, 0], g[0, 0]]))
     assert eq(np.hstack([a[0], b[0]]), np.hstack([h[0], g[0]]))
+    # ndarray's methods on lazy arrays
+    hm = np.random.RandomState(4).standard_normal((5, 7))
+    am = array(hm)
+    assert abs(float(am.std()) - hm.std()) < 1e-14 and bool((am > -9).all()) and not bool((am > 9).any())
+    assert np.array_equal(am.clip(-1, 1).get(), hm.clip(-1, 1)) and np.array_equal(am.cumsum().get(), hm.cumsum())
+    assert np.array_equal(am.swapaxes(0, 1).get(), hm.T) and np.array_equal(am[:1].squeeze().get(), hm[0])
+    assert am[1, 2].item() == hm[1, 2] and am.tolist() == hm.tolist() and am.nbytes == hm.nbytes
+    bm = array(np.zeros(8))
+    bm.fill(3.5)
+    assert np.all(bm.get() == 3.5) and float(am.ptp()) == np.ptp(hm)
     # a loop of x = f(x) that never asks for a value: the expression stops growing at
     # MAX_DEPTH operations (its deepest operand is evaluated), so nothing recurses too far
     x, hx = array(np.full(32, 1.0)), np.full(32, 1.0)

@@ -298,6 +298,13 @@ class TestSurface:
         npt.assert_allclose(float(np.inner(v, v)), np.inner(v0, v0), rtol=1e-13)
         npt.assert_allclose(float(np.vdot(m, m)), np.vdot(m0, m0), rtol=1e-13)
         assert np.array_equal((np.broadcast_to(v, (60, 60)) + m).get(), v0 + m0)
+        npt.assert_allclose(float(m.std()), m0.std(), rtol=1e-13)
+        assert bool((m > -9).all()) and not bool((m > 9).any()) and float(m.ptp()) == np.ptp(m0)
+        assert np.array_equal(m.clip(-1, 1).get(), m0.clip(-1, 1)) and np.array_equal(m.swapaxes(0, 1).get(), m0.T)
+        assert m[1, 2].item() == m0[1, 2] and m[:2, :3].tolist() == m0[:2, :3].tolist() and m.nbytes == m0.nbytes
+        z = array(np.zeros(5000))
+        z.fill(3.5)
+        assert np.all(z.get() == 3.5)
 
     def test_out_keyword_writes_into_the_destination(self):
         """`np.multiply(a, b, out=c)`: one fused kernel writes c (also a view, also with a
