@@ -374,3 +374,29 @@ def test_a_carried_expression_that_is_only_ever_reduced_is_evaluated_on_second_s
     r1, r2 = float(dr.sum(d * d)), float(dr.sum(abs(d)))
     assert "array" not in d.__dict__
     assert abs(r1 - np.sum((hx - hy) ** 2)) <= 1e-12 * r1 and abs(r2 - np.sum(np.abs(hx - hy))) <= 1e-12 * r2
+
+
+def test_evaluations_leave_no_reference_cycles_behind():
+    """Device memory must be freed with its last user, not whenever the cycle collector gets
+    round to it: with the collector switched off, a long loop of fresh results still holds a
+    bounded number of arrays, and a collection afterwards finds no tracer to free."""
+    import gc
+    import delayrepay_amd as dr
+    n = 1 << 18
+    y = dr.array(np.ones(n, np.float32))
+    x = dr.array(np.zeros(n, np.float32))
+    gc.collect()
+    base = hiprt.pool_stats()["bytes_in_use"]
+    gc.disable()
+    try:
+        for k in range(200):
+            x = x * 0.999 + y
+            x.run()
+            if k % 3 == 0:
+                float(dr.sum(x))
+        held = hiprt.pool_stats()["bytes_in_use"] - base
+    finally:
+        gc.enable()
+    assert held <= (hip.MAX_GENERATIONS + 2 + hip._RECENT.maxlen) * 4 * n, held
+    gc.collect()
+    assert not [o for o in gc.get_objects() if isinstance(o, hip.Tracer)]
