@@ -979,6 +979,11 @@ def _over_views(root, view, key=None):
         return walk(root)
     except _TooLarge:
         return None
+    finally:
+        # `walk` refers to itself through its closure, a reference cycle: empty what the
+        # cycle holds (nodes and their arrays) rather than leave it to the cycle collector
+        memo.clear()
+        walk = view = fb = None
 
 
 class _TooLarge(Exception):

@@ -22,6 +22,7 @@ import hashlib
 import os
 import struct
 import warnings
+import weakref
 
 import numpy
 
@@ -938,14 +939,18 @@ def run_multi(exs):
         first = exs[idxs[0]].__dict__
         key = tuple(id(exs[i]) for i in idxs)
         cached = first.get("_multi")
-        if cached is not None and cached[0] == key and cached[1].valid():
+        if cached is not None and cached[0] == key and cached[1].valid() \
+                and all(ref() is not None for ref in cached[2]):
             plan = cached[1]
             STATS["plan_hits"] += 1
         else:
             tracer = Tracer(reuse=True)
             roots = [_trace_root(tracer, exs[i]) for i in idxs]
             plan = _make_plan(tracer, roots)
-            first["_multi"] = (key, plan, [exs[i] for i in idxs])
+            # the other roots are held weakly (the key holds their ids, which are only
+            # theirs while they live); a strong list on the first root would contain that
+            # root itself: a reference cycle that keeps every result until the collector runs
+            first["_multi"] = (key, plan, [weakref.ref(exs[i]) for i in idxs[1:]])
             _remember(exs[idxs[0]])
         outs = _launch_fresh(plan)
         deps = plan.deps()

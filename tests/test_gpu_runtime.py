@@ -400,3 +400,24 @@ def test_evaluations_leave_no_reference_cycles_behind():
     assert held <= (hip.MAX_GENERATIONS + 2 + hip._RECENT.maxlen) * 4 * n, held
     gc.collect()
     assert not [o for o in gc.get_objects() if isinstance(o, hip.Tracer)]
+    # the other entry points: several roots at once, updates in place, slices of lazy
+    # expressions, eager helpers
+    u = dr.array(np.zeros((300, 300), np.float32))
+
+    def work(k):
+        nonlocal x
+        a, b = dr.evaluate(x * 0.5 + y, x - y * float(k))
+        x = a
+        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:]) + float(k)
+        dr.var(u, axis=1)
+        dr.roll(a * 2.0, 3)
+        (u.T * 2.0).run()
+        (a * 2.0 + b)[5:-5].run()
+        np.concatenate([a, b])
+        float(np.linalg.norm(a))
+    for k in range(5):
+        work(k)
+    gc.collect()
+    for k in range(20):
+        work(k + 5)
+    assert gc.collect() <= 10
