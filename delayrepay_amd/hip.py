@@ -22,7 +22,6 @@ import hashlib
 import os
 import struct
 import warnings
-import weakref
 
 import numpy
 
@@ -219,11 +218,13 @@ class Tracer(Visitor):
             else:
                 if reuse:
                     d = child.__dict__
-                    if "array" not in d and getattr(child, "_depth", 0) >= REUSE_DEPTH:
-                        if "_seen" not in d:
-                            d["_seen"] = True
-                        elif id(child) not in self._memo:
-                            # A deep operand that an earlier evaluation already computed
+                    if "array" not in d and getattr(child, "_depth", 0) >= REUSE_DEPTH \
+                            and id(child) not in self._memo:
+                        seen = d.get("_seen", 0)
+                        if seen < REUSE_AFTER:
+                            d["_seen"] = seen + 1
+                        else:
+                            # A deep operand that earlier evaluations already computed
                             # inline (`x = f(x)` carried through a loop that only ever asks
                             # for `sum(g(x))`): computed once on its own now, it is a leaf
                             # here and in everything built on it later.
@@ -510,10 +511,12 @@ class record:
 # older result is asked to become an array in its own right (`node._seal()`), so a loop of
 # `x = f(x)` holds a bounded number of earlier iterates, and of their dependencies, alive.
 MAX_GENERATIONS = 4
-# An unevaluated operand at least this many operations deep that an earlier evaluation has
-# already walked through is evaluated on its own when it is met again (shallower ones are
-# cheaper to compute again than to write and read back).
+# An unevaluated operand at least this many operations deep that two earlier evaluations have
+# already walked through is evaluated on its own when it is met a third time (shallower ones
+# are cheaper to compute again than to write and read back; two roots that share a deep
+# operand, a call and a put price, may well be asked for one after the other).
 REUSE_DEPTH = 8
+REUSE_AFTER = 2       # evaluations that computed it inline before it is computed on its own
 
 _STAMP = 0            # bumped whenever tunables or the fusion mode change
 _RECENT = collections.deque(maxlen=int(os.environ.get("DELAYREPAY_KEEP", "16")))
@@ -939,18 +942,18 @@ def run_multi(exs):
         first = exs[idxs[0]].__dict__
         key = tuple(id(exs[i]) for i in idxs)
         cached = first.get("_multi")
-        if cached is not None and cached[0] == key and cached[1].valid() \
-                and all(ref() is not None for ref in cached[2]):
+        if cached is not None and cached[0] == key and cached[1].valid():
             plan = cached[1]
             STATS["plan_hits"] += 1
         else:
             tracer = Tracer(reuse=True)
             roots = [_trace_root(tracer, exs[i]) for i in idxs]
             plan = _make_plan(tracer, roots)
-            # the other roots are held weakly (the key holds their ids, which are only
-            # theirs while they live); a strong list on the first root would contain that
-            # root itself: a reference cycle that keeps every result until the collector runs
-            first["_multi"] = (key, plan, [weakref.ref(exs[i]) for i in idxs[1:]])
+            # the other roots are kept alive with the entry (the key holds their ids, which
+            # are only theirs while they live); not the first root itself: on its own
+            # attribute that would be a reference cycle, and every result would wait for
+            # the cycle collector
+            first["_multi"] = (key, plan, [exs[i] for i in idxs[1:]])
             _remember(exs[idxs[0]])
         outs = _launch_fresh(plan)
         deps = plan.deps()

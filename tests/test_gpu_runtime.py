@@ -345,10 +345,10 @@ def test_an_expression_never_asked_for_stops_growing():
     assert np.allclose(x.get(), hx, rtol=1e-12)
 
 
-def test_a_carried_expression_that_is_only_ever_reduced_is_evaluated_on_second_sight():
+def test_a_carried_expression_that_is_only_ever_reduced_is_evaluated_on_third_sight():
     """`x = f(x)` carried through a loop that only asks for `sum(g(x))`: the reduction walks
     through x's whole expression.  Once that expression is `hip.REUSE_DEPTH` operations deep
-    and is met in a second evaluation, it is computed once on its own and is a leaf from then
+    and is met in a third evaluation, it is computed once on its own and is a leaf from then
     on, so the work per pass and the number of kernel structures stay bounded."""
     import delayrepay_amd as dr
     n = 1 << 14
@@ -421,3 +421,30 @@ def test_evaluations_leave_no_reference_cycles_behind():
     for k in range(20):
         work(k + 5)
     assert gc.collect() <= 10
+
+
+def test_rebuilding_a_multi_root_expression_reuses_its_plan():
+    """A step that builds call and put prices anew every time and evaluates them together:
+    the nodes are the hash-consed ones of the step before, the cached plan is found, one
+    kernel runs, and no shared operand is computed on its own."""
+    import delayrepay_amd as dr
+    from oracle import numpy_oracle as orc
+    rs = np.random.RandomState(12)
+    S, K, T = (dr.array(rs.uniform(0.5, 2.0, 1 << 14)) for _ in range(3))
+    for step in range(4):
+        call, put = orc.black_scholes_expr(dr, S, K, T, 0.02, 0.3)
+        launches, hits = hip.STATS["launches"], hip.STATS["plan_hits"]
+        outs = hip.run_multi([call, put])
+        del call, put
+        assert hip.STATS["launches"] == launches + 1, step
+        if step:
+            assert hip.STATS["plan_hits"] == hits + 1, step
+    # asked for one after the other (over fresh arrays: operands nobody has walked through
+    # yet), the two prices still share nothing that is written out
+    S2, K2, T2 = (dr.array(a.get()) for a in (S, K, T))
+    call, put = orc.black_scholes_expr(dr, S2, K2, T2, 0.02, 0.3)
+    launches = hip.STATS["launches"]
+    c2 = hip.run(call)
+    p2 = hip.run(put)
+    assert hip.STATS["launches"] == launches + 2
+    assert np.array_equal(c2.get(), outs[0].get()) and np.array_equal(p2.get(), outs[1].get())
