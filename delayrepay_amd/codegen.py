@@ -593,7 +593,7 @@ def packs(prog, vec):
 
 
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
-              reduce_op=None, unaligned=False):
+              reduce_op=None, unaligned=False, one_run=False):
     """Contiguous 1-D kernel.
 
     leaf_class  per leaf 'c' (contiguous, same length as the output) or 'b'
@@ -603,6 +603,10 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     unaligned   some pointer is not 16-byte aligned: vectors at element alignment
     reduce_op   None, or 'add' | 'maximum' | 'minimum': the single root is
                 reduced instead of stored; the output is one partial per block
+    one_run     block c handles run c and nothing else (the grid must have at least
+                n / elements per run blocks); without the loop over runs the compiler
+                needs fewer registers, and the block asks for its operands before it
+                copies the functions' tables into LDS, so one wait covers both
     """
     rs = "__restrict__ " if restrict else ""
     ua = "u" if unaligned else ""
@@ -630,7 +634,8 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     L.append(f'extern "C" __global__ __launch_bounds__({BLOCK})')
     L.append(f"void dr_kernel({', '.join(params)})")
     L.append("{")
-    if mathlib.tables(prog.own_math):
+    staged = bool(mathlib.tables(prog.own_math))
+    if staged and not one_run:
         L.append("    DR_STAGE_TABLES();      // the functions' tables, from memory into LDS")
     for i, c in enumerate(leaf_class):
         if c == "b":
@@ -704,7 +709,11 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     if vec:
         L.append(f"    const long long nvec = n / {E};")
     L.append(f"    const long long nchunk = {count} / {BLOCK * unroll};")
-    L.append("    for (long long c = blockIdx.x; c < nchunk; c += gridDim.x) {")
+    if one_run:
+        L.append("    if (blockIdx.x < nchunk) {")
+        L.append("        const long long c = blockIdx.x;")
+    else:
+        L.append("    for (long long c = blockIdx.x; c < nchunk; c += gridDim.x) {")
     L.append(f"        const long long v = c * {BLOCK * unroll} + threadIdx.x;")
     all_loads, all_work = [], []
     for u in range(unroll):
@@ -747,29 +756,52 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                         else f"({vt + ua}*)o{o} + ({idx})"
                     all_work.append(f"{pad}{{ const {vt} R = {{{items}}}; "
                                     f"{_st(nt_store, 'R', ptr)} }}")
-    L += all_loads + all_work
+    L += all_loads
+    if staged and one_run:
+        L.append("        DR_STAGE_TABLES();      // after the loads: both are in flight together")
+    L += all_work
     L.append("    }")
-    # leftover vectors (fewer than one chunk), spread over the first blocks
-    L.append(f"    for (long long v = nchunk * {BLOCK * unroll} + (long long)blockIdx.x * {BLOCK} "
-             f"+ threadIdx.x; v < {count}; v += (long long)gridDim.x * {BLOCK}) {{")
-    lo, wo = step("", "v", 8)
-    L += lo + wo
-    L.append("    }")
-    if vec and E > 1:
-        # scalar tail: the last n % E elements, by the first threads of block 0
-        L.append(f"    const long long t = nvec * {E} + (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
-        L.append("    if (t < n) {")
+    # what is left over (less than one chunk) is spread over the first blocks; with one run
+    # per block it belongs to the blocks behind the last run (code that follows the main
+    # path would keep its constants in registers across it)
+    if one_run:
+        # one element per thread and pass: this path is short and must not need more
+        # registers than the main one
+        L.append("    else {")
+        if staged:
+            L.append("        DR_STAGE_TABLES();")
+        L.append(f"        for (long long t = nchunk * {BLOCK * unroll * E} + (blockIdx.x - nchunk) * {BLOCK} "
+                 f"+ threadIdx.x; t < n; t += (gridDim.x - nchunk) * {BLOCK}) {{")
         args = [f"b{i}" if c == "b" else f"a{i}[t]" for i, c in enumerate(leaf_class)]
         args = (["t"] if prog.uses_index else []) + args
         decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
         outs = [f"t{o}" for o in range(n_out)]
-        L.append(f"        {decl} dr_body({', '.join(args + scal + outs)});")
-        if reduce_op:
-            L.append(f"        acc0 = {_combine(reduce_op, 'acc0', 't0')};")
-        else:
-            for o in range(n_out):
-                L.append(f"        o{o}[t] = t{o};")
+        L.append(f"            {decl} dr_body({', '.join(args + scal + outs)});")
+        for o in range(n_out):
+            L.append(f"            o{o}[t] = t{o};")
+        L.append("        }")
         L.append("    }")
+    else:
+        L.append(f"    for (long long v = nchunk * {BLOCK * unroll} + (long long)blockIdx.x * {BLOCK} "
+                 f"+ threadIdx.x; v < {count}; v += (long long)gridDim.x * {BLOCK}) {{")
+        lo, wo = step("", "v", 8)
+        L += lo + wo
+        L.append("    }")
+        if vec and E > 1:
+            # scalar tail: the last n % E elements, by the first threads of block 0
+            L.append(f"    const long long t = nvec * {E} + (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
+            L.append("    if (t < n) {")
+            args = [f"b{i}" if c == "b" else f"a{i}[t]" for i, c in enumerate(leaf_class)]
+            args = (["t"] if prog.uses_index else []) + args
+            decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
+            outs = [f"t{o}" for o in range(n_out)]
+            L.append(f"        {decl} dr_body({', '.join(args + scal + outs)});")
+            if reduce_op:
+                L.append(f"        acc0 = {_combine(reduce_op, 'acc0', 't0')};")
+            else:
+                for o in range(n_out):
+                    L.append(f"        o{o}[t] = t{o};")
+            L.append("    }")
     if reduce_op:
         accs = [f"acc{e}" for e in range(max(E, 1))]
         while len(accs) > 1:   # pairwise: (acc0 + acc1) + (acc2 + acc3)

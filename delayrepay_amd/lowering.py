@@ -66,6 +66,7 @@ TUNE = {
     "t_rows": 0,      # transpose tiles: output rows (= contiguous elements of the operand) and
     "t_cols": 0,      # output columns per tile (powers of two; 0: 128 bytes by 1 KB)
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
+    "one_run": 1,     # flat kernels with tables in LDS: one run per block, no loop over runs
     "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
     "smath": 1,       # float32 log/erf/exp from `mathlib32` (0: the device library's)
     "pack": 4,        # elements a thread passes through those functions in lock step
@@ -379,24 +380,35 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         # (29 vs 31 us, 73 vs 83 us): `cache_mib`/`ntl_mib` = 200/320 favour it.
         nts = bool(TUNE["nts"]) and footprint > TUNE["cache_mib"] << 20
         ntl = bool(TUNE["ntl"]) and in_bytes > TUNE["ntl_mib"] << 20
+        # Functions that keep tables in LDS: one run per block and no loop over runs.  The
+        # kernel then needs 80 vector registers instead of 118 (six waves per SIMD instead
+        # of four) and asks for its operands before it copies the tables, so that one wait
+        # covers both.  Black-Scholes float64, 2^25 options: blocks that stay for eight runs
+        # 241.8 us, one run per block with the tables copied first 279, this 233.8-236.8.
+        one_run = bool(mathlib.tables(prog.own_math) and vec and not reduce_op and TUNE["one_run"]
+                       and not TUNE["flat_cap"])
         low.kind = "flat"
         low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
-                   unroll, ntl, nts, ua)
+                   unroll, ntl, nts, ua, one_run)
 
         def emit():
             src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
-                                  restrict=not in_place, reduce_op=reduce_op, unaligned=ua)
+                                  restrict=not in_place, reduce_op=reduce_op, unaligned=ua,
+                                  one_run=one_run)
             return src
         low.emit = emit
         E = cg.flat_elements(prog, leaf_class, out_codes, reduce_op) if vec else 1
         chunks = max(1, (n // E) // (cg.BLOCK * unroll))   # one chunk per block ...
         cap = red_cap if reduce_op else (TUNE["flat_cap"] or (1 << 24) - 1)
-        if mathlib.tables(prog.own_math) and not TUNE["flat_cap"]:
+        if mathlib.tables(prog.own_math) and not TUNE["flat_cap"] and not one_run:
             # the workgroup copies the functions' tables into LDS first: let it stay for
-            # several chunks (Black-Scholes float64: 262 us with a chunk per workgroup, 244 us
-            # with 4096 to 8192 workgroups, 251 us with 1024)
+            # several chunks
             cap = min(cap, TUNE["table_blocks"])
-        low.grid = min(chunks, cap)
+        if one_run:     # block c takes run c; one more block takes what is left over
+            runs = (n // E) // (cg.BLOCK * unroll)
+            low.grid = runs + (1 if n % (E * cg.BLOCK * unroll) else 0)
+        else:
+            low.grid = min(chunks, cap)
         n_out_ptr = 1 if reduce_op else len(out_ptrs)
         low.fmt = "@" + "P" * (len(ptrs) + n_out_ptr) + scal_fmt + "q"
         low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]

@@ -51,6 +51,7 @@ fits on Chebyshev nodes in 50-digit arithmetic).
 DEVICE_MACROS = """\
 #define DR_FN static __device__ __forceinline__
 #define DR_TABLE static __device__ const
+#define DR_ALIGN16 __attribute__((aligned(16)))
 #define DR_RSQ64(x) __builtin_amdgcn_rsq(x)
 #define DR_ANY_LANE(p) (__builtin_amdgcn_ballot_w64(p) != 0)
 /* p * z + k with the constant k in a scalar register pair.  The compiler prefers the
@@ -63,6 +64,7 @@ DEVICE_MACROS = """\
 HOST_MACROS = """\
 #define DR_FN static inline
 #define DR_TABLE static const
+#define DR_ALIGN16 __attribute__((aligned(16)))
 /* a 24-bit estimate of 1/sqrt(x), like the hardware's */
 static inline double dr_rsq64_host(double x)
 {
@@ -84,7 +86,7 @@ STEP = r"""
 LOG_TABLE = r"""
 /* 1/c and log(c) for the 256 intervals of `dr_log_core`; c is the centre of its interval
    moved by less than 2^-23 of itself to a point whose logarithm is a double to within 0.004 ulp. */
-DR_TABLE double dr_log_tab[512] = {
+DR_TABLE DR_ALIGN16 double dr_log_tab[512] = {
     0x1.6a13cd153728dp+0, -0x1.630030b3aac40p-2,
     0x1.691473a88d0e1p+0, -0x1.602d08af0924ap-2,
     0x1.68168155466eap+0, -0x1.5d5bddc0163d9p-2,
@@ -455,7 +457,7 @@ DR_FN void dr_exp_f8(const double (&x)[P], double (&out)[P])
 
 ERF_TABLE = r"""
 /* per interval of `dr_erf_f8`: the point c, then the coefficients of degree 0..8 */
-DR_TABLE double dr_erf_tab[960] = {
+DR_TABLE DR_ALIGN16 double dr_erf_tab[960] = {
     0x0.0p+0, 0x0.0p+0, 0x1.20dd750429b6dp+0, 0x1.543a16bb13eb4p-44, -0x1.812746b0a7461p-2, 0x1.beb969b974784p-29, 0x1.ce2eeac38586cp-4, 0x1.d4661442f6b38p-18, -0x1.ba56e52e23b2dp-6, 0x1.55662ef9e89e4p-10,
     0x1.7fffffff69e3ep-4, 0x1.b0081148008d9p-4, 0x1.1e565bca4204ep+0, -0x1.ad8189aebb061p-4, -0x1.7712743c4144fp-2, 0x1.aafd475beb8f1p-5, 0x1.ba14967ab8217p-4, -0x1.1afca37ae4aacp-6, -0x1.9d46b144eace0p-6, 0x1.17806b6b7b449p-8,
     0x1.3fffffffddf9ap-3, 0x1.662a0bdf55126p-3, 0x1.19e5e92b97c15p+0, -0x1.605f637658332p-3, -0x1.6582e9b69a7a6p-2, 0x1.5aa32b56ce3cap-4, 0x1.97594a5e93b1bp-4, -0x1.c69c44776f897p-6, -0x1.6f81fcdf786dap-6, 0x1.be0ec8845976ap-8,
@@ -635,6 +637,7 @@ TABLES_IN_MEMORY = """\
 """
 
 TABLES_IN_LDS = """\
+typedef double dr_tab2 __attribute__((ext_vector_type(2)));     /* the copies move 16 bytes per lane */
 #define DR_TAB_PTR const __attribute__((address_space(3))) double*
 {arrays}
 {defines}
@@ -672,10 +675,11 @@ def source(names, macros=DEVICE_MACROS, lds=False):
     tabs = tables(names)
     if lds and tabs:
         where = TABLES_IN_LDS.format(
-            arrays="\n".join(f"__shared__ double {TABLE_SIZES[t][0]}_lds[{TABLE_SIZES[t][1]}];" for t in tabs),
+            arrays="\n".join(f"__shared__ DR_ALIGN16 double {TABLE_SIZES[t][0]}_lds[{TABLE_SIZES[t][1]}];" for t in tabs),
             defines="\n".join(f"#define {TABLE_SIZES[t][2]} ((DR_TAB_PTR){TABLE_SIZES[t][0]}_lds)" for t in tabs),
-            copies=" ".join(f"for (int i_ = threadIdx.x; i_ < {TABLE_SIZES[t][1]}; i_ += blockDim.x) "
-                            f"{TABLE_SIZES[t][0]}_lds[i_] = {TABLE_SIZES[t][0]}[i_];" for t in tabs))
+            copies=" ".join(f"for (int i_ = threadIdx.x; i_ < {TABLE_SIZES[t][1] // 2}; i_ += blockDim.x) "
+                            f"((dr_tab2*){TABLE_SIZES[t][0]}_lds)[i_] = ((const dr_tab2*){TABLE_SIZES[t][0]})[i_];"
+                            for t in tabs))
     else:
         where = TABLES_IN_MEMORY.format(
             defines="\n".join(f"#define {TABLE_SIZES[t][2]} {TABLE_SIZES[t][0]}" for t in tabs))
