@@ -401,7 +401,7 @@ def _conv(expr, src, dst):
     return f"({CTYPE[dst]}){expr}"
 
 
-def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=False):
+def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=0, stage_loop=False):
     """Inline device function evaluating the whole program for one element.
 
     Parameters: leaf values, scalar values, then one reference per root."""
@@ -410,7 +410,7 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=Fals
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
     uses_philox = any(name.startswith("philox") for name, _, _, _ in prog.ops)
-    lines = [mathlib.source(prog.own_math, lds=lds_tables) if with_math else "",
+    lines = [mathlib.source(prog.own_math, lds=lds_tables, stage_loop=stage_loop) if with_math else "",
              mathlib32.source(prog.own_math32) if with_math else "",
              PHILOX if uses_philox and with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
@@ -593,7 +593,7 @@ def packs(prog, vec):
 
 
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
-              reduce_op=None, unaligned=False, one_run=False):
+              reduce_op=None, unaligned=False, one_run=False, stage_loop=False):
     """Contiguous 1-D kernel.
 
     leaf_class  per leaf 'c' (contiguous, same length as the output) or 'b'
@@ -613,7 +613,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     n_leaf, n_out = len(prog.leaves), len(out_dtypes)
     red_dt = out_dtypes[0] if reduce_op else None
     E = flat_elements(prog, leaf_class, out_dtypes, reduce_op) if vec else 1
-    src = [PREAMBLE, emit_body(prog, out_dtypes, lds_tables=True)]
+    src = [PREAMBLE, emit_body(prog, out_dtypes, lds_tables=BLOCK, stage_loop=stage_loop)]
     packed = packs(prog, vec)
     if packed:
         src.append(emit_body_packed(prog, out_dtypes, [c == "c" for c in leaf_class], E * unroll,

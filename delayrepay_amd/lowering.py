@@ -66,6 +66,7 @@ TUNE = {
     "t_rows": 0,      # transpose tiles: output rows (= contiguous elements of the operand) and
     "t_cols": 0,      # output columns per tile (powers of two; 0: 128 bytes by 1 KB)
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
+    "stage_loop": 0,  # ... 1: the tables are copied by a loop (one trip to memory per 4 KB)
     "one_run": 1,     # flat kernels with tables in LDS: one run per block, no loop over runs
     "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
     "smath": 1,       # float32 log/erf/exp from `mathlib32` (0: the device library's)
@@ -387,14 +388,15 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         # 241.8 us, one run per block with the tables copied first 279, this 233.8-236.8.
         one_run = bool(mathlib.tables(prog.own_math) and vec and not reduce_op and TUNE["one_run"]
                        and not TUNE["flat_cap"])
+        stage_loop = bool(TUNE["stage_loop"] and mathlib.tables(prog.own_math))
         low.kind = "flat"
         low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
-                   unroll, ntl, nts, ua, one_run)
+                   unroll, ntl, nts, ua, one_run, stage_loop)
 
         def emit():
             src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
                                   restrict=not in_place, reduce_op=reduce_op, unaligned=ua,
-                                  one_run=one_run)
+                                  one_run=one_run, stage_loop=stage_loop)
             return src
         low.emit = emit
         E = cg.flat_elements(prog, leaf_class, out_codes, reduce_op) if vec else 1

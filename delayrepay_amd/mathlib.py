@@ -661,10 +661,11 @@ DR_FN double {fn}_1(double x)
 """
 
 
-def source(names, macros=DEVICE_MACROS, lds=False):
+def source(names, macros=DEVICE_MACROS, lds=0, stage_loop=False):
     """Definitions of the function templates for the ufuncs in `names` (each piece
     once) and of their one-element forms `<function>_1(double)`.  `lds`: the functions
-    read their tables from LDS copies, which the kernel makes with `DR_STAGE_TABLES()`."""
+    read their tables from LDS copies, which a kernel with blocks of `lds` threads makes
+    with `DR_STAGE_TABLES()`."""
     pieces = []
     for name in names:
         for piece in FUNCTIONS[name][1]:
@@ -674,12 +675,29 @@ def source(names, macros=DEVICE_MACROS, lds=False):
         return ""
     tabs = tables(names)
     if lds and tabs:
+        # Every lane first asks for all its 16-byte pieces of all tables and then writes
+        # them: one trip to memory per block, not one per piece (a loop waits for each
+        # piece before it asks for the next).
+        loads, stores = [], []
+        for t in tabs:
+            name, count, _ = TABLE_SIZES[t]
+            for k, first in enumerate(range(0, count // 2, lds)):
+                some = count // 2 - first < lds     # the last piece of a table: some lanes only
+                cond = f"threadIdx.x < {count // 2 - first}" if some else ""
+                var = f"dr_t_{name}_{k}"
+                src = f"((const dr_tab2*){name})[{first} + threadIdx.x]"
+                loads.append(f"dr_tab2 {var}; if ({cond}) {var} = {src};" if some else f"const dr_tab2 {var} = {src};")
+                dst = f"((dr_tab2*){name}_lds)[{first} + threadIdx.x] = {var};"
+                stores.append(f"if ({cond}) {dst}" if some else dst)
+        if stage_loop:
+            loads = [f"for (int i_ = threadIdx.x; i_ < {TABLE_SIZES[t][1] // 2}; i_ += {lds}) "
+                     f"((dr_tab2*){TABLE_SIZES[t][0]}_lds)[i_] = ((const dr_tab2*){TABLE_SIZES[t][0]})[i_];"
+                     for t in tabs]
+            stores = []
         where = TABLES_IN_LDS.format(
             arrays="\n".join(f"__shared__ DR_ALIGN16 double {TABLE_SIZES[t][0]}_lds[{TABLE_SIZES[t][1]}];" for t in tabs),
             defines="\n".join(f"#define {TABLE_SIZES[t][2]} ((DR_TAB_PTR){TABLE_SIZES[t][0]}_lds)" for t in tabs),
-            copies=" ".join(f"for (int i_ = threadIdx.x; i_ < {TABLE_SIZES[t][1] // 2}; i_ += blockDim.x) "
-                            f"((dr_tab2*){TABLE_SIZES[t][0]}_lds)[i_] = ((const dr_tab2*){TABLE_SIZES[t][0]})[i_];"
-                            for t in tabs))
+            copies=" ".join(loads + stores))
     else:
         where = TABLES_IN_MEMORY.format(
             defines="\n".join(f"#define {TABLE_SIZES[t][2]} {TABLE_SIZES[t][0]}" for t in tabs))

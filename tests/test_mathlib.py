@@ -156,10 +156,10 @@ def test_sqrt_is_correctly_rounded(host):
 
 
 def test_device_source_compiles():
-    for lds in (False, True):
+    for lds in (0, 256):
         src = mathlib.source(["log", "erf", "exp", "sqrt"], lds=lds)
         assert src.count("DR_STEP(") >= 13 and src.count("void dr_expm1_reduced(") == 1
-        assert ("__shared__ DR_ALIGN16 double dr_erf_tab_lds[960]" in src) == lds
+        assert ("__shared__ DR_ALIGN16 double dr_erf_tab_lds[960]" in src) == bool(lds)
         stage = "DR_STAGE_TABLES(); " if lds else ""
         kernel = ('extern "C" __global__ void k(const double* a, double* o)\n'
                   "{ " + stage + "int i = threadIdx.x; const double x[2] = {a[2 * i], a[2 * i + 1]}; double p[2], q[2], r[2];\n"
