@@ -126,6 +126,10 @@ def main():
             acc = acc * x + c[i]
         return acc
 
+    def again(leaf):
+        """A new device array with the contents of `leaf`, as a new lazy leaf."""
+        return dr.NPArray(leaf._force().copy())
+
     def sets_for(nbytes):
         """Buffer sets so that a set has left the last-level cache before its next turn."""
         if args.sets:
@@ -141,7 +145,11 @@ def main():
             n = inp["x"].size
             R = sets_for(12 * n)
             sets = [(dr.array(inp["x"]), dr.array(inp["y"])) for _ in range(R)]
-            return dict(dtype="f32", n=n, nbytes=12 * n, desc="SAXPY z=a*x+y f32 n=2^24",
+
+            def fresh(x=sets[0][0], y=sets[0][1]):
+                x, y = again(x), again(y)
+                return lambda: hip.run(inp["a"] * x + y)
+            return dict(dtype="f32", n=n, nbytes=12 * n, desc="SAXPY z=a*x+y f32 n=2^24", fresh=fresh,
                         steps=[(lambda x=x, y=y: hip.run(inp["a"] * x + y)) for x, y in sets],
                         cpu=lambda: orc.saxpy(inp["a"], inp["x"], inp["y"]), cpu_frac=1.0,
                         cpu_code="oracle/numpy_oracle.py::saxpy")
@@ -149,7 +157,11 @@ def main():
             n = inp["x"].size
             R = sets_for(8 * n)
             sets = [dr.array(inp["x"]) for _ in range(R)]
-            return dict(dtype="f32", n=n, nbytes=8 * n,
+
+            def fresh(x=sets[0]):
+                x = again(x)
+                return lambda: hip.run(horner_expr(inp["c"], x))
+            return dict(dtype="f32", n=n, nbytes=8 * n, fresh=fresh,
                         desc="Horner degree-8 polynomial f32 n=2^26",
                         steps=[(lambda x=x: hip.run(horner_expr(inp["c"], x))) for x in sets],
                         cpu=lambda: orc.horner(inp["c"], inp["x"]), cpu_frac=1.0,
@@ -160,7 +172,12 @@ def main():
             R = sets_for(5 * size * n)
             sets = [tuple(dr.array(inp[k]) for k in "SKT") for _ in range(R)]
             m = n // 4       # CPU sample: a quarter of the options
-            return dict(dtype="f32" if size == 4 else "f64", n=n, nbytes=5 * size * n,
+
+            def fresh(first=sets[0]):
+                S, K_, T = (again(a) for a in first)
+                return lambda: hip.run_multi(list(orc.black_scholes_expr(dr, S, K_, T, inp["r"],
+                                                                         inp["sigma"])))
+            return dict(dtype="f32" if size == 4 else "f64", n=n, nbytes=5 * size * n, fresh=fresh,
                         desc=f"Black-Scholes call+put {'f32' if size == 4 else 'f64'} n=2^25",
                         steps=[(lambda S=S, K_=K_, T=T: hip.run_multi(list(orc.black_scholes_expr(
                             dr, S, K_, T, inp["r"], inp["sigma"])))) for S, K_, T in sets],
@@ -175,7 +192,11 @@ def main():
 
             def sweep(u):
                 u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
-            return dict(dtype="f32", n=(N - 2) * (N - 2), nbytes=nbytes,
+
+            def fresh(u=grids[0]):
+                u = again(u)
+                return lambda: sweep(u)
+            return dict(dtype="f32", n=(N - 2) * (N - 2), nbytes=nbytes, fresh=fresh,
                         desc="Jacobi 5-point f32 8192x8192, per sweep",
                         steps=[(lambda u=u: sweep(u)) for u in grids], pair=True,
                         cpu=lambda: orc.jacobi(inp["u"], 1), cpu_frac=1.0,
@@ -185,7 +206,11 @@ def main():
             R = sets_for(24 * n)
             sets = [tuple(dr.array(inp[k]) for k in "xyw") for _ in range(R)]
             m = n // 4
-            return dict(dtype="f64", n=n, nbytes=24 * n, desc="sum((x-y)**2*w) f64 n=2^27",
+
+            def fresh(first=sets[0]):
+                x, y, w = (again(a) for a in first)
+                return lambda: hip.run(ReduceEx(np.add, (x - y) ** 2 * w))
+            return dict(dtype="f64", n=n, nbytes=24 * n, desc="sum((x-y)**2*w) f64 n=2^27", fresh=fresh,
                         steps=[(lambda x=x, y=y, w=w: hip.run(ReduceEx(np.add, (x - y) ** 2 * w)))
                                for x, y, w in sets],
                         cpu=lambda: orc.sumsq(inp["x"][:m], inp["y"][:m], inp["w"][:m]),
@@ -444,6 +469,42 @@ def main():
             "compile_ms": round((c1["compile_ns"] - c0["compile_ns"]) / 1e6, 2),
             "input_gen_s": round(t_gen, 2),
         }
+        if wl.get("fresh") is not None:
+            # A step over arrays never seen before (a new batch of data through the same
+            # expression): neither the nodes nor a plan exist, only the structure has been
+            # met.  F distinct sets of device arrays, more than the evaluated roots that
+            # are kept alive for plan reuse, so that a set's turn never finds its plan.
+            F = max(17, min(K, max(17, (96 << 30) // max(wl["nbytes"], 1))))
+            fresh_steps = [wl["fresh"]() for _ in range(F)]
+            hiprt.sync()
+            hits = {"plan_hits": 0, "seen_hits": 0}
+            walls, hosts = [], []
+            for _ in range(5):
+                t_warm = time.perf_counter()
+                while time.perf_counter() - t_warm < args.settle / 2:
+                    for j in range(R):
+                        ring[j] = steps[j]()
+                    hiprt.sync()
+                s0 = dict(hip.STATS)
+                t0 = time.perf_counter()
+                for i in range(K):
+                    ring[i % R] = fresh_steps[i % F]()
+                t1 = time.perf_counter()
+                hiprt.sync()
+                t2 = time.perf_counter()
+                walls.append((t2 - t0) / K)
+                hosts.append((t1 - t0) / K)
+                for k in hits:
+                    hits[k] += hip.STATS[k] - s0[k]
+            fresh_s = statistics.median(walls)
+            res["fresh_step_us"] = round(fresh_s * 1e6, 2)
+            res["fresh_host_us"] = round(statistics.median(hosts) * 1e6, 2)
+            res["fresh_GBps"] = round(wl["nbytes"] / fresh_s / 1e9, 1)
+            res["fresh_sets"] = F
+            res["fresh_plan_hits"] = hits["plan_hits"]            # 0: no step found a plan
+            res["fresh_structure_hits"] = hits["seen_hits"]       # steps whose structure had been met
+            res["fresh_step_over_kernel"] = round(fresh_s / (kernel_ms * 1e-3), 3)
+            del fresh_steps
         valu = profiled_figure("valu_instructions.txt", name)
         if valu is not None:
             # vector-ALU roofline: one wave instruction per SIMD every 4 cycles = 64 lanes

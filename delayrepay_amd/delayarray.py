@@ -117,6 +117,8 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
     # ---- NumPy protocols -------------------------------------------------
 
     def __array_ufunc__(self, ufunc, method, *inputs, **kwargs):
+        if method == "__call__" and not kwargs and len(inputs) == 1 and ufunc.__name__ != "square":
+            return _unary(ufunc, self)          # `sqrt(x)`, `exp(x)`: the common, short way
         if method == "reduce" and ufunc.__name__ in ("add", "maximum", "minimum"):
             return _reduce(ufunc, inputs[0], **kwargs)
         if method != "__call__":
@@ -480,6 +482,13 @@ def calc_type(func, children):
     return result_dtype(func, tuple(_descr(c) for c in children))
 
 
+class _Ref(weakref.ref):
+    """Weak reference that remembers its table key (`weakref.KeyedRef` does the same
+    through a `__new__` and an `__init__` written in Python, two more frames per node)."""
+
+    __slots__ = ("key",)
+
+
 class _WeakTable:
     """key -> node, holding nodes weakly (a lean WeakValueDictionary: node
     construction is on the host's hot path)."""
@@ -497,7 +506,8 @@ class _WeakTable:
         return ref() if ref is not None else None
 
     def __setitem__(self, key, node):
-        self.data[key] = weakref.KeyedRef(node, self._gone, key)
+        ref = self.data[key] = _Ref(node, self._gone)
+        ref.key = key
 
     def pop(self, key, default=None):
         ref = self.data.pop(key, None)
@@ -517,20 +527,22 @@ class Memoiser(type):
 
     _cache = _WeakTable()
 
-    def __call__(cls, *args, _table=_cache, _get=_cache.data.get, _ref=weakref.KeyedRef):
+    def __call__(cls, *args, _table=_cache, _get=_cache.data.get, _ref=_Ref):
         key = cls._memo_key(*args)
         ref = _get(key)
         node = ref() if ref is not None else None
         if node is None:
             node = type.__call__(cls, *args)
             node._key = key
-            _table.data[key] = _ref(node, _table._gone, key)
+            ref = _table.data[key] = _ref(node, _table._gone)
+            ref.key = key
         return node
 
 
 def reset():
     """Forget every hash-consed node (delayarray.py:234-236) and every cached plan."""
     Memoiser._cache.clear()
+    _NUMBERS.clear()
     forget = getattr(_backend, "forget", None)
     if forget is not None:
         forget()
@@ -990,12 +1002,78 @@ class _TooLarge(Exception):
     pass
 
 
+_NODES = Memoiser._cache.data
+_NODE_GONE = Memoiser._cache._gone
+_new_node = object.__new__
+
+
 def _binary(func, left, right):
+    """`BinaryNumpyEx(func, left, right)` for the arithmetic operators, which are most of
+    what a step that builds its expression anew spends on the host: the table lookup and
+    the constructor's work in one frame."""
     if not isinstance(left, DelayArray):
         left = arg_to_numpy_ex(left)
     if not isinstance(right, DelayArray):
         right = arg_to_numpy_ex(right)
-    return BinaryNumpyEx(func, left, right)
+    key = (BinaryNumpyEx, func, id(left), id(right))
+    ref = _NODES.get(key)
+    if ref is not None:
+        node = ref()
+        if node is not None:
+            return node
+    depth = left._depth
+    if right._depth > depth:
+        depth = right._depth
+    if depth >= MAX_DEPTH:
+        return BinaryNumpyEx(func, left, right)     # evaluates the deep operand first
+    shape = left.shape
+    other = right.shape
+    if shape != other and other:
+        shape = other if not shape else tuple(np.broadcast_shapes(shape, other))
+    node = _new_node(BinaryNumpyEx)
+    node.__dict__ = {"_count": DelayArray.count, "children": [left, right], "_depth": depth + 1,
+                     "func": func, "shape": shape,
+                     "dtype": result_dtype(func, (_descr(left), _descr(right))), "_key": key}
+    DelayArray.count += 1
+    ref = _NODES[key] = _Ref(node, _NODE_GONE)
+    ref.key = key
+    return node
+
+
+def _unary(func, arg):
+    """`UnaryFuncEx(func, arg)` in one frame, like `_binary`."""
+    key = (UnaryFuncEx, func, id(arg))
+    ref = _NODES.get(key)
+    if ref is not None:
+        node = ref()
+        if node is not None:
+            return node
+    if arg._depth >= MAX_DEPTH:
+        return UnaryFuncEx(func, arg)
+    node = _new_node(UnaryFuncEx)
+    node.__dict__ = {"_count": DelayArray.count, "children": [arg], "_depth": arg._depth + 1,
+                     "func": func, "shape": arg.shape,
+                     "dtype": result_dtype(func, (_descr(arg),)), "_key": key}
+    DelayArray.count += 1
+    ref = _NODES[key] = _Ref(node, _NODE_GONE)
+    ref.key = key
+    return node
+
+
+# Numbers that expressions were built with lately, kept alive: a loop that builds its
+# expression anew every pass then finds its constants instead of making them again (a
+# node for a number holds nothing but the number).
+_NUMBERS = {}
+
+
+def _number(val):
+    key = (type(val), val if val else repr(val))
+    node = _NUMBERS.get(key)
+    if node is None:
+        if len(_NUMBERS) >= 512:
+            _NUMBERS.clear()
+        node = _NUMBERS[key] = Scalar(val)
+    return node
 
 
 def arg_to_numpy_ex(arg):
@@ -1003,7 +1081,7 @@ def arg_to_numpy_ex(arg):
     if isinstance(arg, DelayArray):
         return arg
     if type(arg) in _PY_DESCR:
-        return Scalar(arg)
+        return _number(arg)
     if isinstance(arg, (numbers.Number, np.generic)):
         return Scalar(arg)
     if _backend.is_ndarray(arg) or isinstance(arg, np.ndarray):

@@ -45,7 +45,7 @@ COMPILE_OPTS = [
 
 _FUSED = "DELAY_UNFUSED" not in os.environ
 STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0,
-         "lowering_hits": 0, "disk_write_failures": 0}
+         "lowering_hits": 0, "seen_hits": 0, "disk_write_failures": 0}
 
 _COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal") \
     + tuple(cg._PREDICATES)
@@ -135,6 +135,7 @@ class Tracer(Visitor):
         self.scalars = []
         self.scalar_codes = []
         self._scalar_index = {}
+        self.scalar_uses = []     # the slot each use of a number took, in the order of use
         self.ops = []
         self._memo = {}
         self._evaluated = evaluated if evaluated is not None else {}
@@ -167,6 +168,7 @@ class Tracer(Visitor):
             self._scalar_index[key] = idx
             self.scalars.append(_scalar_value(value, code))
             self.scalar_codes.append(code)
+        self.scalar_uses.append(idx)
         return ("s", idx), code
 
     def op(self, name, compute, result, refs):
@@ -710,9 +712,11 @@ def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, 
         low.tail, low.grid, low.fin_count, low.lds = template.tail, template.grid, template.fin_count, template.lds
         low.srcs = [(leaves[i].buf, off) for i, off in recipe]
         low.scal = list(scalars)
+        low.recipe = recipe
         STATS["lowering_hits"] += 1
         return low
     low = _lower(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, reduce_op, in_place)
+    low.recipe = None
     recipe = []
     for buf, off in low.srcs:
         for i, a in enumerate(leaves):
@@ -729,7 +733,161 @@ def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, 
         template.tail, template.grid, template.fin_count, template.lds = (low.tail, low.grid,
                                                                           low.fin_count, low.lds)
         _LOWERED[key] = (template, recipe)
+        low.recipe = recipe
     return low
+
+
+# ---------------------------------------------------------------------------
+# plans for structures seen before
+# ---------------------------------------------------------------------------
+# A step over fresh arrays (a new batch of data through the same expression) finds
+# neither its nodes in the hash-cons table nor a plan on its root.  Tracing, type
+# resolution, the program's key and the lowering's key then cost more host time than
+# a SAXPY kernel of 2^24 elements runs.  `_scan` walks such a DAG once, in the tracer's
+# order, and writes down everything the tracer and the lowering would look at: each
+# node's function, which operand is which earlier node, each number's type, each leaf's
+# geometry.  A structure met before has its plan in `_SEEN`; only buffers and numbers
+# are filled in.
+
+_SEEN = {}
+_SEEN_MAX = 4096
+_CALL_KINDS = frozenset(("BinaryNumpyEx", "BinaryFuncEx", "UnaryFuncEx"))
+
+
+class _Unseen(Exception):
+    """The expression has something in it that the tracer must look at itself."""
+
+
+def _walk(node, key, leaves, uses, deep, index, bufs):
+    """One ufunc node of `_scan`, operands first (a function of the module, not a closure:
+    a closure that calls itself is a reference cycle, and what it holds would wait for the
+    cycle collector)."""
+    index[id(node)] = len(index)
+    add = key.append
+    add(node.func.__name__)
+    children = node.children
+    for child in children:
+        n = index.get(id(child))
+        if n is not None:
+            add(n)
+            continue
+        kind = child.__class__.__name__
+        if kind == "Scalar":
+            index[id(child)] = len(index)
+            add(scalar_descr(child.val))
+        elif kind == "NPArray":
+            index[id(child)] = len(index)
+            arr = child.array
+            buf = arr.buf
+            add((arr.shape, arr._strides, arr.offset, arr.dtype.str,
+                 bufs.setdefault(id(buf), len(bufs)), buf.nbytes, buf.ptr & 255))
+            leaves.append(child)
+        elif kind in _CALL_KINDS:
+            d = child.__dict__
+            if "array" in d:
+                raise _Unseen
+            if child._depth >= REUSE_DEPTH:
+                if d.get("_seen", 0) >= REUSE_AFTER:
+                    raise _Unseen
+                deep.append(d)
+            _walk(child, key, leaves, uses, deep, index, bufs)
+        else:
+            raise _Unseen
+    for child in children:
+        if child.__class__.__name__ == "Scalar":
+            uses.append(child)
+
+
+def _scan(roots, head):
+    """(key, leaf nodes, uses of numbers, deep operands) of the DAG under `roots`, or None
+    when it holds anything but ufunc nodes over arrays and numbers: an evaluated interior
+    node, a generated leaf, a cast, a selection."""
+    key = list(head)
+    leaves, uses, deep = [], [], []
+    index, bufs = {}, {}
+    try:
+        for root in roots:
+            if root.__class__.__name__ not in _CALL_KINDS or "array" in root.__dict__:
+                return None
+            n = index.get(id(root))
+            if n is not None:
+                key.append(n)
+            else:
+                _walk(root, key, leaves, uses, deep, index, bufs)
+            key.append(None)
+    except (_Unseen, AttributeError):
+        return None
+    key.append(_STAMP)
+    return tuple(key), leaves, uses, deep
+
+
+def _seen_before(scan):
+    """The plan of an earlier evaluation of this structure over these arrays and numbers,
+    or None."""
+    key, leaf_nodes, uses, deep = scan
+    hit = _SEEN.get(key)
+    if hit is None:
+        return None
+    model, slots, codes = hit
+    mlow = model.low
+    arrays = [node.array for node in leaf_nodes]
+    scal = [None] * len(codes)
+    for node, slot in zip(uses, slots):
+        scal[slot] = _scalar_value(node.val, codes[slot])
+    low = _Lowered()
+    low.key, low.kind, low.emit, low.fmt = mlow.key, mlow.kind, mlow.emit, mlow.fmt
+    low.tail, low.grid, low.fin_count, low.lds = mlow.tail, mlow.grid, mlow.fin_count, mlow.lds
+    low.recipe = mlow.recipe
+    low.srcs = [(arrays[i].buf, off) for i, off in mlow.recipe]
+    low.scal = scal
+    if model.kern is None:
+        model.kern = _kernel_for(low, model.acc is not None)
+    plan = Plan()
+    plan.low = low
+    plan.kern = model.kern
+    plan.stamp = _STAMP
+    plan.checks = [(node, arr, None) for node, arr in zip(leaf_nodes, arrays)]
+    plan.leaves = arrays
+    plan.shape, plan.out_dtypes, plan.acc = model.shape, model.out_dtypes, model.acc
+    plan.hazard = False
+    plan.region = None
+    plan.empty = False
+    plan.axes = False
+    plan.second = None
+    plan.kern2 = None
+    plan.scratch = 0
+    for d in deep:
+        d["_seen"] = d.get("_seen", 0) + 1
+    STATS["seen_hits"] += 1
+    return plan
+
+
+def _remember_structure(scan, tracer, plan):
+    """Keep `plan` as the model for this structure, if the tracer saw what `_scan` saw
+    (it may have evaluated a deep operand on its own, or met a leaf twice under two
+    nodes) and the lowering can be filled in again from the leaves alone."""
+    key, leaf_nodes, uses, _ = scan
+    low = plan.low
+    if low is None or plan.second is not None or plan.axes or low.recipe is None:
+        return
+    seen_nodes = tracer.leaf_nodes
+    if len(seen_nodes) != len(leaf_nodes) or len(tracer.leaves) != len(leaf_nodes) \
+            or len(tracer.scalar_uses) != len(uses):
+        return
+    for (node, arr, deps), mine in zip(seen_nodes, leaf_nodes):
+        if node is not mine or deps is not None:
+            return
+    if len(_SEEN) >= _SEEN_MAX:
+        _SEEN.clear()
+    model = Plan()
+    mlow = _Lowered()         # holds no buffer alive
+    mlow.key, mlow.kind, mlow.emit, mlow.fmt = low.key, low.kind, low.emit, low.fmt
+    mlow.tail, mlow.grid, mlow.fin_count, mlow.lds = low.tail, low.grid, low.fin_count, low.lds
+    mlow.recipe = low.recipe
+    model.low = mlow
+    model.kern = plan.kern
+    model.shape, model.out_dtypes, model.acc = plan.shape, plan.out_dtypes, plan.acc
+    _SEEN[key] = (model, tuple(tracer.scalar_uses), tuple(tracer.scalar_codes))
 
 
 def _common_shape(leaves, gen_shapes):
@@ -911,14 +1069,23 @@ def run(ex):
     d = ex.__dict__
     plan = d.get("_plan")
     if plan is None or not plan.valid():
-        tracer = Tracer(reuse=True)
-        if _kind(ex) == "ReduceEx":
-            root = tracer.visit(ex.children[0])
-            plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__,
-                              axes=getattr(ex, "axis", None))
+        reduction = _kind(ex) == "ReduceEx"
+        if reduction:
+            axis = getattr(ex, "axis", None)
+            scan = None if axis is not None else _scan(ex.children[:1], ("reduce", ex.func.__name__))
         else:
-            root = _trace_root(tracer, ex)
-            plan = _make_plan(tracer, [root])
+            scan = _scan((ex,), ("run",))
+        plan = _seen_before(scan) if scan is not None else None
+        if plan is None:
+            tracer = Tracer(reuse=True)
+            if reduction:
+                root = tracer.visit(ex.children[0])
+                plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__, axes=axis)
+            else:
+                root = _trace_root(tracer, ex)
+                plan = _make_plan(tracer, [root])
+            if scan is not None:
+                _remember_structure(scan, tracer, plan)
         d["_plan"] = plan
         _remember(ex)
     else:
@@ -946,9 +1113,14 @@ def run_multi(exs):
             plan = cached[1]
             STATS["plan_hits"] += 1
         else:
-            tracer = Tracer(reuse=True)
-            roots = [_trace_root(tracer, exs[i]) for i in idxs]
-            plan = _make_plan(tracer, roots)
+            scan = _scan([exs[i] for i in idxs], ("multi",))
+            plan = _seen_before(scan) if scan is not None else None
+            if plan is None:
+                tracer = Tracer(reuse=True)
+                roots = [_trace_root(tracer, exs[i]) for i in idxs]
+                plan = _make_plan(tracer, roots)
+                if scan is not None:
+                    _remember_structure(scan, tracer, plan)
             # the other roots are kept alive with the entry (the key holds their ids, which
             # are only theirs while they live); not the first root itself: on its own
             # attribute that would be a reference cycle, and every result would wait for

@@ -120,7 +120,8 @@ def merge_dims(shape, stride_sets):
 class Lowered:
     """A kernel choice for one evaluation: cache key, source builder, launch recipe."""
 
-    __slots__ = ("key", "kind", "emit", "fmt", "srcs", "scal", "tail", "grid", "fin_count", "lds")
+    __slots__ = ("key", "kind", "emit", "fmt", "srcs", "scal", "tail", "grid", "fin_count", "lds",
+                 "recipe")
 
 
 # ---------------------------------------------------------------------------

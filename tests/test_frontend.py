@@ -77,13 +77,20 @@ def test_scalar_keys_do_not_collide():
 
 def test_hash_cons_table_holds_nodes_weakly():
     import gc
+    def interior():      # nodes for numbers stay alive for a while (a bounded number of them)
+        return sum(1 for key in Memoiser._cache.data if key[0] is not Scalar)
     a = leaf((8,))
-    before = len(Memoiser._cache)
+    before = interior()
     tmp = [a * float(i) for i in range(50)]
-    assert len(Memoiser._cache) >= before + 50
+    assert interior() >= before + 50
     del tmp
     gc.collect()
-    assert len(Memoiser._cache) <= before + 2
+    assert interior() <= before + 2
+    # the numbers kept alive are bounded
+    tmp = [a * float(i) for i in range(2000)]
+    del tmp
+    gc.collect()
+    assert sum(1 for key in Memoiser._cache.data if key[0] is Scalar) <= 512 + 2
 
 
 def test_nothing_is_computed_while_building():
