@@ -552,3 +552,58 @@ def test_device_random_numbers_cost_no_operand():
     hip.compile_source(hip.lower_only(w)[1])
     with pytest.raises(ValueError):
         dr.random.device(-1)
+
+
+# ---- structures met before (hip._scan) -----------------------------------------------
+
+def test_scan_writes_down_what_tracing_and_lowering_look_at():
+    """Two expressions get the same key exactly when tracing and lowering them gives the
+    same kernel and the same places for buffers and numbers: same functions, same operand
+    identities (x*x is not x*y), same number types, same leaf geometry."""
+    def key(*roots, head=("run",)):
+        scan = hip._scan(roots, head)
+        return None if scan is None else scan[0]
+    a, b, c = leaf((64,)), leaf((64,)), leaf((64,))
+    a2, b2 = leaf((64,)), leaf((64,))
+    assert key(2.0 * a + b) == key(3.5 * a2 + b2)            # other arrays, another number
+    assert key(2.0 * a + b) != key(2 * a + b)                 # a Python int is another type
+    assert key(2.0 * a + b) != key(np.float32(2.0) * a + b)   # and so is a NumPy scalar
+    assert key(a * a + b) != key(a * b + b)                   # which operand is which
+    assert key(a * b + b) == key(a2 * b2 + b2)
+    assert key(a * b + c) != key(a * b + b)
+    assert key(a + b) != key(a - b)
+    assert key(a + b) != key(a + leaf((64,), np.float64))     # dtype
+    assert key(a + b) != key(leaf((32,)) + leaf((32,)))       # shape
+    assert key(a + b) != key(a + leaf((1,)))                  # a broadcast operand
+    d = a - b
+    assert key(d * d) == key((a2 - b2) * (a2 - b2))           # hash-consed: one node, met twice
+    k0, k1 = key(2.0 * a, 2.0 * a + b, head=("multi",)), key(2.0 * a2, 2.0 * a2 + b2, head=("multi",))
+    assert k0 == k1 and k0 != key(2.0 * a + b, 2.0 * a, head=("multi",))
+    # views of one buffer are told from views of two
+    base = hip.placeholder((66,), np.float32)
+    from delayrepay_amd.delayarray import NPArray
+    v0, v1 = NPArray(base[:-2]), NPArray(base[2:])
+    assert key(v0 + v1) != key(a + b)
+    # what the tracer has to look at itself is not scanned
+    assert key(np.where(a > 0, a, b)) is None
+    assert key((a + b).astype(np.float64) * 2.0) is None
+    assert key(a) is None
+
+
+def test_scan_leaves_nothing_behind():
+    """Nothing on the nodes changes and no reference cycle is made by looking."""
+    import gc
+    import weakref
+    a, b = leaf((64,)), leaf((64,))
+    ex = (a - b) * (a - b) + 2.0
+    before = {k: dict(n.__dict__) for k, n in (("ex", ex), ("a", a))}
+    gc.collect()
+    gc.disable()
+    try:
+        scan = hip._scan((ex,), ("run",))
+        ref = weakref.ref(ex)
+        assert {k: dict(n.__dict__) for k, n in (("ex", ex), ("a", a))} == before
+        del scan, ex, before
+        assert ref() is None
+    finally:
+        gc.enable()

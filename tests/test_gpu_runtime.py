@@ -448,3 +448,68 @@ def test_rebuilding_a_multi_root_expression_reuses_its_plan():
     p2 = hip.run(put)
     assert hip.STATS["launches"] == launches + 2
     assert np.array_equal(c2.get(), outs[0].get()) and np.array_equal(p2.get(), outs[1].get())
+
+
+def test_a_structure_met_before_keeps_its_plan_over_fresh_arrays():
+    """Batches of new data through one expression: from the second batch on nothing is
+    traced or lowered (`seen_hits`), and every batch gets its own arrays' and numbers'
+    result.  Operand identities, number types and geometry tell structures apart."""
+    import delayrepay_amd as dr
+    from delayrepay_amd.delayarray import ReduceEx
+    rs = np.random.RandomState(5)
+    n = 1 << 12
+
+    def batch():
+        return [rs.uniform(-1, 1, n).astype(np.float32) for _ in range(3)]
+    cases = [
+        ("saxpy", lambda k, x, y, w: k * x + y, lambda k, x, y, w: np.float32(k) * x + y),
+        ("square", lambda k, x, y, w: x * x + y, lambda k, x, y, w: x * x + y),
+        ("mixed", lambda k, x, y, w: x * y + y, lambda k, x, y, w: x * y + y),
+        ("shared", lambda k, x, y, w: (x - y) * (x - y) * w + k, lambda k, x, y, w: (x - y) * (x - y) * w + np.float32(k)),
+        ("unary", lambda k, x, y, w: np.sqrt(np.abs(x)) / (k + y * y), lambda k, x, y, w: np.sqrt(np.abs(x)) / (np.float32(k) + y * y)),
+    ]
+    for name, lazy, eager in cases:
+        for step in range(4):
+            hx, hy, hw = batch()
+            k = 1.5 + step
+            x, y, w = dr.array(hx), dr.array(hy), dr.array(hw)
+            seen, launches = hip.STATS["seen_hits"], hip.STATS["launches"]
+            got = hip.run(lazy(k, x, y, w)).get()
+            assert hip.STATS["launches"] == launches + 1
+            if step:        # (the first batch may meet a structure that an earlier test left)
+                assert hip.STATS["seen_hits"] == seen + 1, (name, step)
+            assert got.tobytes() == eager(k, hx, hy, hw).astype(np.float32).tobytes(), (name, step)
+    # a reduction root and two roots at once
+    for step in range(3):
+        hx, hy, hw = (a.astype(np.float64) for a in batch())
+        x, y, w = dr.array(hx), dr.array(hy), dr.array(hw)
+        seen = hip.STATS["seen_hits"]
+        s = hip.run(ReduceEx(np.add, (x - y) ** 2 * w)).get()
+        p, q = (r.get() for r in hip.run_multi([x * y + w, x - y * w]))
+        if step:
+            assert hip.STATS["seen_hits"] == seen + 2
+        assert np.isclose(s, ((hx - hy) ** 2 * hw).sum(), rtol=1e-13)
+        assert p.tobytes() == (hx * hy + hw).tobytes() and q.tobytes() == (hx - hy * hw).tobytes()
+    # an operand evaluated beforehand is a leaf, whatever its structure's plan said
+    hx, hy, hw = batch()
+    x, y, w = dr.array(hx), dr.array(hy), dr.array(hw)
+    t = x * y
+    t.run()
+    assert hip.run(t + w).get().tobytes() == (hx * hy + hw).tobytes()
+    hx2, hy2, hw2 = batch()
+    x2, y2, w2 = dr.array(hx2), dr.array(hy2), dr.array(hw2)
+    assert hip.run(x2 * y2 + w2).get().tobytes() == (hx2 * hy2 + hw2).tobytes()
+    # a view with another offset or stride is another geometry
+    big = dr.array(np.concatenate(batch()))
+    hb = big.get()
+    for lo in (0, 4, 5):
+        assert hip.run(big[lo:lo + n] * 2.0 + big[lo + n:lo + 2 * n]).get().tobytes() == \
+            (hb[lo:lo + n] * np.float32(2.0) + hb[lo + n:lo + 2 * n]).tobytes()
+    # switching the tunables makes every remembered plan stale
+    hip.set_tune(nts=0)
+    try:
+        seen = hip.STATS["seen_hits"]
+        assert hip.run(2.5 * x + y).get().tobytes() == (np.float32(2.5) * hx + hy).tobytes()
+        assert hip.STATS["seen_hits"] == seen
+    finally:
+        hip.set_tune(nts=1)
