@@ -401,6 +401,32 @@ def _conv(expr, src, dst):
     return f"({CTYPE[dst]}){expr}"
 
 
+def _op_statement(prog, i):
+    """`const T v<i> = ...;` for operation i of `prog`, one element at a time."""
+    name, cdt, rdt, args = prog.ops[i]
+    cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
+    if name == "cast":
+        expr = cargs[0]
+    elif name == "iota":
+        expr = f"({CTYPE[cdt]})dr_i"
+    elif name in ("philox_raw", "philox_f8"):
+        # operands: key (2 words), counter (4 words), position of element 0 in the stream
+        # (a seventh operand, when the draw starts inside a block: that offset)
+        words = ", ".join(f"(dr_u64){k}{j}" for k, j in args[:6])
+        pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
+        expr = _philox_value(name, f"dr_philox({words}, {pos}(dr_u64)dr_i)")
+    elif cdt == "f8" and name in prog.own_math:
+        expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
+    elif cdt == "f4" and name in prog.own_math32:
+        expr = f"{mathlib32.FUNCTIONS[name][0]}({cargs[0]})"
+    elif name == "where":    # the condition keeps its own type
+        k, j = args[0]
+        expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
+    else:
+        expr = op_expr(name, cdt, cargs)
+    return f"    const {CTYPE[rdt]} v{i} = {expr};"
+
+
 def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=0, stage_loop=False):
     """Inline device function evaluating the whole program for one element.
 
@@ -414,28 +440,8 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=0, s
              mathlib32.source(prog.own_math32) if with_math else "",
              PHILOX if uses_philox and with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
-    for i, (name, cdt, rdt, args) in enumerate(prog.ops):
-        cargs = [_conv(f"{k}{j}", prog.ref_dtype((k, j)), cdt) for k, j in args]
-        if name == "cast":
-            expr = cargs[0]
-        elif name == "iota":
-            expr = f"({CTYPE[cdt]})dr_i"
-        elif name in ("philox_raw", "philox_f8"):
-            # operands: key (2 words), counter (4 words), position of element 0 in the stream
-            # (a seventh operand, when the draw starts inside a block: that offset)
-            words = ", ".join(f"(dr_u64){k}{j}" for k, j in args[:6])
-            pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
-            expr = _philox_value(name, f"dr_philox({words}, {pos}(dr_u64)dr_i)")
-        elif cdt == "f8" and name in prog.own_math:
-            expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
-        elif cdt == "f4" and name in prog.own_math32:
-            expr = f"{mathlib32.FUNCTIONS[name][0]}({cargs[0]})"
-        elif name == "where":    # the condition keeps its own type
-            k, j = args[0]
-            expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
-        else:
-            expr = op_expr(name, cdt, cargs)
-        lines.append(f"    const {CTYPE[rdt]} v{i} = {expr};")
+    for i in range(len(prog.ops)):
+        lines.append(_op_statement(prog, i))
     for i, ((k, j), rdt) in enumerate(prog.roots):
         lines.append(f"    r{i} = {_conv(f'{k}{j}', rdt, out_dtypes[i])};")
     lines.append("}")
@@ -2197,3 +2203,360 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
     L += ["        }", "    }", "}"]
     src.append("\n".join(L))
     return "\n".join(src) + "\n"
+
+
+# ---- rows that are reduced and used again in one kernel -----------------------------
+
+ROW_REDUCE = {"rowsum": "add", "rowmax": "maximum", "rowmin": "minimum"}
+ROW_STEPS_MAX = 16      # 16-byte units a lane holds of one operand's row
+
+
+class RowFusionUnsupported(Exception):
+    """The program or its operands do not fit the row kernel: the reductions inside the
+    expression are evaluated on their own instead."""
+
+
+def row_analysis(prog, leaf_kind):
+    """Where each operation of a program with row reductions is computed.
+
+    A row reduction (`rowsum`, `rowmax`, `rowmin` of a per-element value) yields one value
+    per row.  level[i] counts the reductions on the longest path below operation i; a
+    reduction whose operand has level s is made in stage s, after the stages before it.
+    uniform[i]: the value is the same along a row.  Returns (level, uniform, stages) with
+    stages[s] the reductions made in stage s."""
+    level, uniform = [], []
+    for name, _, _, args in prog.ops:
+        lv, uni = 0, True
+        for k, j in args:
+            if k == "v":
+                lv = max(lv, level[j])
+                uni = uni and uniform[j]
+            elif k == "l":
+                uni = uni and leaf_kind[j] == "k"
+        if name in ROW_REDUCE:
+            if uni:
+                raise RowFusionUnsupported("a reduction of a value that is constant along the row")
+            lv, uni = lv + 1, True
+        elif name in INDEX_OPS:
+            raise RowFusionUnsupported("index-valued operands")
+        level.append(lv)
+        uniform.append(uni)
+    stages = [[] for _ in range(max(level, default=0))]
+    for i, (name, _, _, _) in enumerate(prog.ops):
+        if name in ROW_REDUCE:
+            stages[level[i] - 1].append(i)
+    return level, uniform, stages
+
+
+def _row_needed(prog, targets):
+    """Operations to compute for the values `targets` (refs), in order, the row
+    reductions they read (those are handed in, not computed) and the leaves they read."""
+    need, given = set(), set()
+    leaves = {j for k, j in targets if k == "l"}
+    stack = [j for k, j in targets if k == "v"]
+    while stack:
+        i = stack.pop()
+        if i in need or i in given:
+            continue
+        if prog.ops[i][0] in ROW_REDUCE:
+            given.add(i)
+            continue
+        need.add(i)
+        for k, j in prog.ops[i][3]:
+            if k == "v":
+                stack.append(j)
+            elif k == "l":
+                leaves.add(j)
+    return sorted(need), sorted(given), leaves
+
+
+def _row_function(prog, fname, targets, out_dtypes):
+    """Device function computing `targets` for one element (or one row, when every target
+    is constant along the row): parameters are all leaf values, all scalars, the row
+    reductions it reads, then one reference per target.  Returns (source, reductions read,
+    leaves read)."""
+    need, given, used = _row_needed(prog, targets)
+    params = [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params += [f"const {CTYPE[prog.ops[i][2]]} v{i}" for i in given]
+    params += [f"{CTYPE[dt]}& r{n}" for n, dt in enumerate(out_dtypes)]
+    lines = [f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
+    lines += [_op_statement(prog, i) for i in need]
+    for n, ((k, j), dt) in enumerate(zip(targets, out_dtypes)):
+        lines.append(f"    r{n} = {_conv(f'{k}{j}', prog.ref_dtype((k, j)), dt)};")
+    lines.append("}")
+    return "\n".join(lines), given, used
+
+
+def row_vector(prog, leaf_kind, out_dtypes, out_uniform):
+    """Elements per 16-byte unit, when everything that moves along the row has one item
+    size (4 or 8 bytes); else 1."""
+    widths = {ITEMSIZE[dt] for dt, k in zip(prog.leaves, leaf_kind) if k == "v"}
+    widths |= {ITEMSIZE[dt] for dt, u in zip(out_dtypes, out_uniform) if not u}
+    return 16 // widths.pop() if len(widths) == 1 and widths <= {4, 8} else 1
+
+
+def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt_store=False,
+                   fence=True, recompute=True):
+    """Rows that are reduced and used again: `a - max(a, axis=-1)`, softmax, the variance,
+    layer normalisation.  A group of G lanes (8..64: part of a wave; 256: the block) owns a
+    row of R elements (a compile-time constant, unit stride); lane j takes the 16-byte
+    units j, j + G, ... of it.  An operand flagged in `keep` (default: all) has its share of
+    the row in registers from one stage to the next, so the row is read from memory once;
+    the others are loaded again by every stage that reads them (from the caches: operands
+    that are the same for every row, rows that would not fit).  Stage s computes,
+    per element, the operands of the reductions whose inputs depend on s earlier
+    reductions (per-element values are computed again in every stage that needs them: no
+    value is carried but the row itself), and the group combines them: butterfly of
+    `__shfl_xor` inside the wave, then, for a block, the four waves' values through LDS
+    (two slots in turn, so one barrier per reduction).  The last stage computes the roots
+    and stores them; a root that is constant along the row is stored once per row.
+
+    `fence`: the compiler may not move instructions from one 16-byte unit's work to the
+    next (left to itself it interleaves all sixteen units of a long row for the sake of
+    instruction-level parallelism and needs 205 vector registers for a softmax of rows of
+    16384, which leaves two waves per SIMD).
+
+    leaf_kind    per leaf 'v' (unit stride along the row) or 'k' (constant along it)
+    out_uniform  per root: one value per row
+    Parameters: leaf pointers, output pointers, scalars, K (rows), per leaf the stride
+    between rows, per output the stride between rows (all in elements)."""
+    level, uniform, stages = row_analysis(prog, leaf_kind)
+    if not stages:
+        raise RowFusionUnsupported("no row reduction in the program")
+    V = row_vector(prog, leaf_kind, out_dtypes, out_uniform)
+    units = -(-R // V)
+    full, rem = R // V, R % V
+    steps = -(-units // G)
+    if steps > ROW_STEPS_MAX:
+        raise RowFusionUnsupported("row too long")
+    nl, ns, n_out = len(prog.leaves), len(prog.scalars), len(out_dtypes)
+    block_row = G == BLOCK
+    lanes = min(G, WAVE)
+    per_wave = WAVE // lanes
+    src = [PREAMBLE, mathlib.source(prog.own_math), mathlib32.source(prog.own_math32)]
+
+    # one function per stage, one for the per-element roots, one for the per-row roots
+    stage_fn = []
+    for s, reds in enumerate(stages):
+        targets = [prog.ops[i][3][0] for i in reds]
+        text, given, used = _row_function(prog, f"dr_stage{s}", targets, [prog.ops[i][1] for i in reds])
+        src.append(text)
+        stage_fn.append((given, used))
+    elem_roots = [n for n in range(n_out) if not out_uniform[n]]
+    row_roots = [n for n in range(n_out) if out_uniform[n]]
+    final_given = rowout_given = ()
+    final_used = set()
+    if keep is None:
+        keep = [True] * nl
+    if elem_roots:
+        text, final_given, final_used = _row_function(
+            prog, "dr_final", [prog.roots[n][0] for n in elem_roots], [out_dtypes[n] for n in elem_roots])
+        src.append(text)
+    if row_roots:
+        text, rowout_given, _ = _row_function(
+            prog, "dr_rowout", [prog.roots[n][0] for n in row_roots], [out_dtypes[n] for n in row_roots])
+        src.append(text)
+
+    # combining a value over the group
+    red_types = sorted({(ROW_REDUCE[prog.ops[i][0]], prog.ops[i][2]) for reds in stages for i in reds})
+    n_red = sum(len(reds) for reds in stages)
+    for op, dt in red_types:
+        ct = CTYPE[dt]
+        body = [f"__device__ __forceinline__ {ct} dr_group_{op}_{dt}({ct} v, {ct}* slot)", "{",
+                "#pragma unroll",
+                f"    for (int off = {lanes // 2}; off > 0; off >>= 1) {{",
+                f"        const {ct} o = __shfl_xor(v, off, 64);",
+                f"        v = {_combine(op, 'v', 'o')};",
+                "    }"]
+        if block_row:
+            a, b = _combine(op, "slot[0]", "slot[1]"), _combine(op, "slot[2]", "slot[3]")
+            body += [f"    if ((threadIdx.x & {WAVE - 1}) == 0) slot[threadIdx.x >> 6] = v;",
+                     "    __syncthreads();",
+                     f"    v = {_combine(op, f'({a})', f'({b})')};"]
+        body.append("    return v;")
+        body.append("}")
+        src.append("\n".join(body))
+
+    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
+    params += [f"{CTYPE[dt]}* __restrict__ o{n}" for n, dt in enumerate(out_dtypes)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params.append("const long long K")
+    params += [f"const long long sk{i}" for i in range(nl)]
+    params += [f"const long long so{n}" for n in range(n_out)]
+    scal = [f"s{i}" for i in range(ns)]
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{"]
+    if block_row:
+        widest = max((CTYPE[prog.ops[i][2]] for reds in stages for i in reds),
+                     key=lambda c: 8 if c in ("double", "long long") else 4)
+        L += [f"    __shared__ {widest} dr_slots[2][{max(n_red, 1)}][{BLOCK // WAVE}];",
+              "    const int sub = threadIdx.x;",
+              "    int turn = 0;",
+              "    for (long long row = blockIdx.x; row < K; row += gridDim.x, turn ^= 1) {",
+              "        const long long k = row;"]
+    else:
+        L += [f"    const int sub = threadIdx.x & {G - 1};",
+              f"    const int grp = (threadIdx.x & {WAVE - 1}) >> {G.bit_length() - 1};",
+              f"    const long long stride = (long long)gridDim.x * {BLOCK // WAVE * per_wave};",
+              f"    for (long long first = ((long long)blockIdx.x * {BLOCK // WAVE} + (threadIdx.x >> 6)) * "
+              f"{per_wave}; first < K; first += stride) {{",
+              "        const long long row = first + grp;",
+              "        const long long k = row < K ? row : K - 1;      // idle groups re-read the last row"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind == "v":
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+        else:
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+
+    def vtype(dt):
+        return (VEC16[dt][0] + "u") if V > 1 else CTYPE[dt]
+
+    # which lanes hold what in step j: whole units, the partial last unit, nothing
+    def step_state(j):
+        lo = j * G
+        whole = "" if lo + G <= full else (f"{lo} + sub < {full}" if lo < full else None)
+        part = f"sub == {full - lo}" if rem and lo <= full < lo + G else None
+        return lo, whole, part
+
+    def loads(j, pad, which):
+        """Declarations and loads of step j's units of the row operands in `which`."""
+        lo, whole, part = step_state(j)
+        out = []
+        for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+            if kind != "v" or i not in which:
+                continue
+            vt = vtype(dt)
+            zero = "{0}" if V > 1 else "0"
+            if whole == "":
+                out.append(f"{pad}const {vt} X{j}_{i} = *(const {vt}*)(row{i} + ({lo} + sub) * {V});")
+                continue
+            out.append(f"{pad}{vt} X{j}_{i} = {zero};")
+            if whole is not None:
+                out.append(f"{pad}if ({whole}) X{j}_{i} = *(const {vt}*)(row{i} + ({lo} + sub) * {V});")
+            if part is not None:
+                fill = " ".join(f"X{j}_{i}[{e}] = row{i}[{full * V + e}];" for e in range(rem))
+                out.append(f"{pad}if ({part}) {{ {fill} }}")
+        return out
+
+    def element_args(j, e, used):
+        """Arguments for the leaves: an operand that the function does not read is a zero."""
+        return [(("0" if i not in used else f"X{j}_{i}[{e}]" if V > 1 else f"X{j}_{i}")
+                 if kind == "v" else f"c{i}") for i, kind in enumerate(leaf_kind)]
+
+    def guarded(j, e, stmt, pad):
+        """`stmt` for element e of step j, under the condition that the lane holds it."""
+        lo, whole, part = step_state(j)
+        conds = []
+        if whole == "":
+            return f"{pad}{stmt}"
+        if whole is not None:
+            conds.append(f"({whole})")
+        if part is not None and e < rem:
+            conds.append(f"({part})")
+        if not conds:
+            return None
+        return f"{pad}if ({' || '.join(conds)}) {stmt}"
+
+    pad = "        "
+
+    def relabel(g, tag):
+        """A copy of row value g that the compiler cannot tell is the same value: what one
+        stage computed per element (`exp(x - max)` for the sum) is then not kept in
+        registers for the next stage that computes it (for the quotient), but computed
+        again; a row of 16384 held twice leaves two waves per SIMD."""
+        if not recompute:
+            return f"v{g}"
+        ct = CTYPE[prog.ops[g][2]]
+        L.append(f'{pad}{ct} v{g}_{tag} = v{g}; asm volatile("" : "+v"(v{g}_{tag}));')
+        return f"v{g}_{tag}"
+    kept = {i for i in range(nl) if keep[i] and leaf_kind[i] == "v"}
+    for j in range(steps):
+        L += loads(j, pad, kept)
+    slot = 0
+    for s, reds in enumerate(stages):
+        for i in reds:
+            op, dt = ROW_REDUCE[prog.ops[i][0]], prog.ops[i][2]
+            L.append(f"{pad}{CTYPE[dt]} acc{i} = {_identity(op, dt)};")
+        given = []
+        for g in stage_fn[s][0]:
+            given.append(relabel(g, f"s{s}"))
+        used = stage_fn[s][1]
+        again = {i for i in used if leaf_kind[i] == "v"} - kept
+        outs = [f"t{i}" for i in reds]
+        decl = " ".join(f"{CTYPE[prog.ops[i][1]]} t{i};" for i in reds)
+        for j in range(steps):
+            body = []
+            for e in range(V):
+                acc = " ".join(f"acc{i} = {_combine(ROW_REDUCE[prog.ops[i][0]], f'acc{i}', f't{i}')};"
+                               for i in reds)
+                stmt = (f"{{ {decl} dr_stage{s}({', '.join(element_args(j, e, used) + scal + given + outs)}); "
+                        f"{acc} }}")
+                line = guarded(j, e, stmt, pad + ("    " if again else ""))
+                if line:
+                    body.append(line)
+            if not body:
+                continue
+            if not again:
+                L += body
+            else:
+                L += [f"{pad}{{"] + loads(j, pad + "    ", again) + body + [f"{pad}}}"]
+            if fence and j + 1 < steps:
+                L.append(f"{pad}__builtin_amdgcn_sched_barrier(0);")
+        for i in reds:
+            op, dt = ROW_REDUCE[prog.ops[i][0]], prog.ops[i][2]
+            where = f"({CTYPE[dt]}*)dr_slots[turn][{slot}]" if block_row else "nullptr"
+            L.append(f"{pad}const {CTYPE[dt]} v{i} = dr_group_{op}_{dt}(acc{i}, {where});")
+            slot += 1
+    # the roots
+    store_guard = "" if block_row else "if (row < K) "
+    if elem_roots:
+        given = [relabel(g, "f") for g in final_given]
+        for j in range(steps):
+            lo, whole, part = step_state(j)
+            if whole is None and part is None:
+                continue
+            inner = pad + "    "
+            L.append(f"{pad}{{")
+            L += loads(j, inner, {i for i in final_used if leaf_kind[i] == "v"} - kept)
+            for n in elem_roots:
+                L.append(f"{inner}{vtype(out_dtypes[n])} Y{n};")
+            for e in range(V):
+                outs = [(f"Y{n}[{e}]" if V > 1 else f"Y{n}") for n in elem_roots]
+                # vector components cannot bind to references: through temporaries
+                tmps = [f"y{n}" for n in elem_roots]
+                decl = " ".join(f"{CTYPE[out_dtypes[n]]} y{n};" for n in elem_roots)
+                copy = " ".join(f"{o} = {t};" for o, t in zip(outs, tmps))
+                stmt = (f"{{ {decl} dr_final({', '.join(element_args(j, e, final_used) + scal + given + tmps)}); "
+                        f"{copy} }}")
+                line = guarded(j, e, stmt, inner)
+                if line:
+                    L.append(line)
+            for n in elem_roots:
+                dt = out_dtypes[n]
+                base = f"o{n} + row * so{n}"
+                st = _st(nt_store and V > 1, f"Y{n}", f"({vtype(dt)}*)({base} + ({lo} + sub) * {V})")
+                if whole == "":
+                    L.append(f"{inner}{store_guard}{st}")
+                elif whole is not None:
+                    cond = f"{whole}" if block_row else f"row < K && {whole}"
+                    L.append(f"{inner}if ({cond}) {st}")
+                if part is not None:
+                    tail = " ".join(f"({base})[{full * V + e}] = Y{n}[{e}];" for e in range(rem))
+                    cond = f"{part}" if block_row else f"row < K && {part}"
+                    L.append(f"{inner}if ({cond}) {{ {tail} }}")
+            L.append(f"{pad}}}")
+            if fence and j + 1 < steps:
+                L.append(f"{pad}__builtin_amdgcn_sched_barrier(0);")
+    if row_roots:
+        given = [f"v{g}" for g in rowout_given]
+        outs = [f"z{n}" for n in row_roots]
+        decl = " ".join(f"{CTYPE[out_dtypes[n]]} z{n};" for n in row_roots)
+        # per-row values read no row operand: hand the function zeros for those
+        args = [("0" if kind == "v" else f"c{i}") for i, kind in enumerate(leaf_kind)]
+        cond = "sub == 0" if block_row else "sub == 0 && row < K"
+        stores = " ".join(f"o{n}[row * so{n}] = z{n};" for n in row_roots)
+        L.append(f"{pad}if ({cond}) {{ {decl} dr_rowout({', '.join(args + scal + given + outs)}); {stores} }}")
+    L += ["    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(p for p in src if p) + "\n"

@@ -12,6 +12,7 @@ from .visitor import Visitor
 np = numpy
 fallback = numpy
 GENERATED_LEAVES = True     # FullEx / IotaEx nodes are understood
+LAZY_ROW_REDUCTIONS = True  # reductions that keep their axis may stay lazy nodes
 
 
 def is_ndarray(arr):
@@ -63,7 +64,10 @@ class CpuVisitor(Visitor):
         return self.visit(node.children[0]).astype(node.dtype)
 
     def visit_ReduceEx(self, node):
-        return node.func.reduce(self.visit(node.children[0]), axis=node.axis)
+        if node.__dict__.get("_cut"):
+            return node.array
+        return node.func.reduce(self.visit(node.children[0]), axis=node.axis,
+                                keepdims=getattr(node, "keepdims", False))
 
 
 def run(ex):

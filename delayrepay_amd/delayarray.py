@@ -634,19 +634,22 @@ class ReduceEx(NumpyEx, Funcable):
     over everything (`axis` None) or over a tuple of axes; evaluated as the tail of
     the fused element-wise kernel."""
 
-    def __init__(self, func, arg, axis=None):
+    def __init__(self, func, arg, axis=None, keepdims=False):
         super().__init__(children=[arg])
         self.func = func
         self.axis = axis
-        if axis is None:
+        self.keepdims = keepdims
+        if keepdims:
+            self.shape = tuple(1 if (axis is None or k in axis) else d for k, d in enumerate(arg.shape))
+        elif axis is None:
             self.shape = ()
         else:
             self.shape = tuple(d for k, d in enumerate(arg.shape) if k not in axis)
         self.dtype = arg.dtype
 
     @classmethod
-    def _memo_key(cls, func, arg, axis=None):
-        return (cls, func, id(arg), axis)
+    def _memo_key(cls, func, arg, axis=None, keepdims=False):
+        return (cls, func, id(arg), axis, keepdims)
 
     @property
     def name(self):
@@ -1091,13 +1094,19 @@ def arg_to_numpy_ex(arg):
     raise NotImplementedError(f"cannot use a {type(arg).__name__} in a lazy expression")
 
 
-def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **unused):
+def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **other):
     """Full reduction -> 0-d backend array (what the reference's `sum` returns
-    on its GPU backend, delayarray.py:516-518); axis reductions are eager
-    backend calls on the materialised operand."""
+    on its GPU backend, delayarray.py:516-518); a reduction over some axes -> a new leaf;
+    a reduction along the last axis that keeps it (`keepdims=True`) stays lazy: inside a
+    larger expression (`a - a.max(axis=-1, keepdims=True)`) the backend reduces each row and
+    uses it again in one kernel."""
     arr = arg_to_numpy_ex(arr)
     if out is not None or dtype is not None:
         raise NotImplementedError("reductions with out= or dtype= are not supported")
+    for name, value in other.items():
+        # `where=` and `initial=` change the result: say so instead of leaving them out
+        if not (value is None or value is np._NoValue or (name == "where" and value is True)):
+            raise NotImplementedError(f"reductions with {name}= are not supported on lazy arrays")
     ndim = arr.ndim
     if axis is not None:
         axes = (axis,) if isinstance(axis, (int, np.integer)) else tuple(axis)
@@ -1112,6 +1121,17 @@ def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **unused
         axis = tuple(sorted(norm))
         if len(axis) == ndim:
             axis = None
+    if keepdims and axis == (ndim - 1,) and arr.dtype.kind == "f" and arr.shape[-1] > 1 \
+            and getattr(_backend, "LAZY_ROW_REDUCTIONS", False):
+        return ReduceEx(func, arr, axis, True)
+    if 0 in arr.shape and func is not np.add and arr.dtype == np.bool_ and \
+            (axis is None or 0 in [arr.shape[k] for k in axis]):
+        # `any` / `all` of nothing: the identities of `or` and `and`
+        shape = () if axis is None else tuple(d for k, d in enumerate(arr.shape) if k not in axis)
+        if keepdims:
+            shape = tuple(1 if (axis is None or k in axis) else d for k, d in enumerate(arr.shape))
+        res = _backend.fallback.full(shape, func is np.minimum, dtype=np.bool_)
+        return res if axis is None and not keepdims else NPArray(res)
     res = ReduceEx(func, arr, axis)._force() if axis is not None else ReduceEx(func, arr)._force()
     if keepdims:
         full = tuple(1 if (axis is None or k in axis) else d for k, d in enumerate(arr.shape))

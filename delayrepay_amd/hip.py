@@ -47,6 +47,7 @@ _FUSED = "DELAY_UNFUSED" not in os.environ
 STATS = {"launches": 0, "compiles": 0, "disk_hits": 0, "mem_hits": 0, "plan_hits": 0,
          "lowering_hits": 0, "seen_hits": 0, "disk_write_failures": 0}
 
+_ROW_OPS = {"add": "rowsum", "maximum": "rowmax", "minimum": "rowmin"}
 _COMPARES = ("greater", "less", "greater_equal", "less_equal", "equal", "not_equal") \
     + tuple(cg._PREDICATES)
 
@@ -69,6 +70,7 @@ def set_tune(**kwargs):
     _STAMP += 1
 
 
+LAZY_ROW_REDUCTIONS = True  # a reduction along the last axis that keeps it may stay a lazy node
 GENERATED_LEAVES = True     # FullEx / IotaEx nodes are computed inside kernels
 
 
@@ -126,9 +128,11 @@ class Tracer(Visitor):
     (delayrepay/delayarray.py:434-452,462-467), gets NumPy's result all the same.
     Each handler returns (operand reference, dtype code)."""
 
-    def __init__(self, evaluated=None, reuse=False):
+    def __init__(self, evaluated=None, reuse=False, rows=False):
         super().__init__()
         self._reuse = reuse       # evaluate deep operands met in an earlier evaluation first
+        self._rows = rows         # reductions along the last axis become operations of the program
+        self.row_len = None       # length of the rows those reductions run along
         self.leaves = []
         self.leaf_codes = []
         self._leaf_index = {}
@@ -283,8 +287,24 @@ class Tracer(Visitor):
         return self.op("cast", target, target, [ref]) if code != target else (ref, code)
 
     def visit_ReduceEx(self, node):
-        # a reduction inside a larger expression is evaluated on its own first
-        return self.leaf(node._force())
+        """A reduction inside a larger expression.  Along the last axis, kept (`keepdims`),
+        of a float expression: an operation of the program (`rowsum`, `rowmax`, `rowmin`;
+        the row kernel reduces each row and uses it again, cf. the reference's `ReduceEx`
+        as an interior node, delayarray.py:272-283, cuda.py:87-88).  Anything else is
+        evaluated on its own first and read as a leaf."""
+        child = node.children[0]
+        name = _ROW_OPS.get(node.func.__name__)
+        if self._rows and name and getattr(node, "keepdims", False) \
+                and node.axis == (len(child.shape) - 1,) and child.shape[-1] > 1 \
+                and (self.row_len is None or self.row_len == child.shape[-1]):
+            ref, code = self.visit(child)
+            if code in ("f4", "f8") and ref[0] != "s":
+                self.row_len = child.shape[-1]
+                return self.op(name, code, code, [ref])
+            raise cg.RowFusionUnsupported("a reduction of integers or of a constant")
+        res = self.leaf(node._force())
+        self.leaf_nodes.append((node, node.array, node.__dict__.get("_deps")))
+        return res
 
     def visit_FullEx(self, node):      # a constant array is a scalar parameter
         res = self.scalar(node.val, _code_of(node.dtype), id(node))
@@ -568,7 +588,7 @@ class Plan:
     launch.  `valid()` re-checks what could have changed underneath."""
 
     __slots__ = ("low", "kern", "checks", "stamp", "shape", "out_dtypes", "acc", "leaves",
-                 "hazard", "region", "empty", "axes", "second", "kern2", "scratch")
+                 "hazard", "region", "empty", "axes", "second", "kern2", "scratch", "out_shapes")
 
     def valid(self):
         if self.stamp != _STAMP:
@@ -710,6 +730,7 @@ def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, 
         low = _Lowered()
         low.key, low.kind, low.emit, low.fmt = template.key, template.kind, template.emit, template.fmt
         low.tail, low.grid, low.fin_count, low.lds = template.tail, template.grid, template.fin_count, template.lds
+        low.row_out = template.row_out
         low.srcs = [(leaves[i].buf, off) for i, off in recipe]
         low.scal = list(scalars)
         low.recipe = recipe
@@ -717,6 +738,8 @@ def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, 
         return low
     low = _lower(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, reduce_op, in_place)
     low.recipe = None
+    if low.kind != "rows":
+        low.row_out = None
     recipe = []
     for buf, off in low.srcs:
         for i, a in enumerate(leaves):
@@ -732,6 +755,7 @@ def _lower_memo(prog, leaves, scalars, shape, out_codes, out_ptrs, out_strides, 
         template.key, template.kind, template.emit, template.fmt = low.key, low.kind, low.emit, low.fmt
         template.tail, template.grid, template.fin_count, template.lds = (low.tail, low.grid,
                                                                           low.fin_count, low.lds)
+        template.row_out = low.row_out
         _LOWERED[key] = (template, recipe)
         low.recipe = recipe
     return low
@@ -856,6 +880,7 @@ def _seen_before(scan):
     plan.second = None
     plan.kern2 = None
     plan.scratch = 0
+    plan.out_shapes = None
     for d in deep:
         d["_seen"] = d.get("_seen", 0) + 1
     STATS["seen_hits"] += 1
@@ -928,6 +953,27 @@ def _make_plan(tracer, roots, dst=None, reduce_op=None, axes=None):
     plan.second = None
     plan.kern2 = None
     plan.scratch = 0
+    plan.out_shapes = None
+    if tracer.row_len is not None:
+        # reductions along the last axis inside the expression: rows are reduced and used
+        # again in one kernel, or the caller evaluates those reductions on their own
+        if dst is not None:
+            raise cg.RowFusionUnsupported("row reductions inside a write")
+        shape = _common_shape(leaves, tracer.gen_shapes)
+        if not shape or shape[-1] != tracer.row_len or 0 in shape:
+            raise cg.RowFusionUnsupported("the rows of the reductions are not the rows of the result")
+        if reduce_op:
+            # the root itself is reduced along the rows: one more operation, one value per row
+            if axes != (len(shape) - 1,) or reduce_op not in _ROW_OPS or roots[0][1] not in ("f4", "f8"):
+                raise cg.RowFusionUnsupported("a reduction along other axes than the rows")
+            roots = [tracer.op(_ROW_OPS[reduce_op], roots[0][1], roots[0][1], [roots[0][0]])]
+            prog = tracer.program(roots)
+        out_codes = [code for _, code in roots]
+        plan.out_dtypes = [code_dtype(code) for code in out_codes]
+        plan.shape = shape
+        plan.low = _lower_memo(prog, leaves, tracer.scalars, shape, out_codes, [0] * len(roots), [], None)
+        plan.out_shapes = [shape[:-1] + (1,) if u else shape for u in plan.low.row_out]
+        return plan
     if reduce_op:
         shape = _common_shape(leaves, tracer.gen_shapes)
         code = roots[0][1]
@@ -1025,7 +1071,10 @@ def _launch_fresh(plan):
             _fire(plan, [], out.ptr)
         outs = [out]
     else:
-        outs = [ndarray(plan.shape, dt) for dt in plan.out_dtypes]
+        if plan.out_shapes is not None:
+            outs = [ndarray(shape, dt) for shape, dt in zip(plan.out_shapes, plan.out_dtypes)]
+        else:
+            outs = [ndarray(plan.shape, dt) for dt in plan.out_dtypes]
         if not plan.empty:
             _fire(plan, [o.ptr for o in outs])
     if _RECORDING is not None:
@@ -1034,8 +1083,6 @@ def _launch_fresh(plan):
 
 
 def _trace_root(tracer, node):
-    if _kind(node) == "ReduceEx" and "array" not in node.__dict__:
-        raise TypeError("a reduction must be the root of its own evaluation")
     return tracer.visit(node)
 
 
@@ -1054,6 +1101,8 @@ def _run_unfused(ex, evaluated):
         root = tracer.visit(ex.children[0])
         out = _launch_fresh(_make_plan(tracer, [root], reduce_op=ex.func.__name__,
                                        axes=getattr(ex, "axis", None)))[0]
+        if out.shape != tuple(ex.shape):
+            out = out.reshape(tuple(ex.shape))
     else:
         root = tracer.visit(ex)
         out = _launch_fresh(_make_plan(tracer, [root]))[0]
@@ -1077,13 +1126,21 @@ def run(ex):
             scan = _scan((ex,), ("run",))
         plan = _seen_before(scan) if scan is not None else None
         if plan is None:
-            tracer = Tracer(reuse=True)
-            if reduction:
-                root = tracer.visit(ex.children[0])
-                plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__, axes=axis)
-            else:
-                root = _trace_root(tracer, ex)
-                plan = _make_plan(tracer, [root])
+            for rows in (True, False):
+                # first with reductions along the last axis as operations of the program;
+                # when the row kernel does not take the result, with those evaluated first
+                tracer = Tracer(reuse=True, rows=rows)
+                try:
+                    if reduction:
+                        root = tracer.visit(ex.children[0])
+                        plan = _make_plan(tracer, [root], reduce_op=ex.func.__name__, axes=axis)
+                    else:
+                        root = _trace_root(tracer, ex)
+                        plan = _make_plan(tracer, [root])
+                    break
+                except cg.RowFusionUnsupported:
+                    if not rows:
+                        raise
             if scan is not None:
                 _remember_structure(scan, tracer, plan)
         d["_plan"] = plan
@@ -1091,6 +1148,8 @@ def run(ex):
     else:
         STATS["plan_hits"] += 1
     out = _launch_fresh(plan)[0]
+    if out.shape != tuple(ex.shape) and _kind(ex) == "ReduceEx":
+        out = out.reshape(tuple(ex.shape))      # the reduced axes kept, or a row kernel's column
     d["_deps"] = plan.deps()
     d["_gen"] = plan.generation()
     return out
@@ -1116,9 +1175,15 @@ def run_multi(exs):
             scan = _scan([exs[i] for i in idxs], ("multi",))
             plan = _seen_before(scan) if scan is not None else None
             if plan is None:
-                tracer = Tracer(reuse=True)
-                roots = [_trace_root(tracer, exs[i]) for i in idxs]
-                plan = _make_plan(tracer, roots)
+                for rows in (True, False):
+                    tracer = Tracer(reuse=True, rows=rows)
+                    try:
+                        roots = [_trace_root(tracer, exs[i]) for i in idxs]
+                        plan = _make_plan(tracer, roots)
+                        break
+                    except cg.RowFusionUnsupported:
+                        if not rows:
+                            raise
                 if scan is not None:
                     _remember_structure(scan, tracer, plan)
             # the other roots are kept alive with the entry (the key holds their ids, which
@@ -1294,7 +1359,7 @@ def lower_only(exs, dst=None):
     Works with placeholder arrays on a machine that has no GPU."""
     if not isinstance(exs, (list, tuple)):
         exs = [exs]
-    tracer = Tracer()
+    tracer = Tracer(rows=True)
     if _kind(exs[0]) == "ReduceEx":
         root = tracer.visit(exs[0].children[0])
         low = _make_plan(tracer, [root], reduce_op=exs[0].func.__name__,

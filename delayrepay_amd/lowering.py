@@ -66,6 +66,13 @@ TUNE = {
     "t_rows": 0,      # transpose tiles: output rows (= contiguous elements of the operand) and
     "t_cols": 0,      # output columns per tile (powers of two; 0: 128 bytes by 1 KB)
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
+    "rowfuse": 1,     # reductions along the last axis inside an expression: one kernel per row
+    "row_steps": 4,   # ... 16-byte units of a row per lane before more lanes share the row
+    "row_lanes": 0,   # ... lanes per row (0: from row_steps)
+    "row_regs": 128,  # ... registers that may hold the row between stages (else it is loaded again)
+    "row_fence": 1,   # ... the compiler keeps the work of one 16-byte unit together
+    "row_recompute": 1,   # ... per-element values are computed again by each stage, not kept
+    "row_bpc": 8,     # ... blocks per compute unit at most
     "stage_loop": 0,  # ... 1: the tables are copied by a loop (one trip to memory per 4 KB)
     "one_run": 1,     # flat kernels with tables in LDS: one run per block, no loop over runs
     "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
@@ -121,7 +128,7 @@ class Lowered:
     """A kernel choice for one evaluation: cache key, source builder, launch recipe."""
 
     __slots__ = ("key", "kind", "emit", "fmt", "srcs", "scal", "tail", "grid", "fin_count", "lds",
-                 "recipe")
+                 "recipe", "row_out")
 
 
 # ---------------------------------------------------------------------------
@@ -264,11 +271,87 @@ def _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_pt
     return low
 
 
+def lower_rows(prog, leaves, scalars, shape, out_codes):
+    """Expression with reductions along its last axis inside it (`codegen.emit_row_fused`):
+    every row is read once, reduced, used again and written once.  `shape` is the shape the
+    expression is evaluated at, rows along its last axis; outputs are new dense arrays, of
+    that shape or, for roots that are constant along the row, with a last axis of one.
+    Raises `codegen.RowFusionUnsupported` for layouts the kernel does not take: the caller
+    then evaluates the reductions on their own."""
+    if not TUNE["rowfuse"] or len(shape) < 2 or shape[-1] < 2:
+        raise cg.RowFusionUnsupported("not a matrix of rows")
+    R = shape[-1]
+    strides = [broadcast_strides(a, shape) for a in leaves]
+    kinds = []
+    for st in strides:
+        if st[-1] not in (0, 1):
+            raise cg.RowFusionUnsupported("an operand without unit stride along the row")
+        kinds.append("v" if st[-1] == 1 else "k")
+    dense = [1] * len(shape)             # a new array of `shape`
+    for k in range(len(shape) - 2, -1, -1):
+        dense[k] = dense[k + 1] * shape[k + 1]
+    mshape, msets = merge_dims(shape[:-1], [st[:-1] for st in strides] + [dense[:-1]])
+    if len(mshape) > 1:
+        raise cg.RowFusionUnsupported("rows that do not form one sequence in every operand")
+    K = mshape[0] if mshape else 1
+    sk = [st[0] if st else 0 for st in msets[:-1]]
+    level, uniform, stages = cg.row_analysis(prog, kinds)
+    row_out = []
+    for (kind, j), _ in prog.roots:
+        row_out.append(uniform[j] if kind == "v" else (kind == "s" or kinds[j] == "k"))
+    V = cg.row_vector(prog, kinds, out_codes, row_out)
+    units = -(-R // V)
+    G = TUNE["row_lanes"]
+    if not G:
+        G = 8
+        while G < cg.BLOCK and -(-units // G) > TUNE["row_steps"]:
+            G = G * 2 if G < cg.WAVE else cg.BLOCK
+    steps = -(-units // G)
+    if steps > cg.ROW_STEPS_MAX or K >= 2 ** 40:
+        raise cg.RowFusionUnsupported("row too long")
+    # An operand's share of its row stays in registers between the stages, as long as all
+    # of them fit; operands that are the same for every row (a vector of weights) come from
+    # the caches every time.
+    own = [k == "v" and st != 0 for k, st in zip(kinds, sk)]
+    keep = tuple(o and steps * 4 * sum(own) <= TUNE["row_regs"] for o in own)
+    footprint = sum(a.nbytes for a in leaves) + sum(K * (1 if u else R) * cg.ITEMSIZE[c]
+                                                   for c, u in zip(out_codes, row_out))
+    nts = bool(TUNE["nts"]) and footprint > TUNE["cache_mib"] << 20
+    low = Lowered()
+    low.lds = 0
+    low.fin_count = 0
+    low.kind = "rows"
+    low.row_out = tuple(row_out)
+    fence, recompute = bool(TUNE["row_fence"]), bool(TUNE["row_recompute"])
+    low.key = ("rows", prog.key(), tuple(kinds), tuple(out_codes), low.row_out, R, G, keep, nts,
+               fence, recompute)
+
+    def emit():
+        return cg.emit_row_fused(prog, kinds, out_codes, row_out, R, G, keep=keep, nt_store=nts,
+                                 fence=fence, recompute=recompute)
+    low.emit = emit
+    if G == cg.BLOCK:
+        blocks = K
+    else:
+        blocks = -(-K // (cg.BLOCK // G))
+    low.grid = max(1, min(blocks, grid_cap() * TUNE["row_bpc"] // max(TUNE["bpc"], 1)))
+    low.fmt = "@" + "P" * (len(leaves) + len(out_codes)) + "".join(_SCALAR_FMT[c] for c in prog.scalars) \
+        + "q" * (1 + len(leaves) + len(out_codes))
+    low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+    low.scal = list(scalars)
+    low.tail = [K] + sk + [1 if u else R for u in row_out]
+    return low
+
+
 def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, reduce_op,
            in_place=False):
     """Pick the kernel shape.  `out_ptrs`/`out_strides` describe the destinations
     (element strides at `out_shape`); for a reduction they are empty and the
     partial-sums pointer is appended at launch."""
+    if any(name in cg.ROW_REDUCE for name, _, _, _ in prog.ops):
+        if reduce_op or in_place or any(p for p in out_ptrs):
+            raise cg.RowFusionUnsupported("row reductions inside a write or a reduction over everything")
+        return lower_rows(prog, leaves, scalars, tuple(out_shape), out_codes)
     n = 1
     for d in out_shape:
         n *= d

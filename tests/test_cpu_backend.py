@@ -189,6 +189,15 @@ SCRIPT = textwrap.dedent("""
 """)
 
 
+def run_cpu(script):
+    """stdout of `script` run under DELAY_CPU in a child process."""
+    env = dict(os.environ, DELAY_CPU="1", PYTHONPATH=ROOT)
+    out = subprocess.run([sys.executable, "-c", textwrap.dedent(script)], env=env, capture_output=True,
+                         text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-3000:]
+    return out.stdout
+
+
 def test_delay_cpu_backend_runs_the_reference_suite():
     env = dict(os.environ, DELAY_CPU="1", PYTHONPATH=ROOT)
     out = subprocess.run([sys.executable, "-c", SCRIPT], env=env, capture_output=True, text=True,
@@ -210,3 +219,46 @@ def test_hip_backend_is_the_default_and_fails_loudly_without_the_library(tmp_pat
                          capture_output=True, text=True, timeout=300)
     assert out.returncode != 0
     assert "libdrhip.so is missing" in out.stderr and "no host fall-back" in out.stderr
+
+
+def test_reductions_that_keep_their_axis_stay_lazy_and_give_numpys_values():
+    """`a.max(axis=-1, keepdims=True)` of a float array is a node, not a value: the HIP
+    backend fuses it with what is built on it; this backend applies NumPy's reduction."""
+    script = r"""
+import numpy as np
+import delayrepay_amd as dr
+from delayrepay_amd.delayarray import ReduceEx, DelayArray
+rs = np.random.RandomState(0)
+a = rs.standard_normal((13, 57))
+da = dr.array(a)
+m = da.max(axis=1, keepdims=True)
+assert isinstance(m, ReduceEx) and m.shape == (13, 1) and "array" not in m.__dict__
+e = np.exp(da - m)
+sm = e / e.sum(axis=-1, keepdims=True)
+ref_e = np.exp(a - a.max(axis=1, keepdims=True))
+assert np.array_equal(sm.get(), ref_e / ref_e.sum(axis=-1, keepdims=True))
+assert np.array_equal(m.get(), a.max(axis=1, keepdims=True))
+assert np.array_equal(dr.var(da, axis=1).get(), ((a - a.mean(axis=1, keepdims=True)) ** 2).sum(axis=1) / 57)
+assert np.allclose(dr.std(da, axis=1, keepdims=True).get(), a.std(axis=1, keepdims=True), rtol=1e-14)
+# not along the last axis, not kept, integers: evaluated at once, as before
+assert not isinstance(da.max(axis=0, keepdims=True), ReduceEx)
+assert not isinstance(da.max(axis=1), ReduceEx)
+assert not isinstance(dr.array(np.arange(12).reshape(3, 4)).max(axis=1, keepdims=True), ReduceEx)
+# keywords that change the result are refused, not dropped
+for call in (lambda: np.sum(da, initial=10.0), lambda: np.any(da, where=np.ones((13, 57), bool)),
+             lambda: np.max(da, initial=0.0)):
+    try:
+        call()
+    except NotImplementedError:
+        pass
+    else:
+        raise AssertionError("keyword accepted")
+assert np.sum(da, where=True) == a.sum()
+# any / all of nothing
+z = dr.array(np.zeros((0, 4)))
+assert bool(np.any(z)) is False and bool(np.all(z)) is True
+assert np.array_equal(np.all(z, axis=0).get(), np.ones(4, bool))
+assert np.array_equal(np.any(z, axis=0, keepdims=True).get(), np.zeros((1, 4), bool))
+print("ok")
+"""
+    assert run_cpu(script).strip().endswith("ok")

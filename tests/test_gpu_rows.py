@@ -1,0 +1,213 @@
+"""Reductions along the last axis inside an expression: one kernel reads each row once,
+reduces it, uses the result and writes once (`codegen.emit_row_fused`; the reference's
+`ReduceEx` as an interior node, delayarray.py:272-283, cuda.py:87-88).
+
+Bars: expressions of max / min and + - * / only are bit-equal to NumPy; sums within
+rtol 1e-6 (float32) / 1e-13 (float64) of NumPy's; what follows a sum inherits its
+tolerance."""
+import numpy as np
+import pytest
+
+import delayrepay_amd as dr
+from delayrepay_amd import hip
+from tests.helpers import bits_equal
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(5, 2), (3, 7), (64, 200), (33, 203), (1000, 64), (7, 1000), (9, 1023), (130, 1025),
+          (50, 4096), (17, 4099), (12, 16384), (5, 16381)]
+
+
+def launches(fn):
+    before = hip.STATS["launches"]
+    out = fn()
+    return out, hip.STATS["launches"] - before
+
+
+def softmax(xp, a):
+    e = xp.exp(a - a.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_softmax_is_one_kernel(shape, dtype):
+    rs = np.random.RandomState(hash(shape) % 1000)
+    a = (rs.standard_normal(shape) * 3).astype(dtype)
+    got, n = launches(lambda: softmax(dr, dr.array(a)).get())
+    ref = softmax(np, a)
+    fits = shape[-1] * a.itemsize <= 65536       # a row of at most 64 KB is held by one block
+    assert (n == 1 or not fits) and got.shape == ref.shape and got.dtype == ref.dtype
+    np.testing.assert_allclose(got, ref, rtol=2e-6 if dtype == np.float32 else 1e-13)
+    np.testing.assert_allclose(got.sum(axis=-1), 1.0, rtol=1e-5 if dtype == np.float32 else 1e-13)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_max_min_and_arithmetic_are_bit_equal(shape):
+    rs = np.random.RandomState(3)
+    a = rs.standard_normal(shape).astype(np.float32)
+    da = dr.array(a)
+    got, n = launches(lambda: (da - da.max(axis=1, keepdims=True)).get())
+    assert n == 1 and bits_equal(got, a - a.max(axis=1, keepdims=True))
+    lo, hi = da.min(axis=-1, keepdims=True), da.max(axis=-1, keepdims=True)
+    got, n = launches(lambda: ((da - lo) / (hi - lo)).get())
+    ref = (a - a.min(axis=-1, keepdims=True)) / (a.max(axis=-1, keepdims=True) - a.min(axis=-1, keepdims=True))
+    assert n == 1 and bits_equal(got, ref)
+
+
+def test_nan_and_infinity_in_a_row_follow_numpy():
+    a = np.random.RandomState(4).standard_normal((6, 300)).astype(np.float32)
+    a[1, 17] = np.nan
+    a[2, 5] = np.inf
+    a[3, 299] = -np.inf
+    a[4, :] = -np.inf
+    da = dr.array(a)
+    with np.errstate(invalid="ignore"):
+        ref = a - a.max(axis=1, keepdims=True)
+        ref2 = softmax(np, a)
+    got = (da - da.max(axis=1, keepdims=True)).get()
+    assert np.array_equal(np.isnan(got), np.isnan(ref)) and bits_equal(np.nan_to_num(got), np.nan_to_num(ref))
+    got2 = softmax(dr, da).get()
+    assert np.array_equal(np.isnan(got2), np.isnan(ref2))
+    np.testing.assert_allclose(np.nan_to_num(got2), np.nan_to_num(ref2), rtol=2e-6)
+
+
+@pytest.mark.parametrize("shape", [(64, 200), (33, 1001), (20, 4096), (6, 16384)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_centred_and_normalised_rows(shape, dtype):
+    rs = np.random.RandomState(7)
+    a = (rs.standard_normal(shape) * 2 + 5).astype(dtype)
+    g, b = rs.standard_normal(shape[1]).astype(dtype), rs.standard_normal(shape[1]).astype(dtype)
+    da, dg, db = dr.array(a), dr.array(g), dr.array(b)
+    tol = dict(rtol=2e-5, atol=2e-5) if dtype == np.float32 else dict(rtol=1e-11, atol=1e-11)
+    fits = shape[-1] * a.itemsize <= 65536
+    got, n = launches(lambda: (da - da.mean(axis=1, keepdims=True)).get())
+    assert n == 1 or not fits
+    np.testing.assert_allclose(got, a - a.mean(axis=1, keepdims=True), **tol)
+    # layer normalisation with weights shared by all rows: mean, then variance, then the rows
+    def layer_norm(xp, x, w, c):
+        mu = x.mean(axis=-1, keepdims=True)
+        d = x - mu
+        var = (d * d).mean(axis=-1, keepdims=True)
+        return d / xp.sqrt(var + 1e-5) * w + c
+    got, n = launches(lambda: layer_norm(dr, da, dg, db).get())
+    assert n == 1 or not fits
+    np.testing.assert_allclose(got, layer_norm(np, a, g, b), **tol)
+    # variance and standard deviation along the rows: the mean never leaves the kernel
+    for keep in (False, True):
+        got, n = launches(lambda: dr.var(da, axis=1, keepdims=keep).get())
+        ref = a.var(axis=1, keepdims=keep)
+        # the row kernel, then the division by n (one more when an operand built by the
+        # lines above has been met often enough to be computed on its own)
+        assert got.shape == ref.shape and (n <= 3 or not fits)
+        np.testing.assert_allclose(got, ref, rtol=1e-4 if dtype == np.float32 else 1e-11)
+        got = dr.std(da, axis=1, ddof=1, keepdims=keep).get()
+        np.testing.assert_allclose(got, a.std(axis=1, ddof=1, keepdims=keep),
+                                   rtol=1e-4 if dtype == np.float32 else 1e-11)
+    # z-scores: two reductions of different depth and a quotient of per-row values
+    got, n = launches(lambda: ((da - da.mean(axis=1, keepdims=True)) / da.std(axis=1, keepdims=True)).get())
+    assert n == 1 or not fits
+    np.testing.assert_allclose(got, (a - a.mean(axis=1, keepdims=True)) / a.std(axis=1, keepdims=True), **tol)
+
+
+def test_values_that_are_one_per_row_come_out_as_columns():
+    rs = np.random.RandomState(8)
+    a = rs.standard_normal((40, 700))
+    da = dr.array(a)
+    m = da.max(axis=1, keepdims=True)
+    lse = m + np.log(np.exp(da - m).sum(axis=1, keepdims=True))
+    got, n = launches(lambda: lse.get())
+    mm = a.max(axis=1, keepdims=True)
+    ref = mm + np.log(np.exp(a - mm).sum(axis=1, keepdims=True))
+    assert n == 1 and got.shape == (40, 1)
+    np.testing.assert_allclose(got, ref, rtol=1e-13)
+    # a kept reduction asked for on its own is an ordinary axis reduction
+    got = da.min(axis=1, keepdims=True).get()
+    assert got.shape == (40, 1) and np.array_equal(got, a.min(axis=1, keepdims=True))
+    # the column and the matrix from one kernel
+    sm = softmax(dr, da)
+    peak = sm.max(axis=1, keepdims=True)
+    (_, _), n = launches(lambda: dr.evaluate(sm, peak))
+    np.testing.assert_allclose(sm.get(), softmax(np, a), rtol=1e-13)
+    np.testing.assert_allclose(peak.get(), softmax(np, a).max(axis=1, keepdims=True), rtol=1e-13)
+
+
+def test_stacks_of_matrices_and_operands_of_other_shapes():
+    rs = np.random.RandomState(9)
+    a = rs.standard_normal((6, 10, 300)).astype(np.float32)
+    col = rs.standard_normal((10, 1)).astype(np.float32)
+    da, dcol = dr.array(a), dr.array(col)
+    got, n = launches(lambda: softmax(dr, da).get())
+    assert n == 1
+    np.testing.assert_allclose(got, softmax(np, a), rtol=2e-6)
+    # a per-row operand and a number in the expression
+    got = ((da * 0.5 - (da * 0.5).max(axis=-1, keepdims=True))[1] + dcol).get()
+    ref = (a * np.float32(0.5) - (a * np.float32(0.5)).max(axis=-1, keepdims=True))[1] + col
+    assert bits_equal(got, ref)
+    # rows of a view (a row pitch that is no multiple of 16 bytes)
+    v = dr.array(rs.standard_normal((50, 333)).astype(np.float32))
+    hv = v.get()
+    got = (v[:, 1:-2] - v[:, 1:-2].max(axis=1, keepdims=True)).get()
+    assert bits_equal(got, hv[:, 1:-2] - hv[:, 1:-2].max(axis=1, keepdims=True))
+
+
+def test_what_the_row_kernel_does_not_take_is_computed_the_long_way():
+    rs = np.random.RandomState(10)
+    a = rs.standard_normal((8, 20000)).astype(np.float32)          # rows too long to hold
+    da = dr.array(a)
+    got, n = launches(lambda: (da - da.max(axis=1, keepdims=True)).get())
+    assert n >= 2 and bits_equal(got, a - a.max(axis=1, keepdims=True))
+    b = rs.standard_normal((300, 40))
+    db = dr.array(b)
+    got = (db - db.max(axis=0, keepdims=True)).get()                # not along the rows
+    assert bits_equal(got, b - b.max(axis=0, keepdims=True))
+    t = dr.array(rs.standard_normal((64, 96)))
+    ht = t.get()
+    got = (t.T - t.T.max(axis=1, keepdims=True)).get()              # rows without unit stride
+    assert bits_equal(got, ht.T - ht.T.max(axis=1, keepdims=True))
+    i = dr.array(rs.randint(0, 100, (20, 30)))
+    hi = i.get()
+    got = (i - i.max(axis=1, keepdims=True)).get()                  # integers
+    assert np.array_equal(got, hi - hi.max(axis=1, keepdims=True))
+    wide = dr.array(rs.standard_normal((16, 64)))
+    hw = wide.get()
+    other = dr.array(rs.standard_normal((16, 1)))
+    ho = other.get()
+    got = (other * 2.0 + wide.sum(axis=1, keepdims=True)).get()     # nothing left that has rows
+    np.testing.assert_allclose(got, ho * 2.0 + hw.sum(axis=1, keepdims=True), rtol=1e-13)
+
+
+def test_the_unfused_mode_and_the_tunables_agree():
+    rs = np.random.RandomState(11)
+    a = rs.standard_normal((70, 5000)).astype(np.float32)
+    ref = softmax(np, a)
+    base = softmax(dr, dr.array(a)).get()
+    for tune in (dict(row_recompute=0), dict(row_fence=0), dict(row_regs=0), dict(row_lanes=64),
+                 dict(row_steps=16), dict(rowfuse=0)):
+        old = {k: hip.TUNE[k] for k in tune}
+        hip.set_tune(**tune)
+        try:
+            got = softmax(dr, dr.array(a)).get()
+        finally:
+            hip.set_tune(**old)
+        np.testing.assert_allclose(got, ref, rtol=2e-6)
+        if "row_lanes" not in tune and "rowfuse" not in tune and "row_steps" not in tune:
+            assert bits_equal(got, base), tune      # same order of additions
+    hip.set_fused(False)
+    try:
+        got = softmax(dr, dr.array(a)).get()
+    finally:
+        hip.set_fused(True)
+    np.testing.assert_allclose(got, ref, rtol=2e-6)
+
+
+def test_softmax_full_size():
+    """16384 rows of 16384 float32: every row sums to one, agrees with NumPy on sampled rows."""
+    rs = np.random.RandomState(12)
+    a = rs.standard_normal((16384, 16384)).astype(np.float32)
+    got, n = launches(lambda: softmax(dr, dr.array(a)).get())
+    assert n == 1
+    np.testing.assert_allclose(got.sum(axis=1, dtype=np.float64), 1.0, rtol=1e-5)
+    rows = rs.randint(0, 16384, 64)
+    np.testing.assert_allclose(got[rows], softmax(np, a[rows]), rtol=2e-6)
+    assert np.array_equal(got.argmax(axis=1), a.argmax(axis=1))
