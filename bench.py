@@ -86,7 +86,8 @@ def parse():
     ap.add_argument("--workload", default="all",
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
                          "dot | axis0 | axis1 | axis1_3d | matvec | rows200 | rowbcast | transpose | "
-                         "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | next (all "
+                         "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | softmax | "
+                         "layernorm | next (all "
                          "of these: the operations either side of the five configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
@@ -305,6 +306,38 @@ def main():
                         steps=[(lambda v=v: hip.run(v.T * 2.0)) for v in vols],
                         cpu=lambda: hv[:, :, :256].T * np.float32(2.0), cpu_frac=0.25,
                         cpu_code="numpy.multiply")
+        if name in ("softmax", "layernorm", "rowmax"):
+            N = 16384
+            ha = rs.standard_normal((N, N)).astype(np.float32)
+            mats = [dr.array(ha) for _ in range(sets_for(8 * N * N))]
+            if name == "rowmax":
+                return dict(dtype="f32", n=N * N, nbytes=8 * N * N,
+                            desc="a - max(a, axis=1) f32 16384x16384 (the row kernel with next to no arithmetic)",
+                            steps=[(lambda a=a: hip.run(a - a.max(axis=1, keepdims=True))) for a in mats],
+                            cpu=lambda: ha[:N // 16] - ha[:N // 16].max(axis=1, keepdims=True), cpu_frac=1 / 16,
+                            cpu_code="numpy.max, subtract")
+            if name == "softmax":
+                def soft(xp, a):
+                    e = xp.exp(a - a.max(axis=1, keepdims=True))
+                    return e / e.sum(axis=1, keepdims=True)
+                return dict(dtype="f32", n=N * N, nbytes=8 * N * N,
+                            desc="softmax along the rows f32 16384x16384 (row maximum, sum of "
+                                 "exponentials and quotient in one kernel)",
+                            steps=[(lambda a=a: hip.run(soft(dr, a))) for a in mats],
+                            cpu=lambda: soft(np, ha[:N // 16]), cpu_frac=1 / 16,
+                            cpu_code="numpy.max, subtract, exp, sum, divide")
+            hg, hb = rs.standard_normal(N).astype(np.float32), rs.standard_normal(N).astype(np.float32)
+            g, b = dr.array(hg), dr.array(hb)
+
+            def norm(xp, a, w, c):
+                d = a - a.mean(axis=1, keepdims=True)
+                return d / xp.sqrt((d * d).mean(axis=1, keepdims=True) + 1e-5) * w + c
+            return dict(dtype="f32", n=N * N, nbytes=8 * N * N + 8 * N,
+                        desc="layer normalisation along the rows f32 16384x16384 (mean, variance "
+                             "and the normalised rows in one kernel)",
+                        steps=[(lambda a=a: hip.run(norm(dr, a, g, b))) for a in mats],
+                        cpu=lambda: norm(np, ha[:N // 16], hg, hb), cpu_frac=1 / 16,
+                        cpu_code="numpy.mean, subtract, multiply, sqrt, divide, add")
         if name in ("axis0", "axis1", "rowbcast", "transpose", "interior", "rows200"):
             N = 16384
             ha = rs.standard_normal((N, N)).astype(np.float32)
@@ -594,7 +627,8 @@ def main():
 
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
              "next": ["dot", "axis0", "axis1", "axis1_3d", "matvec", "rows200", "rowbcast", "transpose",
-                      "transpose3d", "interior", "diff2", "stencil9", "stencil3d", "grid", "rand"]}.get(args.workload, [args.workload])
+                      "transpose3d", "interior", "diff2", "stencil9", "stencil3d", "grid", "rand",
+                      "softmax", "layernorm"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:

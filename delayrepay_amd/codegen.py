@@ -2248,9 +2248,12 @@ def row_analysis(prog, leaf_kind):
     return level, uniform, stages
 
 
-def _row_needed(prog, targets):
+def _row_needed(prog, targets, held=None):
     """Operations to compute for the values `targets` (refs), in order, the row
-    reductions they read (those are handed in, not computed) and the leaves they read."""
+    reductions they read (those are handed in, not computed) and the leaves they read.
+    `held` maps an operation to the leaf whose registers hold its value by now: such a
+    value is read from that leaf's slot, and what it was computed from is not needed."""
+    held = held or {}
     need, given = set(), set()
     leaves = {j for k, j in targets if k == "l"}
     stack = [j for k, j in targets if k == "v"]
@@ -2261,6 +2264,10 @@ def _row_needed(prog, targets):
         if prog.ops[i][0] in ROW_REDUCE:
             given.add(i)
             continue
+        if i in held:
+            leaves.add(held[i])
+            need.add(i)
+            continue
         need.add(i)
         for k, j in prog.ops[i][3]:
             if k == "v":
@@ -2270,22 +2277,62 @@ def _row_needed(prog, targets):
     return sorted(need), sorted(given), leaves
 
 
-def _row_function(prog, fname, targets, out_dtypes):
+def _row_function(prog, fname, targets, out_dtypes, held=None):
     """Device function computing `targets` for one element (or one row, when every target
     is constant along the row): parameters are all leaf values, all scalars, the row
     reductions it reads, then one reference per target.  Returns (source, reductions read,
     leaves read)."""
-    need, given, used = _row_needed(prog, targets)
+    held = held or {}
+    need, given, used = _row_needed(prog, targets, held)
     params = [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"const {CTYPE[prog.ops[i][2]]} v{i}" for i in given]
     params += [f"{CTYPE[dt]}& r{n}" for n, dt in enumerate(out_dtypes)]
     lines = [f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
-    lines += [_op_statement(prog, i) for i in need]
+    for i in need:
+        if i in held:       # computed by an earlier stage and kept where its operand was
+            lines.append(f"    const {CTYPE[prog.ops[i][2]]} v{i} = l{held[i]};")
+        else:
+            lines.append(_op_statement(prog, i))
     for n, ((k, j), dt) in enumerate(zip(targets, out_dtypes)):
         lines.append(f"    r{n} = {_conv(f'{k}{j}', prog.ref_dtype((k, j)), dt)};")
     lines.append("}")
     return "\n".join(lines), given, used
+
+
+_ROW_CHEAP = frozenset(("add", "subtract", "multiply", "negative", "positive", "absolute", "fabs",
+                        "maximum", "minimum", "fmax", "fmin", "cast", "copysign", "where", "square"))
+
+
+def _row_carry(prog, need, later_targets, held, kept, uniform):
+    """Which value computed by this stage (operations `need`) to keep for the stages that
+    follow, and where: (operation, leaf) or None.  A value qualifies when later stages read
+    it, when it costs more than a few additions to compute again (an exponential, a
+    quotient), and when there is an operand of its type that is held in registers and that
+    the later stages read only through this value: its registers then hold the value
+    instead.  softmax: exp(a - max) takes the place of a after the sum."""
+    later_need, _, _ = _row_needed(prog, later_targets, held)
+    for v in sorted(set(need) & set(later_need), reverse=True):
+        name, _, rdt, _ = prog.ops[v]
+        if uniform[v] or v in held:
+            continue
+        # what computing v again would cost: the operations below it down to what is at hand
+        below, _, leaves_of_v = _row_needed(prog, [("v", v)], held)
+        if all(prog.ops[i][0] in _ROW_CHEAP for i in below):
+            continue
+        for leaf in sorted(leaves_of_v & kept):
+            if prog.leaves[leaf] != rdt or leaf in held.values():
+                continue
+            trial = dict(held)
+            trial[v] = leaf
+            _, _, still = _row_needed(prog, later_targets, trial)
+            # the leaf's slot may be read later only as the carried value
+            reads_leaf_itself = any(
+                ("l", leaf) in prog.ops[i][3]
+                for i in _row_needed(prog, later_targets, trial)[0] if i not in trial)
+            if not reads_leaf_itself and not any(k == "l" and j == leaf for k, j in later_targets):
+                return v, leaf
+    return None
 
 
 def row_vector(prog, leaf_kind, out_dtypes, out_uniform):
@@ -2297,7 +2344,7 @@ def row_vector(prog, leaf_kind, out_dtypes, out_uniform):
 
 
 def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt_store=False,
-                   fence=True, recompute=True):
+                   fence=True, recompute=True, pipeline=True, carry_values=True, wave_map=False):
     """Rows that are reduced and used again: `a - max(a, axis=-1)`, softmax, the variance,
     layer normalisation.  A group of G lanes (8..64: part of a wave; 256: the block) owns a
     row of R elements (a compile-time constant, unit stride); lane j takes the 16-byte
@@ -2312,6 +2359,9 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     (two slots in turn, so one barrier per reduction).  The last stage computes the roots
     and stores them; a root that is constant along the row is stored once per row.
 
+    A value that a stage computes at some cost and later stages read (softmax's
+    exponentials) takes the place of the operand it was computed from in those registers
+    (`_row_carry`).
     `fence`: the compiler may not move instructions from one 16-byte unit's work to the
     next (left to itself it interleaves all sixteen units of a long row for the sake of
     instruction-level parallelism and needs 205 vector registers for a softmax of rows of
@@ -2337,21 +2387,38 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     src = [PREAMBLE, mathlib.source(prog.own_math), mathlib32.source(prog.own_math32)]
 
     # one function per stage, one for the per-element roots, one for the per-row roots
-    stage_fn = []
-    for s, reds in enumerate(stages):
-        targets = [prog.ops[i][3][0] for i in reds]
-        text, given, used = _row_function(prog, f"dr_stage{s}", targets, [prog.ops[i][1] for i in reds])
-        src.append(text)
-        stage_fn.append((given, used))
-    elem_roots = [n for n in range(n_out) if not out_uniform[n]]
-    row_roots = [n for n in range(n_out) if out_uniform[n]]
-    final_given = rowout_given = ()
-    final_used = set()
     if keep is None:
         keep = [True] * nl
+    kept = {i for i in range(nl) if keep[i] and leaf_kind[i] == "v"}
+    elem_roots = [n for n in range(n_out) if not out_uniform[n]]
+    row_roots = [n for n in range(n_out) if out_uniform[n]]
+    final_targets = [prog.roots[n][0] for n in elem_roots]
+    stage_targets = [[prog.ops[i][3][0] for i in reds] for reds in stages]
+    stage_fn = []
+    held = {}
+    carried_leaves = set()
+    for s, reds in enumerate(stages):
+        targets = stage_targets[s]
+        outs = [prog.ops[i][1] for i in reds]
+        carry = None
+        if carry_values:
+            later = [t for ts in stage_targets[s + 1:] for t in ts] + final_targets
+            need, _, _ = _row_needed(prog, targets, held)
+            carry = _row_carry(prog, need, later, held, kept, uniform)
+        if carry is not None:
+            targets = targets + [("v", carry[0])]
+            outs = outs + [prog.ops[carry[0]][2]]
+        text, given, used = _row_function(prog, f"dr_stage{s}", targets, outs, held)
+        src.append(text)
+        stage_fn.append((given, used, carry))
+        if carry is not None:
+            held[carry[0]] = carry[1]
+            carried_leaves.add(carry[1])
+    final_given = rowout_given = ()
+    final_used = set()
     if elem_roots:
         text, final_given, final_used = _row_function(
-            prog, "dr_final", [prog.roots[n][0] for n in elem_roots], [out_dtypes[n] for n in elem_roots])
+            prog, "dr_final", final_targets, [out_dtypes[n] for n in elem_roots], held)
         src.append(text)
     if row_roots:
         text, rowout_given, _ = _row_function(
@@ -2387,40 +2454,36 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     scal = [f"s{i}" for i in range(ns)]
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{"]
-    if block_row:
-        widest = max((CTYPE[prog.ops[i][2]] for reds in stages for i in reds),
-                     key=lambda c: 8 if c in ("double", "long long") else 4)
-        L += [f"    __shared__ {widest} dr_slots[2][{max(n_red, 1)}][{BLOCK // WAVE}];",
-              "    const int sub = threadIdx.x;",
-              "    int turn = 0;",
-              "    for (long long row = blockIdx.x; row < K; row += gridDim.x, turn ^= 1) {",
-              "        const long long k = row;"]
-    else:
-        L += [f"    const int sub = threadIdx.x & {G - 1};",
-              f"    const int grp = (threadIdx.x & {WAVE - 1}) >> {G.bit_length() - 1};",
-              f"    const long long stride = (long long)gridDim.x * {BLOCK // WAVE * per_wave};",
-              f"    for (long long first = ((long long)blockIdx.x * {BLOCK // WAVE} + (threadIdx.x >> 6)) * "
-              f"{per_wave}; first < K; first += stride) {{",
-              "        const long long row = first + grp;",
-              "        const long long k = row < K ? row : K - 1;      // idle groups re-read the last row"]
-    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
-        if kind == "v":
-            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
-        else:
-            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
-
     def vtype(dt):
         return (VEC16[dt][0] + "u") if V > 1 else CTYPE[dt]
 
+    # Which unit a lane takes in step j: `lo + sub`.  Lanes side by side over the whole
+    # group (sub = lane, lo = j G), or, `wave_map`, every wave of the block its own quarter
+    # of the row (sub = wave * quarter + lane, lo = 64 j): a wave then reads 16 KB of a
+    # 64 KB row in sequence instead of sixteen pieces 4 KB apart, which the memory system
+    # serves faster (copying rows of 64 KB: 75 % of the peak against 66 %; rows of 16 and
+    # 32 KB: 74 against 76 % and 69 against 71 %).
+    wave_map = bool(block_row and wave_map and steps > 1)
+    seg = steps * WAVE
+    step_units = WAVE if wave_map else G
+    max_sub = (BLOCK // WAVE - 1) * seg + WAVE - 1 if wave_map else G - 1
+
+    def holds(sub):
+        """Whether some lane has this `sub`."""
+        if sub < 0:
+            return False
+        return (sub % seg < WAVE and sub // seg < BLOCK // WAVE) if wave_map else sub < G
+
     # which lanes hold what in step j: whole units, the partial last unit, nothing
     def step_state(j):
-        lo = j * G
-        whole = "" if lo + G <= full else (f"{lo} + sub < {full}" if lo < full else None)
-        part = f"sub == {full - lo}" if rem and lo <= full < lo + G else None
+        lo = j * step_units
+        whole = "" if lo + max_sub < full else (f"{lo} + sub < {full}" if lo < full else None)
+        part = f"sub == {full - lo}" if rem and holds(full - lo) else None
         return lo, whole, part
 
-    def loads(j, pad, which):
-        """Declarations and loads of step j's units of the row operands in `which`."""
+    def loads(j, pad, which, base="row", declare=True):
+        """Loads of step j's units of the row operands in `which` from the rows at
+        `base`<i>, into new variables or (`declare` False) into the ones at hand."""
         lo, whole, part = step_state(j)
         out = []
         for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
@@ -2428,16 +2491,97 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
                 continue
             vt = vtype(dt)
             zero = "{0}" if V > 1 else "0"
-            if whole == "":
-                out.append(f"{pad}const {vt} X{j}_{i} = *(const {vt}*)(row{i} + ({lo} + sub) * {V});")
+            # a pointer that is the same for the wave plus a lane's unsigned 32-bit offset:
+            # the load then takes its address from a scalar register pair and one vector
+            # register, instead of a vector register pair per unit of the row
+            ld = f"*(const {vt}*)(({base}{i} + {lo * V}) + usub * {V}u)"
+            if whole == "" and declare:
+                const = "" if i in carried_leaves else "const "
+                out.append(f"{pad}{const}{vt} X{j}_{i} = {ld};")
                 continue
-            out.append(f"{pad}{vt} X{j}_{i} = {zero};")
-            if whole is not None:
-                out.append(f"{pad}if ({whole}) X{j}_{i} = *(const {vt}*)(row{i} + ({lo} + sub) * {V});")
+            if declare:
+                out.append(f"{pad}{vt} X{j}_{i} = {zero};")
+            if whole == "":
+                out.append(f"{pad}X{j}_{i} = {ld};")
+            elif whole is not None:
+                out.append(f"{pad}if ({whole}) X{j}_{i} = {ld};")
             if part is not None:
-                fill = " ".join(f"X{j}_{i}[{e}] = row{i}[{full * V + e}];" for e in range(rem))
+                fill = " ".join(f"X{j}_{i}[{e}] = {base}{i}[{full * V + e}];" for e in range(rem))
                 out.append(f"{pad}if ({part}) {{ {fill} }}")
         return out
+
+    def row_pointers(pad, k, base="row", which=None):
+        out = []
+        for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+            if kind == "v" and (which is None or i in which):
+                out.append(f"{pad}const {CTYPE[dt]}* {base}{i} = a{i} + {k} * sk{i};")
+        return out
+
+    # Rows in turn: the registers that hold a row are filled for the next row as soon as
+    # the last stage has used them, so the next row is on its way while this one is
+    # finished and stored (`rotate`; the first row is loaded ahead of the loop).
+    # (not when the last stage also loads operands that are not held: the wave would wait
+    # for them behind the next row's loads, which return in order)
+    unheld_in_final = {i for i in final_used if leaf_kind[i] == "v"} - kept
+    rotate = bool(kept) and pipeline and not unheld_in_final
+    if rotate:
+        for j in range(steps):
+            for i in sorted(kept):
+                zero = "{0}" if V > 1 else "0"
+                L.append(f"    {vtype(prog.leaves[i])} X{j}_{i} = {zero};")
+    if block_row:
+        widest = max((CTYPE[prog.ops[i][2]] for reds in stages for i in reds),
+                     key=lambda c: 8 if c in ("double", "long long") else 4)
+        L += [f"    __shared__ {widest} dr_slots[2][{max(n_red, 1)}][{BLOCK // WAVE}];",
+              f"    const int sub = (threadIdx.x >> 6) * {seg} + (threadIdx.x & {WAVE - 1});" if wave_map
+              else "    const int sub = threadIdx.x;",
+              "    const unsigned int usub = sub;",
+              "    int turn = 0;"]
+        if rotate:
+            L.append("    if (blockIdx.x < K) {")
+            L += row_pointers("        ", "(long long)blockIdx.x", which=kept)
+            for j in range(steps):
+                L += loads(j, "        ", kept, declare=False)
+            L.append("    }")
+        L += ["    for (long long row = blockIdx.x; row < K; row += gridDim.x, turn ^= 1) {",
+              "        const long long k = row;"]
+        if rotate:
+            L += ["        const bool more = row + gridDim.x < K;",
+                  "        const long long nk = more ? row + gridDim.x : row;"]
+    else:
+        L += [f"    const int sub = threadIdx.x & {G - 1};",
+              f"    const unsigned int usub = threadIdx.x & {G - 1};",
+              f"    const int grp = (threadIdx.x & {WAVE - 1}) >> {G.bit_length() - 1};",
+              f"    const long long stride = (long long)gridDim.x * {BLOCK // WAVE * per_wave};",
+              f"    const long long start = ((long long)blockIdx.x * {BLOCK // WAVE} + (threadIdx.x >> 6)) * "
+              f"{per_wave};"]
+        if rotate:
+            L.append("    if (start < K) {")
+            L.append("        const long long k0 = start + grp < K ? start + grp : K - 1;")
+            L += row_pointers("        ", "k0", which=kept)
+            for j in range(steps):
+                L += loads(j, "        ", kept, declare=False)
+            L.append("    }")
+        L += ["    for (long long first = start; first < K; first += stride) {",
+              "        const long long row = first + grp;",
+              "        const long long k = row < K ? row : K - 1;      // idle groups re-read the last row"]
+        if rotate:
+            L += ["        const bool more = first + stride < K;",
+                  "        const long long nk = more ? (first + stride + grp < K ? first + stride + grp : K - 1) : k;"]
+    for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
+        if kind == "v":
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+        else:
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+    if rotate:
+        L += row_pointers("        ", "nk", base="nrow", which=kept)
+
+    def next_loads(j, pad):
+        """The next row's units of step j, into the registers that step j has just used."""
+        if not rotate:
+            return []
+        inner = loads(j, pad + "    ", kept, base="nrow", declare=False)
+        return [f"{pad}if (more) {{"] + inner + [f"{pad}}}"] if inner else []
 
     def element_args(j, e, used):
         """Arguments for the leaves: an operand that the function does not read is a zero."""
@@ -2470,9 +2614,9 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
         ct = CTYPE[prog.ops[g][2]]
         L.append(f'{pad}{ct} v{g}_{tag} = v{g}; asm volatile("" : "+v"(v{g}_{tag}));')
         return f"v{g}_{tag}"
-    kept = {i for i in range(nl) if keep[i] and leaf_kind[i] == "v"}
-    for j in range(steps):
-        L += loads(j, pad, kept)
+    if not rotate:
+        for j in range(steps):
+            L += loads(j, pad, kept)
     slot = 0
     for s, reds in enumerate(stages):
         for i in reds:
@@ -2482,14 +2626,20 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
         for g in stage_fn[s][0]:
             given.append(relabel(g, f"s{s}"))
         used = stage_fn[s][1]
+        carry = stage_fn[s][2]
         again = {i for i in used if leaf_kind[i] == "v"} - kept
         outs = [f"t{i}" for i in reds]
         decl = " ".join(f"{CTYPE[prog.ops[i][1]]} t{i};" for i in reds)
+        if carry is not None:
+            outs.append("tc")
+            decl += f" {CTYPE[prog.ops[carry[0]][2]]} tc;"
         for j in range(steps):
             body = []
             for e in range(V):
                 acc = " ".join(f"acc{i} = {_combine(ROW_REDUCE[prog.ops[i][0]], f'acc{i}', f't{i}')};"
                                for i in reds)
+                if carry is not None:       # the value takes its operand's place in the registers
+                    acc += f" X{j}_{carry[1]}{f'[{e}]' if V > 1 else ''} = tc;"
                 stmt = (f"{{ {decl} dr_stage{s}({', '.join(element_args(j, e, used) + scal + given + outs)}); "
                         f"{acc} }}")
                 line = guarded(j, e, stmt, pad + ("    " if again else ""))
@@ -2535,7 +2685,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
             for n in elem_roots:
                 dt = out_dtypes[n]
                 base = f"o{n} + row * so{n}"
-                st = _st(nt_store and V > 1, f"Y{n}", f"({vtype(dt)}*)({base} + ({lo} + sub) * {V})")
+                st = _st(nt_store and V > 1, f"Y{n}", f"({vtype(dt)}*)(({base} + {lo * V}) + usub * {V}u)")
                 if whole == "":
                     L.append(f"{inner}{store_guard}{st}")
                 elif whole is not None:
@@ -2545,9 +2695,13 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
                     tail = " ".join(f"({base})[{full * V + e}] = Y{n}[{e}];" for e in range(rem))
                     cond = f"{part}" if block_row else f"row < K && {part}"
                     L.append(f"{inner}if ({cond}) {{ {tail} }}")
+            L += next_loads(j, inner)
             L.append(f"{pad}}}")
             if fence and j + 1 < steps:
                 L.append(f"{pad}__builtin_amdgcn_sched_barrier(0);")
+    elif rotate:
+        for j in range(steps):
+            L += next_loads(j, pad)
     if row_roots:
         given = [f"v{g}" for g in rowout_given]
         outs = [f"z{n}" for n in row_roots]

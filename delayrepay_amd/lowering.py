@@ -67,12 +67,14 @@ TUNE = {
     "t_cols": 0,      # output columns per tile (powers of two; 0: 128 bytes by 1 KB)
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
     "rowfuse": 1,     # reductions along the last axis inside an expression: one kernel per row
-    "row_steps": 4,   # ... 16-byte units of a row per lane before more lanes share the row
-    "row_lanes": 0,   # ... lanes per row (0: from row_steps)
+    "row_lanes": 0,   # ... lanes per row (0: by the cost of idle lanes and of units per lane)
     "row_regs": 128,  # ... registers that may hold the row between stages (else it is loaded again)
+    "row_wavemap": -1,    # ... each wave of a block takes a quarter of the row (-1: rows of 48 KB up)
+    "row_carry": 1,   # ... a costly value read by later stages takes its operand's registers
+    "row_pipe": 1,    # ... the next row is loaded while this one is finished and stored
     "row_fence": 1,   # ... the compiler keeps the work of one 16-byte unit together
     "row_recompute": 1,   # ... per-element values are computed again by each stage, not kept
-    "row_bpc": 8,     # ... blocks per compute unit at most
+    "row_bpc": 0,     # ... blocks per compute unit at most (0: one pass, a block per set of rows)
     "stage_loop": 0,  # ... 1: the tables are copied by a loop (one trip to memory per 4 KB)
     "one_run": 1,     # flat kernels with tables in LDS: one run per block, no loop over runs
     "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
@@ -303,9 +305,20 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     units = -(-R // V)
     G = TUNE["row_lanes"]
     if not G:
-        G = 8
-        while G < cg.BLOCK and -(-units // G) > TUNE["row_steps"]:
-            G = G * 2 if G < cg.WAVE else cg.BLOCK
+        # Lanes per row: few units per lane (a lane with one load in flight per row keeps
+        # more rows in flight per wave), but no group much wider than its row (rows of 100
+        # units on a block of 256 lanes leave 60 % of them idle and pay for barriers).
+        best = None
+        for lanes in (8, 16, 32, 64, cg.BLOCK):
+            n = -(-units // lanes)
+            if n > cg.ROW_STEPS_MAX:
+                continue
+            # lane slots per unit of the row, dearer with every further unit per lane and
+            # with the barriers of a block
+            cost = lanes * n / units * (1 + 0.25 * (n - 1)) * (1.1 if lanes == cg.BLOCK else 1.0)
+            if best is None or cost < best[0]:
+                best = (cost, lanes)
+        G = best[1] if best else cg.BLOCK
     steps = -(-units // G)
     if steps > cg.ROW_STEPS_MAX or K >= 2 ** 40:
         raise cg.RowFusionUnsupported("row too long")
@@ -322,19 +335,27 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     low.fin_count = 0
     low.kind = "rows"
     low.row_out = tuple(row_out)
-    fence, recompute = bool(TUNE["row_fence"]), bool(TUNE["row_recompute"])
+    fence, recompute, pipe = bool(TUNE["row_fence"]), bool(TUNE["row_recompute"]), bool(TUNE["row_pipe"])
+    carry = bool(TUNE["row_carry"])
+    wmap = G == cg.BLOCK and (steps >= 12 if TUNE["row_wavemap"] < 0 else bool(TUNE["row_wavemap"]))
     low.key = ("rows", prog.key(), tuple(kinds), tuple(out_codes), low.row_out, R, G, keep, nts,
-               fence, recompute)
+               fence, recompute, pipe, carry, wmap)
 
     def emit():
         return cg.emit_row_fused(prog, kinds, out_codes, row_out, R, G, keep=keep, nt_store=nts,
-                                 fence=fence, recompute=recompute)
+                                 fence=fence, recompute=recompute, pipeline=pipe, carry_values=carry,
+                                 wave_map=wmap)
     low.emit = emit
     if G == cg.BLOCK:
         blocks = K
     else:
         blocks = -(-K // (cg.BLOCK // G))
-    low.grid = max(1, min(blocks, grid_cap() * TUNE["row_bpc"] // max(TUNE["bpc"], 1)))
+    # One pass: every block takes its rows and ends.  Blocks that stay and stride through
+    # the matrix are slower here as they are for flat kernels (`a - max(a, axis=1)` float32,
+    # percent of the HBM peak, 2048 blocks that stay / one pass: rows of 64: 67 / 79, of
+    # 200: 62 / 74, of 1000: 63 / 80, of 4096: 69 / 72, of 16384: 70 / 71).
+    cap = grid_cap() * TUNE["row_bpc"] // max(TUNE["bpc"], 1) if TUNE["row_bpc"] else (1 << 24) - 1
+    low.grid = max(1, min(blocks, cap))
     low.fmt = "@" + "P" * (len(leaves) + len(out_codes)) + "".join(_SCALAR_FMT[c] for c in prog.scalars) \
         + "q" * (1 + len(leaves) + len(out_codes))
     low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]

@@ -15,7 +15,7 @@ from tests.helpers import bits_equal
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(5, 2), (3, 7), (64, 200), (33, 203), (1000, 64), (7, 1000), (9, 1023), (130, 1025),
-          (50, 4096), (17, 4099), (12, 16384), (5, 16381)]
+          (50, 4096), (17, 4099), (12, 16384), (5, 16381), (9, 13001), (6, 12289)]
 
 
 def launches(fn):
@@ -183,7 +183,8 @@ def test_the_unfused_mode_and_the_tunables_agree():
     ref = softmax(np, a)
     base = softmax(dr, dr.array(a)).get()
     for tune in (dict(row_recompute=0), dict(row_fence=0), dict(row_regs=0), dict(row_lanes=64),
-                 dict(row_steps=16), dict(rowfuse=0)):
+                 dict(row_lanes=256, row_bpc=2), dict(rowfuse=0), dict(row_pipe=0), dict(row_carry=0),
+                 dict(row_wavemap=1), dict(row_wavemap=0, row_lanes=256)):
         old = {k: hip.TUNE[k] for k in tune}
         hip.set_tune(**tune)
         try:
@@ -191,7 +192,7 @@ def test_the_unfused_mode_and_the_tunables_agree():
         finally:
             hip.set_tune(**old)
         np.testing.assert_allclose(got, ref, rtol=2e-6)
-        if "row_lanes" not in tune and "rowfuse" not in tune and "row_steps" not in tune:
+        if not {"row_lanes", "rowfuse", "row_wavemap"} & set(tune):
             assert bits_equal(got, base), tune      # same order of additions
     hip.set_fused(False)
     try:
