@@ -48,19 +48,24 @@ METRIC = "fused-kernel effective HBM GB/s (% of MI355X peak); Gelem/s vs unfused
 
 
 def measured_traffic(name):
-    """HBM bytes per launch of a workload's kernel as measured with rocprofv3
-    counters (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel); the figures
-    live in profiles/hbm_traffic.txt as `<workload> <bytes>` lines."""
+    """(HBM bytes per launch, kernel names) of a workload as measured with rocprofv3
+    counters (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel); the figures live
+    in profiles/hbm_traffic.txt as `<workload> <bytes>   # <kernel>[, <kernel>]: ...`
+    lines.  The kernel names carry a digest of everything that shapes the generated
+    source, so a figure taken from another version of a kernel can be told."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
     try:
         with open(path) as fh:
             for ln in fh:
                 parts = ln.split()
                 if len(parts) >= 2 and parts[0] == name:
-                    return int(float(parts[1]))
+                    kernels = []
+                    if "#" in ln:
+                        kernels = [k.strip() for k in ln.split("#", 1)[1].split(":", 1)[0].split(",")]
+                    return int(float(parts[1])), sorted(k for k in kernels if k)
     except OSError:
         pass
-    return None
+    return None, []
 
 
 def profiled_figure(fname, name):
@@ -559,6 +564,25 @@ def main():
                            for k, e in r["subsets"].items() if k in (1, 4, 8)}}
                 for which, r in rep.items()}
             res["parity"]["subsets"] = "k: options with |oracle price| >= 2^-k max(S, K)"
+            if name == "bs32":
+                # Why the float32 bar is wider than two ulp: NumPy's own float32 prices are
+                # several ulp from the true ones (the float64 evaluation of the same
+                # inputs).  Largest distance from that value, in float32 ulp, of this
+                # backend's prices and of NumPy's, on options with |price| >= 2^-k max(S, K).
+                truth = orc.black_scholes(*(inp[k].astype(np.float64) for k in "SKT"),
+                                          inp["r"], inp["sigma"])
+                scale = np.maximum(inp["S"], inp["K"]).astype(np.float64)
+                vs = {}
+                for which, got, ref, t in (("call", call, ocall, truth[0]), ("put", put, oput, truth[1])):
+                    ulp = np.spacing(np.abs(t).astype(np.float32)).astype(np.float64)
+                    for k in (1, 2, 4):
+                        m = np.abs(t) >= scale * 2.0 ** -k
+                        if m.any():
+                            vs[f"{which}_k{k}"] = {
+                                "device_ulp": round(float(np.max(np.abs(got - t)[m] / ulp[m])), 2),
+                                "numpy_float32_ulp": round(float(np.max(np.abs(ref - t)[m] / ulp[m])), 2)}
+                res["parity"]["ulp_from_float64_value"] = vs
+                del truth, scale
             del call, put, ocall, oput
         if "sets" in wl and not args.no_parity:
             # The stream mix alone: the same three loads and two stores per element with a
@@ -690,10 +714,25 @@ def main():
     }
     if copy is not None:
         line["copy_kernel"] = copy
-    traffic = measured_traffic(HEADLINE)
-    if traffic is not None:
-        line["roofline"]["traffic"] = traffic
+    # HBM traffic per launch comes from a profiler run (counters cannot be read here): it
+    # is quoted only for the very kernels this run launched; a figure taken from another
+    # version of a kernel is dropped and flagged
+    for name, res in results.items():
+        traffic, kernels = measured_traffic(name)
+        if traffic is None:
+            continue
+        ran = sorted(k for k in res["kernel"] if not k.endswith("_fin"))
+        if kernels == ran:
+            res["hbm_traffic_bytes"] = traffic
+            res["hbm_traffic_over_algorithmic"] = round(traffic / res["algorithmic_bytes"], 4)
+        else:
+            res["hbm_traffic_bytes"] = None
+            res["hbm_traffic_stale"] = {"profiled": kernels, "ran": ran}
+    if head.get("hbm_traffic_bytes") is not None:
+        line["roofline"]["traffic"] = head["hbm_traffic_bytes"]
         line["roofline"]["traffic_source"] = "profiles/hbm_traffic.txt (rocprofv3 --pmc, calibrated)"
+    elif "hbm_traffic_stale" in head:
+        line["roofline"]["traffic_stale"] = True
     if "cpu" in head:
         line["cpu_baseline"] = {
             "value": head["cpu"]["GBps"], "unit": "GB/s", "cores": 1, "kind": "port",

@@ -308,8 +308,12 @@ static __device__ __forceinline__ void dr_philox_block(dr_u64 k0, dr_u64 k1, dr_
     x[3] = c3 + carry;
 #pragma unroll
     for (int round = 0; round < 10; ++round) {
-        const dr_u64 hi0 = dr_mulhi64(0xD2E7470EE14C6C93ULL, x[0]), lo0 = 0xD2E7470EE14C6C93ULL * x[0];
-        const dr_u64 hi1 = dr_mulhi64(0xCA5A826395121157ULL, x[2]), lo1 = 0xCA5A826395121157ULL * x[2];
+        /* one 128-bit product gives both halves (asked for separately, the low half is
+           multiplied out a second time) */
+        const unsigned __int128 p0 = (unsigned __int128)0xD2E7470EE14C6C93ULL * x[0];
+        const unsigned __int128 p1 = (unsigned __int128)0xCA5A826395121157ULL * x[2];
+        const dr_u64 hi0 = (dr_u64)(p0 >> 64), lo0 = (dr_u64)p0;
+        const dr_u64 hi1 = (dr_u64)(p1 >> 64), lo1 = (dr_u64)p1;
         x[0] = hi1 ^ x[1] ^ k0;
         x[2] = hi0 ^ x[3] ^ k1;
         x[1] = lo1;

@@ -420,7 +420,9 @@ int drhip_launch_scratch(void* func, unsigned grid_x, unsigned block_x, unsigned
     unsigned char block[DRHIP_MAX_ARGS_BYTES];
     if (!args || args_bytes > sizeof block)
         return fail(DRHIP_EINVAL, "drhip_launch_scratch", "argument block missing or larger than DRHIP_MAX_ARGS_BYTES");
-    if (scratch_arg_offset % sizeof(void*) || scratch_arg_offset + sizeof(void*) > args_bytes)
+    // (compared without adding to the offset: an offset close to SIZE_MAX must not wrap)
+    if (scratch_arg_offset % sizeof(void*) || args_bytes < sizeof(void*) ||
+        scratch_arg_offset > args_bytes - sizeof(void*))
         return fail(DRHIP_EINVAL, "drhip_launch_scratch", "scratch pointer slot outside the argument block or misaligned");
     if (scratch_bytes > drhip_k_scratch_bytes())
         return fail(DRHIP_EINVAL, "drhip_launch_scratch", "request exceeds the static scratch array (drhip_scratch_bytes())");

@@ -126,10 +126,7 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         target = None
         if kwargs:
             out = kwargs.get("out")
-            if isinstance(out, tuple) and len(out) == 1 and out[0] is inputs[0]:
-                # `x += y`: like the reference, build a new node and let Python rebind x
-                kwargs = {k: v for k, v in kwargs.items() if k != "out"}
-            elif isinstance(out, tuple) and len(out) == 1 and isinstance(out[0], DelayArray):
+            if isinstance(out, tuple) and len(out) == 1 and isinstance(out[0], DelayArray):
                 # `np.multiply(a, b, out=c)`: the fused kernel writes straight into c
                 target = out[0]
                 kwargs = {k: v for k, v in kwargs.items() if k != "out"}
@@ -294,12 +291,19 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         (the reference evaluates it to a temporary first, delayarray.py:114-121)."""
         arr = self._force()
         # written to by hand, the result is an array in its own right from now on: it
-        # must not be recomputed (and the write lost) when one of its inputs changes
+        # must not be recomputed (and the write lost) when one of its inputs changes,
+        # the same expression built again must not find it (`b = a * 2; b[0] = 100;
+        # c = a * 2`: c is a new node), and a backend that walks through evaluated nodes
+        # stops here
         d = self.__dict__
-        if "_deps" in d:
+        if self.children:
             d.pop("_deps", None)
             d.pop("_plan", None)
             d.pop("_multi", None)
+            d["_cut"] = True
+            own = d.get("_key")
+            if own is not None and Memoiser._cache.get(own) is self:
+                Memoiser._cache.pop(own)
         key = _unwrap(key)
         if isinstance(item, DelayArray) and "array" not in item.__dict__:
             _backend.run_into(item, arr[key])
@@ -1147,6 +1151,7 @@ def evaluate(*arrays):
         results = _backend.run_multi(todo)
         for node, res in zip(todo, results):
             node.array = res
+            node._depth = 0     # a leaf of whatever is built on it from now on
     return arrays
 
 

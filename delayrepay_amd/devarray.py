@@ -264,9 +264,18 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
             dim += 1
         return self._view(shape, strides, offset)
 
+    def check_writable(self):
+        """A view that repeats elements (a stride of zero along an axis longer than one, as
+        `broadcast_to` makes them) is read-only, as in NumPy: one write would land on
+        every repeat and on the source."""
+        for d, s in zip(self.shape, self._strides):
+            if d > 1 and s == 0:
+                raise ValueError("assignment destination is read-only")
+
     def __setitem__(self, key, value):
         from . import hip
         dst = self[key]
+        dst.check_writable()
         hip.assign(dst, value)
 
     def broadcast_to(self, shape):

@@ -1295,6 +1295,7 @@ def _write(plan, dst):
 
 def run_into(ex, dst):
     """`dst[...] = ex` as one fused kernel writing the destination view directly."""
+    dst.check_writable()
     if not _FUSED:
         assign(dst, run(ex))
         return

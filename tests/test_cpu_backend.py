@@ -262,3 +262,29 @@ assert np.array_equal(np.any(z, axis=0, keepdims=True).get(), np.zeros((1, 4), b
 print("ok")
 """
     assert run_cpu(script).strip().endswith("ok")
+
+
+def test_a_result_written_to_by_hand_is_an_array_of_its_own():
+    """After `b = a * 2; b[0] = 100` the node of `a * 2` holds a value that is no longer
+    `a * 2`: the same expression built again is a new node, and what is built on `b` sees
+    the write (this backend walks through evaluated nodes; it must stop at this one)."""
+    script = r"""
+    import numpy as np
+    import delayrepay_amd as dr
+    a = dr.array(np.arange(5.0))
+    b = a * 2
+    b.run()
+    b[0] = 100.0
+    c = a * 2
+    assert c is not b and np.array_equal(c.get(), np.arange(5.0) * 2)
+    assert np.array_equal((b + 1).get(), np.array([101.0, 3, 5, 7, 9]))
+    # an explicit out= that is also the first operand writes into it
+    x = dr.array(np.arange(5.0)); y = dr.array(np.ones(5))
+    back = np.add(x, y, out=x)
+    assert back is x and np.array_equal(x.get(), np.arange(5.0) + 1)
+    # several results evaluated together are leaves of what is built on them
+    p, q = dr.evaluate(x * 3, x + 7)
+    assert p._depth == 0 and q._depth == 0
+    print("ok")
+    """
+    assert run_cpu(script).strip().endswith("ok")

@@ -513,3 +513,25 @@ def test_a_structure_met_before_keeps_its_plan_over_fresh_arrays():
         assert hip.STATS["seen_hits"] == seen
     finally:
         hip.set_tune(nts=1)
+
+
+def test_writes_by_hand_aliasing_out_and_stretched_views():
+    """The same program as on the CPU backend gives the same values here; a view that
+    repeats elements is read-only."""
+    import delayrepay_amd as dr
+    a = dr.array(np.arange(5.0))
+    b = a * 2
+    b.run()
+    b[0] = 100.0
+    c = a * 2
+    assert c is not b and np.array_equal(c.get(), np.arange(5.0) * 2)
+    assert np.array_equal((b + 1).get(), np.array([101.0, 3, 5, 7, 9]))
+    x, y = dr.array(np.arange(5.0)), dr.array(np.ones(5))
+    back = np.add(x, y, out=x)
+    assert back is x and np.array_equal(x.get(), np.arange(5.0) + 1)
+    wide = np.broadcast_to(dr.array(np.arange(4.0)), (3, 4))
+    assert np.array_equal(wide.get(), np.broadcast_to(np.arange(4.0), (3, 4)))
+    with pytest.raises(ValueError, match="read-only"):
+        wide[0, 0] = 5.0
+    with pytest.raises(ValueError, match="read-only"):
+        wide[...] = dr.array(np.ones((3, 4))) * 2.0

@@ -99,6 +99,10 @@ def test_launch_scratch_refuses_what_it_cannot_hold():
                                     len(args), 64) == 20002            # slot outside the block
     assert lib.drhip_launch_scratch(kern.func, low.grid, cg.BLOCK, 0, args, len(args), slot + 4,
                                     64) == 20002                       # misaligned slot
+    # an offset near the top of size_t must not wrap round the bound check (it is refused on
+    # the host; nothing is launched)
+    assert lib.drhip_launch_scratch(kern.func, low.grid, cg.BLOCK, 0, args, len(args),
+                                    ctypes.c_size_t(0xFFFFFFFFFFFFFFF8), 64) == 20002
     huge = ctypes.create_string_buffer(8192)
     assert lib.drhip_launch_scratch(kern.func, low.grid, cg.BLOCK, 0, huge, 8192, 0, 64) == 20002
 
