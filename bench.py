@@ -613,9 +613,13 @@ def main():
             hip.set_tune(cache_mib=200, ntl_mib=320)
             hip.set_fused(False)
             try:
-                l0 = hip.STATS["launches"]
+                l0, k0 = hip.STATS["launches"], hiprt.counters()
+                t0 = time.perf_counter()
                 ring[0] = steps[0]()
                 hiprt.sync()
+                # first call: every node's kernel compiled, as one translation unit
+                res["unfused_first_call_ms"] = round((time.perf_counter() - t0) * 1e3, 2)
+                res["unfused_compile_ms"] = round((hiprt.counters()["compile_ns"] - k0["compile_ns"]) / 1e6, 2)
                 res["unfused_kernels"] = hip.STATS["launches"] - l0
                 ring[0] = steps[0]()
                 hiprt.sync()

@@ -305,6 +305,9 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
             if own is not None and Memoiser._cache.get(own) is self:
                 Memoiser._cache.pop(own)
         key = _unwrap(key)
+        check = getattr(arr, "check_writable", None)
+        if check is not None:
+            check()             # a stretched view is read-only as a whole, as in NumPy
         if isinstance(item, DelayArray) and "array" not in item.__dict__:
             _backend.run_into(item, arr[key])
         else:

@@ -274,8 +274,8 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
 
     def __setitem__(self, key, value):
         from . import hip
+        self.check_writable()
         dst = self[key]
-        dst.check_writable()
         hip.assign(dst, value)
 
     def broadcast_to(self, shape):

@@ -655,8 +655,68 @@ def _partials(nbytes):
     return hiprt.malloc(nbytes), False
 
 
+_DEFER = None         # a list while launches are being collected (`_together`)
+
+
+def _compile_together(entries):
+    """Kernels that the collected launches need and that are not compiled yet, as ONE
+    translation unit: the run-time compiler's fixed cost (120-190 ms here, whatever the
+    kernel) is then paid once, not once per kernel.  The un-fused mode needs 46 kernels
+    for Black-Scholes (cf. the reference's compile per evaluation, cuda.py:35-43)."""
+    todo = {}
+    for plan, _, reduce_out in entries:
+        for low, kern, fin in ((plan.low, plan.kern, reduce_out is not None and plan.second is None),
+                               (plan.second, plan.kern2, False)):
+            if low is not None and kern is None and low.key not in _KERNELS:
+                todo.setdefault(low.key, (low, fin))
+    if len(todo) < 2:
+        return
+    parts, names = [], []
+    for i, (low, fin) in enumerate(todo.values()):
+        source, name = _source(low)
+        # every kernel's source is complete in itself: its own namespace, and the macros
+        # that differ from kernel to kernel start afresh
+        parts.append("#undef DR_TAB_PTR\n#undef DR_LOG_TAB\n#undef DR_ERF_TAB\n#undef DR_STAGE_TABLES\n"
+                     f"namespace dr_unit_{i} {{\n{source}\n}}\n")
+        names.append((low, name, fin, source))
+    module = _load_or_compile("".join(parts))
+    for low, name, fin, source in names:
+        kern = Kernel()
+        kern.source = source
+        kern.func = hiprt.get_function(module, name)
+        kern.finalize = hiprt.get_function(module, name + "_fin") if fin else None
+        kern.packer = struct.Struct(low.fmt)
+        _KERNELS[low.key] = kern
+
+
+class _together:
+    """Context: the launches inside are collected, their kernels compiled in one go, then
+    issued in order."""
+
+    def __enter__(self):
+        global _DEFER
+        self.outer = _DEFER
+        if _DEFER is None:
+            _DEFER = []
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        global _DEFER
+        if self.outer is not None:       # nested: the outermost context issues everything
+            return False
+        entries, _DEFER = _DEFER, None
+        if exc_type is None:
+            _compile_together(entries)
+            for plan, out_ptrs, reduce_out in entries:
+                _fire(plan, out_ptrs, reduce_out)
+        return False
+
+
 def _fire(plan, out_ptrs, reduce_out=None):
     """Compile on first use, pack the argument block, launch."""
+    if _DEFER is not None:
+        _DEFER.append((plan, out_ptrs, reduce_out))
+        return
     low = plan.low
     kern = plan.kern
     if kern is None:
@@ -1114,7 +1174,8 @@ def run(ex):
     """Evaluate one DAG root; returns a new device array owned by the caller
     (cf. cuda.py:91-96)."""
     if not _FUSED:
-        return _run_unfused(ex, {})
+        with _together():
+            return _run_unfused(ex, {})
     d = ex.__dict__
     plan = d.get("_plan")
     if plan is None or not plan.valid():
@@ -1159,7 +1220,9 @@ def run_multi(exs):
     """Evaluate several roots; roots of equal shape share one kernel (and their
     common sub-expressions)."""
     if not _FUSED:
-        return [run(ex) for ex in exs]
+        with _together():       # one kernel per node, a node shared by two roots once
+            evaluated = {}
+            return [_run_unfused(ex, evaluated) for ex in exs]
     by_shape = {}
     for i, ex in enumerate(exs):
         by_shape.setdefault(tuple(ex.shape), []).append(i)

@@ -331,8 +331,10 @@ class TestSurface:
         with pytest.raises(ValueError):
             np.add(a, b, out=array(np.zeros((5, 9))))
         x = array(a0.copy())
-        y = np.add(x, 1.0, out=x)                  # the destination is an operand: a new node,
-        assert y is not x and np.array_equal(y.get(), a0 + 1)    # as for `x += 1` (delayarray.py:46-61)
+        y = np.add(x, 1.0, out=x)                  # the destination is an operand: written in place,
+        assert y is x and np.array_equal(x.get(), a0 + 1)        # as NumPy does (`x += 1` rebinds x
+        x += 1.0                                                 # to a new node, delayarray.py:46-61)
+        assert np.array_equal(x.get(), a0 + 2)
 
     def test_a_write_into_an_evaluated_expression_survives(self):
         x0 = np.arange(8.0)
