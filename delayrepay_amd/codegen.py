@@ -129,6 +129,10 @@ _FLOAT_FUNCS2 = {
     "power": "pow", "arctan2": "atan2", "hypot": "hypot", "copysign": "copysign",
     "fmod": "fmod", "fmax": "fmax", "fmin": "fmin",
 }
+# functions whose results carry a rounding error of their own (about an ulp)
+_INEXACT = frozenset(("sin", "cos", "tan", "arcsin", "arccos", "arctan", "sinh", "cosh", "tanh", "exp",
+                      "exp2", "expm1", "log", "log2", "log10", "log1p", "cbrt", "erf", "erfc", "power",
+                      "arctan2", "hypot"))
 _INFIX = {"add": "+", "subtract": "-", "multiply": "*", "divide": "/", "true_divide": "/"}
 _COMPARE = {"greater": ">", "less": "<", "greater_equal": ">=", "less_equal": "<=",
             "equal": "==", "not_equal": "!="}
@@ -367,9 +371,10 @@ class Program:
     roots    list of (ref, dtype code)
     """
 
-    __slots__ = ("leaves", "scalars", "ops", "roots", "own_math", "own_math32", "uses_index")
+    __slots__ = ("leaves", "scalars", "ops", "roots", "own_math", "own_math32", "uses_index",
+                 "soft_div")
 
-    def __init__(self, leaves, scalars, ops, roots, own_math=True, own_math32=True):
+    def __init__(self, leaves, scalars, ops, roots, own_math=True, own_math32=True, soft_div=True):
         self.leaves = tuple(leaves)
         self.scalars = tuple(scalars)
         self.ops = tuple(ops)
@@ -384,9 +389,32 @@ class Program:
             if own_math32 else ()
         # these operations read the element index: only the flat kernel supplies it
         self.uses_index = any(name in INDEX_OPS for name, _, _, _ in self.ops)
+        self.soft_div = self._quotients_nobody_sees() if soft_div and own_math else ()
+
+    def _quotients_nobody_sees(self):
+        """float64 divisions whose result reaches a root only through functions that round
+        on their own (`log(S / K)`, `erf(d / s)`): their last bit cannot be seen in any
+        result beyond what those functions' own error already hides, so they may be
+        computed to within one ulp instead of correctly rounded (`mathlib.DIV_F8`).  A
+        quotient that a root can see through exact operations alone (+ - * /, sqrt, the
+        selections, the reductions) stays the correctly rounded one: expressions of those
+        remain equal to NumPy's to the bit."""
+        seen = [False] * len(self.ops)      # visible at a root through exact operations only
+        for (kind, j), _ in self.roots:
+            if kind == "v":
+                seen[j] = True
+        for i in range(len(self.ops) - 1, -1, -1):
+            name = self.ops[i][0]
+            if seen[i] and name not in _INEXACT:
+                for kind, j in self.ops[i][3]:
+                    if kind == "v":
+                        seen[j] = True
+        return tuple(i for i, (name, cdt, _, _) in enumerate(self.ops)
+                     if name in ("divide", "true_divide") and cdt == "f8" and not seen[i])
 
     def key(self):
-        return (self.leaves, self.scalars, self.ops, self.roots, self.own_math, self.own_math32)
+        return (self.leaves, self.scalars, self.ops, self.roots, self.own_math, self.own_math32,
+                self.soft_div)
 
     def ref_dtype(self, ref):
         kind, i = ref
@@ -423,6 +451,8 @@ def _op_statement(prog, i):
         expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
     elif cdt == "f4" and name in prog.own_math32:
         expr = f"{mathlib32.FUNCTIONS[name][0]}({cargs[0]})"
+    elif i in prog.soft_div:
+        expr = f"dr_div_f8_1({cargs[0]}, {cargs[1]})"
     elif name == "where":    # the condition keeps its own type
         k, j = args[0]
         expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
@@ -440,7 +470,8 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=0, s
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
     uses_philox = any(name.startswith("philox") for name, _, _, _ in prog.ops)
-    lines = [mathlib.source(prog.own_math, lds=lds_tables, stage_loop=stage_loop) if with_math else "",
+    lines = [mathlib.source(prog.own_math, lds=lds_tables, stage_loop=stage_loop,
+                            soft_div=bool(prog.soft_div)) if with_math else "",
              mathlib32.source(prog.own_math32) if with_math else "",
              PHILOX if uses_philox and with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
@@ -504,6 +535,17 @@ def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"
             else:       # converted or broadcast argument: gather it first
                 lines.append(f"    {{ double t_[{P}]; {loop} t_[e] = {cargs[0]}; "
                              f"{mathlib.FUNCTIONS[name][0]}<{P}>(t_, v{i}); }}")
+            continue
+        if i in prog.soft_div:
+            gather = []
+            names = []
+            for pos, (k, j) in enumerate(args):
+                if prog.ref_dtype((k, j)) == "f8" and ref(k, j).endswith("[e]"):
+                    names.append(f"{k}{j}")
+                else:       # converted or broadcast operand: gather it first
+                    gather.append(f"double q{pos}_[{P}]; {loop} q{pos}_[e] = {cargs[pos]};")
+                    names.append(f"q{pos}_")
+            lines.append(f"    {{ {' '.join(gather)} dr_div_f8<{P}>({names[0]}, {names[1]}, v{i}); }}")
             continue
         if name == "cast":
             expr = cargs[0]
@@ -2388,7 +2430,8 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     block_row = G == BLOCK
     lanes = min(G, WAVE)
     per_wave = WAVE // lanes
-    src = [PREAMBLE, mathlib.source(prog.own_math), mathlib32.source(prog.own_math32)]
+    src = [PREAMBLE, mathlib.source(prog.own_math, soft_div=bool(prog.soft_div)),
+           mathlib32.source(prog.own_math32)]
 
     # one function per stage, one for the per-element roots, one for the per-row roots
     if keep is None:

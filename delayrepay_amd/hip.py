@@ -344,7 +344,8 @@ class Tracer(Visitor):
         self.iotas = []
 
     def program(self, roots):
-        return Program(self.leaf_codes, self.scalar_codes, self.ops, roots, TUNE["dmath"], TUNE["smath"])
+        return Program(self.leaf_codes, self.scalar_codes, self.ops, roots, TUNE["dmath"], TUNE["smath"],
+                       TUNE["softdiv"])
 
 
 # ---------------------------------------------------------------------------

@@ -53,6 +53,7 @@ DEVICE_MACROS = """\
 #define DR_TABLE static __device__ const
 #define DR_ALIGN16 __attribute__((aligned(16)))
 #define DR_RSQ64(x) __builtin_amdgcn_rsq(x)
+#define DR_RCP64(x) __builtin_amdgcn_rcp(x)
 #define DR_ANY_LANE(p) (__builtin_amdgcn_ballot_w64(p) != 0)
 /* p * z + k with the constant k in a scalar register pair.  The compiler prefers the
    two-address v_fmac_f64 for a Horner step and then copies every 64-bit constant into
@@ -73,6 +74,14 @@ static inline double dr_rsq64_host(double x)
     return ldexp((double)(float)mant, ex);
 }
 #define DR_RSQ64(x) dr_rsq64_host(x)
+/* a 24-bit estimate of 1/x, like the hardware's */
+static inline double dr_rcp64_host(double x)
+{
+    int ex;
+    const double mant = frexp(1.0 / x, &ex);
+    return ldexp((double)(float)mant, ex);
+}
+#define DR_RCP64(x) dr_rcp64_host(x)
 #define DR_ANY_LANE(p) (p)
 #define DR_FMA_K(p, z, k) __builtin_fma(p, z, k)
 """
@@ -615,6 +624,48 @@ DR_FN void dr_sqrt_f8(const double (&x)[P], double (&out)[P])
     }
 }"""
 
+DIV_F8 = r"""
+/* a / b for quotients that nothing reads but functions which round on their own
+   (log(a / b), erf(x / s)): the reciprocal estimate, two refinements, the product and
+   one correction by the exact residual, eight operations where the correctly rounded
+   division takes thirteen (it scales both operands first, so that no intermediate
+   result leaves the normal range, and fixes up the special cases afterwards).  The
+   result is the correctly rounded quotient except in about one case in 2^20, then the
+   neighbouring double (checked against exact quotients in tests/test_mathlib.py).
+   Operands that need the scaling or the special cases show in the result (not a normal
+   number: a NaN from 0 or infinity times its reciprocal, an infinity, a denormal, a zero,
+   whose sign the correction would lose) and take the compiler's division, on a path a
+   wave skips when none of its lanes needs it. */
+template <int P>
+DR_FN void dr_div_f8(const double (&a)[P], const double (&b)[P], double (&out)[P])
+{
+    bool rare = false;
+    _Pragma("unroll") for (int e = 0; e < P; ++e) {
+        double y = DR_RCP64(b[e]);
+        double t = __builtin_fma(-b[e], y, 1.0);
+        y = __builtin_fma(y, t, y);
+        t = __builtin_fma(-b[e], y, 1.0);
+        y = __builtin_fma(y, t, y);
+        double q = a[e] * y;
+        const double r = __builtin_fma(-b[e], q, a[e]);
+        q = __builtin_fma(r, y, q);
+        out[e] = q;
+        rare |= !__builtin_isnormal(q);
+    }
+    if (DR_ANY_LANE(rare)) {
+        _Pragma("unroll") for (int e = 0; e < P; ++e)
+            if (!__builtin_isnormal(out[e]))
+                out[e] = a[e] / b[e];
+    }
+}
+DR_FN double dr_div_f8_1(double a, double b)
+{
+    const double x[1] = {a}, y[1] = {b};
+    double r[1];
+    dr_div_f8<1>(x, y, r);
+    return r[0];
+}"""
+
 # ufunc name -> (device function template, sources it needs in order), float64 only
 FUNCTIONS = {
     "log": ("dr_log_f8", (STEP, LOG_TABLE, LOG_CORE, LOG_F8)),
@@ -661,7 +712,7 @@ DR_FN double {fn}_1(double x)
 """
 
 
-def source(names, macros=DEVICE_MACROS, lds=0, stage_loop=False):
+def source(names, macros=DEVICE_MACROS, lds=0, stage_loop=False, soft_div=False):
     """Definitions of the function templates for the ufuncs in `names` (each piece
     once) and of their one-element forms `<function>_1(double)`.  `lds`: the functions
     read their tables from LDS copies, which a kernel with blocks of `lds` threads makes
@@ -672,7 +723,7 @@ def source(names, macros=DEVICE_MACROS, lds=0, stage_loop=False):
             if piece not in pieces:
                 pieces.append(piece)
     if not pieces:
-        return ""
+        return macros + DIV_F8 if soft_div else ""
     tabs = tables(names)
     if lds and tabs:
         # Every lane first asks for all its 16-byte pieces of all tables and then writes
@@ -705,4 +756,4 @@ def source(names, macros=DEVICE_MACROS, lds=0, stage_loop=False):
     table_text = [p for p in pieces if p in (LOG_TABLE, ERF_TABLE)]
     rest = [p for p in pieces if p not in (LOG_TABLE, ERF_TABLE)]
     wrappers = "".join(SCALAR_WRAPPER.format(fn=FUNCTIONS[name][0]) for name in names)
-    return macros + "".join(table_text) + "\n" + where + "".join(rest) + wrappers
+    return macros + "".join(table_text) + "\n" + where + "".join(rest) + wrappers + (DIV_F8 if soft_div else "")

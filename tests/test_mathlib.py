@@ -20,7 +20,13 @@ def host(tmp_path_factory):
     """The device source built for the host with g++.  Arrays go through the 4-element
     pack (the form the kernels use) and the remainder through the 1-element form."""
     d = tmp_path_factory.mktemp("mathlib")
-    src = "#include <math.h>\n" + mathlib.source(sorted(mathlib.FUNCTIONS), mathlib.HOST_MACROS)
+    src = "#include <math.h>\n" + mathlib.source(sorted(mathlib.FUNCTIONS), mathlib.HOST_MACROS, soft_div=True)
+    src += ('extern "C" void v_div(const double* a, const double* b, double* y, long n)\n'
+            "{ long i = 0;\n"
+            "  for (; i + 4 <= n; i += 4) { const double p[4] = {a[i], a[i+1], a[i+2], a[i+3]}, "
+            "q[4] = {b[i], b[i+1], b[i+2], b[i+3]}; double r[4]; dr_div_f8<4>(p, q, r); "
+            "for (int e = 0; e < 4; e++) y[i+e] = r[e]; }\n"
+            "  for (; i < n; i++) y[i] = dr_div_f8_1(a[i], b[i]); }\n")
     for name, (fn, _) in mathlib.FUNCTIONS.items():
         src += (f'extern "C" void v_{name}(const double* x, double* y, long n)\n'
                 "{ long i = 0;\n"
@@ -32,7 +38,14 @@ def host(tmp_path_factory):
                     str(d / "m.cpp")], check=True)
     lib = ctypes.CDLL(str(d / "m.so"))
 
-    def call(name, x):
+    def call(name, x, other=None):
+        if name == "div":
+            a = np.ascontiguousarray(x, dtype=np.float64)
+            b = np.ascontiguousarray(other, dtype=np.float64)
+            y = np.empty_like(a)
+            lib.v_div(a.ctypes.data_as(ctypes.c_void_p), b.ctypes.data_as(ctypes.c_void_p),
+                      y.ctypes.data_as(ctypes.c_void_p), ctypes.c_long(a.size))
+            return y
         x = np.ascontiguousarray(x, dtype=np.float64)
         y = np.empty_like(x)
         getattr(lib, "v_" + name)(x.ctypes.data_as(ctypes.c_void_p),
@@ -378,3 +391,49 @@ def test_float32_device_source_compiles_to_the_hardware_functions():
         asm = open(f"{d}/k.s").read()
     assert len(re.findall(r"^\s+v_exp_f32", asm, re.M)) >= 2 and len(re.findall(r"^\s+v_log_f32", asm, re.M)) >= 1
     assert not re.findall(r"^\s+v_pk_\w+_f32", asm, re.M)
+
+
+def test_quotients_that_only_inexact_functions_read(host):
+    """`dr_div_f8` (eight operations instead of the correctly rounded division's thirteen):
+    the correctly rounded quotient nearly always, never more than one ulp from it; zero,
+    infinite, NaN, denormal and overflowing cases are NumPy's."""
+    rs = np.random.RandomState(11)
+    n = 1 << 20
+    a = np.concatenate([rs.uniform(-100, 100, n), np.exp(rs.uniform(-300, 300, n)) * rs.choice([-1, 1], n)])
+    b = np.concatenate([rs.uniform(0.1, 100, n) * rs.choice([-1, 1], n), np.exp(rs.uniform(-300, 300, n))])
+    got, ref = host("div", a, b), a / b
+    off = np.abs(got - ref) / np.spacing(np.abs(ref))
+    assert off.max() <= 1.0
+    assert np.count_nonzero(off) <= a.size // 50000         # measured: none in 2^21
+    with np.errstate(all="ignore"):
+        sa = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1.0, 0.0, np.inf, 1e308, 1e-308,
+                       5e-324, 1.0, 1e-320, 3.0, 1e300, -1e-300, 2.0, 7.0])
+        sb = np.array([1.0, 2.0, 0.0, -0.0, 2.0, -3.0, 1.0, np.nan, 0.0, np.inf, 1e-308, 1e308,
+                       2.0, 5e-324, 1e-320, np.inf, 1e-300, 1e300, 1e-310, 1.7976931348623157e308])
+        want = sa / sb
+    res = host("div", sa, sb)
+    assert np.array_equal(np.isnan(res), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(res[ok], want[ok]) and np.array_equal(np.signbit(res[ok]), np.signbit(want[ok]))
+    # one at a time and in packs: the same arithmetic
+    assert np.array_equal(host("div", a[:1001], b[:1001]),
+                          np.concatenate([host("div", a[i:i + 1], b[i:i + 1]) for i in range(1001)]))
+
+
+def test_only_quotients_that_no_root_can_see_are_computed_that_way():
+    from delayrepay_amd import codegen as cg
+    def soft(ops, roots):
+        return cg.Program(["f8", "f8"], [], ops, roots).soft_div
+    div = ("divide", "f8", "f8", (("l", 0), ("l", 1)))
+    log = lambda j: ("log", "f8", "f8", (("v", j),))
+    add = lambda i, j: ("add", "f8", "f8", (("v", i), ("v", j)))
+    assert soft([div, log(0)], [(("v", 1), "f8")]) == (0,)                       # log(a / b)
+    assert soft([div], [(("v", 0), "f8")]) == ()                                 # a / b itself
+    assert soft([div, log(0), add(0, 1)], [(("v", 2), "f8")]) == ()              # a / b + log(a / b)
+    assert soft([div, log(0)], [(("v", 1), "f8"), (("v", 0), "f8")]) == ()       # both are roots
+    assert soft([div, ("sqrt", "f8", "f8", (("v", 0),))], [(("v", 1), "f8")]) == ()      # sqrt is exact
+    assert soft([div, ("multiply", "f8", "f8", (("v", 0), ("l", 0))), ("erf", "f8", "f8", (("v", 1),))],
+                [(("v", 2), "f8")]) == (0,)                                      # erf(a / b * a)
+    assert soft([("divide", "f4", "f4", (("l", 0), ("l", 1))), ("log", "f4", "f4", (("v", 0),))],
+                [(("v", 1), "f4")]) == ()                                        # float32: untouched
+    assert cg.Program(["f8", "f8"], [], [div, log(0)], [(("v", 1), "f8")], soft_div=False).soft_div == ()
