@@ -389,13 +389,19 @@ class Program:
             if own_math32 else ()
         # these operations read the element index: only the flat kernel supplies it
         self.uses_index = any(name in INDEX_OPS for name, _, _, _ in self.ops)
-        self.soft_div = self._quotients_nobody_sees() if soft_div and own_math else ()
+        # float64 only: in float32 the short division (`mathlib32.DIV_F4`) with its branch for
+        # the rare cases measures slower than the compiler's branch-free sequence
+        # (Black-Scholes float32: 120 against 115 us); soft_div=2 asks for it all the same
+        self.soft_div = self._quotients_nobody_sees(("f8",) * bool(own_math)
+                                                    + ("f4",) * bool(own_math32 and soft_div == 2)) \
+            if soft_div else ()
 
-    def _quotients_nobody_sees(self):
-        """float64 divisions whose result reaches a root only through functions that round
+    def _quotients_nobody_sees(self, types):
+        """Divisions (in the float types `types`) whose result reaches a root only through functions that round
         on their own (`log(S / K)`, `erf(d / s)`): their last bit cannot be seen in any
         result beyond what those functions' own error already hides, so they may be
-        computed to within one ulp instead of correctly rounded (`mathlib.DIV_F8`).  A
+        computed to within one ulp instead of correctly rounded (`mathlib.DIV_F8`,
+        `mathlib32.DIV_F4`).  A
         quotient that a root can see through exact operations alone (+ - * /, sqrt, the
         selections, the reductions) stays the correctly rounded one: expressions of those
         remain equal to NumPy's to the bit."""
@@ -410,7 +416,7 @@ class Program:
                     if kind == "v":
                         seen[j] = True
         return tuple(i for i, (name, cdt, _, _) in enumerate(self.ops)
-                     if name in ("divide", "true_divide") and cdt == "f8" and not seen[i])
+                     if name in ("divide", "true_divide") and cdt in types and not seen[i])
 
     def key(self):
         return (self.leaves, self.scalars, self.ops, self.roots, self.own_math, self.own_math32,
@@ -452,7 +458,7 @@ def _op_statement(prog, i):
     elif cdt == "f4" and name in prog.own_math32:
         expr = f"{mathlib32.FUNCTIONS[name][0]}({cargs[0]})"
     elif i in prog.soft_div:
-        expr = f"dr_div_f8_1({cargs[0]}, {cargs[1]})"
+        expr = f"dr_div_f8_1({cargs[0]}, {cargs[1]})" if cdt == "f8" else f"dr_div_f4({cargs[0]}, {cargs[1]})"
     elif name == "where":    # the condition keeps its own type
         k, j = args[0]
         expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
@@ -470,9 +476,11 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=0, s
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
     uses_philox = any(name.startswith("philox") for name, _, _, _ in prog.ops)
+    soft8 = any(prog.ops[i][1] == "f8" for i in prog.soft_div)
+    soft4 = any(prog.ops[i][1] == "f4" for i in prog.soft_div)
     lines = [mathlib.source(prog.own_math, lds=lds_tables, stage_loop=stage_loop,
-                            soft_div=bool(prog.soft_div)) if with_math else "",
-             mathlib32.source(prog.own_math32) if with_math else "",
+                            soft_div=soft8) if with_math else "",
+             mathlib32.source(prog.own_math32, soft_div=soft4) if with_math else "",
              PHILOX if uses_philox and with_math else "",
              f"__device__ __forceinline__ void {fname}({', '.join(params)})", "{"]
     for i in range(len(prog.ops)):
@@ -535,6 +543,9 @@ def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"
             else:       # converted or broadcast argument: gather it first
                 lines.append(f"    {{ double t_[{P}]; {loop} t_[e] = {cargs[0]}; "
                              f"{mathlib.FUNCTIONS[name][0]}<{P}>(t_, v{i}); }}")
+            continue
+        if i in prog.soft_div and cdt == "f4":
+            lines.append(f"    {loop} v{i}[e] = dr_div_f4({cargs[0]}, {cargs[1]});")
             continue
         if i in prog.soft_div:
             gather = []
@@ -2430,8 +2441,9 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     block_row = G == BLOCK
     lanes = min(G, WAVE)
     per_wave = WAVE // lanes
-    src = [PREAMBLE, mathlib.source(prog.own_math, soft_div=bool(prog.soft_div)),
-           mathlib32.source(prog.own_math32)]
+    src = [PREAMBLE,
+           mathlib.source(prog.own_math, soft_div=any(prog.ops[i][1] == "f8" for i in prog.soft_div)),
+           mathlib32.source(prog.own_math32, soft_div=any(prog.ops[i][1] == "f4" for i in prog.soft_div))]
 
     # one function per stage, one for the per-element roots, one for the per-row roots
     if keep is None:

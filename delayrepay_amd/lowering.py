@@ -67,6 +67,7 @@ TUNE = {
     "t_cols": 0,      # output columns per tile (powers of two; 0: 128 bytes by 1 KB)
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
     "softdiv": 1,     # float64 quotients that only inexact functions read: to one ulp, 8 operations
+                      # (2: float32 quotients as well, 4 operations; measured slower)
     "rowfuse": 1,     # reductions along the last axis inside an expression: one kernel per row
     "row_lanes": 0,   # ... lanes per row (0: by the cost of idle lanes and of units per lane)
     "row_regs": 128,  # ... registers that may hold the row between stages (else it is loaded again)

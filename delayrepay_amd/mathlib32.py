@@ -27,12 +27,16 @@ DEVICE_MACROS = """\
 #define DR_FN4 static __device__ __forceinline__
 #define DR_EXP2F(x) __builtin_amdgcn_exp2f(x)
 #define DR_LOG2F(x) __builtin_amdgcn_logf(x)
+#define DR_RCPF(x) __builtin_amdgcn_rcpf(x)
+#define DR_ANY_LANE4(p) (__builtin_amdgcn_ballot_w64(p) != 0)
 """
 
 HOST_MACROS = """\
 #define DR_FN4 static inline
 #define DR_EXP2F(x) exp2f(x)
 #define DR_LOG2F(x) log2f(x)
+#define DR_RCPF(x) (1.0f / (x))
+#define DR_ANY_LANE4(p) (p)
 """
 
 EXP_F4 = r"""
@@ -89,6 +93,27 @@ DR_FN4 float dr_erf_f4(float x)
     return a >= 0.875f ? far : near;                        /* NaN takes `near` and stays NaN */
 }"""
 
+DIV_F4 = r"""
+/* a / b for quotients that nothing reads but functions which round on their own: the
+   hardware's reciprocal (1 ulp), the product and one correction by the exact residual,
+   four operations where the correctly rounded division takes ten and two changes of the
+   denormal mode.  Within one ulp of the exact quotient.  Whatever needs the long way
+   (zero, infinite, NaN, denormal or overflowing operands and results) shows as a result
+   that is not a normal number and takes the compiler's division, on a path that a wave
+   skips when none of its lanes needs it. */
+DR_FN4 float dr_div_f4(float a, float b)
+{
+    const float y = DR_RCPF(b);
+    float q = a * y;
+    const float r = __builtin_fmaf(-b, q, a);
+    q = __builtin_fmaf(r, y, q);
+    if (DR_ANY_LANE4(!__builtin_isnormal(q))) {
+        if (!__builtin_isnormal(q))
+            q = a / b;
+    }
+    return q;
+}"""
+
 # ufunc name -> (device function, sources it needs in order), float32 only
 FUNCTIONS = {
     "exp": ("dr_exp_f4", (EXP_F4,)),
@@ -97,11 +122,14 @@ FUNCTIONS = {
 }
 
 
-def source(names, macros=DEVICE_MACROS):
-    """Definitions of the functions for the ufuncs in `names`, each piece once."""
+def source(names, macros=DEVICE_MACROS, soft_div=False):
+    """Definitions of the functions for the ufuncs in `names`, each piece once (and of the
+    short division, when the program has quotients that qualify for it)."""
     pieces = []
     for name in names:
         for piece in FUNCTIONS[name][1]:
             if piece not in pieces:
                 pieces.append(piece)
+    if soft_div:
+        pieces.append(DIV_F4)
     return macros + "".join(pieces) if pieces else ""

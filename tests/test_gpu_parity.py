@@ -1556,3 +1556,47 @@ def test_device_random_numbers_fuse_without_memory_traffic():
     y = x[10:20] + 1.0
     want = ref.random(5000)
     assert np.array_equal(y.get(), want[10:20] + 1.0) and np.array_equal(x.get(), want)
+
+
+# ---- quotients that only inexact functions read ---------------------------------------------
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_quotients_inside_functions_and_quotients_that_are_results(dtype):
+    """`log(a / b)`: the quotient is computed the short way (within one ulp), the result
+    stays within the bar for functions; special operands give what NumPy gives.  The same
+    quotient asked for as a result as well is the correctly rounded one, to the bit."""
+    rs = np.random.RandomState(21)
+    n = 1 << 18
+    wide = 30 if dtype == np.float32 else 250
+    a = np.concatenate([rs.uniform(0.01, 100, n), np.exp(rs.uniform(-wide, wide, n))]).astype(dtype)
+    b = np.concatenate([rs.uniform(0.01, 100, n), np.exp(rs.uniform(-wide, wide, n))]).astype(dtype)
+    special = np.array([0.0, -0.0, 1.0, np.inf, np.nan, 5e-324 if dtype == np.float64 else 1e-45,
+                        np.finfo(dtype).max, np.finfo(dtype).tiny], dtype=dtype)
+    a = np.concatenate([a, np.repeat(special, special.size)])
+    b = np.concatenate([b, np.tile(special, special.size)])
+    da, db = dr.array(a), dr.array(b)
+    low, _ = hip.lower_only([np.log(da / db)])
+    assert low.key[1][-1] == ((0,) if dtype == np.float64 else ())     # the quotient is marked
+    with np.errstate(all="ignore"):
+        ref = np.log(a / b)
+        got = np.log(da / db).get()
+        assert np.array_equal(np.isnan(got), np.isnan(ref))
+        fin = np.isfinite(ref)
+        assert np.array_equal(got[~fin & ~np.isnan(ref)], ref[~fin & ~np.isnan(ref)])
+        # near log(1) = 0 one ulp of the quotient is many ulps of the logarithm, for NumPy's
+        # quotient as for this one: the bar is on the quotient's scale there
+        err = np.abs(got[fin].astype(np.float64) - ref[fin].astype(np.float64))
+        eps = float(np.finfo(dtype).eps)
+        bound = (2 if dtype == np.float32 else 450) * eps * np.maximum(np.abs(ref[fin]).astype(np.float64), 1.0)
+        assert np.all(err <= bound), float(np.max(err / bound))
+        q = da / db
+        lg = np.log(q)
+        dr.evaluate(lg, q)
+        assert bits_equal(q.get(), a / b)
+        both = np.log(da / db) + da / db           # seen through an addition: exact as well
+        want = ref + a / b
+        g2 = both.get()
+        ok = np.isfinite(want)
+        assert np.array_equal(np.isnan(g2), np.isnan(want))
+        tol = (4 if dtype == np.float32 else 900) * eps * np.maximum(np.abs(want[ok]).astype(np.float64), 1.0)
+        assert np.all(np.abs(g2[ok].astype(np.float64) - want[ok].astype(np.float64)) <= tol)

@@ -293,16 +293,25 @@ def host32(tmp_path_factory):
     special cases; the device's own 1-ulp versions are measured in the GPU tests."""
     from delayrepay_amd import mathlib32
     d = tmp_path_factory.mktemp("mathlib32")
-    src = "#include <math.h>\n" + mathlib32.source(sorted(mathlib32.FUNCTIONS), mathlib32.HOST_MACROS)
+    src = "#include <math.h>\n" + mathlib32.source(sorted(mathlib32.FUNCTIONS), mathlib32.HOST_MACROS,
+                                                   soft_div=True)
     for name, (fn, _) in mathlib32.FUNCTIONS.items():
         src += (f"void v_{name}(const float* x, float* y, long n)\n"
                 f"{{ for (long i = 0; i < n; i++) y[i] = {fn}(x[i]); }}\n")
+    src += ("void v_div(const float* a, const float* b, float* y, long n)\n"
+            "{ for (long i = 0; i < n; i++) y[i] = dr_div_f4(a[i], b[i]); }\n")
     (d / "m.c").write_text(src)
     subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
                     str(d / "m.c"), "-lm"], check=True)
     lib = ctypes.CDLL(str(d / "m.so"))
 
-    def call(name, x):
+    def call(name, x, other=None):
+        if name == "div":
+            a, b = (np.ascontiguousarray(v, dtype=np.float32) for v in (x, other))
+            y = np.empty_like(a)
+            lib.v_div(a.ctypes.data_as(ctypes.c_void_p), b.ctypes.data_as(ctypes.c_void_p),
+                      y.ctypes.data_as(ctypes.c_void_p), ctypes.c_long(a.size))
+            return y
         x = np.ascontiguousarray(x, dtype=np.float32)
         y = np.empty_like(x)
         getattr(lib, "v_" + name)(x.ctypes.data_as(ctypes.c_void_p),
@@ -434,6 +443,31 @@ def test_only_quotients_that_no_root_can_see_are_computed_that_way():
     assert soft([div, ("sqrt", "f8", "f8", (("v", 0),))], [(("v", 1), "f8")]) == ()      # sqrt is exact
     assert soft([div, ("multiply", "f8", "f8", (("v", 0), ("l", 0))), ("erf", "f8", "f8", (("v", 1),))],
                 [(("v", 2), "f8")]) == (0,)                                      # erf(a / b * a)
-    assert soft([("divide", "f4", "f4", (("l", 0), ("l", 1))), ("log", "f4", "f4", (("v", 0),))],
-                [(("v", 1), "f4")]) == ()                                        # float32: untouched
+    f4 = [("divide", "f4", "f4", (("l", 0), ("l", 1))), ("log", "f4", "f4", (("v", 0),))]
+    assert soft(f4, [(("v", 1), "f4")]) == ()                                    # float32: only on request
+    assert cg.Program(["f4", "f4"], [], f4, [(("v", 1), "f4")], soft_div=2).soft_div == (0,)
     assert cg.Program(["f8", "f8"], [], [div, log(0)], [(("v", 1), "f8")], soft_div=False).soft_div == ()
+
+
+def test_float32_quotients_that_only_inexact_functions_read(host32):
+    """`dr_div_f4`: within one ulp of the exact quotient (here with a correctly rounded
+    reciprocal standing in for the hardware's, which is within one ulp: the device build is
+    measured in the GPU tests), special cases as NumPy's."""
+    rs = np.random.RandomState(12)
+    n = 1 << 21
+    a = np.concatenate([rs.uniform(-100, 100, n), np.exp(rs.uniform(-40, 40, n))]).astype(np.float32)
+    b = np.concatenate([rs.uniform(0.1, 100, n) * rs.choice([-1, 1], n), np.exp(rs.uniform(-40, 40, n))]
+                       ).astype(np.float32)
+    got = host32("div", a, b)
+    exact = a.astype(np.float64) / b.astype(np.float64)
+    assert ulp32(got, exact).max() <= 1.0
+    with np.errstate(all="ignore"):
+        sa = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1.0, 0.0, np.inf, 1e38, 1e-38,
+                       1e-45, 1.0, 1e-40, 3.0, 1e30, -1e-30, 2.0], dtype=np.float32)
+        sb = np.array([1.0, 2.0, 0.0, -0.0, 2.0, -3.0, 1.0, np.nan, 0.0, np.inf, 1e-38, 1e38,
+                       2.0, 1e-45, 1e-40, np.inf, 1e-30, 1e30, 1e-39], dtype=np.float32)
+        want = sa / sb
+    res = host32("div", sa, sb)
+    assert np.array_equal(np.isnan(res), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(res[ok], want[ok]) and np.array_equal(np.signbit(res[ok]), np.signbit(want[ok]))
