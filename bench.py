@@ -92,7 +92,7 @@ def parse():
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
                          "dot | axis0 | axis1 | axis1_3d | matvec | rows200 | rowbcast | transpose | "
                          "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | softmax | "
-                         "layernorm | next (all "
+                         "layernorm | rowmax | strided | next (all "
                          "of these: the operations either side of the five configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
@@ -278,6 +278,15 @@ def main():
                         desc="a @ x f32 16384x16384 (the fused row reduction `@` builds)",
                         steps=[(lambda a=a: hip.run(ReduceEx(np.add, a * x, (1,)))) for a in mats],
                         cpu=lambda: ha[:N // 4] @ hx, cpu_frac=0.25, cpu_code="numpy.matmul")
+        if name == "strided":
+            n = 1 << 27
+            hx = rs.standard_normal(n).astype(np.float32)
+            vecs = [dr.array(hx) for _ in range(sets_for(6 * n))]
+            return dict(dtype="f32", n=n // 2, nbytes=4 * n,
+                        desc="x[::2] * 2 f32 n=2^27 (every second element: 8 B per result are needed, "
+                             "12 B are fetched and written, whole cache lines)",
+                        steps=[(lambda v=v: hip.run(v[::2] * 2.0)) for v in vecs],
+                        cpu=lambda: hx[:n // 4:2] * np.float32(2.0), cpu_frac=0.25, cpu_code="numpy.multiply")
         if name == "diff2":
             n = 1 << 27
             hx = rs.standard_normal(n).astype(np.float32)
@@ -656,7 +665,7 @@ def main():
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
              "next": ["dot", "axis0", "axis1", "axis1_3d", "matvec", "rows200", "rowbcast", "transpose",
                       "transpose3d", "interior", "diff2", "stencil9", "stencil3d", "grid", "rand",
-                      "softmax", "layernorm"]}.get(args.workload, [args.workload])
+                      "softmax", "layernorm", "rowmax", "strided"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:

@@ -84,6 +84,9 @@ typedef unsigned int u4x2u __attribute__((ext_vector_type(2), aligned(4)));
 typedef unsigned char u1x2u __attribute__((ext_vector_type(2), aligned(1)));
 typedef unsigned char u1x4u __attribute__((ext_vector_type(4), aligned(1)));
 typedef unsigned char u1x8u __attribute__((ext_vector_type(8), aligned(1)));
+// between accesses of one wave's lanes to the wave's own LDS: the hardware keeps them in order
+#define DR_WAVE_SYNC() do { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); \
+    __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront"); } while (0)
 """
 
 
@@ -351,7 +354,7 @@ def flat_elements(prog, leaf_class, out_dtypes, reduce_op):
     of its stretch once per vector: float32 x float64 68 % of the HBM peak, a mask beside
     two float32 operands 31 %); four when the program draws Philox numbers, whose blocks
     hold four outputs (a thread then makes each block once)."""
-    widths = [ITEMSIZE[dt] for dt, c in zip(prog.leaves, leaf_class) if c == "c"]
+    widths = [ITEMSIZE[dt] for dt, c in zip(prog.leaves, leaf_class) if c != "b"]
     if not reduce_op:
         widths += [ITEMSIZE[dt] for dt in out_dtypes]
     if any(name.startswith("philox") for name, _, _, _ in prog.ops):
@@ -656,11 +659,15 @@ def packs(prog, vec):
 
 
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
-              reduce_op=None, unaligned=False, one_run=False, stage_loop=False):
+              reduce_op=None, unaligned=False, one_run=False, stage_loop=False, exchange=True,
+              guard=False):
     """Contiguous 1-D kernel.
 
-    leaf_class  per leaf 'c' (contiguous, same length as the output) or 'b'
-                (single element broadcast to every position)
+    leaf_class  per leaf 'c' (contiguous, same length as the output), 'b' (single
+                element broadcast to every position) or 's2' .. 's8' (every k-th element
+                of a contiguous stretch: a thread loads the k vectors that hold its
+                elements and picks them out of the registers; the lines in between
+                are fetched whichever way the elements are read)
     vec         True: 16-byte vector accesses (all element types 4 or 8 bytes wide);
                 False: one element per access
     unaligned   some pointer is not 16-byte aligned: vectors at element alignment
@@ -670,16 +677,30 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                 n / elements per run blocks); without the loop over runs the compiler
                 needs fewer registers, and the block asks for its operands before it
                 copies the functions' tables into LDS, so one wait covers both
+    guard       the last vector of a strided operand would reach past its buffer's end:
+                the last few elements are left to the element-wise tail
+    exchange    outputs of which a lane holds several adjacent vectors (random numbers:
+                four doubles per lane) change lanes through LDS before they are stored
     """
     rs = "__restrict__ " if restrict else ""
     ua = "u" if unaligned else ""
+
+    def step_of(c):
+        return int(c[1:]) if c[0] == "s" else 1
+
+    def element(i, dt, c, e, tag):
+        """Element e of leaf i among the values a thread has loaded for one step."""
+        per, K = flat_vec(dt, E)[1], step_of(c)
+        if K > 1 and K >= per:
+            return f"L{i}_{e}{tag}"
+        return f"L{i}_{e * K // per}{tag}[{e * K % per}]"
     n_leaf, n_out = len(prog.leaves), len(out_dtypes)
     red_dt = out_dtypes[0] if reduce_op else None
     E = flat_elements(prog, leaf_class, out_dtypes, reduce_op) if vec else 1
     src = [PREAMBLE, emit_body(prog, out_dtypes, lds_tables=BLOCK, stage_loop=stage_loop)]
     packed = packs(prog, vec)
     if packed:
-        src.append(emit_body_packed(prog, out_dtypes, [c == "c" for c in leaf_class], E * unroll,
+        src.append(emit_body_packed(prog, out_dtypes, [c != "b" for c in leaf_class], E * unroll,
                                     group=E))
     if reduce_op:
         src.append(emit_block_reduce(reduce_op, red_dt))
@@ -698,6 +719,13 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     L.append(f"void dr_kernel({', '.join(params)})")
     L.append("{")
     staged = bool(mathlib.tables(prog.own_math))
+    xch = sorted({(ITEMSIZE[dt],) + flat_vec(dt, E)[::2] for dt in out_dtypes
+                  if flat_vec(dt, E)[2] > 1}) if packed and exchange and not reduce_op else []
+    for size, vt, chunks in xch:
+        L.append(f"    __shared__ {vt} dr_xch{size}[{BLOCK * chunks}];")
+    if xch:
+        L.append(f"    const int dr_lane = threadIdx.x & {WAVE - 1};")
+    exchange = bool(xch)
     if staged and not one_run:
         L.append("    DR_STAGE_TABLES();      // the functions' tables, from memory into LDS")
     for i, c in enumerate(leaf_class):
@@ -714,18 +742,28 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
         pad = " " * indent
         loads, work = [], []
         for i, (dt, c) in enumerate(zip(prog.leaves, leaf_class)):
-            if c != "c":
+            if c == "b":
                 continue
-            if vec:
+            K = step_of(c)
+            if vec and K > 1 and K >= flat_vec(dt, E)[1]:
+                # no vector would hold two of the thread's elements: element loads
+                for e in range(E):
+                    loads.append(f"{pad}const {CTYPE[dt]} L{i}_{e}{tag} = "
+                                 f"{_ld(nt_load, f'a{i} + (({idx}) * {E} + {e}) * {K}')};")
+            elif vec:
                 vt, per, chunks = flat_vec(dt, E)
                 vt += ua
+                chunks *= K
                 for ch in range(chunks):
+                    if not any((e * K) // per == ch for e in range(E)):
+                        continue        # a vector that holds none of the thread's elements
                     ptr = f"(const {vt}*)a{i} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
                         else f"(const {vt}*)a{i} + ({idx})"
                     loads.append(f"{pad}const {vt} L{i}_{ch}{tag} = {_ld(nt_load, ptr)};")
             else:
+                at = f"({idx}) * {K}" if K > 1 else f"({idx})"
                 loads.append(f"{pad}const {CTYPE[dt]} L{i}{tag} = "
-                             f"{_ld(nt_load, f'a{i} + ({idx})')};")
+                             f"{_ld(nt_load, f'a{i} + {at}')};")
         if vec and not reduce_op:
             for o, dt in enumerate(out_dtypes):
                 vt, per, chunks = flat_vec(dt, E)
@@ -737,8 +775,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                 if c == "b":
                     args.append(f"b{i}")
                 elif vec:
-                    per = flat_vec(dt, E)[1]
-                    args.append(f"L{i}_{e // per}{tag}[{e % per}]")
+                    args.append(element(i, dt, c, e, tag))
                 else:
                     args.append(f"L{i}{tag}")
             outs = [f"t{o}" for o in range(n_out)]
@@ -770,7 +807,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     # persistent blocks striding through memory.
     count = "nvec" if vec else "n"
     if vec:
-        L.append(f"    const long long nvec = n / {E};")
+        L.append(f"    const long long nvec = (n - {E}) / {E};" if guard else f"    const long long nvec = n / {E};")
     L.append(f"    const long long nchunk = {count} / {BLOCK * unroll};")
     if one_run:
         L.append("    if (blockIdx.x < nchunk) {")
@@ -796,9 +833,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
             if c == "b":
                 args.append(f"b{i}")
                 continue
-            per = flat_vec(dt, E)[1]
-            items = ", ".join(f"L{i}_{e // per}_u{u}[{e % per}]" for u in range(unroll)
-                              for e in range(E))
+            items = ", ".join(element(i, dt, c, e, f"_u{u}") for u in range(unroll) for e in range(E))
             all_work.append(f"{pad}const {CTYPE[dt]} P{i}[{P}] = {{{items}}};")
             args.append(f"P{i}")
         for o, dt in enumerate(out_dtypes):
@@ -812,9 +847,27 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                 continue
             for o, dt in enumerate(out_dtypes):
                 vt, per, chunks = flat_vec(dt, E)
+                idx = f"v + {u * BLOCK}" if u else "v"
+                if chunks > 1 and exchange:
+                    # A lane holds `chunks` adjacent vectors.  Stored as they are, every store
+                    # of the wave would write 16 bytes in every 16 * chunks; the lanes swap
+                    # vectors through the wave's own stretch of LDS instead, so that each
+                    # store covers 1 KB without gaps.  A wave's LDS accesses complete in
+                    # order; the fences keep the compiler from reordering them.
+                    xv = f"dr_xch{ITEMSIZE[dt]}"
+                    for ch in range(chunks):
+                        items = ", ".join(f"T{o}[{u * E + ch * per + k}]" for k in range(per))
+                        all_work.append(f"{pad}{{ const {vt} R = {{{items}}}; "
+                                        f"{xv}[threadIdx.x * {chunks} + {ch}] = R; }}")
+                    all_work.append(f"{pad}DR_WAVE_SYNC();")
+                    for ch in range(chunks):
+                        ptr = f"({vt + ua}*)o{o} + (({idx}) - dr_lane) * {chunks} + {ch * WAVE} + dr_lane"
+                        all_work.append(f"{pad}{{ const {vt} R = {xv}[(threadIdx.x - dr_lane) * {chunks} "
+                                        f"+ {ch * WAVE} + dr_lane]; {_st(nt_store, 'R', ptr)} }}")
+                    all_work.append(f"{pad}DR_WAVE_SYNC();")
+                    continue
                 for ch in range(chunks):
                     items = ", ".join(f"T{o}[{u * E + ch * per + k}]" for k in range(per))
-                    idx = f"v + {u * BLOCK}" if u else "v"
                     ptr = f"({vt + ua}*)o{o} + ({idx}) * {chunks} + {ch}" if chunks > 1 \
                         else f"({vt + ua}*)o{o} + ({idx})"
                     all_work.append(f"{pad}{{ const {vt} R = {{{items}}}; "
@@ -835,7 +888,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
             L.append("        DR_STAGE_TABLES();")
         L.append(f"        for (long long t = nchunk * {BLOCK * unroll * E} + (blockIdx.x - nchunk) * {BLOCK} "
                  f"+ threadIdx.x; t < n; t += (gridDim.x - nchunk) * {BLOCK}) {{")
-        args = [f"b{i}" if c == "b" else f"a{i}[t]" for i, c in enumerate(leaf_class)]
+        args = [f"b{i}" if c == "b" else f"a{i}[t * {step_of(c)}]" for i, c in enumerate(leaf_class)]
         args = (["t"] if prog.uses_index else []) + args
         decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
         outs = [f"t{o}" for o in range(n_out)]
@@ -854,7 +907,7 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
             # scalar tail: the last n % E elements, by the first threads of block 0
             L.append(f"    const long long t = nvec * {E} + (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
             L.append("    if (t < n) {")
-            args = [f"b{i}" if c == "b" else f"a{i}[t]" for i, c in enumerate(leaf_class)]
+            args = [f"b{i}" if c == "b" else f"a{i}[t * {step_of(c)}]" for i, c in enumerate(leaf_class)]
             args = (["t"] if prog.uses_index else []) + args
             decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
             outs = [f"t{o}" for o in range(n_out)]

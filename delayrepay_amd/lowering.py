@@ -77,6 +77,8 @@ TUNE = {
     "row_fence": 1,   # ... the compiler keeps the work of one 16-byte unit together
     "row_recompute": 1,   # ... per-element values are computed again by each stage, not kept
     "row_bpc": 0,     # ... blocks per compute unit at most (0: one pass, a block per set of rows)
+    "strided": 1,     # every k-th element of a vector: the flat kernel (0: the general one)
+    "xch": 1,         # a lane's adjacent output vectors change lanes through LDS before the store
     "stage_loop": 0,  # ... 1: the tables are copied by a loop (one trip to memory per 4 KB)
     "one_run": 1,     # flat kernels with tables in LDS: one run per block, no loop over runs
     "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
@@ -390,6 +392,12 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
 
     flat = ndim <= 1 and all(s == [1] or s == [0] or s == [] for s in m_leaf) \
         and all(s == [1] or s == [] for s in m_out)
+    if not flat and ndim == 1 and TUNE["strided"] and all(s == [1] for s in m_out) \
+            and all(len(s) == 1 and 0 <= s[0] <= 8 for s in m_leaf):
+        # Every k-th element of a vector (`a[::2]`): the flat kernel with the k vectors that
+        # hold a thread's elements loaded whole.  The general kernel computes an index per
+        # element and stores element by element.
+        flat = True
     if flat and ndim == 1 and not reduce_op and TUNE["lds"] and TUNE["svec"] and TUNE["row1d"] \
             and 4096 <= n < 2 ** 31 - 4096:
         # Shifted views of one vector (differences, 1-D stencils): every view would fetch the
@@ -418,12 +426,13 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         m_leaf = [[0 if st == [0] else far] + list(st) for st in m_leaf]
         m_out = [[far] + list(st) for st in m_out]
     if flat:
-        leaf_class = tuple("b" if (s == [0] and n > 1) else "c" for s in m_leaf)
+        leaf_class = tuple("b" if (s == [0] and n > 1) else f"s{s[0]}" if s and s[0] > 1 else "c"
+                           for s in m_leaf)
         ptrs = [a.ptr for a in leaves]
         # bytes (masks) move as vectors of sixteen; the wider operands beside them then take
         # four or eight vectors per thread
-        widths_ok = all(c in cg.VEC16 for c, k in zip(prog.leaves, leaf_class) if k == "c")
-        align_ok = all(p % 16 == 0 for p, k in zip(ptrs, leaf_class) if k == "c")
+        widths_ok = all(c in cg.VEC16 for c, k in zip(prog.leaves, leaf_class) if k != "b")
+        align_ok = all(p % 16 == 0 for p, k in zip(ptrs, leaf_class) if k != "b")
         if not reduce_op:
             widths_ok = widths_ok and all(c in cg.VEC16 for c in out_codes)
             align_ok = align_ok and all(p % 16 == 0 for p in out_ptrs)
@@ -438,7 +447,7 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             # 1 / 2 / 3 vectors 65.8 / 89.3 / 86.6; 384 blocks 81.6; 128 blocks 72.3.  dot of
             # two operands: 256 blocks x 2 / 4 vectors 77.5 / 89.5.  A body with many
             # operations per element needs more waves than that to keep the vector unit busy.
-            n_in = max(1, sum(c == "c" for c in leaf_class))
+            n_in = max(1, sum(c != "b" for c in leaf_class))
             cheap = {"floor", "ceil", "trunc", "rint", "copysign", "fmax", "fmin"}
             cost = sum(10 if (name in cg._FLOAT_FUNCS1 or name in cg._FLOAT_FUNCS2 or name in
                               ("divide", "true_divide", "reciprocal")) and name not in cheap else 1
@@ -469,13 +478,13 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             # loads and one store (SAXPY, 2^24) 76.3 / 78.9 / 78.8; three float64 loads and
             # two stores with a trivial body 75.0 / 77.6 / 78.8, with Black-Scholes' float32
             # body 73.2 / 73.5 / 71.7.
-            streams = sum(c == "c" for c in leaf_class) + len(out_codes)
+            streams = sum(c != "b" for c in leaf_class) + len(out_codes)
             unroll = 1 if streams <= 2 else 2
         if packed:
             # float64 functions evaluate a pack of elements in lock step: at least `pack`
             # elements per thread (a vector of doubles holds two)
             unroll = max(unroll, TUNE["pack"] // cg.flat_elements(prog, leaf_class, out_codes, reduce_op))
-        in_bytes = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k == "c")
+        in_bytes = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k != "b")
         footprint = in_bytes
         if not reduce_op:
             footprint += sum(n * cg.ITEMSIZE[c] for c in out_codes)
@@ -493,17 +502,23 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         # of four) and asks for its operands before it copies the tables, so that one wait
         # covers both.  Black-Scholes float64, 2^25 options: blocks that stay for eight runs
         # 241.8 us, one run per block with the tables copied first 279, this 233.8-236.8.
+        # the vectors of a strided operand may reach up to k - 1 elements past the last one
+        # used: where that is past the buffer's end the last vector step is left to the tail
+        guard = any(k[0] == "s" and a.offset + n * int(k[1:]) > a.buf.nbytes // a.dtype.itemsize
+                    for a, k in zip(leaves, leaf_class))
+        strided = any(k[0] == "s" for k in leaf_class)
         one_run = bool(mathlib.tables(prog.own_math) and vec and not reduce_op and TUNE["one_run"]
-                       and not TUNE["flat_cap"])
+                       and not TUNE["flat_cap"] and not strided)
         stage_loop = bool(TUNE["stage_loop"] and mathlib.tables(prog.own_math))
         low.kind = "flat"
         low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
-                   unroll, ntl, nts, ua, one_run, stage_loop)
+                   unroll, ntl, nts, ua, one_run, stage_loop, bool(TUNE["xch"]), guard)
 
         def emit():
             src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
                                   restrict=not in_place, reduce_op=reduce_op, unaligned=ua,
-                                  one_run=one_run, stage_loop=stage_loop)
+                                  one_run=one_run, stage_loop=stage_loop, exchange=bool(TUNE["xch"]),
+                                  guard=guard)
             return src
         low.emit = emit
         E = cg.flat_elements(prog, leaf_class, out_codes, reduce_op) if vec else 1

@@ -496,6 +496,45 @@ def test_flipped_views_are_read_as_reversed_vectors(dtype):
     assert np.array_equal((dr.array(m0)[:, ::-1] * dr.array(d0)).get(), m0[:, ::-1] * d0)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.uint8])
+def test_every_kth_element_of_a_vector_takes_the_flat_kernel(dtype):
+    """`a[::2]`, `a[1::3]`, `a[5:-3:4]`: the vectors that hold a thread's elements are loaded
+    whole and the elements picked out of the registers; lengths around the vector and run
+    sizes, views that end on the buffer's last element (the last vector is left to the
+    element-wise tail), strided beside dense operands, a reduction, a float64 result."""
+    rs = np.random.RandomState(47)
+    mk = (lambda n: rs.randint(0, 99, n).astype(dtype)) if np.dtype(dtype).kind in "iu" else \
+        (lambda n: rs.uniform(-1, 1, n).astype(dtype))
+    for n in (64, 1000, 4096, 8192, 100003, 1 << 20):
+        a0 = mk(n)
+        a = dr.array(a0)
+        for k in (2, 3, 4, 5, 8):
+            for lo in (0, 1, k - 1):
+                assert np.array_equal((a[lo::k] * 2).get(), a0[lo::k] * 2), (n, k, lo)
+            low = hip.lower_only(a[::k] * 3)[0]          # not yet evaluated
+            assert low.kind == "flat" and low.key[2] == (f"s{k}",), (n, k)
+        m = a0[::2].size
+        b0 = mk(m)
+        assert np.array_equal((a[::2] + dr.array(b0)).get(), a0[::2] + b0), n
+        assert np.array_equal((a[1::2] - a[::2][:a0[1::2].size]).get(), a0[1::2] - a0[::2][:a0[1::2].size]), n
+        assert np.array_equal((a[5:-3:4] * 3).get(), a0[5:-3:4] * 3), n
+        d0 = rs.uniform(-1, 1, m)
+        assert np.array_equal((a[::2] * dr.array(d0)).get(), a0[::2] * d0), n
+    a0 = mk(1 << 16)
+    a = dr.array(a0)
+    # the view's last vector would end past the buffer: left to the tail
+    assert hip.lower_only(a[1::2] * 2)[0].key[-1] is True
+    assert hip.lower_only(a[::2] * 2)[0].key[-1] is False
+    got, want = dr.sum(a[::2] * a[1::2]), np.sum(a0[::2] * a0[1::2])
+    if np.dtype(dtype).kind == "f":
+        assert abs(float(got) - float(want)) <= 1e-5 * (1 << 15)
+    else:
+        assert int(got) == int(want)
+    m0 = mk(300 * 64).reshape(300, 64)
+    assert np.array_equal((dr.array(m0)[:, ::2] * 2).get(), m0[:, ::2] * 2)     # rows merge: one stride
+    assert np.array_equal((dr.array(m0)[:, 1::3] * 2).get(), m0[:, 1::3] * 2)   # they do not: general kernel
+
+
 def test_boundary_change_between_sweeps_is_seen():
     """The ping-pong copy is refreshed when something else writes the buffer."""
     u0 = np.zeros((20, 24), np.float32)
