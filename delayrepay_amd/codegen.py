@@ -660,7 +660,7 @@ def packs(prog, vec):
 
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,
               reduce_op=None, unaligned=False, one_run=False, stage_loop=False, exchange=True,
-              guard=False):
+              guard=False, runs=1):
     """Contiguous 1-D kernel.
 
     leaf_class  per leaf 'c' (contiguous, same length as the output), 'b' (single
@@ -677,6 +677,8 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
                 n / elements per run blocks); without the loop over runs the compiler
                 needs fewer registers, and the block asks for its operands before it
                 copies the functions' tables into LDS, so one wait covers both
+    runs        with `one_run`: a block handles this many adjacent runs one after the other
+                (straight-line code, no loop) and copies the tables once for all of them
     guard       the last vector of a strided operand would reach past its buffer's end:
                 the last few elements are left to the element-wise tail
     exchange    outputs of which a lane holds several adjacent vectors (random numbers:
@@ -808,10 +810,16 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     count = "nvec" if vec else "n"
     if vec:
         L.append(f"    const long long nvec = (n - {E}) / {E};" if guard else f"    const long long nvec = n / {E};")
-    L.append(f"    const long long nchunk = {count} / {BLOCK * unroll};")
+    if one_run and runs > 1:
+        L.append(f"    const long long nchunk = {count} / {BLOCK * unroll * runs} * {runs};")
+        L.append(f"    const long long nblk = nchunk / {runs};")
+    else:
+        L.append(f"    const long long nchunk = {count} / {BLOCK * unroll};")
+        if one_run:
+            L.append("    const long long nblk = nchunk;")
     if one_run:
-        L.append("    if (blockIdx.x < nchunk) {")
-        L.append("        const long long c = blockIdx.x;")
+        L.append("    if (blockIdx.x < nblk) {")
+        L.append(f"        const long long c = blockIdx.x * {runs}LL;")
     else:
         L.append("    for (long long c = blockIdx.x; c < nchunk; c += gridDim.x) {")
     L.append(f"        const long long v = c * {BLOCK * unroll} + threadIdx.x;")
@@ -876,6 +884,10 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
     if staged and one_run:
         L.append("        DR_STAGE_TABLES();      // after the loads: both are in flight together")
     L += all_work
+    for r in range(1, runs if one_run else 1):
+        L.append(f"        {{ const long long v = (c + {r}) * {BLOCK * unroll} + threadIdx.x;")
+        L += all_loads + all_work
+        L.append("        }")
     L.append("    }")
     # what is left over (less than one chunk) is spread over the first blocks; with one run
     # per block it belongs to the blocks behind the last run (code that follows the main
@@ -886,8 +898,8 @@ def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, rest
         L.append("    else {")
         if staged:
             L.append("        DR_STAGE_TABLES();")
-        L.append(f"        for (long long t = nchunk * {BLOCK * unroll * E} + (blockIdx.x - nchunk) * {BLOCK} "
-                 f"+ threadIdx.x; t < n; t += (gridDim.x - nchunk) * {BLOCK}) {{")
+        L.append(f"        for (long long t = nchunk * {BLOCK * unroll * E} + (blockIdx.x - nblk) * {BLOCK} "
+                 f"+ threadIdx.x; t < n; t += (gridDim.x - nblk) * {BLOCK}) {{")
         args = [f"b{i}" if c == "b" else f"a{i}[t * {step_of(c)}]" for i, c in enumerate(leaf_class)]
         args = (["t"] if prog.uses_index else []) + args
         decl = " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes))
@@ -2454,7 +2466,8 @@ def row_vector(prog, leaf_kind, out_dtypes, out_uniform):
 
 
 def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt_store=False,
-                   fence=True, recompute=True, pipeline=True, carry_values=True, wave_map=False):
+                   fence=True, recompute=True, pipeline=True, carry_values=True, wave_map=False,
+                   nt_load=False):
     """Rows that are reduced and used again: `a - max(a, axis=-1)`, softmax, the variance,
     layer normalisation.  A group of G lanes (8..64: part of a wave; 256: the block) owns a
     row of R elements (a compile-time constant, unit stride); lane j takes the 16-byte
@@ -2606,7 +2619,9 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
             # a pointer that is the same for the wave plus a lane's unsigned 32-bit offset:
             # the load then takes its address from a scalar register pair and one vector
             # register, instead of a vector register pair per unit of the row
-            ld = f"*(const {vt}*)(({base}{i} + {lo * V}) + usub * {V}u)"
+            # (an operand that stays in registers is read once: past the caches, `nt_load`)
+            ld = _ld(nt_load and V > 1 and i in kept,
+                     f"(const {vt}*)(({base}{i} + {lo * V}) + usub * {V}u)")
             if whole == "" and declare:
                 const = "" if i in carried_leaves else "const "
                 out.append(f"{pad}{const}{vt} X{j}_{i} = {ld};")

@@ -78,6 +78,8 @@ TUNE = {
     "row_recompute": 1,   # ... per-element values are computed again by each stage, not kept
     "row_bpc": 0,     # ... blocks per compute unit at most (0: one pass, a block per set of rows)
     "strided": 1,     # every k-th element of a vector: the flat kernel (0: the general one)
+    "table_runs": 1,  # ... and takes this many adjacent runs, one after the other
+    "row_ntl": 1,     # row kernels read the operands they keep in registers past the caches
     "xch": 1,         # a lane's adjacent output vectors change lanes through LDS before the store
     "stage_loop": 0,  # ... 1: the tables are copied by a loop (one trip to memory per 4 KB)
     "one_run": 1,     # flat kernels with tables in LDS: one run per block, no loop over runs
@@ -334,6 +336,7 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     footprint = sum(a.nbytes for a in leaves) + sum(K * (1 if u else R) * cg.ITEMSIZE[c]
                                                    for c, u in zip(out_codes, row_out))
     nts = bool(TUNE["nts"]) and footprint > TUNE["cache_mib"] << 20
+    ntl = bool(TUNE["ntl"]) and bool(TUNE["row_ntl"]) and sum(a.nbytes for a in leaves) > TUNE["ntl_mib"] << 20
     low = Lowered()
     low.lds = 0
     low.fin_count = 0
@@ -343,12 +346,12 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     carry = bool(TUNE["row_carry"])
     wmap = G == cg.BLOCK and (steps >= 12 if TUNE["row_wavemap"] < 0 else bool(TUNE["row_wavemap"]))
     low.key = ("rows", prog.key(), tuple(kinds), tuple(out_codes), low.row_out, R, G, keep, nts,
-               fence, recompute, pipe, carry, wmap)
+               fence, recompute, pipe, carry, wmap, ntl)
 
     def emit():
         return cg.emit_row_fused(prog, kinds, out_codes, row_out, R, G, keep=keep, nt_store=nts,
                                  fence=fence, recompute=recompute, pipeline=pipe, carry_values=carry,
-                                 wave_map=wmap)
+                                 wave_map=wmap, nt_load=ntl)
     low.emit = emit
     if G == cg.BLOCK:
         blocks = K
@@ -510,15 +513,16 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         one_run = bool(mathlib.tables(prog.own_math) and vec and not reduce_op and TUNE["one_run"]
                        and not TUNE["flat_cap"] and not strided)
         stage_loop = bool(TUNE["stage_loop"] and mathlib.tables(prog.own_math))
+        runs = max(1, TUNE["table_runs"]) if one_run else 1
         low.kind = "flat"
         low.key = ("flat", prog.key(), leaf_class, tuple(out_codes), vec, reduce_op, in_place,
-                   unroll, ntl, nts, ua, one_run, stage_loop, bool(TUNE["xch"]), guard)
+                   unroll, ntl, nts, ua, one_run, stage_loop, bool(TUNE["xch"]), guard, runs)
 
         def emit():
             src, _ = cg.emit_flat(prog, leaf_class, out_codes, vec, unroll, ntl, nts,
                                   restrict=not in_place, reduce_op=reduce_op, unaligned=ua,
                                   one_run=one_run, stage_loop=stage_loop, exchange=bool(TUNE["xch"]),
-                                  guard=guard)
+                                  guard=guard, runs=runs)
             return src
         low.emit = emit
         E = cg.flat_elements(prog, leaf_class, out_codes, reduce_op) if vec else 1
@@ -529,8 +533,8 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
             # several chunks
             cap = min(cap, TUNE["table_blocks"])
         if one_run:     # block c takes run c; one more block takes what is left over
-            runs = (n // E) // (cg.BLOCK * unroll)
-            low.grid = runs + (1 if n % (E * cg.BLOCK * unroll) else 0)
+            whole = (n // E) // (cg.BLOCK * unroll * runs)
+            low.grid = whole + (1 if n % (E * cg.BLOCK * unroll * runs) else 0)
         else:
             low.grid = min(chunks, cap)
         n_out_ptr = 1 if reduce_op else len(out_ptrs)
