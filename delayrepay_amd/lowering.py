@@ -279,6 +279,55 @@ def _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_pt
     return low
 
 
+def _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V):
+    """Lanes per row for the row kernel: the candidate with the least estimated time per
+    row.  The estimate has a memory term and an arithmetic term, fitted to measurements on
+    MI355X (`a - max(a)` and softmax, float32 and float64, rows of 16 to 4096 elements,
+    every candidate; the choice is within 2 points of the best candidate in all but one of
+    those 38 cases):
+
+    memory      a wave's load covers `min(lanes, units) * 16` contiguous bytes of a row.  Rows
+                whose pitch is no multiple of 128 bytes start inside a cache line, so a short
+                stretch touches one line more than it fills (rows of 300 float32, percent of
+                the HBM peak with 8 / 16 / 32 / 64 lanes: 44 / 62 / 68 / 77), and a stretch
+                below 128 bytes never fills the line it touches (rows of 32 float32 with 2
+                lanes of 4 units each: 23); more than four units per lane cost a little, and
+                so does a single one;
+    arithmetic  idle lanes of the last step and the butterfly (log2 lanes steps per
+                reduction, spread over a lane's units) take issue slots that the body needs:
+                softmax on rows of 128 float32 with 8 / 16 / 32 lanes: 77 / 75 / 66, on rows
+                of 300 with 16 / 32 / 64 lanes: 57 / 68 / 59.
+    A block per row pays only from 512 units on (rows of 1024 float32: 64 lanes 79 / 78,
+    a block 76 / 63)."""
+    units = -(-R // V)
+    pitches = [st * a.dtype.itemsize for a, k, st in zip(leaves, kinds, sk) if k == "v" and st]
+    pitches += [R * cg.ITEMSIZE[c] for c, u in zip(out_codes, row_out) if not u]
+    extra = 0 if all(p % 128 == 0 for p in pitches) else 32 if all(p % 64 == 0 for p in pitches) else 96
+    dense = all(st == R for k, st in zip(kinds, sk) if k == "v" and st)
+    moved = sum(a.dtype.itemsize for a, k, st in zip(leaves, kinds, sk) if k == "v" and st) \
+        + sum(cg.ITEMSIZE[c] for c, u in zip(out_codes, row_out) if not u)
+    work = sum(10 if (name in cg._FLOAT_FUNCS1 or name in cg._FLOAT_FUNCS2 or name in
+                      ("divide", "true_divide", "reciprocal")) else 1 for name, _, _, _ in prog.ops)
+    if any(cdt == "f8" for _, cdt, _, _ in prog.ops):
+        work *= 2
+    ratio = 0.26 * work / max(moved, 1)
+    best = None
+    for lanes in (1, 2, 4, 8, 16, 32, 64, cg.BLOCK):
+        n = -(-units // lanes)
+        if n > cg.ROW_STEPS_MAX:
+            continue
+        # what one load of a wave covers without a gap: a lane group's stretch of its row
+        # or, with one unit per lane and rows that follow each other, the wave's 1 KB
+        piece = 1024 if n == 1 and dense else min(lanes, units) * 16
+        t_mem = max(128, piece + extra) / piece / (0.95 if n == 1 else 1.0 if n <= 4 else 0.97 if n <= 8 else 0.88)
+        butterfly = 8 if lanes == cg.BLOCK else lanes.bit_length() - 1
+        t_alu = ratio * lanes * n / units * (1 + 0.15 * butterfly / n)
+        t = max(t_mem, t_alu) + 0.25 * min(t_mem, t_alu)
+        if best is None or t < best[0]:
+            best = (t, lanes)
+    return best[1] if best else cg.BLOCK
+
+
 def lower_rows(prog, leaves, scalars, shape, out_codes):
     """Expression with reductions along its last axis inside it (`codegen.emit_row_fused`):
     every row is read once, reduced, used again and written once.  `shape` is the shape the
@@ -311,20 +360,7 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     units = -(-R // V)
     G = TUNE["row_lanes"]
     if not G:
-        # Lanes per row: few units per lane (a lane with one load in flight per row keeps
-        # more rows in flight per wave), but no group much wider than its row (rows of 100
-        # units on a block of 256 lanes leave 60 % of them idle and pay for barriers).
-        best = None
-        for lanes in (8, 16, 32, 64, cg.BLOCK):
-            n = -(-units // lanes)
-            if n > cg.ROW_STEPS_MAX:
-                continue
-            # lane slots per unit of the row, dearer with every further unit per lane and
-            # with the barriers of a block
-            cost = lanes * n / units * (1 + 0.25 * (n - 1)) * (1.1 if lanes == cg.BLOCK else 1.0)
-            if best is None or cost < best[0]:
-                best = (cost, lanes)
-        G = best[1] if best else cg.BLOCK
+        G = _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V)
     steps = -(-units // G)
     if steps > cg.ROW_STEPS_MAX or K >= 2 ** 40:
         raise cg.RowFusionUnsupported("row too long")
