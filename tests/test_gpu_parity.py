@@ -523,8 +523,8 @@ def test_every_kth_element_of_a_vector_takes_the_flat_kernel(dtype):
     a0 = mk(1 << 16)
     a = dr.array(a0)
     # the view's last vector would end past the buffer: left to the tail
-    assert hip.lower_only(a[1::2] * 2)[0].key[-1] is True
-    assert hip.lower_only(a[::2] * 2)[0].key[-1] is False
+    assert hip.lower_only(a[1::2] * 2)[0].key[-2] is True
+    assert hip.lower_only(a[::2] * 5)[0].key[-2] is False
     got, want = dr.sum(a[::2] * a[1::2]), np.sum(a0[::2] * a0[1::2])
     if np.dtype(dtype).kind == "f":
         assert abs(float(got) - float(want)) <= 1e-5 * (1 << 15)
