@@ -81,7 +81,7 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
             if deps is None or all(buf.version == ver for buf, ver in deps):
                 return arr
             del self.array  # a leaf was written to since: recompute
-        self.array = _backend.run(self)
+        self.array = _evaluate(_backend.run, self)
         self._depth = 0     # a leaf of whatever is built on it from now on
         return self.array
 
@@ -309,7 +309,7 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         if check is not None:
             check()             # a stretched view is read-only as a whole, as in NumPy
         if isinstance(item, DelayArray) and "array" not in item.__dict__:
-            _backend.run_into(item, arr[key])
+            _evaluate(_backend.run_into, item, arr[key])
         else:
             arr[key] = _unwrap(item)
 
@@ -1146,12 +1146,51 @@ def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **other)
     return res if axis is None and not keepdims else NPArray(res)
 
 
+def _evaluate(entry, roots, *more):
+    """`entry(roots, *more)` of the backend.  An expression is at most MAX_DEPTH operations
+    deep, but evaluated operands whose leaves have been written to since are computed
+    again as part of whatever reads them, and a chain of such operands (the iterates of a
+    loop, each MAX_DEPTH deep, after a write to the array they all started from) can be
+    deeper than the interpreter's stack allows.  Then the stale operands are brought up
+    to date one by one, deepest first, and the evaluation is tried again."""
+    try:
+        return entry(roots, *more)
+    except RecursionError:
+        for root in (roots if isinstance(roots, (list, tuple)) else [roots]):
+            _refresh_operands(root)
+        return entry(roots, *more)
+
+
+def _refresh_operands(root):
+    """Evaluate again, children before parents and without recursion, every evaluated
+    node below `root` whose leaves were written to after it was computed."""
+    stack = [(root, False)]
+    seen = set()
+    while stack:
+        node, after = stack.pop()
+        if after:
+            node._force()       # its operands are up to date: a walk of MAX_DEPTH at most
+            continue
+        if id(node) in seen:
+            continue
+        seen.add(id(node))
+        d = node.__dict__
+        if "array" in d and node is not root:
+            deps = d.get("_deps")
+            if deps is None or all(buf.version == ver for buf, ver in deps):
+                continue        # a leaf, or a result that is up to date
+            stack.append((node, True))
+        for child in d.get("children", ()):
+            if isinstance(child, DelayArray):
+                stack.append((child, False))
+
+
 def evaluate(*arrays):
     """Evaluate several lazy arrays together, in one fused kernel when their
     shapes agree, sharing common sub-expressions.  Returns the same objects."""
     todo = [a for a in arrays if isinstance(a, DelayArray) and "array" not in a.__dict__]
     if todo:
-        results = _backend.run_multi(todo)
+        results = _evaluate(_backend.run_multi, todo)
         for node, res in zip(todo, results):
             node.array = res
             node._depth = 0     # a leaf of whatever is built on it from now on

@@ -293,6 +293,42 @@ def test_matrix_product_on_the_matrix_cores(dtype, tol):
                        atol=1e-4 if dtype == np.float32 else 1e-12)
 
 
+def test_a_deep_chain_of_stale_results_is_brought_up_to_date_without_recursion():
+    """Three iterates, each 120 operations deep and each evaluated, then a write to the
+    array they started from: the last iterate is asked for again and would be re-walked
+    through all 360 operations, more frames than the interpreter allows; the stale
+    operands are then recomputed one by one, deepest first."""
+    import sys
+    import delayrepay_amd as dr
+    h0 = np.linspace(0.0, 1.0, 5000)
+    base = dr.array(h0.copy())
+
+    def grow(x):
+        for _ in range(60):
+            x = x * 0.999 + 0.25
+        return x
+    x1 = grow(base); x1.run()
+    x2 = grow(x1); x2.run()
+    x3 = grow(x2); x3.run()
+    want_old = grow(grow(grow(h0)))
+    assert np.array_equal(x3.get(), want_old)
+    base[:] = base * 2.0 + 1.0
+    from delayrepay_amd import delayarray
+    calls = []
+    refresh = delayarray._refresh_operands
+    delayarray._refresh_operands = lambda root: (calls.append(root), refresh(root))
+    limit = sys.getrecursionlimit()
+    sys.setrecursionlimit(1000)
+    try:
+        got = x3.get()
+    finally:
+        sys.setrecursionlimit(limit)
+        delayarray._refresh_operands = refresh
+    assert calls, "the chain was walked in one go: make it deeper"
+    assert np.array_equal(got, grow(grow(grow(h0 * 2.0 + 1.0))))
+    assert np.array_equal(x1.get(), grow(h0 * 2.0 + 1.0))
+
+
 def test_a_loop_of_functional_updates_holds_a_bounded_history():
     """`x = f(x)` evaluated every pass: results computed from results are a chain; past
     `hip.MAX_GENERATIONS` links the older result becomes an array in its own right, so the
