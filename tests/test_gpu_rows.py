@@ -212,3 +212,92 @@ def test_softmax_full_size():
     rows = rs.randint(0, 16384, 64)
     np.testing.assert_allclose(got[rows], softmax(np, a[rows]), rtol=2e-6)
     assert np.array_equal(got.argmax(axis=1), a.argmax(axis=1))
+
+
+# ---- seeded random expressions with row maxima and minima inside ----------------------------
+
+def _fuzz_leaf(rs, shape):
+    """(lazy leaf, host array) of a shape that broadcasts to `shape`: dense, a view with a row
+    pitch, one row for all, one value per row, every second column (which the row kernel
+    does not take: the reductions are then evaluated on their own)."""
+    dtype = [np.float32, np.float64][rs.randint(2)]
+    rows, R = shape
+    kind = rs.randint(7)
+
+    def host(s):
+        v = rs.uniform(-2, 2, s)
+        v[rs.uniform(size=s) < 0.02] = 0.0
+        return v.astype(dtype)
+    if kind == 3:
+        h = host((rows, R + 5))
+        lo = int(rs.randint(0, 6))
+        return dr.array(h)[:, lo:lo + R], h[:, lo:lo + R]
+    if kind == 4:
+        h = host((1, R))
+        return dr.array(h), h
+    if kind == 5:
+        h = host((rows, 1))
+        return dr.array(h), h
+    if kind == 6 and R * 2 * rows < (1 << 22):
+        h = host((rows, 2 * R))
+        return dr.array(h)[:, ::2], h[:, ::2]
+    h = host(shape)
+    return dr.array(h), h
+
+
+_FUZZ_UNARY = [np.negative, np.absolute, lambda x: x * x, lambda x: 0.5 * x, lambda x: x + 1, lambda x: 3 - x,
+               lambda x: np.sqrt(np.absolute(x))]
+_FUZZ_BINARY = [np.add, np.subtract, np.multiply, np.true_divide, np.maximum, np.minimum,
+                lambda a, b: np.where(a > b, a, b * 2)]
+
+
+def _fuzz_expr(rs, shape, depth, reductions):
+    """Random expression; with probability growing towards the root a sub-expression is
+    replaced by its maximum or minimum along the row (exact, whatever the order)."""
+    if depth == 0:
+        return _fuzz_leaf(rs, shape)
+    if reductions and rs.uniform() < 0.3:
+        d, o = _fuzz_expr(rs, shape, depth - 1, reductions - 1)
+        if o.shape != shape:        # reduce something that has whole rows
+            d2, o2 = _fuzz_leaf(rs, shape)
+            while o2.shape != shape:
+                d2, o2 = _fuzz_leaf(rs, shape)
+            d, o = d + d2, o + o2
+        if rs.randint(2):
+            return d.max(axis=-1, keepdims=True), o.max(axis=-1, keepdims=True)
+        return d.min(axis=-1, keepdims=True), o.min(axis=-1, keepdims=True)
+    if rs.uniform() < 0.3:
+        fn = _FUZZ_UNARY[rs.randint(len(_FUZZ_UNARY))]
+        d, o = _fuzz_expr(rs, shape, depth - 1, reductions)
+        return fn(d), fn(o)
+    fn = _FUZZ_BINARY[rs.randint(len(_FUZZ_BINARY))]
+    d1, o1 = _fuzz_expr(rs, shape, depth - 1, reductions)
+    d2, o2 = _fuzz_expr(rs, shape, depth - 1, reductions)
+    return fn(d1, d2), fn(o1, o2)
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_random_expressions_with_row_maxima_inside_are_bit_equal(seed):
+    rs = np.random.RandomState(7000 + seed)
+    shape = (int(rs.choice([1, 3, 64, 130, 1000])),
+             int(rs.choice([2, 3, 5, 16, 33, 64, 100, 257, 1000, 4099, 9000, 20000])))
+    if shape[0] * shape[1] > (1 << 22):
+        shape = (64, shape[1])
+    with np.errstate(all="ignore"):
+        d, o = _fuzz_expr(rs, shape, depth=int(rs.randint(2, 6)), reductions=3)
+        anchor_d, anchor_o = _fuzz_leaf(rs, shape)
+        d, o = d + anchor_d, o + anchor_o
+        got = d.get()
+    ref = np.broadcast_to(o, got.shape) if o.shape != got.shape else o
+    assert got.shape == np.broadcast_shapes(o.shape, got.shape) and bits_equal(got, np.asarray(ref)), (seed, shape)
+
+
+def test_the_random_expressions_reached_the_row_kernel():
+    """Runs after the cases above: many of them must have taken the row kernel, in
+    several lane-group sizes, and some the fallback (reductions evaluated on their own)."""
+    groups = {}
+    for key in hip._KERNELS:
+        if key[0] == "rows":
+            groups[key[6]] = groups.get(key[6], 0) + 1
+    print("row kernels by lanes per row:", groups)
+    assert sum(groups.values()) >= 20 and len(groups) >= 4, groups
