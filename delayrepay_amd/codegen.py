@@ -288,7 +288,7 @@ def op_expr(name, dt, args):
 
 
 # operations computed from the element index instead of from operands
-INDEX_OPS = ("iota", "philox_raw", "philox_f8")
+INDEX_OPS = ("iota", "philox_raw", "philox_f8", "philox_f4")
 
 # Philox-4x64-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11),
 # the counter-based generator behind numpy.random.Philox.  Output r of the stream that
@@ -347,6 +347,13 @@ def _philox_value(name, raw):
     return f"(long long){raw}" if name == "philox_raw" else f"(double)({raw} >> 11) * 0x1p-53"
 
 
+def _philox_float(raw, half):
+    """A float in [0, 1) from the top 24 bits of one half of a raw output: what
+    numpy.random.Generator.random(dtype=float32) makes of it (a 64-bit output serves two
+    numbers, its low half first)."""
+    return f"(float)((unsigned int)({raw} >> (32 * ({half}))) >> 8) * 0x1p-24f"
+
+
 def flat_elements(prog, leaf_class, out_dtypes, reduce_op):
     """Elements one thread handles per vector step of the flat kernel: a 16-byte vector of
     the widest streamed type (narrower streams move shorter vectors, see `flat_vec`: with
@@ -357,9 +364,9 @@ def flat_elements(prog, leaf_class, out_dtypes, reduce_op):
     widths = [ITEMSIZE[dt] for dt, c in zip(prog.leaves, leaf_class) if c != "b"]
     if not reduce_op:
         widths += [ITEMSIZE[dt] for dt in out_dtypes]
-    if any(name.startswith("philox") for name, _, _, _ in prog.ops):
-        widths.append(4)
-    if any(name.startswith("philox") for name, _, _, _ in prog.ops):
+    draws = {name for name, _, _, _ in prog.ops if name.startswith("philox")}
+    if draws:       # a block of four outputs: four 64-bit numbers or eight floats
+        widths.append(2 if "philox_f4" in draws else 4)
         return 16 // min(widths)
     return 16 // max(widths) if widths else 4
 
@@ -456,6 +463,12 @@ def _op_statement(prog, i):
         words = ", ".join(f"(dr_u64){k}{j}" for k, j in args[:6])
         pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
         expr = _philox_value(name, f"dr_philox({words}, {pos}(dr_u64)dr_i)")
+    elif name == "philox_f4":
+        # the same operands, the position counted in halves of outputs
+        words = ", ".join(f"(dr_u64){k}{j}" for k, j in args[:6])
+        pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
+        at = f"({pos}(dr_u64)dr_i)"
+        expr = _philox_float(f"dr_philox({words}, {at} >> 1)", f"(int)({at} & 1)")
     elif cdt == "f8" and name in prog.own_math:
         expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
     elif cdt == "f4" and name in prog.own_math32:
@@ -524,20 +537,31 @@ def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"
         if name == "iota":
             lines.append(f"    {loop} v{i}[e] = ({CTYPE[cdt]}){index};")
             continue
-        if name in ("philox_raw", "philox_f8"):
+        if name in ("philox_raw", "philox_f8", "philox_f4"):
             words = ", ".join(f"(dr_u64){k}{j}" for k, j in args[:6])
-            if len(args) == 6 and group == 4:
-                # the draw starts on a block and a group is four consecutive elements
-                # from a multiple of four: one block per group
-                for g in range(P // 4):
-                    vals = " ".join(f"v{i}[{4 * g + w}] = {_philox_value(name, f'x_[{w}]')};"
-                                    for w in range(4))
-                    lines.append(f"    {{ dr_u64 x_[4]; dr_philox_block({words}, (dr_u64)dr_g[{g}] >> 2, x_); "
-                                 f"{vals} }}")
+            per = 8 if name == "philox_f4" else 4       # numbers that one block serves
+            if len(args) == 6 and group % per == 0:
+                # the draw starts on a block and a group is consecutive elements from a
+                # multiple of a block's numbers: every block is made once
+                for g in range(P // group):
+                    for b in range(group // per):
+                        at = group * g + per * b
+                        if name == "philox_f4":
+                            vals = " ".join(f"v{i}[{at + 2 * w + h}] = {_philox_float(f'x_[{w}]', h)};"
+                                            for w in range(4) for h in range(2))
+                        else:
+                            vals = " ".join(f"v{i}[{at + w}] = {_philox_value(name, f'x_[{w}]')};"
+                                            for w in range(4))
+                        blk = f"((dr_u64)dr_g[{g}] >> {per.bit_length() - 1}) + {b}"
+                        lines.append(f"    {{ dr_u64 x_[4]; dr_philox_block({words}, {blk}, x_); {vals} }}")
             else:
                 pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
-                raw = f"dr_philox({words}, {pos}(dr_u64){index})"
-                lines.append(f"    {loop} v{i}[e] = {_philox_value(name, raw)};")
+                at = f"({pos}(dr_u64){index})"
+                if name == "philox_f4":
+                    value = _philox_float(f"dr_philox({words}, {at} >> 1)", f"(int)({at} & 1)")
+                else:
+                    value = _philox_value(name, f"dr_philox({words}, {at})")
+                lines.append(f"    {loop} v{i}[e] = {value};")
             continue
         if cdt == "f8" and name in prog.own_math:
             k, j = args[0]

@@ -52,6 +52,13 @@ class CpuVisitor(Visitor):
             return arr
         # numpy.random.Philox steps its counter before it makes a block, so the block
         # that holds output `pos` is made from `counter + pos // 4`, entered one lower
+        if node.dtype == numpy.float32:     # two numbers per output, its low half first
+            start = (node.counter - 1) % (1 << 256)
+            bits = numpy.random.Philox(key=node.key, counter=start)
+            raw = bits.random_raw((node.pos + node.shape[0] + 1) // 2)
+            halves = numpy.stack([raw & numpy.uint64(0xffffffff), raw >> numpy.uint64(32)], axis=1).ravel()
+            halves = halves[node.pos:node.pos + node.shape[0]].astype(numpy.uint32)
+            return (halves >> numpy.uint32(8)).astype(numpy.float32) * numpy.float32(1.0 / 16777216.0)
         first, skip = divmod(node.pos, 4)
         start = (node.counter + first - 1) % (1 << 256)
         bits = numpy.random.Philox(key=node.key, counter=start)

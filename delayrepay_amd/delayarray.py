@@ -918,17 +918,19 @@ class IotaEx(_Generated):
 class RandEx(_Generated):
     """`n` consecutive outputs of a Philox-4x64-10 stream (`numpy.random.Philox` with
     the same key and counter), starting `pos` outputs into it: raw 64-bit words (dtype
-    int64, the same bits as NumPy's uint64) or doubles in [0, 1) made from their top 53
-    bits as `numpy.random.Generator.random` makes them.  Every element is a function of
-    its index alone, so inside a 1-d expression of the same length it is computed in
-    the kernel and costs no memory traffic; made by `random.device(seed)`."""
+    int64, the same bits as NumPy's uint64), doubles in [0, 1) made from their top 53
+    bits as `numpy.random.Generator.random` makes them, or floats in [0, 1) made from the
+    top 24 bits of each half of an output, low half first, as `random(dtype=float32)`
+    makes them (`pos` then counts halves).  Every element is a function of its index
+    alone, so inside a 1-d expression of the same length it is computed in the kernel
+    and costs no memory traffic; made by `random.device(seed)`."""
 
     def __init__(self, n, key, counter, pos, dtype):
         super().__init__()
         self.shape = (int(n),)
         self.dtype = np.dtype(dtype)
-        if self.dtype not in (np.int64, np.float64):
-            raise TypeError("a Philox stream yields int64 words or float64 numbers")
+        if self.dtype not in (np.int64, np.float64, np.float32):
+            raise TypeError("a Philox stream yields int64 words, float64 or float32 numbers")
         self.key = int(key)
         self.counter = int(counter)        # counter of the block that holds output 0
         self.pos = int(pos)

@@ -318,7 +318,7 @@ class Tracer(Visitor):
         if node.pos:        # the draw starts inside a block
             refs.append(self.scalar(node.pos, "i8", ("pos", id(node)))[0])
         code = _code_of(node.dtype)
-        res = self.op("philox_raw" if code == "i8" else "philox_f8", code, code, refs)
+        res = self.op({"i8": "philox_raw", "f8": "philox_f8", "f4": "philox_f4"}[code], code, code, refs)
         self.gen_shapes.append(node.shape)
         self.iotas.append((res[0][1], node))
         self.leaf_nodes.append((node, None, None))

@@ -61,6 +61,13 @@ SCRIPT = textwrap.dedent("""
     assert np.array_equal(gen.uniform(-3.0, 5.0, 1001).get(), ref.uniform(-3.0, 5.0, 1001))
     raw = gen.random_raw(10).get()
     assert raw.dtype == np.int64 and np.array_equal(raw.view(np.uint64), ref.bit_generator.random_raw(10))
+    # float32: two numbers from every output, the low half first; the high half of the last
+    # output waits for the next float32 draw, whatever else is drawn in between
+    gen, ref = dnp.random.device(5), np.random.Generator(np.random.Philox(key=5))
+    for size, dt in ((7, np.float32), (3, np.float64), (4, np.float32), (1001, np.float32), (2, np.float64),
+                     ((5, 3), np.float32), (1, np.float32), (64, np.float32)):
+        got, want = gen.random(size, dtype=dt).get(), ref.random(size, dtype=dt)
+        assert got.dtype == want.dtype and np.array_equal(got, want), (size, dt)
     big = dnp.random.device(3, counter=(1 << 256) - 2)
     assert np.array_equal(big.random(20).get(),
                           np.random.Generator(np.random.Philox(key=3, counter=(1 << 256) - 2)).random(20))

@@ -550,6 +550,13 @@ def test_device_random_numbers_cost_no_operand():
     w = odd.random_raw(1 << 12)                                   # starts in the middle of a block
     assert (w.pos, w.dtype) == (3, np.int64)
     hip.compile_source(hip.lower_only(w)[1])
+    f = dr.random.device(9).random(1 << 14, dtype=np.float32)     # eight floats per block
+    low, src = hip.lower_only(f * 2)
+    assert f.dtype == np.float32 and low.kind == "flat" and low.srcs == [] and src.count("dr_philox_block(") == 3
+    hip.compile_source(src)
+    gen = dr.random.device(9)
+    gen.random(3, dtype=np.float32)                              # leaves the high half of output 1 waiting
+    assert gen._half == 1 and gen.pos == 2                       # (taken first by the next float32 draw)
     with pytest.raises(ValueError):
         dr.random.device(-1)
 

@@ -1572,6 +1572,17 @@ def test_device_random_stream_is_numpys_philox(seed, counter):
         assert np.array_equal(gen.random(n).get(), ref.random(n)), n
     assert np.array_equal(gen.uniform(-2.5, 7.0, 100003).get(), ref.uniform(-2.5, 7.0, 100003))
     assert np.array_equal(gen.random((33, 65)).get(), ref.random((33, 65)))
+    # float32 numbers take half an output each, low half first, and an odd draw leaves the
+    # high half of its last output to the next float32 draw, whatever is drawn in between
+    for n, dt in ((7, np.float32), (5, np.float64), (1 << 16, np.float32), (3, np.int64), (70001, np.float32),
+                  ((1 << 18) + 5, np.float32), (2, np.float32), ((17, 33), np.float32)):
+        if dt == np.int64:
+            assert np.array_equal(gen.random_raw(n).get().view(np.uint64), ref.bit_generator.random_raw(n))
+            continue
+        got, want = gen.random(n, dtype=dt).get(), ref.random(n, dtype=dt)
+        assert got.dtype == want.dtype and np.array_equal(got, want), (n, dt)
+    f = gen.random(1 << 12, dtype=np.float32)
+    assert np.array_equal((f * 2 + 1).get(), ref.random(1 << 12, dtype=np.float32) * np.float32(2) + np.float32(1))
 
 
 def test_device_random_numbers_fuse_without_memory_traffic():
