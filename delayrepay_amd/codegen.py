@@ -407,11 +407,12 @@ class Program:
             if soft_div else ()
 
     def _quotients_nobody_sees(self, types):
-        """Divisions (in the float types `types`) whose result reaches a root only through functions that round
-        on their own (`log(S / K)`, `erf(d / s)`): their last bit cannot be seen in any
+        """Divisions (in the float types `types`) and float64 square roots whose result
+        reaches a root only through functions that round on their own (`log(S / K)`,
+        `erf(d / (s * sqrt(t)))`): their last bit cannot be seen in any
         result beyond what those functions' own error already hides, so they may be
         computed to within one ulp instead of correctly rounded (`mathlib.DIV_F8`,
-        `mathlib32.DIV_F4`).  A
+        `dr_sqrt_near_f8`, `mathlib32.DIV_F4`).  A
         quotient that a root can see through exact operations alone (+ - * /, sqrt, the
         selections, the reductions) stays the correctly rounded one: expressions of those
         remain equal to NumPy's to the bit."""
@@ -426,7 +427,9 @@ class Program:
                     if kind == "v":
                         seen[j] = True
         return tuple(i for i, (name, cdt, _, _) in enumerate(self.ops)
-                     if name in ("divide", "true_divide") and cdt in types and not seen[i])
+                     if not seen[i] and cdt in types
+                     and (name in ("divide", "true_divide")
+                          or (name == "sqrt" and cdt == "f8" and "sqrt" in self.own_math)))
 
     def key(self):
         return (self.leaves, self.scalars, self.ops, self.roots, self.own_math, self.own_math32,
@@ -469,6 +472,8 @@ def _op_statement(prog, i):
         pos = f"(dr_u64){args[6][0]}{args[6][1]} + " if len(args) > 6 else ""
         at = f"({pos}(dr_u64)dr_i)"
         expr = _philox_float(f"dr_philox({words}, {at} >> 1)", f"(int)({at} & 1)")
+    elif cdt == "f8" and name == "sqrt" and i in prog.soft_div:
+        expr = f"dr_sqrt_near_f8_1({cargs[0]})"
     elif cdt == "f8" and name in prog.own_math:
         expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
     elif cdt == "f4" and name in prog.own_math32:
@@ -492,7 +497,7 @@ def emit_body(prog, out_dtypes, fname="dr_body", with_math=True, lds_tables=0, s
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"{CTYPE[dt]}& r{i}" for i, dt in enumerate(out_dtypes)]
     uses_philox = any(name.startswith("philox") for name, _, _, _ in prog.ops)
-    soft8 = any(prog.ops[i][1] == "f8" for i in prog.soft_div)
+    soft8 = any(prog.ops[i][1] == "f8" and prog.ops[i][0] != "sqrt" for i in prog.soft_div)
     soft4 = any(prog.ops[i][1] == "f4" for i in prog.soft_div)
     lines = [mathlib.source(prog.own_math, lds=lds_tables, stage_loop=stage_loop,
                             soft_div=soft8) if with_math else "",
@@ -565,11 +570,12 @@ def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"
             continue
         if cdt == "f8" and name in prog.own_math:
             k, j = args[0]
+            fn = "dr_sqrt_near_f8" if name == "sqrt" and i in prog.soft_div else mathlib.FUNCTIONS[name][0]
             if prog.ref_dtype((k, j)) == "f8" and ref(k, j).endswith("[e]"):
-                lines.append(f"    {mathlib.FUNCTIONS[name][0]}<{P}>({k}{j}, v{i});")
+                lines.append(f"    {fn}<{P}>({k}{j}, v{i});")
             else:       # converted or broadcast argument: gather it first
                 lines.append(f"    {{ double t_[{P}]; {loop} t_[e] = {cargs[0]}; "
-                             f"{mathlib.FUNCTIONS[name][0]}<{P}>(t_, v{i}); }}")
+                             f"{fn}<{P}>(t_, v{i}); }}")
             continue
         if i in prog.soft_div and cdt == "f4":
             lines.append(f"    {loop} v{i}[e] = dr_div_f4({cargs[0]}, {cargs[1]});")
@@ -2532,7 +2538,8 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     lanes = min(G, WAVE)
     per_wave = WAVE // lanes
     src = [PREAMBLE,
-           mathlib.source(prog.own_math, soft_div=any(prog.ops[i][1] == "f8" for i in prog.soft_div)),
+           mathlib.source(prog.own_math, soft_div=any(prog.ops[i][1] == "f8" and prog.ops[i][0] != "sqrt"
+                                                      for i in prog.soft_div)),
            mathlib32.source(prog.own_math32, soft_div=any(prog.ops[i][1] == "f4" for i in prog.soft_div))]
 
     # one function per stage, one for the per-element roots, one for the per-row roots

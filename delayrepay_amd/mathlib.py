@@ -622,39 +622,74 @@ DR_FN void dr_sqrt_f8(const double (&x)[P], double (&out)[P])
             if (!(x[e] >= 0x1p-767 && x[e] < __builtin_inf()))
                 out[e] = __builtin_sqrt(x[e]);
     }
+}
+/* The same for square roots that nothing reads but functions which round on their own
+   (erf(x / (s * sqrt(t)))): the estimate, the coupled step for g alone and one correction
+   by the residual, seven operations instead of ten.  The result is the correctly
+   rounded root except in about one case in 2^20, then the neighbouring double. */
+template <int P>
+DR_FN void dr_sqrt_near_f8(const double (&x)[P], double (&out)[P])
+{
+    _Pragma("unroll") for (int e = 0; e < P; ++e) {
+        const double y = DR_RSQ64(x[e]);
+        double g = x[e] * y;
+        const double h = 0.5 * y;
+        const double r = __builtin_fma(-h, g, 0.5);
+        g = __builtin_fma(g, r, g);
+        const double d = __builtin_fma(-g, g, x[e]);
+        out[e] = __builtin_fma(d, h, g);
+    }
+    bool rare = false;
+    _Pragma("unroll") for (int e = 0; e < P; ++e)
+        rare |= !(x[e] >= 0x1p-767 && x[e] < __builtin_inf());
+    if (DR_ANY_LANE(rare)) {
+        _Pragma("unroll") for (int e = 0; e < P; ++e)
+            if (!(x[e] >= 0x1p-767 && x[e] < __builtin_inf()))
+                out[e] = __builtin_sqrt(x[e]);
+    }
+}
+DR_FN double dr_sqrt_near_f8_1(double x)
+{
+    const double a[1] = {x};
+    double r[1];
+    dr_sqrt_near_f8<1>(a, r);
+    return r[0];
 }"""
 
 DIV_F8 = r"""
 /* a / b for quotients that nothing reads but functions which round on their own
-   (log(a / b), erf(x / s)): the reciprocal estimate, two refinements, the product and
-   one correction by the exact residual, eight operations where the correctly rounded
-   division takes thirteen (it scales both operands first, so that no intermediate
-   result leaves the normal range, and fixes up the special cases afterwards).  The
-   result is the correctly rounded quotient except in about one case in 2^20, then the
-   neighbouring double (checked against exact quotients in tests/test_mathlib.py).
+   (log(a / b), erf(x / s)): the reciprocal estimate, one refinement, the product and
+   one correction by the exact residual, six operations where the correctly rounded
+   division takes thirteen (it refines twice, scales both operands first, so that no
+   intermediate result leaves the normal range, and fixes up the special cases
+   afterwards).  An estimate good to e makes the refined reciprocal good to e^2, the
+   product likewise, and the correction squares that again: from 14 bits on the quotient
+   is right to 2^-56 before it is rounded.  The result is the correctly rounded
+   quotient except in about one case in 2^20, then the neighbouring double (checked
+   against exact quotients in tests/test_mathlib.py, and on the device).
    Operands that need the scaling or the special cases show in the result (not a normal
    number: a NaN from 0 or infinity times its reciprocal, an infinity, a denormal, a zero,
-   whose sign the correction would lose) and take the compiler's division, on a path a
-   wave skips when none of its lanes needs it. */
+   whose sign the correction would lose) or in the numerator (below 2^-1000 its residual,
+   2^-48 of it, falls among the denormals and corrects nothing) and take the compiler's
+   division, on a path a wave skips when none of its lanes needs it. */
+#define DR_DIV_RARE(q, a) (!(__builtin_isnormal(q) && __builtin_fabs(a) >= 0x1p-1000))
 template <int P>
 DR_FN void dr_div_f8(const double (&a)[P], const double (&b)[P], double (&out)[P])
 {
     bool rare = false;
     _Pragma("unroll") for (int e = 0; e < P; ++e) {
         double y = DR_RCP64(b[e]);
-        double t = __builtin_fma(-b[e], y, 1.0);
-        y = __builtin_fma(y, t, y);
-        t = __builtin_fma(-b[e], y, 1.0);
+        const double t = __builtin_fma(-b[e], y, 1.0);
         y = __builtin_fma(y, t, y);
         double q = a[e] * y;
         const double r = __builtin_fma(-b[e], q, a[e]);
         q = __builtin_fma(r, y, q);
         out[e] = q;
-        rare |= !__builtin_isnormal(q);
+        rare |= DR_DIV_RARE(q, a[e]);
     }
     if (DR_ANY_LANE(rare)) {
         _Pragma("unroll") for (int e = 0; e < P; ++e)
-            if (!__builtin_isnormal(out[e]))
+            if (DR_DIV_RARE(out[e], a[e]))
                 out[e] = a[e] / b[e];
     }
 }

@@ -1608,6 +1608,46 @@ def test_device_random_numbers_fuse_without_memory_traffic():
     assert np.array_equal(y.get(), want[10:20] + 1.0) and np.array_equal(x.get(), want)
 
 
+# ---- the short division and square root, on the device itself ---------------------------------
+
+def test_short_division_and_square_root_are_within_one_ulp_on_the_device():
+    """`dr_div_f8` and `dr_sqrt_near_f8` start from the hardware's reciprocal and reciprocal
+    square root estimates, which the host build of the same source only imitates: here the
+    device's own results, 2^22 random operands each over the whole exponent range and the
+    special values, against NumPy's correctly rounded ones."""
+    import struct
+    from delayrepay_amd import hiprt, mathlib
+    from delayrepay_amd.devarray import ndarray
+    src = mathlib.source(["sqrt"], soft_div=True) + """
+extern "C" __global__ void dr_kernel(const double* a, const double* b, double* q, double* r, long long n)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) { q[i] = dr_div_f8_1(a[i], b[i]); r[i] = dr_sqrt_near_f8_1(b[i]); }
+}
+"""
+    fn = hiprt.get_function(hip._load_or_compile(src), "dr_kernel")
+    rs = np.random.RandomState(31)
+    n = 1 << 21
+    special = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 5e-324, 1e-310, 2.2250738585072014e-308,
+                        1.7976931348623157e308, 1e-250, 3.0])
+    a = np.concatenate([rs.uniform(-100, 100, n), np.exp(rs.uniform(-300, 300, n)) * rs.choice([-1, 1], n),
+                        np.repeat(special, special.size)])
+    b = np.concatenate([rs.uniform(0.01, 100, n), np.exp(rs.uniform(-300, 300, n)), np.tile(special, special.size)])
+    da, db = dr.array(a)._force(), dr.array(b)._force()
+    q, r = ndarray(a.shape, np.float64), ndarray(a.shape, np.float64)
+    args = struct.pack("@PPPPq", da.ptr, db.ptr, q.ptr, r.ptr, a.size)
+    hiprt.launch(fn, -(-a.size // 256), 256, 0, args, len(args))
+    with np.errstate(all="ignore"):
+        for got, want in ((q.get(), a / b), (r.get(), np.sqrt(b))):
+            assert np.array_equal(np.isnan(got), np.isnan(want))
+            fin = np.isfinite(want)
+            assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+            assert np.array_equal(np.signbit(got[fin]), np.signbit(want[fin]))
+            off = np.abs(got[fin] - want[fin]) / np.spacing(np.abs(want[fin]))
+            assert off.max() <= 1.0, off.max()
+            assert np.count_nonzero(off) <= a.size // 20000, np.count_nonzero(off)
+
+
 # ---- quotients that only inexact functions read ---------------------------------------------
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])

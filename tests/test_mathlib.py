@@ -33,6 +33,11 @@ def host(tmp_path_factory):
                 "  for (; i + 4 <= n; i += 4) { const double a[4] = {x[i], x[i+1], x[i+2], x[i+3]}; "
                 f"double r[4]; {fn}<4>(a, r); for (int e = 0; e < 4; e++) y[i+e] = r[e]; }}\n"
                 f"  for (; i < n; i++) y[i] = {fn}_1(x[i]); }}\n")
+    src += ('extern "C" void v_sqrt_near(const double* x, double* y, long n)\n'
+            "{ long i = 0;\n"
+            "  for (; i + 4 <= n; i += 4) { const double a[4] = {x[i], x[i+1], x[i+2], x[i+3]}; "
+            "double r[4]; dr_sqrt_near_f8<4>(a, r); for (int e = 0; e < 4; e++) y[i+e] = r[e]; }\n"
+            "  for (; i < n; i++) y[i] = dr_sqrt_near_f8_1(x[i]); }\n")
     (d / "m.cpp").write_text(src)
     subprocess.run(["g++", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
                     str(d / "m.cpp")], check=True)
@@ -416,9 +421,10 @@ def test_quotients_that_only_inexact_functions_read(host):
     assert np.count_nonzero(off) <= a.size // 50000         # measured: none in 2^21
     with np.errstate(all="ignore"):
         sa = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1.0, 0.0, np.inf, 1e308, 1e-308,
-                       5e-324, 1.0, 1e-320, 3.0, 1e300, -1e-300, 2.0, 7.0])
+                       5e-324, 1.0, 1e-320, 3.0, 1e300, -1e-300, 2.0, 7.0, 1e-310, 5e-324, 3e-305])
         sb = np.array([1.0, 2.0, 0.0, -0.0, 2.0, -3.0, 1.0, np.nan, 0.0, np.inf, 1e-308, 1e308,
-                       2.0, 5e-324, 1e-320, np.inf, 1e-300, 1e300, 1e-310, 1.7976931348623157e308])
+                       2.0, 5e-324, 1e-320, np.inf, 1e-300, 1e300, 1e-310, 1.7976931348623157e308,
+                       1e-250, 1e-250, 7e-200])
         want = sa / sb
     res = host("div", sa, sb)
     assert np.array_equal(np.isnan(res), np.isnan(want))
@@ -427,6 +433,27 @@ def test_quotients_that_only_inexact_functions_read(host):
     # one at a time and in packs: the same arithmetic
     assert np.array_equal(host("div", a[:1001], b[:1001]),
                           np.concatenate([host("div", a[i:i + 1], b[i:i + 1]) for i in range(1001)]))
+
+
+def test_square_roots_that_only_inexact_functions_read(host):
+    """`dr_sqrt_near_f8` (seven operations instead of ten): the correctly rounded root nearly
+    always, never more than one ulp from it; zero, negative, infinite, NaN and tiny
+    arguments give what `sqrt` gives."""
+    rs = np.random.RandomState(12)
+    n = 1 << 20
+    x = np.concatenate([rs.uniform(0, 100, n), np.exp(rs.uniform(-500, 700, n))])
+    got, ref = host("sqrt_near", x), np.sqrt(x)
+    off = np.abs(got - ref) / np.spacing(ref)
+    assert off.max() <= 1.0
+    assert np.count_nonzero(off) <= x.size // 50000
+    with np.errstate(all="ignore"):
+        sx = np.array([0.0, -0.0, -1.0, np.inf, -np.inf, np.nan, 5e-324, 1e-310, 2.2250738585072014e-308,
+                       1e-250, 1.7976931348623157e308, 4.0, 2.0])
+        want = np.sqrt(sx)
+    res = host("sqrt_near", sx)
+    assert np.array_equal(np.isnan(res), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(res[ok], want[ok]) and np.array_equal(np.signbit(res[ok]), np.signbit(want[ok]))
 
 
 def test_only_quotients_that_no_root_can_see_are_computed_that_way():
@@ -441,6 +468,11 @@ def test_only_quotients_that_no_root_can_see_are_computed_that_way():
     assert soft([div, log(0), add(0, 1)], [(("v", 2), "f8")]) == ()              # a / b + log(a / b)
     assert soft([div, log(0)], [(("v", 1), "f8"), (("v", 0), "f8")]) == ()       # both are roots
     assert soft([div, ("sqrt", "f8", "f8", (("v", 0),))], [(("v", 1), "f8")]) == ()      # sqrt is exact
+    root = ("sqrt", "f8", "f8", (("l", 0),))
+    erf = lambda j: ("erf", "f8", "f8", (("v", j),))
+    assert soft([root, erf(0)], [(("v", 1), "f8")]) == (0,)                      # erf(sqrt(a)): the root too
+    assert soft([root, erf(0), add(0, 1)], [(("v", 2), "f8")]) == ()             # sqrt(a) + erf(sqrt(a))
+    assert cg.Program(["f8", "f8"], [], [root, erf(0)], [(("v", 1), "f8")], own_math=False).soft_div == ()
     assert soft([div, ("multiply", "f8", "f8", (("v", 0), ("l", 0))), ("erf", "f8", "f8", (("v", 1),))],
                 [(("v", 2), "f8")]) == (0,)                                      # erf(a / b * a)
     f4 = [("divide", "f4", "f4", (("l", 0), ("l", 1))), ("log", "f4", "f4", (("v", 0),))]
