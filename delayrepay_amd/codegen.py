@@ -399,9 +399,9 @@ class Program:
             if own_math32 else ()
         # these operations read the element index: only the flat kernel supplies it
         self.uses_index = any(name in INDEX_OPS for name, _, _, _ in self.ops)
-        # float64 only: in float32 the short division (`mathlib32.DIV_F4`) with its branch for
-        # the rare cases measures slower than the compiler's branch-free sequence
-        # (Black-Scholes float32: 120 against 115 us); soft_div=2 asks for it all the same
+        # soft_div: 1 float64 only, 2 float32 as well.  The float32 forms are used by bodies
+        # that evaluate packs of elements (one test for the rare cases per pack: element by
+        # element the test costs more than the short forms save)
         self.soft_div = self._quotients_nobody_sees(("f8",) * bool(own_math)
                                                     + ("f4",) * bool(own_math32 and soft_div == 2)) \
             if soft_div else ()
@@ -429,7 +429,7 @@ class Program:
         return tuple(i for i, (name, cdt, _, _) in enumerate(self.ops)
                      if not seen[i] and cdt in types
                      and (name in ("divide", "true_divide")
-                          or (name == "sqrt" and cdt == "f8" and "sqrt" in self.own_math)))
+                          or (name == "sqrt" and (cdt == "f4" or "sqrt" in self.own_math))))
 
     def key(self):
         return (self.leaves, self.scalars, self.ops, self.roots, self.own_math, self.own_math32,
@@ -478,8 +478,8 @@ def _op_statement(prog, i):
         expr = f"{mathlib.FUNCTIONS[name][0]}_1({cargs[0]})"
     elif cdt == "f4" and name in prog.own_math32:
         expr = f"{mathlib32.FUNCTIONS[name][0]}({cargs[0]})"
-    elif i in prog.soft_div:
-        expr = f"dr_div_f8_1({cargs[0]}, {cargs[1]})" if cdt == "f8" else f"dr_div_f4({cargs[0]}, {cargs[1]})"
+    elif i in prog.soft_div and cdt == "f8":
+        expr = f"dr_div_f8_1({cargs[0]}, {cargs[1]})"
     elif name == "where":    # the condition keeps its own type
         k, j = args[0]
         expr = f"(({k}{j} != 0) ? {cargs[1]} : {cargs[2]})"
@@ -577,19 +577,25 @@ def emit_body_packed(prog, out_dtypes, leaf_is_array, pack, fname="dr_body_pack"
                 lines.append(f"    {{ double t_[{P}]; {loop} t_[e] = {cargs[0]}; "
                              f"{fn}<{P}>(t_, v{i}); }}")
             continue
-        if i in prog.soft_div and cdt == "f4":
-            lines.append(f"    {loop} v{i}[e] = dr_div_f4({cargs[0]}, {cargs[1]});")
+        if i in prog.soft_div and name == "sqrt":       # float32 (float64 went above)
+            k, j = args[0]
+            if prog.ref_dtype((k, j)) == "f4" and ref(k, j).endswith("[e]"):
+                lines.append(f"    dr_sqrt_near_f4_pack<{P}>({k}{j}, v{i});")
+            else:
+                lines.append(f"    {{ float t_[{P}]; {loop} t_[e] = {cargs[0]}; "
+                             f"dr_sqrt_near_f4_pack<{P}>(t_, v{i}); }}")
             continue
         if i in prog.soft_div:
             gather = []
             names = []
             for pos, (k, j) in enumerate(args):
-                if prog.ref_dtype((k, j)) == "f8" and ref(k, j).endswith("[e]"):
+                if prog.ref_dtype((k, j)) == cdt and ref(k, j).endswith("[e]"):
                     names.append(f"{k}{j}")
                 else:       # converted or broadcast operand: gather it first
-                    gather.append(f"double q{pos}_[{P}]; {loop} q{pos}_[e] = {cargs[pos]};")
+                    gather.append(f"{CTYPE[cdt]} q{pos}_[{P}]; {loop} q{pos}_[e] = {cargs[pos]};")
                     names.append(f"q{pos}_")
-            lines.append(f"    {{ {' '.join(gather)} dr_div_f8<{P}>({names[0]}, {names[1]}, v{i}); }}")
+            fn = "dr_div_f8" if cdt == "f8" else "dr_div_f4_pack"
+            lines.append(f"    {{ {' '.join(gather)} {fn}<{P}>({names[0]}, {names[1]}, v{i}); }}")
             continue
         if name == "cast":
             expr = cargs[0]
@@ -685,7 +691,8 @@ def packs(prog, vec):
     """Whether the flat kernel evaluates this program on packs of elements: programs
     that use the float64 functions of `mathlib` or draw Philox numbers, in vector
     kernels."""
-    return bool(vec and (prog.own_math or any(name.startswith("philox") for name, _, _, _ in prog.ops)))
+    return bool(vec and (prog.own_math or any(name.startswith("philox") for name, _, _, _ in prog.ops)
+                         or any(prog.ops[i][1] == "f4" for i in prog.soft_div)))
 
 
 def emit_flat(prog, leaf_class, out_dtypes, vec, unroll, nt_load, nt_store, restrict=True,

@@ -66,7 +66,8 @@ TUNE = {
     "t_rows": 0,      # transpose tiles: output rows (= contiguous elements of the operand) and
     "t_cols": 0,      # output columns per tile (powers of two; 0: 128 bytes by 1 KB)
     "dmath": 1,       # float64 log/erf from `mathlib` (0: the device library's)
-    "softdiv": 1,     # float64 quotients that only inexact functions read: to one ulp, 8 operations
+    "softdiv": 2,     # quotients and square roots that only inexact functions read: to one ulp, in
+                      # fewer operations (1: float64 only, 2: float32 too, in packed bodies; 0: never)
                       # (2: float32 quotients as well, 4 operations; measured slower)
     "rowfuse": 1,     # reductions along the last axis inside an expression: one kernel per row
     "row_lanes": 0,   # ... lanes per row (0: by the cost of idle lanes and of units per lane)
@@ -86,6 +87,7 @@ TUNE = {
     "table_blocks": 4096,  # most workgroups of a flat kernel whose functions keep tables in LDS
     "smath": 1,       # float32 log/erf/exp from `mathlib32` (0: the device library's)
     "pack": 4,        # elements a thread passes through those functions in lock step
+    "pack32": 8,      # ... a float32 body with short divisions or square roots
 }
 for _kv in filter(None, os.environ.get("DELAYREPAY_TUNE", "").split(",")):
     _k, _v = _kv.split("=")
@@ -522,7 +524,9 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         if packed:
             # float64 functions evaluate a pack of elements in lock step: at least `pack`
             # elements per thread (a vector of doubles holds two)
-            unroll = max(unroll, TUNE["pack"] // cg.flat_elements(prog, leaf_class, out_codes, reduce_op))
+            size = TUNE["pack"] if prog.own_math or not any(prog.ops[i][1] == "f4" for i in prog.soft_div) \
+                else TUNE["pack32"]
+            unroll = max(unroll, size // cg.flat_elements(prog, leaf_class, out_codes, reduce_op))
         in_bytes = sum(a.nbytes for a, k in zip(leaves, leaf_class) if k != "b")
         footprint = in_bytes
         if not reduce_op:

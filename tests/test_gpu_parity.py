@@ -1646,6 +1646,41 @@ extern "C" __global__ void dr_kernel(const double* a, const double* b, double* q
             off = np.abs(got[fin] - want[fin]) / np.spacing(np.abs(want[fin]))
             assert off.max() <= 1.0, off.max()
             assert np.count_nonzero(off) <= a.size // 20000, np.count_nonzero(off)
+    # the float32 forms (packs of four): the hardware's reciprocal with one correction, and
+    # its square root as it is
+    from delayrepay_amd import mathlib32
+    src = mathlib32.source([], soft_div=True) + """
+extern "C" __global__ void dr_kernel(const float* a, const float* b, float* q, float* r, long long n)
+{
+    const long long i = 4 * ((long long)blockIdx.x * 256 + threadIdx.x);
+    if (i + 4 <= n) {
+        const float x[4] = {a[i], a[i + 1], a[i + 2], a[i + 3]}, y[4] = {b[i], b[i + 1], b[i + 2], b[i + 3]};
+        float u[4], v[4];
+        dr_div_f4_pack<4>(x, y, u); dr_sqrt_near_f4_pack<4>(y, v);
+        for (int e = 0; e < 4; ++e) { q[i + e] = u[e]; r[i + e] = v[e]; }
+    }
+}
+"""
+    fn = hiprt.get_function(hip._load_or_compile(src), "dr_kernel")
+    sp = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, 1e-40, 1.1754944e-38, 3.4028235e38,
+                   1e-30, 3.0], dtype=np.float32)
+    a4 = np.concatenate([rs.uniform(-100, 100, n), np.exp(rs.uniform(-80, 80, n)) * rs.choice([-1, 1], n),
+                         np.repeat(sp, sp.size), [1.0, 1.0, 1.0]]).astype(np.float32)
+    b4 = np.concatenate([rs.uniform(0.01, 100, n), np.exp(rs.uniform(-80, 80, n)), np.tile(sp, sp.size),
+                         [1.0, 1.0, 1.0]]).astype(np.float32)
+    assert a4.size % 4 == 0
+    da, db = dr.array(a4)._force(), dr.array(b4)._force()
+    q, r = ndarray(a4.shape, np.float32), ndarray(a4.shape, np.float32)
+    args = struct.pack("@PPPPq", da.ptr, db.ptr, q.ptr, r.ptr, a4.size)
+    hiprt.launch(fn, -(-a4.size // 1024), 256, 0, args, len(args))
+    with np.errstate(all="ignore"):
+        for got, want in ((q.get(), a4 / b4), (r.get(), np.sqrt(b4))):
+            assert np.array_equal(np.isnan(got), np.isnan(want))
+            fin = np.isfinite(want)
+            assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+            assert np.array_equal(np.signbit(got[fin]), np.signbit(want[fin]))
+            off = np.abs(got[fin].astype(np.float64) - want[fin]) / np.spacing(np.abs(want[fin])).astype(np.float64)
+            assert off.max() <= 1.0, off.max()
 
 
 # ---- quotients that only inexact functions read ---------------------------------------------
@@ -1666,7 +1701,7 @@ def test_quotients_inside_functions_and_quotients_that_are_results(dtype):
     b = np.concatenate([b, np.tile(special, special.size)])
     da, db = dr.array(a), dr.array(b)
     low, _ = hip.lower_only([np.log(da / db)])
-    assert low.key[1][-1] == ((0,) if dtype == np.float64 else ())     # the quotient is marked
+    assert low.key[1][-1] == (0,)                                      # the quotient is marked
     with np.errstate(all="ignore"):
         ref = np.log(a / b)
         got = np.log(da / db).get()

@@ -301,13 +301,18 @@ def host32(tmp_path_factory):
     src = "#include <math.h>\n" + mathlib32.source(sorted(mathlib32.FUNCTIONS), mathlib32.HOST_MACROS,
                                                    soft_div=True)
     for name, (fn, _) in mathlib32.FUNCTIONS.items():
-        src += (f"void v_{name}(const float* x, float* y, long n)\n"
+        src += (f'extern "C" void v_{name}(const float* x, float* y, long n)\n'
                 f"{{ for (long i = 0; i < n; i++) y[i] = {fn}(x[i]); }}\n")
-    src += ("void v_div(const float* a, const float* b, float* y, long n)\n"
-            "{ for (long i = 0; i < n; i++) y[i] = dr_div_f4(a[i], b[i]); }\n")
-    (d / "m.c").write_text(src)
-    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
-                    str(d / "m.c"), "-lm"], check=True)
+    # the short division: packs of four (the form the kernels use), then one at a time
+    src += ('extern "C" void v_div(const float* a, const float* b, float* y, long n)\n'
+            "{ long i = 0;\n"
+            "  for (; i + 4 <= n; i += 4) { const float p[4] = {a[i], a[i+1], a[i+2], a[i+3]}, "
+            "q[4] = {b[i], b[i+1], b[i+2], b[i+3]}; float r[4]; dr_div_f4_pack<4>(p, q, r); "
+            "for (int e = 0; e < 4; e++) y[i+e] = r[e]; }\n"
+            "  for (; i < n; i++) y[i] = dr_div_f4(a[i], b[i]); }\n")
+    (d / "m.cpp").write_text(src)
+    subprocess.run(["g++", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", str(d / "m.so"),
+                    str(d / "m.cpp"), "-lm"], check=True)
     lib = ctypes.CDLL(str(d / "m.so"))
 
     def call(name, x, other=None):
