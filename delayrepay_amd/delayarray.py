@@ -246,6 +246,14 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         return np.transpose(self)
 
     def reshape(self, *args, **kwargs):
+        if "array" not in self.__dict__ and not kwargs and self.ndim:
+            want = args[0] if len(args) == 1 and not isinstance(args[0], (int, np.integer)) else args
+            want = tuple(want) if isinstance(want, (tuple, list)) else None
+            if want is not None and len(want) == self.ndim + 1 and want[-1] == 1 and \
+                    builtins.all(w == d or w == -1 for w, d in zip(want, self.shape)) and want.count(-1) <= 1:
+                res = _keep_last_axis(self)         # `a.sum(axis=1).reshape(-1, 1)`
+                if res is not None:
+                    return res
         return NPArray(self._force().reshape(*args, **kwargs))
 
     def copy(self):
@@ -279,6 +287,10 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         same expression over slices of its leaves: only the part asked for is ever
         computed, and shifted slices of one expression fuse into one stencil."""
         key = _unwrap(key)
+        if "array" not in self.__dict__ and _adds_last_axis(key, self.ndim):
+            res = _keep_last_axis(self)
+            if res is not None:
+                return res
         if "array" not in self.__dict__ and type(self) in _ELEMENTWISE and _basic_key(key):
             res = _over_views(self, lambda arr: arr[key], key)
             if res is not None:
@@ -1014,6 +1026,63 @@ class _TooLarge(Exception):
     pass
 
 
+def _adds_last_axis(key, ndim):
+    """Whether indexing with `key` only appends an axis of one: `[:, None]`, `[..., None]`."""
+    key = key if isinstance(key, tuple) else (key,)
+    if len(key) < 2 or key[-1] is not None:
+        return False
+    head = key[:-1]
+    if len(head) == 1 and head[0] is Ellipsis:
+        return True
+    return len(head) == ndim and builtins.all(isinstance(k, slice) and k == slice(None) for k in head)
+
+
+def _keep_last_axis(root):
+    """`root[..., None]` of an unevaluated expression over reductions along the last axis
+    that are still lazy (`a.sum(axis=1)`, `a.max(axis=1) * 2`): the same expression over their
+    `keepdims` twins, which the backend's row kernel takes as operands, so that
+    `a / a.sum(axis=1)[:, None]` reads every row once.  None when the expression holds no
+    such reduction (the caller then indexes as usual)."""
+    memo = {}
+    found = [False]
+    budget = [PUSH_VIEWS_UP_TO]
+
+    def walk(node):
+        hit = memo.get(id(node))
+        if hit is not None:
+            return hit
+        kind = type(node)
+        arr = node.__dict__.get("array")
+        if kind is Scalar:
+            res = node
+        elif kind is ReduceEx and arr is None and not node.keepdims and node.axis is not None \
+                and node.axis == (node.children[0].ndim - 1,):
+            found[0] = True
+            res = ReduceEx(node.func, node.children[0], node.axis, True)
+        elif arr is not None or kind is NPArray:
+            res = NPArray(node._force()[..., None])
+        elif kind in _ELEMENTWISE and kind is not CastEx:
+            budget[0] -= 1
+            if budget[0] < 0:
+                raise _TooLarge
+            res = kind(node.func, *[walk(c) for c in node.children])
+        elif kind is CastEx:
+            res = CastEx(node.dtype, walk(node.children[0]))
+        else:
+            raise _TooLarge
+        memo[id(node)] = res
+        return res
+
+    try:
+        res = walk(root)
+        return res if found[0] else None
+    except _TooLarge:
+        return None
+    finally:
+        memo.clear()
+        walk = None
+
+
 _NODES = Memoiser._cache.data
 _NODE_GONE = Memoiser._cache._gone
 _new_node = object.__new__
@@ -1130,9 +1199,13 @@ def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **other)
         axis = tuple(sorted(norm))
         if len(axis) == ndim:
             axis = None
-    if keepdims and axis == (ndim - 1,) and arr.dtype.kind == "f" and arr.shape[-1] > 1 \
+    if axis == (ndim - 1,) and arr.dtype.kind == "f" and arr.shape[-1] > 1 \
             and getattr(_backend, "LAZY_ROW_REDUCTIONS", False):
-        return ReduceEx(func, arr, axis, True)
+        # with `keepdims` it is an operand of the row kernel as it is; without, it becomes
+        # one when a last axis of one is put back (`a.sum(axis=1)[:, None]`,
+        # `.reshape(-1, 1)`, `expand_dims(..., -1)`: `_keep_last_axis`), and is evaluated
+        # on its own by whatever else reads it
+        return ReduceEx(func, arr, axis, bool(keepdims))
     if 0 in arr.shape and func is not np.add and arr.dtype == np.bool_ and \
             (axis is None or 0 in [arr.shape[k] for k in axis]):
         # `any` / `all` of nothing: the identities of `or` and `and`

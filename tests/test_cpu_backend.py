@@ -247,10 +247,26 @@ assert np.array_equal(sm.get(), ref_e / ref_e.sum(axis=-1, keepdims=True))
 assert np.array_equal(m.get(), a.max(axis=1, keepdims=True))
 assert np.array_equal(dr.var(da, axis=1).get(), ((a - a.mean(axis=1, keepdims=True)) ** 2).sum(axis=1) / 57)
 assert np.allclose(dr.std(da, axis=1, keepdims=True).get(), a.std(axis=1, keepdims=True), rtol=1e-14)
-# not along the last axis, not kept, integers: evaluated at once, as before
+# not along the last axis, integers: evaluated at once, as before
 assert not isinstance(da.max(axis=0, keepdims=True), ReduceEx)
-assert not isinstance(da.max(axis=1), ReduceEx)
 assert not isinstance(dr.array(np.arange(12).reshape(3, 4)).max(axis=1, keepdims=True), ReduceEx)
+# along the last axis without keepdims: lazy too, and putting the axis back gives the kept twin,
+# so the usual spellings of a normalisation fuse as well
+s = da.sum(axis=1)
+assert isinstance(s, ReduceEx) and s.shape == (13,) and "array" not in s.__dict__
+for kept in (s[:, None], s[..., None], s[:, np.newaxis], s.reshape(-1, 1), s.reshape(13, 1), np.expand_dims(s, -1),
+             np.expand_dims(s, 1)):
+    assert isinstance(kept, ReduceEx) and kept.keepdims and kept.shape == (13, 1) and kept is s[:, None]
+assert "array" not in s.__dict__
+assert np.array_equal((da / da.sum(axis=1)[:, None]).get(), a / a.sum(axis=1)[:, None])
+assert np.array_equal((da - da.mean(axis=1).reshape(-1, 1)).get(), a - a.mean(axis=1).reshape(-1, 1))
+mx = (da.max(axis=1) * 2.0)[:, None]            # an expression over the reduction
+assert isinstance(mx, DelayArray) and mx.shape == (13, 1) and "array" not in mx.__dict__
+assert np.array_equal((da - mx).get(), a - (a.max(axis=1) * 2.0)[:, None])
+assert np.array_equal(s.get(), a.sum(axis=1)) and np.array_equal(s[3:7].get(), a.sum(axis=1)[3:7])
+assert np.array_equal((s * 2 + 1).get(), a.sum(axis=1) * 2 + 1) and float(s[2]) == a.sum(axis=1)[2]
+t3 = dr.array(rs.standard_normal((3, 4, 5)))
+assert np.array_equal((t3 / t3.sum(axis=-1)[..., None]).get(), t3.get() / t3.get().sum(axis=-1)[..., None])
 # keywords that change the result are refused, not dropped
 for call in (lambda: np.sum(da, initial=10.0), lambda: np.any(da, where=np.ones((13, 57), bool)),
              lambda: np.max(da, initial=0.0)):

@@ -301,3 +301,33 @@ def test_the_random_expressions_reached_the_row_kernel():
             groups[key[6]] = groups.get(key[6], 0) + 1
     print("row kernels by lanes per row:", groups)
     assert sum(groups.values()) >= 20 and len(groups) >= 4, groups
+
+
+def test_the_usual_spellings_of_a_normalisation_are_one_kernel_too():
+    """`a.sum(axis=1)` stays lazy; `[:, None]`, `.reshape(-1, 1)` and `expand_dims(..., -1)`
+    turn it into its kept twin, so these expressions take the row kernel like their
+    `keepdims=True` forms; used in any other way the reduction is evaluated on its own."""
+    rs = np.random.RandomState(8)
+    a = rs.uniform(0.5, 2.0, (300, 1000)).astype(np.float32)
+    da = dr.array(a)
+    got, n = launches(lambda: (da / da.sum(axis=1)[:, None]).get())
+    assert n == 1
+    np.testing.assert_allclose(got, a / a.sum(axis=1)[:, None], rtol=2e-6)
+    got, n = launches(lambda: (da - da.max(axis=1).reshape(-1, 1)).get())
+    assert n == 1 and bits_equal(got, a - a.max(axis=1).reshape(-1, 1))
+    got, n = launches(lambda: (da - np.expand_dims(da.min(axis=-1), -1) * 2.0).get())
+    assert n == 1 and bits_equal(got, a - np.expand_dims(a.min(axis=-1), -1) * 2.0)
+    e = np.exp(da - da.max(axis=1)[:, None])
+    got, n = launches(lambda: (e / e.sum(axis=1)[:, None]).get())
+    ref = np.exp(a - a.max(axis=1)[:, None])
+    assert n == 1
+    np.testing.assert_allclose(got, ref / ref.sum(axis=1)[:, None], rtol=2e-6)
+    # on its own, sliced, or inside an expression of its own shape: evaluated as before
+    s = da.sum(axis=1)
+    np.testing.assert_allclose(s.get(), a.sum(axis=1), rtol=1e-5)
+    np.testing.assert_allclose((s * 2 + 1)[5:9].get(), (a.sum(axis=1) * 2 + 1)[5:9], rtol=1e-5)
+    assert bits_equal(da.max(axis=1).get(), a.max(axis=1))
+    t3 = rs.standard_normal((7, 9, 130))
+    d3 = dr.array(t3)
+    got, n = launches(lambda: (d3 - d3.max(axis=-1)[..., None]).get())
+    assert n == 1 and bits_equal(got, t3 - t3.max(axis=-1)[..., None])
