@@ -876,6 +876,14 @@ def _walk(node, key, leaves, uses, deep, index, bufs):
                     raise _Unseen
                 deep.append(d)
             _walk(child, key, leaves, uses, deep, index, bufs)
+        elif kind == "ReduceEx":
+            # a reduction along the last axis that keeps it: an operation of the row kernel
+            # (anything else the tracer evaluates on its own: not a structure to remember)
+            if "array" in child.__dict__ or not getattr(child, "keepdims", False) \
+                    or child.axis != (len(child.children[0].shape) - 1,):
+                raise _Unseen
+            add(("rows", child.children[0].shape[-1]))
+            _walk(child, key, leaves, uses, deep, index, bufs)
         else:
             raise _Unseen
     for child in children:
@@ -941,7 +949,8 @@ def _seen_before(scan):
     plan.second = None
     plan.kern2 = None
     plan.scratch = 0
-    plan.out_shapes = None
+    plan.out_shapes = model.out_shapes
+    low.row_out = mlow.row_out
     for d in deep:
         d["_seen"] = d.get("_seen", 0) + 1
     STATS["seen_hits"] += 1
@@ -970,8 +979,10 @@ def _remember_structure(scan, tracer, plan):
     mlow.key, mlow.kind, mlow.emit, mlow.fmt = low.key, low.kind, low.emit, low.fmt
     mlow.tail, mlow.grid, mlow.fin_count, mlow.lds = low.tail, low.grid, low.fin_count, low.lds
     mlow.recipe = low.recipe
+    mlow.row_out = low.row_out
     model.low = mlow
     model.kern = plan.kern
+    model.out_shapes = plan.out_shapes
     model.shape, model.out_dtypes, model.acc = plan.shape, plan.out_dtypes, plan.acc
     _SEEN[key] = (model, tuple(tracer.scalar_uses), tuple(tracer.scalar_codes))
 

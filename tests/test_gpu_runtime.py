@@ -526,6 +526,26 @@ def test_a_structure_met_before_keeps_its_plan_over_fresh_arrays():
             assert hip.STATS["seen_hits"] == seen + 2
         assert np.isclose(s, ((hx - hy) ** 2 * hw).sum(), rtol=1e-13)
         assert p.tobytes() == (hx * hy + hw).tobytes() and q.tobytes() == (hx - hy * hw).tobytes()
+    # rows that are reduced and used again: the row kernel's plan is kept as well, per row
+    # length and per way the rows are laid out
+    for shape in ((64, 64), (32, 128), (64, 64)):
+        for step in range(3):
+            ha = rs.uniform(-2, 2, shape).astype(np.float32)
+            hb = rs.uniform(1, 2, (shape[0] + 2, shape[1] + 4)).astype(np.float32)
+            a, b = dr.array(ha), dr.array(hb)[1:-1, 2:-2]
+            seen, launches = hip.STATS["seen_hits"], hip.STATS["launches"]
+            e = np.exp(a - a.max(axis=1, keepdims=True))
+            got = hip.run(e / e.sum(axis=1, keepdims=True) * b).get()
+            assert hip.STATS["launches"] == launches + 1
+            if step:
+                assert hip.STATS["seen_hits"] == seen + 1, (shape, step)
+            ref = np.exp(ha - ha.max(axis=1, keepdims=True))
+            np.testing.assert_allclose(got, ref / ref.sum(axis=1, keepdims=True) * hb[1:-1, 2:-2], rtol=3e-6)
+            seen = hip.STATS["seen_hits"]
+            got = hip.run(a / a.max(axis=1)[:, None]).get()
+            assert got.tobytes() == (ha / ha.max(axis=1)[:, None]).tobytes()
+            if step:
+                assert hip.STATS["seen_hits"] == seen + 1, (shape, step)
     # an operand evaluated beforehand is a leaf, whatever its structure's plan said
     hx, hy, hw = batch()
     x, y, w = dr.array(hx), dr.array(hy), dr.array(hw)
