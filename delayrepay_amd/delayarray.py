@@ -328,13 +328,16 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
     # ---- reductions and friends -----------------------------------------
 
     def sum(self, *args, **kwargs):
-        return np.sum(self, *args, **kwargs)
+        node = _row_reduce(np.add, self, args, kwargs)
+        return node if node is not None else np.sum(self, *args, **kwargs)
 
     def max(self, *args, **kwargs):
-        return np.max(self, *args, **kwargs)
+        node = _row_reduce(np.maximum, self, args, kwargs)
+        return node if node is not None else np.max(self, *args, **kwargs)
 
     def min(self, *args, **kwargs):
-        return np.min(self, *args, **kwargs)
+        node = _row_reduce(np.minimum, self, args, kwargs)
+        return node if node is not None else np.min(self, *args, **kwargs)
 
     def mean(self, *args, **kwargs):
         return np.mean(self, *args, **kwargs)
@@ -1110,7 +1113,7 @@ def _binary(func, left, right):
     shape = left.shape
     other = right.shape
     if shape != other and other:
-        shape = other if not shape else tuple(np.broadcast_shapes(shape, other))
+        shape = other if not shape else _broadcast2(shape, other)
     node = _new_node(BinaryNumpyEx)
     node.__dict__ = {"_count": DelayArray.count, "children": [left, right], "_depth": depth + 1,
                      "func": func, "shape": shape,
@@ -1119,6 +1122,59 @@ def _binary(func, left, right):
     ref = _NODES[key] = _Ref(node, _NODE_GONE)
     ref.key = key
     return node
+
+
+def _row_reduce(func, arr, args, kwargs):
+    """`arr.sum(axis=-1)`, `arr.max(axis=1, keepdims=True)` ... of a float matrix as the lazy
+    node `_reduce` would return, in one frame (a step that builds softmax anew calls this
+    twice); None for every other call, which then goes the long way."""
+    shape = arr.shape
+    ndim = len(shape)
+    if ndim < 2 or len(args) > 1 or arr.dtype.kind != "f" or shape[-1] < 2 \
+            or not getattr(_backend, "LAZY_ROW_REDUCTIONS", False):
+        return None
+    axis = args[0] if args else kwargs.get("axis")
+    if not isinstance(axis, int) or (axis != -1 and axis != ndim - 1):
+        return None
+    keep = False
+    for name, value in kwargs.items():
+        if name == "keepdims" and isinstance(value, bool):
+            keep = value
+        elif name != "axis":
+            return None
+    axis = (ndim - 1,)
+    key = (ReduceEx, func, id(arr), axis, keep)
+    ref = _NODES.get(key)
+    if ref is not None:
+        node = ref()
+        if node is not None:
+            return node
+    if arr._depth >= MAX_DEPTH:
+        return None
+    node = _new_node(ReduceEx)
+    node.__dict__ = {"_count": DelayArray.count, "children": [arr], "_depth": arr._depth + 1,
+                     "func": func, "axis": axis, "keepdims": keep,
+                     "shape": shape[:-1] + (1,) if keep else shape[:-1], "dtype": arr.dtype, "_key": key}
+    DelayArray.count += 1
+    ref = _NODES[key] = _Ref(node, _NODE_GONE)
+    ref.key = key
+    return node
+
+
+def _broadcast2(a, b):
+    """Broadcast shape of two shapes (NumPy's own routine takes several microseconds)."""
+    if len(a) == len(b):
+        out = []
+        for x, y in zip(a, b):
+            if x == y or y == 1:
+                out.append(x)
+            elif x == 1:
+                out.append(y)
+            else:
+                break
+        else:
+            return tuple(out)
+    return tuple(np.broadcast_shapes(a, b))       # other ranks, or NumPy's error message
 
 
 def _unary(func, arg):
