@@ -92,7 +92,7 @@ def parse():
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
                          "dot | axis0 | axis1 | axis1_3d | matvec | rows200 | rowbcast | transpose | "
                          "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | softmax | "
-                         "layernorm | rowmax | strided | next (all "
+                         "layernorm | rowmax | strided | strided2d | next (all "
                          "of these: the operations either side of the five configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
@@ -287,6 +287,15 @@ def main():
                              "12 B are fetched and written, whole cache lines)",
                         steps=[(lambda v=v: hip.run(v[::2] * 2.0)) for v in vecs],
                         cpu=lambda: hx[:n // 4:2] * np.float32(2.0), cpu_frac=0.25, cpu_code="numpy.multiply")
+        if name == "strided2d":
+            rows, cols = 8192, 16383
+            hm = rs.standard_normal((rows, cols)).astype(np.float32)
+            mats = [dr.array(hm) for _ in range(sets_for(4 * rows * cols + 4 * rows * 5461))]
+            return dict(dtype="f32", n=rows * 5461, nbytes=8 * rows * 5461,
+                        desc="m[:, ::3] * 2 f32 8192x16383 (every third element of every row: 8 B per result "
+                             "are needed, 16 B are fetched and written)",
+                        steps=[(lambda m=m: hip.run(m[:, ::3] * 2.0)) for m in mats],
+                        cpu=lambda: hm[:rows // 4, ::3] * np.float32(2.0), cpu_frac=0.25, cpu_code="numpy.multiply")
         if name == "diff2":
             n = 1 << 27
             hx = rs.standard_normal(n).astype(np.float32)
@@ -665,7 +674,7 @@ def main():
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
              "next": ["dot", "axis0", "axis1", "axis1_3d", "matvec", "rows200", "rowbcast", "transpose",
                       "transpose3d", "interior", "diff2", "stencil9", "stencil3d", "grid", "rand",
-                      "softmax", "layernorm", "rowmax", "strided"]}.get(args.workload, [args.workload])
+                      "softmax", "layernorm", "rowmax", "strided", "strided2d"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:

@@ -434,10 +434,15 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     flat = ndim <= 1 and all(s == [1] or s == [0] or s == [] for s in m_leaf) \
         and all(s == [1] or s == [] for s in m_out)
     if not flat and ndim == 1 and TUNE["strided"] and all(s == [1] for s in m_out) \
-            and all(len(s) == 1 and 0 <= s[0] <= 8 for s in m_leaf):
-        # Every k-th element of a vector (`a[::2]`): the flat kernel with the k vectors that
-        # hold a thread's elements loaded whole.  The general kernel computes an index per
-        # element and stores element by element.
+            and all(len(s) == 1 and (0 <= s[0] <= 1 or (s[0] == 2 and a.dtype.itemsize <= 4))
+                    for a, s in zip(leaves, m_leaf)):
+        # Every second element of a vector (`a[::2]`): the flat kernel with the two vectors
+        # that hold a thread's elements loaded whole (x[::2] * 2, 2^26 float32 results: 129 us;
+        # the general kernel, which computes an index per element and stores element by
+        # element, 139).  From every third element on, two thirds and more of what such
+        # vectors bring into the registers is thrown away and the general kernel, one
+        # element per lane, is the faster one (x[::3] * 2: 126 us against 141 with vectors
+        # and 170 with four element loads per thread).
         flat = True
     if flat and ndim == 1 and not reduce_op and TUNE["lds"] and TUNE["svec"] and TUNE["row1d"] \
             and 4096 <= n < 2 ** 31 - 4096:
