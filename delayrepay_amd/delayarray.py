@@ -1237,6 +1237,10 @@ def _reduce(func, arr, axis=None, dtype=None, out=None, keepdims=False, **other)
     arr = arg_to_numpy_ex(arr)
     if out is not None or dtype is not None:
         raise NotImplementedError("reductions with out= or dtype= are not supported")
+    if not other and isinstance(axis, int) and isinstance(keepdims, bool):
+        node = _row_reduce(func, arr, (axis,), {"keepdims": keepdims})      # the common case, in one frame
+        if node is not None:
+            return node
     for name, value in other.items():
         # `where=` and `initial=` change the result: say so instead of leaving them out
         if not (value is None or value is np._NoValue or (name == "where" and value is True)):
