@@ -15,6 +15,9 @@ GENERATED_LEAVES = True     # FullEx / IotaEx nodes are understood
 LAZY_ROW_REDUCTIONS = True  # reductions that keep their axis may stay lazy nodes
 
 
+COUNTS_WRITES = True    # ndarrays have no version: the front end counts the writes instead
+
+
 def is_ndarray(arr):
     return isinstance(arr, numpy.ndarray)
 

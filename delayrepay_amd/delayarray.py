@@ -38,6 +38,12 @@ from . import backend as be
 from .promote import PY_DESCR, result_dtype, scalar_descr
 
 _backend = be.backend
+# A backend whose arrays carry no version of their own (NumPy's) cannot tell which results
+# a write has made stale, so every write through `__setitem__` is counted and a result
+# evaluated before the latest one is computed again when it is next asked for: on every
+# backend an evaluated expression follows its leaves.
+_COUNTS_WRITES = bool(getattr(_backend, "COUNTS_WRITES", False))
+_WRITES = [0]
 
 
 def cast(func):
@@ -75,14 +81,20 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
 
     def _force(self):
         """Evaluate (once) and return the backend array."""
-        arr = self.__dict__.get("array")
+        d = self.__dict__
+        arr = d.get("array")
         if arr is not None:
-            deps = self.__dict__.get("_deps")
-            if deps is None or all(buf.version == ver for buf, ver in deps):
+            deps = d.get("_deps")
+            if deps is None:
+                if d.get("_epoch", _WRITES[0]) == _WRITES[0]:
+                    return arr
+            elif all(buf.version == ver for buf, ver in deps):
                 return arr
             del self.array  # a leaf was written to since: recompute
         self.array = _evaluate(_backend.run, self)
         self._depth = 0     # a leaf of whatever is built on it from now on
+        if _COUNTS_WRITES and self.children:
+            self._epoch = _WRITES[0]
         return self.array
 
     def __array__(self, dtype=None, copy=None):
@@ -308,10 +320,12 @@ class DelayArray(numpy.lib.mixins.NDArrayOperatorsMixin):
         # c = a * 2`: c is a new node), and a backend that walks through evaluated nodes
         # stops here
         d = self.__dict__
+        _WRITES[0] += 1
         if self.children:
             d.pop("_deps", None)
             d.pop("_plan", None)
             d.pop("_multi", None)
+            d.pop("_epoch", None)
             d["_cut"] = True
             own = d.get("_key")
             if own is not None and Memoiser._cache.get(own) is self:
@@ -1329,6 +1343,8 @@ def evaluate(*arrays):
         for node, res in zip(todo, results):
             node.array = res
             node._depth = 0     # a leaf of whatever is built on it from now on
+            if _COUNTS_WRITES and node.children:
+                node._epoch = _WRITES[0]
     return arrays
 
 

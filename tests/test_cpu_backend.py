@@ -311,3 +311,41 @@ def test_a_result_written_to_by_hand_is_an_array_of_its_own():
     print("ok")
     """
     assert run_cpu(script).strip().endswith("ok")
+
+
+def test_an_evaluated_result_follows_its_leaves_on_this_backend_too():
+    """The device backend computes an evaluated result again when a leaf under it has been
+    written to (its buffers carry versions).  NumPy's arrays carry none, so the front end
+    counts writes: asked for directly or used as an operand, a result evaluated before the
+    latest write is computed again, and the two backends agree on the same program
+    (the same cases run on the device in tests/test_gpu_reference_suite.py)."""
+    script = r"""
+    import numpy as np
+    import delayrepay_amd as dr
+    a = dr.array(np.ones(16))
+    b = a * 2 + 1
+    assert np.all(b.get() == 3) and b.get() is b.get()      # nothing written: the same array
+    c = b + 1
+    assert np.all(c.get() == 4)
+    p, q = dr.evaluate(b * 2, b - 1)
+    assert np.all(p.get() == 6) and np.all(q.get() == 2)
+    a[:] = 5.0
+    assert np.all(c.get() == 12) and np.all(b.get() == 11)
+    assert np.all(p.get() == 22) and np.all(q.get() == 10)
+    # reductions along the rows are expressions like any other
+    m = dr.array(np.arange(24.0).reshape(4, 6))
+    s, k = m.sum(axis=1), m.max(axis=1, keepdims=True)
+    assert s.get()[1] == 51 and k.get()[1, 0] == 11
+    m[1, 1] = -50.0
+    assert s.get()[1] == -6 and k.get()[1, 0] == 11
+    m[1, 5] = 99.0
+    assert k.get()[1, 0] == 99
+    # a result written to by hand keeps the write whatever happens to its operands
+    h = a * 3
+    h.run()
+    h[0] = -1.0
+    a[:] = 2.0
+    assert h.get()[0] == -1 and h.get()[1] == 15
+    print("ok")
+    """
+    assert run_cpu(script).strip().endswith("ok")
