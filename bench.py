@@ -91,7 +91,7 @@ def parse():
     ap.add_argument("--workload", default="all",
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
                          "dot | axis0 | axis1 | axis1_3d | matvec | rows200 | rowbcast | transpose | "
-                         "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | softmax | "
+                         "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | softmax | softmax32k | "
                          "layernorm | rowmax | strided | strided2d | next (all "
                          "of these: the operations either side of the five configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
@@ -329,6 +329,20 @@ def main():
                         steps=[(lambda v=v: hip.run(v.T * 2.0)) for v in vols],
                         cpu=lambda: hv[:, :, :256].T * np.float32(2.0), cpu_frac=0.25,
                         cpu_code="numpy.multiply")
+        if name == "softmax32k":
+            R, N = 32000, 8192
+            ha = rs.standard_normal((N, R)).astype(np.float32)
+            mats = [dr.array(ha) for _ in range(sets_for(8 * N * R))]
+
+            def soft(xp, a):
+                e = xp.exp(a - a.max(axis=1, keepdims=True))
+                return e / e.sum(axis=1, keepdims=True)
+            return dict(dtype="f32", n=N * R, nbytes=8 * N * R,
+                        desc="softmax along rows of 32000 f32, 8192 rows (a row of 128 KB held in "
+                             "one block's registers)",
+                        steps=[(lambda a=a: hip.run(soft(dr, a))) for a in mats],
+                        cpu=lambda: soft(np, ha[:N // 16]), cpu_frac=1 / 16,
+                        cpu_code="numpy.max, subtract, exp, sum, divide")
         if name in ("softmax", "layernorm", "rowmax"):
             N = 16384
             ha = rs.standard_normal((N, N)).astype(np.float32)
@@ -674,7 +688,7 @@ def main():
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
              "next": ["dot", "axis0", "axis1", "axis1_3d", "matvec", "rows200", "rowbcast", "transpose",
                       "transpose3d", "interior", "diff2", "stencil9", "stencil3d", "grid", "rand",
-                      "softmax", "layernorm", "rowmax", "strided", "strided2d"]}.get(args.workload, [args.workload])
+                      "softmax", "softmax32k", "layernorm", "rowmax", "strided", "strided2d"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:
