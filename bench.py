@@ -339,7 +339,7 @@ def main():
                 return e / e.sum(axis=1, keepdims=True)
             return dict(dtype="f32", n=N * R, nbytes=8 * N * R,
                         desc="softmax along rows of 32000 f32, 8192 rows (a row of 128 KB held in "
-                             "one block's registers)",
+                             "the registers of a block of 512 lanes)",
                         steps=[(lambda a=a: hip.run(soft(dr, a))) for a in mats],
                         cpu=lambda: soft(np, ha[:N // 16]), cpu_frac=1 / 16,
                         cpu_code="numpy.max, subtract, exp, sum, divide")

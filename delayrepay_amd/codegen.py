@@ -2367,10 +2367,14 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
 # ---- rows that are reduced and used again in one kernel -----------------------------
 
 ROW_REDUCE = {"rowsum": "add", "rowmax": "maximum", "rowmin": "minimum"}
-# 16-byte units a lane holds of one operand's row: a block of 256 lanes takes rows of up to
-# 128 KB.  With 32 units kept (128 registers) a softmax still runs three waves a SIMD and
-# moves rows of 32000 float32 at 65 % of the peak, against 34 % for a kernel per reduction.
-ROW_STEPS_MAX = 32
+# 16-byte units a lane holds of one operand's row.  A block of 256 lanes takes rows of up to
+# 64 KB; longer ones, up to 256 KB, a block of 512 lanes with up to 32 units each (rows of
+# 128 KB: 16 units in 512 lanes move 71 % of the peak, 32 units in 256 lanes 68 %, with
+# 150-165 registers; 1024 lanes leave each 128 registers and a layer normalisation of
+# 50257 float32 then spills: 20 %).
+ROW_STEPS_MAX = 16
+ROW_STEPS_LONG = 32
+ROW_BLOCKS = (256, 512)             # lanes of a block that holds one row
 
 
 class RowFusionUnsupported(Exception):
@@ -2509,7 +2513,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
                    fence=True, recompute=True, pipeline=True, carry_values=True, wave_map=False,
                    nt_load=False):
     """Rows that are reduced and used again: `a - max(a, axis=-1)`, softmax, the variance,
-    layer normalisation.  A group of G lanes (8..64: part of a wave; 256: the block) owns a
+    layer normalisation.  A group of G lanes (1..64: part of a wave; 256 or 512: the block) owns a
     row of R elements (a compile-time constant, unit stride); lane j takes the 16-byte
     units j, j + G, ... of it.  An operand flagged in `keep` (default: all) has its share of
     the row in registers from one stage to the next, so the row is read from memory once;
@@ -2541,10 +2545,13 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     units = -(-R // V)
     full, rem = R // V, R % V
     steps = -(-units // G)
-    if steps > ROW_STEPS_MAX:
+    if steps > (ROW_STEPS_LONG if G > BLOCK else ROW_STEPS_MAX):
         raise RowFusionUnsupported("row too long")
     nl, ns, n_out = len(prog.leaves), len(prog.scalars), len(out_dtypes)
-    block_row = G == BLOCK
+    block_row = G >= BLOCK
+    B = G if block_row else BLOCK          # lanes of a block: 256, or 512 for one long row
+    if B not in ROW_BLOCKS:
+        raise RowFusionUnsupported("no such block")
     lanes = min(G, WAVE)
     per_wave = WAVE // lanes
     src = [PREAMBLE,
@@ -2603,10 +2610,18 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
                 f"        v = {_combine(op, 'v', 'o')};",
                 "    }"]
         if block_row:
-            a, b = _combine(op, "slot[0]", "slot[1]"), _combine(op, "slot[2]", "slot[3]")
             body += [f"    if ((threadIdx.x & {WAVE - 1}) == 0) slot[threadIdx.x >> 6] = v;",
-                     "    __syncthreads();",
-                     f"    v = {_combine(op, f'({a})', f'({b})')};"]
+                     "    __syncthreads();"]
+            terms = [f"slot[{w}]" for w in range(B // WAVE)]
+            if len(terms) == 4:
+                terms = [f"({_combine(op, terms[t], terms[t + 1])})" for t in (0, 2)]
+            level = 0
+            while len(terms) > 2:       # the waves' values pairwise, in one order for every lane
+                body += [f"    const {ct} w{level}_{t // 2} = {_combine(op, terms[t], terms[t + 1])};"
+                         for t in range(0, len(terms), 2)]
+                terms = [f"w{level}_{t}" for t in range(len(terms) // 2)]
+                level += 1
+            body.append(f"    v = {_combine(op, terms[0], terms[1])};")
         body.append("    return v;")
         body.append("}")
         src.append("\n".join(body))
@@ -2618,7 +2633,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     params += [f"const long long sk{i}" for i in range(nl)]
     params += [f"const long long so{n}" for n in range(n_out)]
     scal = [f"s{i}" for i in range(ns)]
-    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+    L = [f'extern "C" __global__ __launch_bounds__({B})',
          f"void dr_kernel({', '.join(params)})", "{"]
     def vtype(dt):
         return (VEC16[dt][0] + "u") if V > 1 else CTYPE[dt]
@@ -2626,20 +2641,19 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     # Which unit a lane takes in step j: `lo + sub`.  Lanes side by side over the whole
     # group (sub = lane, lo = j G), or, `wave_map`, every wave of the block its own quarter
     # of the row (sub = wave * quarter + lane, lo = 64 j): a wave then reads 16 KB of a
-    # 64 KB row in sequence instead of sixteen pieces 4 KB apart (32 KB of a 128 KB row
-    # instead of thirty-two pieces), which the memory system
+    # 64 KB row in sequence instead of sixteen pieces 4 KB apart, which the memory system
     # serves faster (copying rows of 64 KB: 75 % of the peak against 66 %; rows of 16 and
     # 32 KB: 74 against 76 % and 69 against 71 %).
     wave_map = bool(block_row and wave_map and steps > 1)
     seg = steps * WAVE
     step_units = WAVE if wave_map else G
-    max_sub = (BLOCK // WAVE - 1) * seg + WAVE - 1 if wave_map else G - 1
+    max_sub = (B // WAVE - 1) * seg + WAVE - 1 if wave_map else G - 1
 
     def holds(sub):
         """Whether some lane has this `sub`."""
         if sub < 0:
             return False
-        return (sub % seg < WAVE and sub // seg < BLOCK // WAVE) if wave_map else sub < G
+        return (sub % seg < WAVE and sub // seg < B // WAVE) if wave_map else sub < G
 
     # which lanes hold what in step j: whole units, the partial last unit, nothing
     def step_state(j):
@@ -2701,7 +2715,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     if block_row:
         widest = max((CTYPE[prog.ops[i][2]] for reds in stages for i in reds),
                      key=lambda c: 8 if c in ("double", "long long") else 4)
-        L += [f"    __shared__ {widest} dr_slots[2][{max(n_red, 1)}][{BLOCK // WAVE}];",
+        L += [f"    __shared__ {widest} dr_slots[2][{max(n_red, 1)}][{B // WAVE}];",
               f"    const int sub = (threadIdx.x >> 6) * {seg} + (threadIdx.x & {WAVE - 1});" if wave_map
               else "    const int sub = threadIdx.x;",
               "    const unsigned int usub = sub;",

@@ -32,7 +32,7 @@ from .codegen import Program, dtype_code, code_dtype
 from .promote import result_dtype, scalar_descr
 from .visitor import Visitor
 from .lowering import (TUNE, Lowered as _Lowered, broadcast_strides as _broadcast_strides,
-                       lower as _lower,
+                       lower as _lower, block_lanes as _block_lanes,
                        lower_axis_reduce as _lower_axis_reduce)
 
 hiprt.lib()  # fail at import when libdrhip.so has not been built
@@ -405,6 +405,11 @@ def _load_or_compile(source):
     return module
 
 
+# Lanes per block of the kernels that are not launched with `codegen.BLOCK` of them (a row
+# kernel whose block of 512 or 1024 lanes holds one long row), by function handle.
+_BLOCK_OF = {}
+
+
 def _kernel_name(low):
     """Symbol of the generated kernel: shape kind plus a digest of the cache key, so
     that profilers list structurally different kernels separately."""
@@ -429,6 +434,9 @@ def _kernel_for(low, with_finalize):
     kern.func = hiprt.get_function(module, name)
     kern.finalize = hiprt.get_function(module, name + "_fin") if with_finalize else None
     kern.packer = struct.Struct(low.fmt)
+    block = _block_lanes(low)
+    if block != cg.BLOCK:
+        _BLOCK_OF[kern.func] = block
     _KERNELS[low.key] = kern
     return kern
 
@@ -486,9 +494,9 @@ class Replay:
     def _issue_all(self):
         for func, grid, lds, args, slot, scratch in self.launches:
             if slot is None:
-                hiprt.launch(func, grid, cg.BLOCK, lds, args, len(args))
+                hiprt.launch(func, grid, _BLOCK_OF.get(func, cg.BLOCK), lds, args, len(args))
             else:
-                hiprt.launch_scratch(func, grid, cg.BLOCK, lds, args, len(args), slot, scratch)
+                hiprt.launch_scratch(func, grid, _BLOCK_OF.get(func, cg.BLOCK), lds, args, len(args), slot, scratch)
 
     def as_graph(self):
         """Capture the recorded launches into a HIP graph; later calls replay the
@@ -635,9 +643,9 @@ def _issue(func, grid, args, slot=None, scratch=0):
     that takes the library's static scratch array, of which the kernel uses
     `scratch` bytes; None for a kernel without one."""
     if slot is None:
-        hiprt.launch(func, grid, cg.BLOCK, 0, args, len(args))
+        hiprt.launch(func, grid, _BLOCK_OF.get(func, cg.BLOCK), 0, args, len(args))
     else:
-        hiprt.launch_scratch(func, grid, cg.BLOCK, 0, args, len(args), slot, scratch)
+        hiprt.launch_scratch(func, grid, _BLOCK_OF.get(func, cg.BLOCK), 0, args, len(args), slot, scratch)
     if _RECORDING is not None:
         _RECORDING.launches.append((func, grid, 0, args, slot, scratch))
     STATS["launches"] += 1

@@ -327,7 +327,23 @@ def _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V):
         t = max(t_mem, t_alu) + 0.25 * min(t_mem, t_alu)
         if best is None or t < best[0]:
             best = (t, lanes)
+    if best is None and -(-units // cg.ROW_BLOCKS[-1]) <= cg.ROW_STEPS_LONG:
+        return cg.ROW_BLOCKS[-1]        # longer than 256 lanes hold: a block of 512
     return best[1] if best else cg.BLOCK
+
+
+def block_lanes(low):
+    """Lanes per block that the kernel of `low` is launched with: `codegen.BLOCK`, except
+    for a row kernel whose block of 512 lanes holds one long row (read from the cache key,
+    which every copy of a lowering carries)."""
+    if low.kind == "rows" and low.key[6] > cg.BLOCK:
+        return low.key[6]
+    return cg.BLOCK
+
+
+def _row_steps_max(G):
+    """Units a lane may hold of one operand's row."""
+    return cg.ROW_STEPS_LONG if G > cg.BLOCK else cg.ROW_STEPS_MAX
 
 
 def lower_rows(prog, leaves, scalars, shape, out_codes):
@@ -364,7 +380,7 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     if not G:
         G = _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V)
     steps = -(-units // G)
-    if steps > cg.ROW_STEPS_MAX or K >= 2 ** 40:
+    if steps > _row_steps_max(G) or K >= 2 ** 40:
         raise cg.RowFusionUnsupported("row too long")
     # An operand's share of its row stays in registers between the stages, as long as all
     # of them fit; operands that are the same for every row (a vector of weights) come from
@@ -382,7 +398,7 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     low.row_out = tuple(row_out)
     fence, recompute, pipe = bool(TUNE["row_fence"]), bool(TUNE["row_recompute"]), bool(TUNE["row_pipe"])
     carry = bool(TUNE["row_carry"])
-    wmap = G == cg.BLOCK and (steps >= 12 if TUNE["row_wavemap"] < 0 else bool(TUNE["row_wavemap"]))
+    wmap = G >= cg.BLOCK and (steps >= 12 if TUNE["row_wavemap"] < 0 else bool(TUNE["row_wavemap"]))
     low.key = ("rows", prog.key(), tuple(kinds), tuple(out_codes), low.row_out, R, G, keep, nts,
                fence, recompute, pipe, carry, wmap, ntl)
 
@@ -391,7 +407,7 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
                                  fence=fence, recompute=recompute, pipeline=pipe, carry_values=carry,
                                  wave_map=wmap, nt_load=ntl)
     low.emit = emit
-    if G == cg.BLOCK:
+    if G >= cg.BLOCK:
         blocks = K
     else:
         blocks = -(-K // (cg.BLOCK // G))

@@ -615,3 +615,26 @@ def test_scan_leaves_nothing_behind():
         assert ref() is None
     finally:
         gc.enable()
+
+
+def test_long_rows_take_a_block_of_512_lanes_and_compile():
+    """Lowering of softmax by row length: a lane group or a block of 256 lanes up to 64 KB,
+    a block of 512 lanes up to 256 KB (with the waves' partial results combined over eight
+    slots), and nothing beyond (`RowFusionUnsupported`: the caller evaluates the reductions
+    on their own).  The generated source goes through hiprtc here, without a device."""
+    def soft(a):
+        e = np.exp(a - a.max(axis=1, keepdims=True))
+        return e / e.sum(axis=1, keepdims=True)
+    for R, dtype, lanes in ((16384, np.float32, 256), (16385, np.float32, 512), (50257, np.float32, 512),
+                            (65536, np.float32, 512), (32768, np.float64, 512), (8192, np.float64, 256)):
+        low, src = hip.lower_only(soft(leaf((64, R), dtype)))
+        assert low.kind == "rows" and lowering.block_lanes(low) == lanes, (R, dtype)
+        assert f"__launch_bounds__({lanes})" in src and f"[{lanes // 64}];" in src
+        if lanes == 512:
+            assert "slot[7]" in src and "slot[8]" not in src
+            hip.compile_source(src)
+    for R, dtype in ((65537, np.float32), (32769, np.float64)):
+        with pytest.raises(cg.RowFusionUnsupported):
+            hip.lower_only(soft(leaf((64, R), dtype)))
+    low, _ = hip.lower_only(leaf((64, 50257)) * 2.0)
+    assert lowering.block_lanes(low) == cg.BLOCK

@@ -9,15 +9,15 @@ import numpy as np
 import pytest
 
 import delayrepay_amd as dr
-from delayrepay_amd import hip
+from delayrepay_amd import hip, lowering
 from tests.helpers import bits_equal
 
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(5, 2), (3, 7), (64, 200), (33, 203), (1000, 64), (7, 1000), (9, 1023), (130, 1025),
           (50, 4096), (17, 4099), (12, 16384), (5, 16381), (9, 13001), (6, 12289),
-          (4, 32768), (3, 32000), (3, 20001), (2, 40000)]
-ROW_BYTES = 131072      # a row of at most 128 KB is held by one block, 512 bytes a lane
+          (4, 32768), (3, 32000), (3, 20001), (2, 40000), (2, 65536), (2, 70001)]
+ROW_BYTES = 262144      # a row of at most 256 KB is held by one block (of 512 lanes above 64 KB)
 
 
 def launches(fn):
@@ -156,7 +156,7 @@ def test_stacks_of_matrices_and_operands_of_other_shapes():
 
 def test_what_the_row_kernel_does_not_take_is_computed_the_long_way():
     rs = np.random.RandomState(10)
-    a = rs.standard_normal((8, 40000)).astype(np.float32)          # rows too long to hold
+    a = rs.standard_normal((8, 70000)).astype(np.float32)          # rows too long to hold
     da = dr.array(a)
     got, n = launches(lambda: (da - da.max(axis=1, keepdims=True)).get())
     assert n >= 2 and bits_equal(got, a - a.max(axis=1, keepdims=True))
@@ -334,3 +334,29 @@ def test_the_usual_spellings_of_a_normalisation_are_one_kernel_too():
     d3 = dr.array(t3)
     got, n = launches(lambda: (d3 - d3.max(axis=-1)[..., None]).get())
     assert n == 1 and bits_equal(got, t3 - t3.max(axis=-1)[..., None])
+
+
+def test_rows_held_by_a_block_of_512_lanes_replay_with_that_block():
+    """Rows of 64 to 256 KB take a block of 512 lanes; recorded launches and the HIP graph
+    made of them must launch that many (a replay with 256 would leave half of every row
+    unwritten)."""
+    rs = np.random.RandomState(12)
+    a = rs.standard_normal((24, 50257)).astype(np.float32)
+    b = rs.standard_normal((24, 50257)).astype(np.float32)
+    da = dr.array(a)
+    low, src = hip.lower_only(softmax(dr, da))
+    assert low.kind == "rows" and lowering.block_lanes(low) == 512 and "__launch_bounds__(512)" in src
+    with hip.record() as rep:
+        out = hip.run(softmax(dr, da))
+    assert len(rep.launches) == 1
+    ref = softmax(np, a)
+    np.testing.assert_allclose(out.get(), ref, rtol=2e-6)
+    da[...] = b                                        # same buffers, new values
+    rep()
+    np.testing.assert_allclose(out.get(), softmax(np, b), rtol=2e-6)
+    rep.as_graph()
+    for k in range(3):
+        da[...] = (a, b)[k % 2]
+        rep()
+        hip.synchronize()
+        np.testing.assert_allclose(out.get(), (ref, softmax(np, b))[k % 2], rtol=2e-6)
