@@ -2414,20 +2414,23 @@ def row_analysis(prog, leaf_kind):
     return level, uniform, stages
 
 
-def _row_needed(prog, targets, held=None):
+def _row_needed(prog, targets, held=None, pre=()):
     """Operations to compute for the values `targets` (refs), in order, the row
     reductions they read (those are handed in, not computed) and the leaves they read.
     `held` maps an operation to the leaf whose registers hold its value by now: such a
-    value is read from that leaf's slot, and what it was computed from is not needed."""
+    value is read from that leaf's slot, and what it was computed from is not needed.
+    `pre`: operations computed once per row beforehand, handed in like the reductions
+    (a target is computed even when it is listed there)."""
     held = held or {}
     need, given = set(), set()
     leaves = {j for k, j in targets if k == "l"}
     stack = [j for k, j in targets if k == "v"]
+    own = set(stack)
     while stack:
         i = stack.pop()
         if i in need or i in given:
             continue
-        if prog.ops[i][0] in ROW_REDUCE:
+        if prog.ops[i][0] in ROW_REDUCE or (i in pre and i not in own):
             given.add(i)
             continue
         if i in held:
@@ -2443,13 +2446,13 @@ def _row_needed(prog, targets, held=None):
     return sorted(need), sorted(given), leaves
 
 
-def _row_function(prog, fname, targets, out_dtypes, held=None):
+def _row_function(prog, fname, targets, out_dtypes, held=None, pre=()):
     """Device function computing `targets` for one element (or one row, when every target
     is constant along the row): parameters are all leaf values, all scalars, the row
     reductions it reads, then one reference per target.  Returns (source, reductions read,
     leaves read)."""
     held = held or {}
-    need, given, used = _row_needed(prog, targets, held)
+    need, given, used = _row_needed(prog, targets, held, pre)
     params = [f"const {CTYPE[dt]} l{i}" for i, dt in enumerate(prog.leaves)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params += [f"const {CTYPE[prog.ops[i][2]]} v{i}" for i in given]
@@ -2470,20 +2473,20 @@ _ROW_CHEAP = frozenset(("add", "subtract", "multiply", "negative", "positive", "
                         "maximum", "minimum", "fmax", "fmin", "cast", "copysign", "where", "square"))
 
 
-def _row_carry(prog, need, later_targets, held, kept, uniform):
+def _row_carry(prog, need, later_targets, held, kept, uniform, pre=()):
     """Which value computed by this stage (operations `need`) to keep for the stages that
     follow, and where: (operation, leaf) or None.  A value qualifies when later stages read
     it, when it costs more than a few additions to compute again (an exponential, a
     quotient), and when there is an operand of its type that is held in registers and that
     the later stages read only through this value: its registers then hold the value
     instead.  softmax: exp(a - max) takes the place of a after the sum."""
-    later_need, _, _ = _row_needed(prog, later_targets, held)
+    later_need, _, _ = _row_needed(prog, later_targets, held, pre)
     for v in sorted(set(need) & set(later_need), reverse=True):
         name, _, rdt, _ = prog.ops[v]
         if uniform[v] or v in held:
             continue
         # what computing v again would cost: the operations below it down to what is at hand
-        below, _, leaves_of_v = _row_needed(prog, [("v", v)], held)
+        below, _, leaves_of_v = _row_needed(prog, [("v", v)], held, pre)
         if all(prog.ops[i][0] in _ROW_CHEAP for i in below):
             continue
         for leaf in sorted(leaves_of_v & kept):
@@ -2491,11 +2494,11 @@ def _row_carry(prog, need, later_targets, held, kept, uniform):
                 continue
             trial = dict(held)
             trial[v] = leaf
-            _, _, still = _row_needed(prog, later_targets, trial)
+            _, _, still = _row_needed(prog, later_targets, trial, pre)
             # the leaf's slot may be read later only as the carried value
             reads_leaf_itself = any(
                 ("l", leaf) in prog.ops[i][3]
-                for i in _row_needed(prog, later_targets, trial)[0] if i not in trial)
+                for i in _row_needed(prog, later_targets, trial, pre)[0] if i not in trial)
             if not reads_leaf_itself and not any(k == "l" and j == leaf for k, j in later_targets):
                 return v, leaf
     return None
@@ -2511,7 +2514,7 @@ def row_vector(prog, leaf_kind, out_dtypes, out_uniform):
 
 def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt_store=False,
                    fence=True, recompute=True, pipeline=True, carry_values=True, wave_map=False,
-                   nt_load=False):
+                   nt_load=False, hoist=True):
     """Rows that are reduced and used again: `a - max(a, axis=-1)`, softmax, the variance,
     layer normalisation.  A group of G lanes (1..64: part of a wave; 256 or 512: the block) owns a
     row of R elements (a compile-time constant, unit stride); lane j takes the 16-byte
@@ -2567,6 +2570,27 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     row_roots = [n for n in range(n_out) if out_uniform[n]]
     final_targets = [prog.roots[n][0] for n in elem_roots]
     stage_targets = [[prog.ops[i][3][0] for i in reds] for reds in stages]
+    # Values that are the same along a row and that per-element work reads (the mean
+    # `sum / n`, `sqrt(var + eps)`, `log(sum)`) are computed once per row, as soon as the
+    # reductions they depend on are made, and handed to the per-element functions like the
+    # reductions themselves: left inside, the compiler computes them for every element (a
+    # log-softmax of rows of 16384 issued 65 logarithms per lane for its 64 elements).
+    pre = set()
+    if hoist:
+        for n, (name, _, _, args) in enumerate(prog.ops):
+            if not uniform[n]:
+                pre |= {j for k, j in args
+                        if k == "v" and uniform[j] and prog.ops[j][0] not in ROW_REDUCE}
+    pre_by_level = {}
+    for i in sorted(pre):
+        pre_by_level.setdefault(level[i], []).append(i)
+    pre_fn = {}
+    for lv, ops_lv in sorted(pre_by_level.items()):
+        lower_pre = {i for i in pre if level[i] < lv}
+        text, given, _ = _row_function(prog, f"dr_once{lv}", [("v", i) for i in ops_lv],
+                                       [prog.ops[i][2] for i in ops_lv], pre=lower_pre)
+        src.append(text)
+        pre_fn[lv] = (ops_lv, given)
     stage_fn = []
     held = {}
     carried_leaves = set()
@@ -2576,12 +2600,12 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
         carry = None
         if carry_values:
             later = [t for ts in stage_targets[s + 1:] for t in ts] + final_targets
-            need, _, _ = _row_needed(prog, targets, held)
-            carry = _row_carry(prog, need, later, held, kept, uniform)
+            need, _, _ = _row_needed(prog, targets, held, pre)
+            carry = _row_carry(prog, need, later, held, kept, uniform, pre)
         if carry is not None:
             targets = targets + [("v", carry[0])]
             outs = outs + [prog.ops[carry[0]][2]]
-        text, given, used = _row_function(prog, f"dr_stage{s}", targets, outs, held)
+        text, given, used = _row_function(prog, f"dr_stage{s}", targets, outs, held, pre)
         src.append(text)
         stage_fn.append((given, used, carry))
         if carry is not None:
@@ -2591,7 +2615,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     final_used = set()
     if elem_roots:
         text, final_given, final_used = _row_function(
-            prog, "dr_final", final_targets, [out_dtypes[n] for n in elem_roots], held)
+            prog, "dr_final", final_targets, [out_dtypes[n] for n in elem_roots], held, pre)
         src.append(text)
     if row_roots:
         text, rowout_given, _ = _row_function(
@@ -2759,6 +2783,17 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     if rotate:
         L += row_pointers("        ", "nk", base="nrow", which=kept)
 
+    def once(lv, pad):
+        """The per-row values of level lv: computed by every lane (all get the same)."""
+        if lv not in pre_fn:
+            return []
+        ops_lv, given = pre_fn[lv]
+        args = [("0" if kind == "v" else f"c{i}") for i, kind in enumerate(leaf_kind)]
+        args += [f"s{i}" for i in range(ns)] + [f"v{g}" for g in given] + [f"v{i}" for i in ops_lv]
+        return [f"{pad}{CTYPE[prog.ops[i][2]]} v{i};" for i in ops_lv] + \
+               [f"{pad}dr_once{lv}({', '.join(args)});"]
+    L += once(0, "        ")
+
     def next_loads(j, pad):
         """The next row's units of step j, into the registers that step j has just used."""
         if not rotate:
@@ -2841,6 +2876,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
             where = f"({CTYPE[dt]}*)dr_slots[turn][{slot}]" if block_row else "nullptr"
             L.append(f"{pad}const {CTYPE[dt]} v{i} = dr_group_{op}_{dt}(acc{i}, {where});")
             slot += 1
+        L += once(s + 1, pad)
     # the roots
     store_guard = "" if block_row else "if (row < K) "
     if elem_roots:

@@ -73,6 +73,7 @@ TUNE = {
     "row_lanes": 0,   # ... lanes per row (0: by the cost of idle lanes and of units per lane)
     "row_regs": 128,  # ... registers that may hold the row between stages (else it is loaded again)
     "row_wavemap": -1,    # ... each wave of a block takes a quarter of the row (-1: rows of 48 KB up)
+    "row_hoist": 1,   # ... values that are the same along a row are computed once per row
     "row_carry": 1,   # ... a costly value read by later stages takes its operand's registers
     "row_pipe": 1,    # ... the next row is loaded while this one is finished and stored
     "row_fence": 1,   # ... the compiler keeps the work of one 16-byte unit together
@@ -399,13 +400,14 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     fence, recompute, pipe = bool(TUNE["row_fence"]), bool(TUNE["row_recompute"]), bool(TUNE["row_pipe"])
     carry = bool(TUNE["row_carry"])
     wmap = G >= cg.BLOCK and (steps >= 12 if TUNE["row_wavemap"] < 0 else bool(TUNE["row_wavemap"]))
+    hoist = bool(TUNE["row_hoist"])
     low.key = ("rows", prog.key(), tuple(kinds), tuple(out_codes), low.row_out, R, G, keep, nts,
-               fence, recompute, pipe, carry, wmap, ntl)
+               fence, recompute, pipe, carry, wmap, ntl) + (() if hoist else ("per element",))
 
     def emit():
         return cg.emit_row_fused(prog, kinds, out_codes, row_out, R, G, keep=keep, nt_store=nts,
                                  fence=fence, recompute=recompute, pipeline=pipe, carry_values=carry,
-                                 wave_map=wmap, nt_load=ntl)
+                                 wave_map=wmap, nt_load=ntl, hoist=hoist)
     low.emit = emit
     if G >= cg.BLOCK:
         blocks = K

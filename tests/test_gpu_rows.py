@@ -360,3 +360,41 @@ def test_rows_held_by_a_block_of_512_lanes_replay_with_that_block():
         rep()
         hip.synchronize()
         np.testing.assert_allclose(out.get(), (ref, softmax(np, b))[k % 2], rtol=2e-6)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_values_computed_once_per_row_give_the_same_bits_as_per_element(dtype):
+    """The mean `sum / n`, `sqrt(var + eps)`, `log(sum)` are the same along a row: computed
+    once per row and handed to the per-element work, or computed for every element
+    (`row_hoist=0`), the results are the same bits; both agree with NumPy."""
+    rs = np.random.RandomState(13)
+    a = (rs.standard_normal((40, 3001)) * 2 + 1).astype(dtype)
+    w = rs.standard_normal(3001).astype(dtype)
+    col = rs.standard_normal((40, 1)).astype(dtype)
+
+    def layer_norm(xp, x, g):
+        mu = x.mean(axis=-1, keepdims=True)
+        d = x - mu
+        return d / xp.sqrt((d * d).mean(axis=-1, keepdims=True) + 1e-5) * g
+
+    def log_softmax(xp, x, g):
+        s = x - x.max(axis=-1, keepdims=True)
+        return s - xp.log(xp.exp(s).sum(axis=-1, keepdims=True))
+
+    def scaled(xp, x, g, c):            # a value per row that no reduction feeds: level 0
+        return x * xp.exp(c) + x.sum(axis=-1, keepdims=True) / xp.exp(c)
+    tol = dict(rtol=3e-5, atol=3e-5) if dtype == np.float32 else dict(rtol=1e-11, atol=1e-11)
+    for fn, extra in ((layer_norm, ()), (log_softmax, ()), (scaled, (col,))):
+        got = {}
+        for hoist in (1, 0):
+            hip.set_tune(row_hoist=hoist)
+            try:
+                args = [dr.array(a), dr.array(w)] + [dr.array(e) for e in extra]
+                low, src = hip.lower_only(fn(dr, *args))
+                assert low.kind == "rows" and ("dr_once" in src) == bool(hoist), fn.__name__
+                got[hoist], n = launches(lambda: fn(dr, *args).get())
+                assert n == 1
+            finally:
+                hip.set_tune(row_hoist=1)
+        assert bits_equal(got[0], got[1]), fn.__name__
+        np.testing.assert_allclose(got[1], fn(np, a, w, *extra), **tol)
