@@ -282,7 +282,7 @@ def _lower_stencil3d(low, prog, leaves, m_leaf, m_out, mshape, out_codes, out_pt
     return low
 
 
-def _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V):
+def _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V, uniform=None):
     """Lanes per row for the row kernel: the candidate with the least estimated time per
     row.  The estimate has a memory term and an arithmetic term, fitted to measurements on
     MI355X (`a - max(a)` and softmax, float32 and float64, rows of 16 to 4096 elements,
@@ -309,8 +309,11 @@ def _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V):
     dense = all(st == R for k, st in zip(kinds, sk) if k == "v" and st)
     moved = sum(a.dtype.itemsize for a, k, st in zip(leaves, kinds, sk) if k == "v" and st) \
         + sum(cg.ITEMSIZE[c] for c, u in zip(out_codes, row_out) if not u)
+    # per element: what is the same along the row is computed once per row
     work = sum(10 if (name in cg._FLOAT_FUNCS1 or name in cg._FLOAT_FUNCS2 or name in
-                      ("divide", "true_divide", "reciprocal")) else 1 for name, _, _, _ in prog.ops)
+                      ("divide", "true_divide", "reciprocal")) else 1
+               for i, (name, _, _, _) in enumerate(prog.ops)
+               if uniform is None or not uniform[i] or name in cg.ROW_REDUCE)
     if any(cdt == "f8" for _, cdt, _, _ in prog.ops):
         work *= 2
     ratio = 0.26 * work / max(moved, 1)
@@ -379,7 +382,8 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     units = -(-R // V)
     G = TUNE["row_lanes"]
     if not G:
-        G = _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V)
+        G = _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V,
+                       uniform if TUNE["row_hoist"] else None)
     steps = -(-units // G)
     if steps > _row_steps_max(G) or K >= 2 ** 40:
         raise cg.RowFusionUnsupported("row too long")
