@@ -387,7 +387,9 @@ def test_values_computed_once_per_row_give_the_same_bits_as_per_element(dtype):
     for fn, extra in ((layer_norm, ()), (log_softmax, ()), (scaled, (col,))):
         got = {}
         for hoist in (1, 0):
-            hip.set_tune(row_hoist=hoist)
+            # the same lanes per row both times (the choice counts per-element work, which
+            # differs between the two, and the order of a sum follows the lanes)
+            hip.set_tune(row_hoist=hoist, row_lanes=256)
             try:
                 args = [dr.array(a), dr.array(w)] + [dr.array(e) for e in extra]
                 low, src = hip.lower_only(fn(dr, *args))
@@ -395,6 +397,6 @@ def test_values_computed_once_per_row_give_the_same_bits_as_per_element(dtype):
                 got[hoist], n = launches(lambda: fn(dr, *args).get())
                 assert n == 1
             finally:
-                hip.set_tune(row_hoist=1)
+                hip.set_tune(row_hoist=1, row_lanes=0)
         assert bits_equal(got[0], got[1]), fn.__name__
         np.testing.assert_allclose(got[1], fn(np, a, w, *extra), **tol)
