@@ -400,3 +400,27 @@ def test_values_computed_once_per_row_give_the_same_bits_as_per_element(dtype):
                 hip.set_tune(row_hoist=1, row_lanes=0)
         assert bits_equal(got[0], got[1]), fn.__name__
         np.testing.assert_allclose(got[1], fn(np, a, w, *extra), **tol)
+
+
+def test_rows_beyond_2_to_31_elements():
+    """Row kernels address with 64 bits: 70000 rows of 32768 float32 (2.29e9 elements,
+    9.2 GB in, 9.2 GB out, a block of 512 lanes per row); rows on both sides of the
+    2^31-element boundary and the last row agree with NumPy."""
+    K, R = 70000, 32768
+    rs = np.random.RandomState(14)
+    x = dr.zeros((K, R), dtype=np.float32)
+    edge = (1 << 31) // R                       # first row that starts at element 2^31
+    picked = {0: None, edge - 1: None, edge: None, edge + 1: None, K - 1: None}
+    for k in picked:
+        picked[k] = rs.standard_normal(R).astype(np.float32)
+        x[k] = picked[k]
+    out, n = launches(lambda: hip.run(softmax(dr, x)))
+    assert n == 1 and out.shape == (K, R)
+    for k, row in picked.items():
+        np.testing.assert_allclose(out[k].get(), softmax(np, row[None])[0], rtol=2e-6, err_msg=str(k))
+    np.testing.assert_allclose(out[edge + 7].get(), np.full(R, 1.0 / R, np.float32), rtol=1e-6)
+    del out
+    small, n = launches(lambda: hip.run(x[:, :96] - x[:, :96].max(axis=1, keepdims=True)))
+    assert n == 1                               # lane groups, rows 128 KB apart
+    for k, row in picked.items():
+        assert bits_equal(small[k].get(), row[:96] - row[:96].max())
