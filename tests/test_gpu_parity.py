@@ -1730,3 +1730,23 @@ def test_quotients_inside_functions_and_quotients_that_are_results(dtype):
         assert np.array_equal(np.isnan(g2), np.isnan(want))
         tol = (4 if dtype == np.float32 else 900) * eps * np.maximum(np.abs(want[ok]).astype(np.float64), 1.0)
         assert np.all(np.abs(g2[ok].astype(np.float64) - want[ok].astype(np.float64)) <= tol)
+
+
+def test_device_random_draws_of_more_than_2_to_31_numbers():
+    """One draw of 2^31 + 2^20 + 3 doubles (17 GB): positions are 64-bit, so the numbers
+    around element 2^31 and the last ones equal NumPy's stream advanced to that place, and
+    the draw after it continues where NumPy's would."""
+    n = (1 << 31) + (1 << 20) + 3
+    gen = dr.random.device(21)
+    big = gen.random(n)
+    big.run()
+
+    def numpy_at(start, count):
+        bits = np.random.Philox(key=21)
+        bits.advance(start // 4)                    # four outputs per block
+        return np.random.Generator(bits).random(start % 4 + count)[start % 4:]
+    for start, count in ((0, 9), ((1 << 31) - 5, 11), (n - 7, 7)):
+        assert np.array_equal(big[start:start + count].get(), numpy_at(start, count)), start
+    assert np.array_equal(gen.random(6).get(), numpy_at(n, 6))
+    total = float(dr.sum(big))
+    assert abs(total / n - 0.5) < 1e-4
