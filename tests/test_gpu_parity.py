@@ -1750,3 +1750,75 @@ def test_device_random_draws_of_more_than_2_to_31_numbers():
     assert np.array_equal(gen.random(6).get(), numpy_at(n, 6))
     total = float(dr.sum(big))
     assert abs(total / n - 0.5) < 1e-4
+
+
+def test_two_dimensional_kernels_on_more_than_2_to_31_elements():
+    """A 46400 x 46400 float32 matrix (2.15e9 elements, 8.6 GB) built on the device as
+    `col[:, None] + row[None, :]`, so that NumPy can compute any entry: the tiled kernels
+    (transpose, broadcast, stencil), the axis reductions, strided columns and the row kernel
+    address rows and tiles on both sides of element 2^31 correctly."""
+    N = M = 46400
+    rs = np.random.RandomState(0)
+    col = rs.standard_normal(N).astype(np.float32)
+    row = rs.standard_normal(M).astype(np.float32)
+    a = dr.array(col)[:, None] + dr.array(row)[None, :]
+    a.run()
+
+    def entries(i, j):
+        return (col[i][:, None] + row[j][None, :]).astype(np.float32)
+    I = np.array([0, 1, 46339, 46340, 46341, N - 2, N - 1])       # 2^31 / 46400 = 46282.4
+    I = np.concatenate([I, [46281, 46282, 46283]])
+    J = np.array([0, 5, 4095, 4096, M - 3, M - 1])
+    t = hip.run(a.T * 2.0)
+    assert np.array_equal(np.stack([t[j].get()[I] for j in J]), (entries(I, J) * 2).T)
+    del t
+    b = hip.run(a + dr.array(row))
+    assert np.array_equal(np.stack([b[i].get()[J] for i in I]), entries(I, J) + row[J])
+    del b
+    st = hip.run(0.25 * (a[:-2, 1:-1] + a[2:, 1:-1] + a[1:-1, :-2] + a[1:-1, 2:]))
+    ii, jj = np.array([0, 46280, 46281, 46282, 46283, N - 3]), np.array([0, 4094, 4095, M - 3])
+    ref = np.float32(0.25) * (((entries(ii, jj + 1) + entries(ii + 2, jj + 1)) + entries(ii + 1, jj))
+                              + entries(ii + 1, jj + 2))
+    assert np.array_equal(np.stack([st[i].get()[jj] for i in ii]), ref)
+    del st
+    s0, s1 = dr.sum(a, axis=0).get(), dr.sum(a, axis=1).get()
+    np.testing.assert_allclose(s0[J], col.astype(np.float64).sum() + N * row[J].astype(np.float64), rtol=1e-5, atol=0.5)
+    np.testing.assert_allclose(s1[I], M * col[I].astype(np.float64) + row.astype(np.float64).sum(), rtol=1e-5, atol=0.5)
+    v = hip.run(a[:, ::2] * 2.0)
+    assert np.array_equal(np.stack([v[i].get()[J[:4] // 2] for i in I]), entries(I, (J[:4] // 2) * 2) * 2)
+    del v
+    r = hip.run(a[:, :4096] - a[:, :4096].max(axis=1, keepdims=True))
+    assert np.array_equal(np.stack([r[i].get()[:64] for i in I]),
+                          entries(I, np.arange(64)) - (col[I] + row[:4096].max())[:, None])
+
+
+def test_three_dimensional_kernels_on_more_than_2_to_31_elements():
+    """1300^3 float32 (2.2e9 elements) built on the device as x[i] + y[j] + z[k]: the
+    transpose over all axes, the 7-point stencil and a reduction along the middle axis,
+    checked at entries on both sides of element 2^31 (plane 1270.7)."""
+    N = 1300
+    rs = np.random.RandomState(1)
+    x, y, z = (rs.standard_normal(N).astype(np.float32) for _ in range(3))
+    a = (dr.array(x)[:, None, None] + dr.array(y)[None, :, None]) + dr.array(z)[None, None, :]
+    a.run()
+
+    def entries(i, j, k):
+        return ((x[i][:, None, None] + y[j][None, :, None]) + z[k][None, None, :]).astype(np.float32)
+
+    def pick(arr, I, J, K):
+        return np.stack([np.stack([arr[i, j].get()[K] for j in J]) for i in I])
+    I, J = np.array([0, 1269, 1270, 1271, 1272, N - 3]), np.array([0, 700, 1000, N - 3])
+    K = np.array([0, 3, 4, 1023, 1024, N - 3])
+    t = hip.run(a.T * 2.0)
+    assert np.array_equal(pick(t, K, J, I), np.transpose(entries(I, J, K) * 2, (2, 1, 0)))
+    del t
+    st = hip.run((1.0 / 6.0) * (a[:-2, 1:-1, 1:-1] + a[2:, 1:-1, 1:-1] + a[1:-1, :-2, 1:-1]
+                                + a[1:-1, 2:, 1:-1] + a[1:-1, 1:-1, :-2] + a[1:-1, 1:-1, 2:]))
+    ref = np.float32(1.0 / 6.0) * (((((entries(I, J + 1, K + 1) + entries(I + 2, J + 1, K + 1))
+                                      + entries(I + 1, J, K + 1)) + entries(I + 1, J + 2, K + 1))
+                                    + entries(I + 1, J + 1, K)) + entries(I + 1, J + 1, K + 2))
+    assert np.array_equal(pick(st, I, J, K), ref)
+    del st
+    s = dr.sum(a, axis=1).get()
+    np.testing.assert_allclose(s[I][:, K], N * (x[I][:, None] + z[K][None, :]).astype(np.float64)
+                               + y.astype(np.float64).sum(), rtol=1e-5, atol=0.5)
