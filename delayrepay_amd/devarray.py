@@ -9,6 +9,7 @@ returns views of the same buffer, as the front end's `__getitem__` /
 goes through libdrhip; nothing here computes on the host.
 """
 import numbers
+import warnings
 
 import numpy as np
 import numpy.lib.mixins
@@ -17,6 +18,7 @@ from . import hiprt
 
 _CHECKED_DTYPES = set()
 SUPPORTED_DTYPES = ("float32", "float64", "int32", "int64", "bool", "uint8", "uint32")
+_WIDENED = set()        # types whose widening on upload has been announced
 
 
 class Buffer:
@@ -146,12 +148,24 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
         if not host.flags.c_contiguous:       # (ascontiguousarray would make 0-d into 1-d)
             host = np.ascontiguousarray(host)
         if host.dtype.name not in SUPPORTED_DTYPES:
+            # Types without a device form are widened to one that holds every value (said
+            # once per type: the result's dtype, and with it the rounding or wrap-around
+            # of later arithmetic, is then the wider type's, not NumPy's for the narrow one).
             if host.dtype.kind in "iu":
-                host = host.astype(np.int64)
-            elif host.dtype.kind == "f":
-                host = host.astype(np.float64)
+                if host.dtype == np.uint64 and host.size and int(host.max()) > np.iinfo(np.int64).max:
+                    raise OverflowError("uint64 values of 2**63 and more have no device form "
+                                        "(uint64 arrays are held as int64)")
+                wide = np.int64
+            elif host.dtype.kind == "f" and host.dtype.itemsize < 4:
+                wide = np.float64
             else:
                 raise TypeError(f"dtype {host.dtype} is not supported on the device")
+            if host.dtype.name not in _WIDENED:
+                _WIDENED.add(host.dtype.name)
+                warnings.warn(f"delayrepay_amd: {host.dtype.name} arrays are held as "
+                              f"{np.dtype(wide).name} on the device; results have that type",
+                              RuntimeWarning, stacklevel=3)
+            host = host.astype(wide)
         out = cls(host.shape, host.dtype)
         if host.nbytes:
             hiprt.memcpy_h2d(out.buf.ptr, host.ctypes.data, host.nbytes)

@@ -1421,8 +1421,8 @@ def test_transposes_of_arrays_with_more_than_two_dimensions_go_through_the_lds_t
     import itertools
     rs = np.random.RandomState(37)
     for shape, dt in [((5, 70, 33), np.float32), ((3, 4, 130, 9), np.float64), ((40, 36, 64), np.float32),
-                      ((6, 50, 20), np.int8)]:
-        h = (rs.uniform(-3, 3, shape) if dt != np.int8 else rs.randint(-9, 9, shape)).astype(dt)
+                      ((6, 50, 20), np.int64)]:
+        h = (rs.uniform(-3, 3, shape) if dt != np.int64 else rs.randint(-9, 9, shape)).astype(dt)
         a = dr.array(h)
         for perm in itertools.permutations(range(len(shape))):
             if perm[-1] == len(shape) - 1:
@@ -1822,3 +1822,31 @@ def test_three_dimensional_kernels_on_more_than_2_to_31_elements():
     s = dr.sum(a, axis=1).get()
     np.testing.assert_allclose(s[I][:, K], N * (x[I][:, None] + z[K][None, :]).astype(np.float64)
                                + y.astype(np.float64).sum(), rtol=1e-5, atol=0.5)
+
+
+def test_types_without_a_device_form_are_widened_aloud_or_refused():
+    """float16, int8, int16, uint16 and uint64 arrays are held as float64 / int64: every
+    value is kept, the results have the wide type, and the first upload of each type says
+    so.  What cannot be kept is refused: uint64 values of 2^63 and more, long double,
+    complex numbers."""
+    import warnings
+    from delayrepay_amd import devarray
+    rs = np.random.RandomState(5)
+    for dt, wide in ((np.float16, np.float64), (np.int8, np.int64), (np.int16, np.int64),
+                     (np.uint16, np.int64), (np.uint64, np.int64)):
+        h = rs.standard_normal(1000) * 10
+        h = (np.abs(h) if np.dtype(dt).kind == "u" else h).astype(dt)
+        devarray._WIDENED.discard(np.dtype(dt).name)
+        with pytest.warns(RuntimeWarning, match=np.dtype(dt).name):
+            a = dr.array(h)
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")              # said once per type
+            b = dr.array(h)
+        assert a.dtype == wide and b.dtype == wide
+        got = (a * 3 + b).get()
+        assert got.dtype == wide and np.array_equal(got, h.astype(wide) * 3 + h.astype(wide))
+    with pytest.raises(OverflowError):
+        dr.array(np.array([1, 2 ** 63], dtype=np.uint64))
+    for bad in (np.ones(3, np.longdouble), np.ones(3, np.complex64), np.ones(3, np.complex128)):
+        with pytest.raises(TypeError):
+            dr.array(bad)
