@@ -157,7 +157,7 @@ class ndarray(numpy.lib.mixins.NDArrayOperatorsMixin):
                                         "(uint64 arrays are held as int64)")
                 wide = np.int64
             elif host.dtype.kind == "f" and host.dtype.itemsize < 4:
-                wide = np.float64
+                wide = np.float32
             else:
                 raise TypeError(f"dtype {host.dtype} is not supported on the device")
             if host.dtype.name not in _WIDENED:

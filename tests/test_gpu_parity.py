@@ -1825,14 +1825,14 @@ def test_three_dimensional_kernels_on_more_than_2_to_31_elements():
 
 
 def test_types_without_a_device_form_are_widened_aloud_or_refused():
-    """float16, int8, int16, uint16 and uint64 arrays are held as float64 / int64: every
+    """float16, int8, int16, uint16 and uint64 arrays are held as float32 / int64: every
     value is kept, the results have the wide type, and the first upload of each type says
     so.  What cannot be kept is refused: uint64 values of 2^63 and more, long double,
     complex numbers."""
     import warnings
     from delayrepay_amd import devarray
     rs = np.random.RandomState(5)
-    for dt, wide in ((np.float16, np.float64), (np.int8, np.int64), (np.int16, np.int64),
+    for dt, wide in ((np.float16, np.float32), (np.int8, np.int64), (np.int16, np.int64),
                      (np.uint16, np.int64), (np.uint64, np.int64)):
         h = rs.standard_normal(1000) * 10
         h = (np.abs(h) if np.dtype(dt).kind == "u" else h).astype(dt)
