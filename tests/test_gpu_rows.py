@@ -360,6 +360,14 @@ def test_rows_held_by_a_block_of_512_lanes_replay_with_that_block():
         rep()
         hip.synchronize()
         np.testing.assert_allclose(out.get(), (ref, softmax(np, b))[k % 2], rtol=2e-6)
+    # fresh arrays through the same expression: plans made from the remembered structure
+    hits = hip.STATS["seen_hits"]
+    for k in range(6):
+        h = rs.standard_normal((24, 50257)).astype(np.float32)
+        got, n = launches(lambda: softmax(dr, dr.array(h)).get())
+        assert n == 1
+        np.testing.assert_allclose(got, softmax(np, h), rtol=2e-6)
+    assert hip.STATS["seen_hits"] > hits
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
