@@ -1879,9 +1879,9 @@ def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
          "        const long long k = row < K ? row : K - 1;      // idle groups re-read the last row"]
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
-            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + {row_at(i, 'k')};")
         else:
-            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[{row_at(i, 'k')}];")
     L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
 
     def element(args, pad):
@@ -2514,7 +2514,7 @@ def row_vector(prog, leaf_kind, out_dtypes, out_uniform):
 
 def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt_store=False,
                    fence=True, recompute=True, pipeline=True, carry_values=True, wave_map=False,
-                   nt_load=False, hoist=True):
+                   nt_load=False, hoist=True, outer2=False):
     """Rows that are reduced and used again: `a - max(a, axis=-1)`, softmax, the variance,
     layer normalisation.  A group of G lanes (1..64: part of a wave; 256 or 512: the block) owns a
     row of R elements (a compile-time constant, unit stride); lane j takes the 16-byte
@@ -2656,6 +2656,19 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     params.append("const long long K")
     params += [f"const long long sk{i}" for i in range(nl)]
     params += [f"const long long so{n}" for n in range(n_out)]
+    if outer2:
+        # rows counted over two levels, K = K0 * K1, that some operand does not walk as one
+        # sequence (a matrix repeated for every item of a batch): row k of operand i starts
+        # at (k / K1) * sk_i + (k % K1) * sj_i
+        params.append("const unsigned int K1")
+        params += [f"const long long sj{i}" for i in range(nl)]
+        src.append("__device__ __forceinline__ long long dr_row_at(const long long k, const unsigned int K1, "
+                   "const long long s0, const long long s1)\n{\n"
+                   "    const unsigned int q = (unsigned int)k / K1;\n"
+                   "    return (long long)q * s0 + (long long)((unsigned int)k - q * K1) * s1;\n}")
+
+    def row_at(i, k):
+        return f"dr_row_at({k}, K1, sk{i}, sj{i})" if outer2 else f"{k} * sk{i}"
     scal = [f"s{i}" for i in range(ns)]
     L = [f'extern "C" __global__ __launch_bounds__({B})',
          f"void dr_kernel({', '.join(params)})", "{"]
@@ -2721,7 +2734,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
         out = []
         for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
             if kind == "v" and (which is None or i in which):
-                out.append(f"{pad}const {CTYPE[dt]}* {base}{i} = a{i} + {k} * sk{i};")
+                out.append(f"{pad}const {CTYPE[dt]}* {base}{i} = a{i} + {row_at(i, k)};")
         return out
 
     # Rows in turn: the registers that hold a row are filled for the next row as soon as
@@ -2777,9 +2790,9 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
                   "        const long long nk = more ? (first + stride + grp < K ? first + stride + grp : K - 1) : k;"]
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
-            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + {row_at(i, 'k')};")
         else:
-            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[{row_at(i, 'k')}];")
     if rotate:
         L += row_pointers("        ", "nk", base="nrow", which=kept)
 

@@ -370,10 +370,18 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     for k in range(len(shape) - 2, -1, -1):
         dense[k] = dense[k + 1] * shape[k + 1]
     mshape, msets = merge_dims(shape[:-1], [st[:-1] for st in strides] + [dense[:-1]])
-    if len(mshape) > 1:
+    sj = None
+    if len(mshape) == 2 and mshape[0] * mshape[1] < 2 ** 31:
+        # two levels of rows (a matrix added to every item of a batch before the rows are
+        # normalised): the kernel splits the row number
+        K, K1 = mshape[0] * mshape[1], mshape[1]
+        sk = [st[0] for st in msets[:-1]]
+        sj = [st[1] for st in msets[:-1]]
+    elif len(mshape) > 1:
         raise cg.RowFusionUnsupported("rows that do not form one sequence in every operand")
-    K = mshape[0] if mshape else 1
-    sk = [st[0] if st else 0 for st in msets[:-1]]
+    else:
+        K = mshape[0] if mshape else 1
+        sk = [st[0] if st else 0 for st in msets[:-1]]
     level, uniform, stages = cg.row_analysis(prog, kinds)
     row_out = []
     for (kind, j), _ in prog.roots:
@@ -382,7 +390,8 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     units = -(-R // V)
     G = TUNE["row_lanes"]
     if not G:
-        G = _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V,
+        G = _row_lanes(prog, leaves, kinds, [b or a for a, b in zip(sk, sj)] if sj else sk,
+                       out_codes, row_out, R, V,
                        uniform if TUNE["row_hoist"] else None)
     steps = -(-units // G)
     if steps > _row_steps_max(G) or K >= 2 ** 40:
@@ -390,7 +399,8 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     # An operand's share of its row stays in registers between the stages, as long as all
     # of them fit; operands that are the same for every row (a vector of weights) come from
     # the caches every time.
-    own = [k == "v" and st != 0 for k, st in zip(kinds, sk)]
+    own = [k == "v" and (st != 0 or (sj is not None and sj[i] != 0))
+           for i, (k, st) in enumerate(zip(kinds, sk))]
     keep = tuple(o and steps * 4 * sum(own) <= TUNE["row_regs"] for o in own)
     footprint = sum(a.nbytes for a in leaves) + sum(K * (1 if u else R) * cg.ITEMSIZE[c]
                                                    for c, u in zip(out_codes, row_out))
@@ -406,12 +416,13 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     wmap = G >= cg.BLOCK and (steps >= 12 if TUNE["row_wavemap"] < 0 else bool(TUNE["row_wavemap"]))
     hoist = bool(TUNE["row_hoist"])
     low.key = ("rows", prog.key(), tuple(kinds), tuple(out_codes), low.row_out, R, G, keep, nts,
-               fence, recompute, pipe, carry, wmap, ntl) + (() if hoist else ("per element",))
+               fence, recompute, pipe, carry, wmap, ntl) + (() if hoist else ("per element",)) \
+        + (("two levels",) if sj else ())
 
     def emit():
         return cg.emit_row_fused(prog, kinds, out_codes, row_out, R, G, keep=keep, nt_store=nts,
                                  fence=fence, recompute=recompute, pipeline=pipe, carry_values=carry,
-                                 wave_map=wmap, nt_load=ntl, hoist=hoist)
+                                 wave_map=wmap, nt_load=ntl, hoist=hoist, outer2=bool(sj))
     low.emit = emit
     if G >= cg.BLOCK:
         blocks = K
@@ -424,10 +435,10 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     cap = grid_cap() * TUNE["row_bpc"] // max(TUNE["bpc"], 1) if TUNE["row_bpc"] else (1 << 24) - 1
     low.grid = max(1, min(blocks, cap))
     low.fmt = "@" + "P" * (len(leaves) + len(out_codes)) + "".join(_SCALAR_FMT[c] for c in prog.scalars) \
-        + "q" * (1 + len(leaves) + len(out_codes))
+        + "q" * (1 + len(leaves) + len(out_codes)) + ("I" + "q" * len(leaves) if sj else "")
     low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
     low.scal = list(scalars)
-    low.tail = [K] + sk + [1 if u else R for u in row_out]
+    low.tail = [K] + sk + [1 if u else R for u in row_out] + ([K1] + sj if sj else [])
     return low
 
 

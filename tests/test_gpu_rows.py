@@ -432,3 +432,47 @@ def test_rows_beyond_2_to_31_elements():
     assert n == 1                               # lane groups, rows 128 KB apart
     for k, row in picked.items():
         assert bits_equal(small[k].get(), row[:96] - row[:96].max())
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_operands_repeated_over_a_batch_stay_in_the_row_kernel(dtype):
+    """`softmax(scores + mask)` with a mask per (row, column) shared by every item of the
+    batch, `layer_norm(x + positions)`, a vector per batch item: the rows are counted over two
+    levels (batch, row) that the repeated operand does not walk as one sequence; one
+    kernel, which splits the row number."""
+    rs = np.random.RandomState(15)
+    B, N = 6, 37
+    for R in (40, 257, 1000, 5000):
+        x = rs.standard_normal((B, N, R)).astype(dtype)
+        mask = np.where(rs.uniform(size=(N, R)) < 0.2, -np.inf, 0.0).astype(dtype)
+        mask[:, 0] = 0.0                                       # no row without a finite entry
+        pos = rs.standard_normal((N, R)).astype(dtype)
+        per_item = rs.standard_normal((B, 1, R)).astype(dtype)
+        dx, dm, dp, dv = dr.array(x), dr.array(mask), dr.array(pos), dr.array(per_item)
+        got, n = launches(lambda: softmax(dr, dx + dm).get())
+        assert n == 1, R
+        np.testing.assert_allclose(got, softmax(np, x + mask), rtol=2e-6 if dtype == np.float32 else 1e-13)
+        got, n = launches(lambda: ((dx + dp) - (dx + dp).max(axis=-1, keepdims=True)).get())
+        assert n == 1 and bits_equal(got, (x + pos) - (x + pos).max(axis=-1, keepdims=True))
+        got, n = launches(lambda: ((dx * dv + dp) - (dx * dv + dp).min(axis=-1, keepdims=True)).get())
+        ref = (x * per_item + pos) - (x * per_item + pos).min(axis=-1, keepdims=True)
+        assert n == 1 and bits_equal(got, ref)
+
+        def layer_norm(xp, a, p):
+            s = a + p
+            d = s - s.mean(axis=-1, keepdims=True)
+            return d / xp.sqrt((d * d).mean(axis=-1, keepdims=True) + 1e-5)
+        got, n = launches(lambda: layer_norm(dr, dx, dp).get())
+        assert n == 1
+        tol = dict(rtol=3e-5, atol=3e-5) if dtype == np.float32 else dict(rtol=1e-11, atol=1e-11)
+        np.testing.assert_allclose(got, layer_norm(np, x, pos), **tol)
+        # the batch as a view: every second item, rows still two levels
+        got, n = launches(lambda: softmax(dr, dx[::2] + dm).get())
+        assert n == 1
+        np.testing.assert_allclose(got, softmax(np, x[::2] + mask), rtol=2e-6 if dtype == np.float32 else 1e-13)
+    # three levels that do not merge: the long way, same values
+    y = rs.standard_normal((3, 4, 5, 64)).astype(dtype)
+    m2 = rs.standard_normal((4, 1, 64)).astype(dtype)
+    dy, dm2 = dr.array(y), dr.array(m2)
+    got = ((dy + dm2) - (dy + dm2).max(axis=-1, keepdims=True)).get()
+    assert bits_equal(got, (y + m2) - (y + m2).max(axis=-1, keepdims=True))
