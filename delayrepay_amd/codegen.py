@@ -1879,9 +1879,9 @@ def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
          "        const long long k = row < K ? row : K - 1;      // idle groups re-read the last row"]
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
-            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + {row_at(i, 'k')};")
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
         else:
-            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[{row_at(i, 'k')}];")
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
     L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
 
     def element(args, pad):

@@ -638,3 +638,18 @@ def test_long_rows_take_a_block_of_512_lanes_and_compile():
             hip.lower_only(soft(leaf((64, R), dtype)))
     low, _ = hip.lower_only(leaf((64, 50257)) * 2.0)
     assert lowering.block_lanes(low) == cg.BLOCK
+
+
+def test_every_axis_reduction_kernel_shape_is_emitted_and_compiles():
+    """One case per strategy of the reductions along axes (a block, a lane group or a wave
+    per output row, a thread per output column, streams over a middle axis, the narrow and
+    short forms): lowered over placeholders, the source generated and put through hiprtc."""
+    cases = {"axis_block": ((16384, 16384), (1,)), "axis_stream": ((256, 512, 1024), (1,)),
+             "axis_group": ((1342177, 200), (1,)), "axis_row": ((37, 70, 129), (0, 2)),
+             "axis_col": ((129, 70), (0,)), "axis_narrow": ((1 << 22, 8), (0,)),
+             "axis_short": ((1 << 20, 4), (1,))}
+    for kind, (shape, axes) in cases.items():
+        for func, dtype in ((np.add, np.float32), (np.maximum, np.float64)):
+            low, src = hip.lower_only(ReduceEx(func, leaf(shape, dtype) * 2.0, axes))
+            assert low.kind == kind, (kind, low.kind, dtype)
+            hip.compile_source(src)
