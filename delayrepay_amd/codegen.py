@@ -1781,7 +1781,7 @@ def emit_narrow_cols(prog, leaf_kind, acc_dt, op, K):
     return "\n".join(src) + "\n", V, LW
 
 
-def emit_short_rows(prog, leaf_kind, acc_dt, op, R):
+def emit_short_rows(prog, leaf_kind, acc_dt, op, R, outer2=False):
     """Reduction over a short unit-stride last dimension: a lane owns one output and
     walks its own row of R elements (R is a compile-time constant) with 16-byte loads
     at element alignment.  The lanes' loads are a row pitch apart, but a wave's R
@@ -1802,6 +1802,10 @@ def emit_short_rows(prog, leaf_kind, acc_dt, op, R):
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params.append("const long long K")
     params += [f"const long long sk{i}" for i in range(nl)]
+    if outer2:
+        params.append("const unsigned int K1")
+        params += [f"const long long sj{i}" for i in range(nl)]
+        src.append(ROW_AT)
     call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
          f"void dr_kernel({', '.join(params)})", "{",
@@ -1809,9 +1813,9 @@ def emit_short_rows(prog, leaf_kind, acc_dt, op, R):
          "    if (k >= K) return;"]
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
-            L.append(f"    const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+            L.append(f"    const {CTYPE[dt]}* row{i} = a{i} + {_row_at(outer2, i, 'k')};")
         else:
-            L.append(f"    const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+            L.append(f"    const {CTYPE[dt]} c{i} = a{i}[{_row_at(outer2, i, 'k')}];")
     L.append(f"    {ct} acc = {_identity(op, acc_dt)};")
 
     def element(args):
@@ -1838,7 +1842,7 @@ def emit_short_rows(prog, leaf_kind, acc_dt, op, R):
     return "\n".join(src) + "\n"
 
 
-def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
+def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G, outer2=False):
     """Reduction over a unit-stride last dimension of R elements (a compile-time
     constant) by groups of G lanes (G a power of two, 8..64): a wave holds 64 / G rows at a
     time, lane j of a group takes the 16-byte units j, j + G, ... of its row (a group reads
@@ -1864,6 +1868,10 @@ def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params.append("const long long K")
     params += [f"const long long sk{i}" for i in range(nl)]
+    if outer2:
+        params.append("const unsigned int K1")
+        params += [f"const long long sj{i}" for i in range(nl)]
+        src.append(ROW_AT)
     call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
     shfl = "__shfl_xor(acc, off, 64)"
     if acc_dt in ("u1", "b1"):
@@ -1879,9 +1887,9 @@ def emit_group_rows(prog, leaf_kind, acc_dt, op, R, G):
          "        const long long k = row < K ? row : K - 1;      // idle groups re-read the last row"]
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
-            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + k * sk{i};")
+            L.append(f"        const {CTYPE[dt]}* row{i} = a{i} + {_row_at(outer2, i, 'k')};")
         else:
-            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[k * sk{i}];")
+            L.append(f"        const {CTYPE[dt]} c{i} = a{i}[{_row_at(outer2, i, 'k')}];")
     L.append(f"        {ct} acc = {_identity(op, acc_dt)};")
 
     def element(args, pad):
@@ -2018,7 +2026,7 @@ def emit_col_stream(prog, leaf_kind, acc_dt, op, unroll=8, outer=False, stagger=
     return "\n".join(src) + "\n"
 
 
-def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False, shared=()):
+def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False, shared=(), outer2=False):
     """Reduction over a long unit-stride last dimension: a block per (row, slice) streams
     its stretch of the row like a flat reduction (256 lanes x 16 bytes x `unroll` per step,
     one accumulator per vector element), combines through `dr_block_reduce` and writes one
@@ -2049,6 +2057,11 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False, shared=(
     if outer:
         params.append("const long long RO")
         params += [f"const long long so{i}" for i in range(nl)]
+    if outer2:
+        assert not outer
+        params.append("const unsigned int K1")
+        params += [f"const long long sj{i}" for i in range(nl)]
+        src.append(ROW_AT)
     call_tail = [f"s{i}" for i in range(len(prog.scalars))] + ["t0"]
     ident = _identity(op, acc_dt)
     L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
@@ -2069,8 +2082,8 @@ def emit_block_rows(prog, leaf_kind, acc_dt, op, unroll=4, outer=False, shared=(
         first, pad = f"(long long)threadIdx.x * {V}", "    "
     else:
         L.append("        const long long r_end = (sl + 1) * RS < R ? (sl + 1) * RS : R;")
-        base = lambda i: f"a{i} + k * sk{i}"
-        const = lambda i: f"a{i}[k * sk{i}]"
+        base = lambda i: f"a{i} + {_row_at(outer2, i, 'k')}"
+        const = lambda i: f"a{i}[{_row_at(outer2, i, 'k')}]"
         first, pad = f"sl * RS + (long long)threadIdx.x * {V}", ""
     for i, (dt, kind) in enumerate(zip(prog.leaves, leaf_kind)):
         if kind == "v":
@@ -2362,6 +2375,20 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
     L += ["        }", "    }", "}"]
     src.append("\n".join(L))
     return "\n".join(src) + "\n"
+
+
+# Rows counted over two levels, K = K0 * K1, that some operand does not walk as one sequence
+# (a matrix repeated for every item of a batch): row k of operand i starts at
+# (k / K1) * sk_i + (k % K1) * sj_i.  Kernels that take such rows have the parameters K1 and
+# sj_i after their others.
+ROW_AT = ("__device__ __forceinline__ long long dr_row_at(const long long k, const unsigned int K1, "
+          "const long long s0, const long long s1)\n{\n"
+          "    const unsigned int q = (unsigned int)k / K1;\n"
+          "    return (long long)q * s0 + (long long)((unsigned int)k - q * K1) * s1;\n}")
+
+
+def _row_at(outer2, i, k):
+    return f"dr_row_at({k}, K1, sk{i}, sj{i})" if outer2 else f"{k} * sk{i}"
 
 
 # ---- rows that are reduced and used again in one kernel -----------------------------
@@ -2657,18 +2684,12 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     params += [f"const long long sk{i}" for i in range(nl)]
     params += [f"const long long so{n}" for n in range(n_out)]
     if outer2:
-        # rows counted over two levels, K = K0 * K1, that some operand does not walk as one
-        # sequence (a matrix repeated for every item of a batch): row k of operand i starts
-        # at (k / K1) * sk_i + (k % K1) * sj_i
         params.append("const unsigned int K1")
         params += [f"const long long sj{i}" for i in range(nl)]
-        src.append("__device__ __forceinline__ long long dr_row_at(const long long k, const unsigned int K1, "
-                   "const long long s0, const long long s1)\n{\n"
-                   "    const unsigned int q = (unsigned int)k / K1;\n"
-                   "    return (long long)q * s0 + (long long)((unsigned int)k - q * K1) * s1;\n}")
+        src.append(ROW_AT)
 
     def row_at(i, k):
-        return f"dr_row_at({k}, K1, sk{i}, sj{i})" if outer2 else f"{k} * sk{i}"
+        return _row_at(outer2, i, k)
     scal = [f"s{i}" for i in range(ns)]
     L = [f'extern "C" __global__ __launch_bounds__({B})',
          f"void dr_kernel({', '.join(params)})", "{"]

@@ -948,6 +948,13 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
         K *= d
     for d in rmerged:
         R *= d
+    # kept dimensions that merge into one sequence of rows, or into two levels of them that
+    # the row-wise kernels split again (an operand shared by every item of a batch)
+    two = len(kmerged) == 2 and K < 2 ** 31
+    one_or_two = len(kmerged) == 1 or two
+    two_fmt = "I" + "q" * len(leaves) if two else ""
+    two_tail = [kmerged[1]] + [k[1] for k in ksets] if two else []
+    two_key = ("two levels",) if two else ()
     # coalescing decides the strategy: which side holds the unit-stride dimension
     # (judged by the operands that carry the traffic: a column of weights beside a matrix
     # must not turn a sum over rows into the strategy for sums along rows)
@@ -990,7 +997,7 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
         low.scal, low.tail = list(scalars), [U]
         return low, S, K, "col"
     if (strategy == "row" and slices is None and R <= TUNE["ax_short"] and K >= 4096
-            and len(kmerged) == 1 and len(rmerged) == 1
+            and one_or_two and len(rmerged) == 1
             and all(r[0] in (0, 1) for r in rsets) and K < 2 ** 40):
         # many short rows: a lane per output walking its own row, no combining step
         kinds = tuple("v" if r[0] == 1 else "k" for r in rsets)
@@ -998,19 +1005,19 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
         low.lds = 0
         low.fin_count = 0
         low.kind = "axis_short"
-        low.key = ("axis_short", prog.key(), kinds, acc, reduce_op, R)
+        low.key = ("axis_short", prog.key(), kinds, acc, reduce_op, R) + two_key
 
         def emit_short():
-            return cg.emit_short_rows(prog, kinds, acc, reduce_op, R)
+            return cg.emit_short_rows(prog, kinds, acc, reduce_op, R, outer2=two)
         low.emit = emit_short
         low.grid = -(-K // cg.BLOCK)
         low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
-                   + "q" + "q" * len(leaves))
+                   + "q" + "q" * len(leaves) + two_fmt)
         low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
-        low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets]
+        low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets] + two_tail
         return low, 1, K, "short"
     if (strategy == "row" and slices is None and TUNE["ax_short"] < R <= TUNE["ax_group"]
-            and K >= 1024 and len(kmerged) == 1 and len(rmerged) == 1 and TUNE["uvec"]
+            and K >= 1024 and one_or_two and len(rmerged) == 1 and TUNE["uvec"]
             and all(r[0] in (0, 1) for r in rsets) and K < 2 ** 40):
         widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == 1}
         if len(widths) == 1 and widths <= {4, 8} and all(
@@ -1030,19 +1037,19 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
             low.lds = 0
             low.fin_count = 0
             low.kind = "axis_group"
-            low.key = ("axis_group", prog.key(), kinds, acc, reduce_op, R, G)
+            low.key = ("axis_group", prog.key(), kinds, acc, reduce_op, R, G) + two_key
 
             def emit_group():
-                return cg.emit_group_rows(prog, kinds, acc, reduce_op, R, G)
+                return cg.emit_group_rows(prog, kinds, acc, reduce_op, R, G, outer2=two)
             low.emit = emit_group
             rows_per_block = (cg.BLOCK // cg.WAVE) * (cg.WAVE // G)
             # one pass over the rows per wave (rows of 200 float32: 80.6 % of the HBM peak; four
             # passes 76.5, sixteen 72.9)
             low.grid = max(1, min(-(-K // rows_per_block), 1 << 20))
             low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
-                       + "q" + "q" * len(leaves))
+                       + "q" + "q" * len(leaves) + two_fmt)
             low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
-            low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets]
+            low.scal, low.tail = list(scalars), [K] + [k[0] for k in ksets] + two_tail
             return low, 1, K, "group"
     if (strategy == "col" and slices is None and len(rmerged) == 1 and len(kmerged) == 1
             and TUNE["ax_stream"] > 0 and TUNE["uvec"] and all(k[0] in (0, 1) for k in ksets)):
@@ -1139,7 +1146,7 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
             low.scal = list(scalars)
             low.tail = [K, RI, S, QS] + [k[0] for k in ksets] + [RO] + [r[0] for r in rsets]
             return low, S, K, "row"
-    if (strategy == "row" and slices is None and len(rmerged) == 1 and len(kmerged) == 1
+    if (strategy == "row" and slices is None and len(rmerged) == 1 and one_or_two
             and R >= TUNE["ax_block"] > 0 and TUNE["uvec"] and all(r[0] in (0, 1) for r in rsets)):
         widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == 1}
         if len(widths) == 1 and widths <= {4, 8} and all(
@@ -1154,14 +1161,14 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
             # an operand that is the same for every row (the vector of a matrix-vector
             # product) stays in the caches; `a @ x` on 16384^2 float32: 76.8 % of the HBM
             # peak with every load non-temporal
-            shared = tuple(i for i, (k, r) in enumerate(zip(ksets, rsets)) if r[0] == 1 and k[0] == 0)
+            shared = tuple(i for i, (k, r) in enumerate(zip(ksets, rsets)) if r[0] == 1 and not any(k))
             low = Lowered()
             low.lds = 0
             low.fin_count = 0
             low.kind = "axis_block"
-            low.key = ("axis_block", prog.key(), kinds, acc, reduce_op, shared)
+            low.key = ("axis_block", prog.key(), kinds, acc, reduce_op, shared) + two_key
             rows = TUNE["ax_block_rows"]
-            if shared and S == 1 and rows > 1 and K >= 1024 * rows:
+            if shared and S == 1 and rows > 1 and K >= 1024 * rows and not two:
                 # several rows per block: the shared operand is loaded once for all of them
                 unroll = TUNE["ax_block_rows_unroll"]
                 low.key = ("axis_block", prog.key(), kinds, acc, reduce_op, shared, unroll, rows)
@@ -1177,13 +1184,13 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
                 return low, 1, K, "row"
 
             def emit_block():
-                return cg.emit_block_rows(prog, kinds, acc, reduce_op, shared=shared)
+                return cg.emit_block_rows(prog, kinds, acc, reduce_op, shared=shared, outer2=two)
             low.emit = emit_block
             low.grid = max(1, min(K * S, 1 << 20))
             low.fmt = ("@" + "P" * (len(leaves) + 1) + "".join(_SCALAR_FMT[c] for c in prog.scalars)
-                       + "qqqq" + "q" * len(leaves))
+                       + "qqqq" + "q" * len(leaves) + two_fmt)
             low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
-            low.scal, low.tail = list(scalars), [K, R, S, RS] + [k[0] for k in ksets]
+            low.scal, low.tail = list(scalars), [K, R, S, RS] + [k[0] for k in ksets] + two_tail
             return low, S, K, "row"
     # enough independent pieces to fill the device: cut the reduced extent into slices
     if slices is not None:

@@ -653,3 +653,17 @@ def test_every_axis_reduction_kernel_shape_is_emitted_and_compiles():
             low, src = hip.lower_only(ReduceEx(func, leaf(shape, dtype) * 2.0, axes))
             assert low.kind == kind, (kind, low.kind, dtype)
             hip.compile_source(src)
+
+
+def test_reductions_along_rows_of_a_batch_with_a_shared_operand_keep_the_row_wise_kernels():
+    """`sum(x + m, axis=-1)`, x (batch, rows, columns), m (rows, columns): two levels of
+    kept dimensions; the lane, lane-group and block kernels take them with the row number
+    split by the inner level (`dr_row_at`), and their sources compile."""
+    for (B, N, R), kind in (((256, 8192, 8), "axis_short"), ((256, 8192, 64), "axis_group"),
+                            ((64, 1000, 1000), "axis_group"), ((16, 512, 16384), "axis_block")):
+        low, src = hip.lower_only(ReduceEx(np.add, leaf((B, N, R)) + leaf((N, R)), (2,)))
+        assert low.kind == kind and "dr_row_at(k, K1, sk0, sj0)" in src, (B, N, R, low.kind)
+        assert low.tail[-3:] == [N, R, R] and low.fmt.endswith("Iqq")
+        hip.compile_source(src)
+        plain, src1 = hip.lower_only(ReduceEx(np.add, leaf((B, N, R)) * 2.0, (2,)))
+        assert plain.kind == kind and "dr_row_at" not in src1

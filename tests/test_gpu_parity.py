@@ -1850,3 +1850,29 @@ def test_types_without_a_device_form_are_widened_aloud_or_refused():
     for bad in (np.ones(3, np.longdouble), np.ones(3, np.complex64), np.ones(3, np.complex128)):
         with pytest.raises(TypeError):
             dr.array(bad)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_row_reductions_with_an_operand_shared_by_a_batch(dtype):
+    """`sum(x + m, axis=-1)` with x of shape (batch, rows, columns) and m (rows, columns):
+    the kept dimensions are two levels that m does not walk as one sequence.  The row-wise
+    reduction kernels (a lane, a lane group or a block per row) split the row number
+    instead of leaving the case to the general wave-per-row kernel."""
+    rs = np.random.RandomState(16)
+    for (B, N, R), kind in (((40, 300, 8), "axis_short"), ((6, 200, 64), "axis_group"),
+                            ((5, 210, 1000), "axis_group"), ((3, 7, 16384), "axis_block"),
+                            ((1, 1500, 200), "axis_group")):
+        x = rs.standard_normal((B, N, R)).astype(dtype)
+        m = rs.standard_normal((N, R)).astype(dtype)
+        v = rs.standard_normal((B, 1, R)).astype(dtype)
+        dx, dm, dv = dr.array(x), dr.array(m), dr.array(v)
+        low, _ = hip.lower_only(ReduceEx(np.add, dx + dm, (2,)))
+        assert low.kind == kind, (B, N, R, low.kind)
+        tol = dict(rtol=2e-5, atol=1e-4) if dtype == np.float32 else dict(rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(dr.sum(dx + dm, axis=-1).get(), (x + m).sum(axis=-1), **tol)
+        np.testing.assert_allclose(dr.sum(dx * dv + dm, axis=2).get(), (x * v + m).sum(axis=2), **tol)
+        assert np.array_equal(dr.max(dx + dm, axis=-1).get(), (x + m).max(axis=-1))
+        assert np.array_equal(dr.min(dx[::2] * dv[::2], axis=-1).get(), (x[::2] * v[::2]).min(axis=-1))
+        kd = dr.sum(dx + dm, axis=-1, keepdims=True).get()
+        assert kd.shape == (B, N, 1)
+        np.testing.assert_allclose(kd, (x + m).sum(axis=-1, keepdims=True), **tol)
