@@ -92,7 +92,7 @@ def parse():
                     help="sumsq (headline) | saxpy | horner | bs32 | bs64 | jacobi | all (these six); "
                          "dot | axis0 | axis1 | axis1_3d | matvec | rows200 | rowbcast | transpose | "
                          "transpose3d | interior | diff2 | stencil9 | stencil3d | grid | rand | softmax | softmax32k | "
-                         "layernorm | rowmax | strided | strided2d | next (all "
+                         "layernorm | rowmax | strided | strided2d | points3 | next (all "
                          "of these: the operations either side of the five configurations); "
                          "matmul32 | matmul64 (the eager matrix product)")
     ap.add_argument("--settle", type=float, default=0.25,
@@ -329,6 +329,18 @@ def main():
                         steps=[(lambda v=v: hip.run(v.T * 2.0)) for v in vols],
                         cpu=lambda: hv[:, :, :256].T * np.float32(2.0), cpu_frac=0.25,
                         cpu_code="numpy.multiply")
+        if name == "points3":
+            n = 1 << 25
+            hx = rs.standard_normal((n, 3)).astype(np.float32)
+            hs, ht = rs.standard_normal(3).astype(np.float32), rs.standard_normal(3).astype(np.float32)
+            pts = [dr.array(hx) for _ in range(sets_for(8 * n * 3))]
+            sc, sh = dr.array(hs), dr.array(ht)
+            return dict(dtype="f32", n=n * 3, nbytes=8 * n * 3,
+                        desc="points * scale + shift f32, 2^25 points of 3 coordinates (rows of 12 "
+                             "bytes: the row kernel without reductions, a lane per row)",
+                        steps=[(lambda p=p: hip.run(p * sc + sh)) for p in pts],
+                        cpu=lambda: hx[:n // 16] * hs + ht, cpu_frac=1 / 16,
+                        cpu_code="numpy.multiply, add")
         if name == "softmax32k":
             R, N = 32000, 8192
             ha = rs.standard_normal((N, R)).astype(np.float32)
@@ -688,7 +700,7 @@ def main():
     names = {"all": ["sumsq", "saxpy", "horner", "bs32", "bs64", "jacobi"],
              "next": ["dot", "axis0", "axis1", "axis1_3d", "matvec", "rows200", "rowbcast", "transpose",
                       "transpose3d", "interior", "diff2", "stencil9", "stencil3d", "grid", "rand",
-                      "softmax", "softmax32k", "layernorm", "rowmax", "strided", "strided2d"]}.get(args.workload, [args.workload])
+                      "softmax", "softmax32k", "layernorm", "rowmax", "strided", "strided2d", "points3"]}.get(args.workload, [args.workload])
     HEADLINE = "sumsq" if "sumsq" in names else names[0]
     results = {}
     for name in names:

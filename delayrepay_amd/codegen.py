@@ -2569,8 +2569,6 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
     Parameters: leaf pointers, output pointers, scalars, K (rows), per leaf the stride
     between rows, per output the stride between rows (all in elements)."""
     level, uniform, stages = row_analysis(prog, leaf_kind)
-    if not stages:
-        raise RowFusionUnsupported("no row reduction in the program")
     V = row_vector(prog, leaf_kind, out_dtypes, out_uniform)
     units = -(-R // V)
     full, rem = R // V, R % V
@@ -2771,7 +2769,7 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
                 zero = "{0}" if V > 1 else "0"
                 L.append(f"    {vtype(prog.leaves[i])} X{j}_{i} = {zero};")
     if block_row:
-        widest = max((CTYPE[prog.ops[i][2]] for reds in stages for i in reds),
+        widest = max((CTYPE[prog.ops[i][2]] for reds in stages for i in reds), default="float",
                      key=lambda c: 8 if c in ("double", "long long") else 4)
         L += [f"    __shared__ {widest} dr_slots[2][{max(n_red, 1)}][{B // WAVE}];",
               f"    const int sub = (threadIdx.x >> 6) * {seg} + (threadIdx.x & {WAVE - 1});" if wave_map

@@ -69,6 +69,8 @@ TUNE = {
     "softdiv": 2,     # quotients and square roots that only inexact functions read: to one ulp, in
                       # fewer operations (1: float64 only, 2: float32 too, in packed bodies; 0: never)
                       # (2: float32 quotients as well, 4 operations; measured slower)
+    "rows_elem": 4096,    # element-wise work on rows of at most this many bytes with repeated
+                      # operands takes the row kernel (0: the tiled kernel)
     "rowfuse": 1,     # reductions along the last axis inside an expression: one kernel per row
     "row_lanes": 0,   # ... lanes per row (0: by the cost of idle lanes and of units per lane)
     "row_regs": 128,  # ... registers that may hold the row between stages (else it is loaded again)
@@ -350,7 +352,7 @@ def _row_steps_max(G):
     return cg.ROW_STEPS_LONG if G > cg.BLOCK else cg.ROW_STEPS_MAX
 
 
-def lower_rows(prog, leaves, scalars, shape, out_codes):
+def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False):
     """Expression with reductions along its last axis inside it (`codegen.emit_row_fused`):
     every row is read once, reduced, used again and written once.  `shape` is the shape the
     expression is evaluated at, rows along its last axis; outputs are new dense arrays, of
@@ -386,6 +388,10 @@ def lower_rows(prog, leaves, scalars, shape, out_codes):
     row_out = []
     for (kind, j), _ in prog.roots:
         row_out.append(uniform[j] if kind == "v" else (kind == "s" or kinds[j] == "k"))
+    if whole_rows and any(row_out):
+        # the caller's results all have the full shape: one that is the same along a row
+        # (a column repeated) would be stored once per row here
+        raise cg.RowFusionUnsupported("a result that is constant along the rows")
     V = cg.row_vector(prog, kinds, out_codes, row_out)
     units = -(-R // V)
     G = TUNE["row_lanes"]
@@ -622,6 +628,27 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         if reduce_op:
             low.fin_count = low.grid
         return low
+
+    # Short rows with operands that repeat along or across them (`points * scale` with
+    # points of shape (n, 3), `(x - mean) / std` over a few dozen features): a tile of 256
+    # columns leaves most lanes idle (x * v, percent of the HBM peak, tiled / row kernel:
+    # rows of 3 float32: 4 / 71, of 16: 10 / 78, of 64: 38 / 77, of 200: 65 / 73, of 300:
+    # 55 / 67, of 1024: 76 / 79; of 2000: 72 / 69, of 4096: 77 / 76).  The row kernel without
+    # reductions gives each row to a group of lanes sized to it; results go to dense arrays.
+    if (TUNE["rows_elem"] and not reduce_op and not in_place and ndim >= 2 and out_codes
+            and out_shape[-1] * max(cg.ITEMSIZE[c] for c in out_codes) <= TUNE["rows_elem"]
+            and all(s[-1] in (0, 1) for s in m_leaf)
+            and len({id(a.buf) for a in leaves}) == len(leaves)):     # no shifted views: those share an LDS window
+        dense = []
+        step = 1
+        for d in reversed(out_shape):
+            dense.insert(0, step)
+            step *= d
+        if all(list(st) == dense for st in out_strides):
+            try:
+                return lower_rows(prog, leaves, scalars, tuple(out_shape), out_codes, whole_rows=True)
+            except cg.RowFusionUnsupported:
+                pass
 
     # Tiled family: the last merged dimension is walked with unit stride by every output
     # and with stride 1 or 0 by every operand; the dimensions in front of it are the

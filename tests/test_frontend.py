@@ -252,7 +252,7 @@ def test_misaligned_view_moves_vectors_at_element_alignment():
     aligned = hip.lower_only(NPArray(base[4:]) * 2.0)[1].split('extern "C"')[1]
     assert "(const f4x4*)a0" in aligned and "f4x4u" not in aligned
     # rows whose pitch is not a multiple of 16 bytes: vector tiles all the same
-    m = NPArray(hip.placeholder((1022, 1022), np.float32, strides=(1024, 1), offset=1025))
+    m = NPArray(hip.placeholder((2046, 2046), np.float32, strides=(2048, 1), offset=2049))
     low, src = hip.lower_only(m * 2.0 + m)
     assert low.key[0] == "tile2dv" and "(const f4x4u*)(a0" in src and "(f4x4u*)(o0" in src
     hip.compile_source(src)
@@ -274,14 +274,29 @@ def test_broadcast_scalar_leaf_and_mixed_dtypes():
 
 
 def test_strided_and_broadcast_operands_use_nd():
-    a, b = leaf((64, 1, 32), np.float64), leaf((1, 48, 32), np.float32)
+    a, b = leaf((64, 1, 1320), np.float64), leaf((1, 48, 1320), np.float32)
     low, src = hip.lower_only(a * b + 1)         # unit inner stride: tiled, rows = 64 * 48
     assert low.kind == "tile2d" and "rem_o / e1" in src
     hip.compile_source(src)
     col = leaf((64, 1))
-    low, src = hip.lower_only(leaf((64, 32)) * col)          # column broadcast: one load per row
+    low, src = hip.lower_only(leaf((64, 1320)) * col)        # column broadcast: one load per row
     assert low.kind == "tile2d" and ("r",) in low.key[2]
     hip.compile_source(src)
+    # rows of at most 4 KB: the row kernel, a group of lanes per row, also over two levels
+    a, b = leaf((64, 1, 32), np.float64), leaf((1, 48, 32), np.float32)
+    low, src = hip.lower_only(a * b + 1)
+    assert low.kind == "rows" and "dr_row_at" in src and "dr_final" in src and "dr_stage" not in src
+    hip.compile_source(src)
+    low, src = hip.lower_only(leaf((1 << 20, 3)) * leaf((3,)) + leaf((1 << 20, 1)))
+    assert low.kind == "rows" and low.key[6] == 1 and low.key[2] == ("v", "v", "k")
+    hip.compile_source(src)
+    lowering.TUNE["rows_elem"] = 0
+    try:
+        assert hip.lower_only(leaf((1 << 20, 5)) * leaf((5,)))[0].kind == "tile2d"
+    finally:
+        lowering.TUNE["rows_elem"] = 4096
+    dst = hip.placeholder((64, 32), np.float32, strides=(64, 1))           # a destination with
+    assert hip.lower_only(leaf((64, 32)) * col, dst=dst)[0].kind == "tile2d"   # its own pitch
     m = hip.placeholder((100, 200), np.float32)
     low, src = hip.lower_only(NPArray(m.T) * 2.0)           # transposed operand: through LDS
     assert low.kind == "tile2dt" and "__shared__ float tt0[" in src
@@ -503,7 +518,7 @@ def test_views_of_lazy_expressions_are_pushed_to_the_leaves():
     r = e[1:-1, 4:-4]
     assert type(r) is BinaryNumpyEx and r.shape == (510, 1016) and "array" not in e.__dict__
     low, src = hip.lower_only(r)
-    assert len(low.srcs) == 2 and low.kind.startswith("tile2d")
+    assert len(low.srcs) == 2 and low.kind in ("tile2d", "rows")
     # shifted slices of one expression become one LDS stencil over the expression's leaf
     s = a + 1.0
     lap = s[:-2, 1:-1] + s[2:, 1:-1] + s[1:-1, :-2] + s[1:-1, 2:]

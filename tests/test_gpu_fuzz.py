@@ -97,7 +97,7 @@ def test_random_expression(seed):
     if rs.uniform() < 0.4:
         shape = (int(rs.choice([1, 5, 63, 64, 257, 1000, 4099])),)
     else:
-        shape = (int(rs.choice([1, 3, 8, 33, 64, 130])), int(rs.choice([1, 4, 7, 64, 129, 260])))
+        shape = (int(rs.choice([1, 3, 8, 33, 64, 130])), int(rs.choice([1, 4, 7, 64, 129, 260, 1300])))
     with np.errstate(all="ignore"):
         d, o = random_expr(rs, shape, depth=int(rs.randint(1, 5)))
         anchor_d, anchor_o = full_shape_leaf(rs, shape)
@@ -147,8 +147,8 @@ def test_fuzz_reached_every_kernel_shape():
     for key in hip._KERNELS:
         kinds[key[0]] = kinds.get(key[0], 0) + 1
     print("kernel kinds compiled:", kinds)
-    for kind in ("flat", "nd", "tile2d", "tile2dv", "tile2dt", "axis", "axis_short", "axis_narrow",
-                 "axis_group"):
+    for kind in ("flat", "nd", "tile2dv", "tile2dt", "axis", "axis_short", "axis_narrow",
+                 "axis_group", "rows"):
         assert kinds.get(kind, 0) > 0, kind
 
 

@@ -1876,3 +1876,50 @@ def test_row_reductions_with_an_operand_shared_by_a_batch(dtype):
         kd = dr.sum(dx + dm, axis=-1, keepdims=True).get()
         assert kd.shape == (B, N, 1)
         np.testing.assert_allclose(kd, (x + m).sum(axis=-1, keepdims=True), **tol)
+
+
+def test_element_wise_work_on_short_rows_takes_the_row_kernel():
+    """`points * scale + shift` with points (n, 3), standardising a few dozen features, an
+    operand per batch item: rows of at most 4 KB with operands that repeat go through the
+    row kernel without reductions (a lane group per row); bit-equal to NumPy.  A result
+    that is constant along the rows (a column repeated), a destination with its own pitch,
+    shifted views of one buffer and longer rows keep the tiled kernels."""
+    rs = np.random.RandomState(17)
+    for dtype in (np.float32, np.float64, np.int32):
+        for n, R in ((100003, 3), (5000, 8), (4099, 33), (1000, 64), (513, 200), (130, 500)):
+            mk = (lambda *s: rs.standard_normal(s).astype(dtype)) if dtype != np.int32 else \
+                 (lambda *s: rs.randint(-50, 50, s).astype(dtype))
+            x, v, c = mk(n, R), mk(R), mk(n, 1)
+            dx, dv, dc = dr.array(x), dr.array(v), dr.array(c)
+            ex = dx * dv + dc
+            assert hip.lower_only(ex)[0].kind == "rows", (dtype, n, R)
+            assert bits_equal(ex.get(), x * v + c)
+            p, q = dr.evaluate(dx - dv, (dx + dc) * dv)                   # two results, one kernel
+            assert bits_equal(p.get(), x - v) and bits_equal(q.get(), (x + c) * v)
+            assert bits_equal((dx[::2] * dv > dc[::2]).get(), x[::2] * v > c[::2])      # masks
+            if dtype != np.int32:
+                assert bits_equal((dx / dv).get(), x / v)
+    # batches: an operand per item, one shared by all items
+    x, m, w = rs.standard_normal((7, 50, 40)), rs.standard_normal((50, 40)), rs.standard_normal((7, 1, 40))
+    dx, dm, dw = dr.array(x), dr.array(m), dr.array(w)
+    assert hip.lower_only(dx * dw + dm)[0].kind == "rows"
+    assert bits_equal((dx * dw + dm).get(), x * w + m)
+    # what stays with the tiled kernels
+    c = rs.standard_normal((300, 1))
+    dc = dr.array(c)
+    rep = dc * 2.0 + dr.zeros((300, 5))
+    assert bits_equal(np.repeat(dr.array(c[:, 0]), 5).get(), np.repeat(c[:, 0], 5))
+    a = rs.standard_normal((64, 48))
+    da = dr.array(a)
+    assert hip.lower_only(da[:, 1:] - da[:, :-1])[0].kind.startswith("tile2d")   # shifted views
+    assert bits_equal((da[:, 1:] - da[:, :-1]).get(), a[:, 1:] - a[:, :-1])
+    wide = rs.standard_normal((40, 1300)).astype(np.float32)
+    other = rs.standard_normal((40, 1300))
+    col = rs.standard_normal((40, 1))
+    mixed = dr.array(wide) * dr.array(other) + dr.array(col)
+    assert hip.lower_only(mixed)[0].kind == "tile2d"                          # longer rows, mixed types
+    assert bits_equal(mixed.get(), wide * other + col)
+    dst = dr.zeros((64, 60))
+    dst[:, 4:52] = da * dr.array(c[:64])                                         # its own pitch
+    ref = np.zeros((64, 60)); ref[:, 4:52] = a * c[:64]
+    assert bits_equal(dst.get(), ref)
