@@ -856,6 +856,23 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
                   if k[0] == "t") >= 1 << 20
         t_r = TUNE["t_rows"] or (512 if far else 128) // widest
         t_c = TUNE["t_cols"] or (256 if far else 1024) // widest
+        if not TUNE["t_rows"] and not TUNE["t_cols"]:
+            # A matrix with one short side (points as rows of three coordinates and the three
+            # coordinate vectors: `pts.T`): a tile that fits the short side instead of leaving
+            # most of its lanes outside the matrix.  `a.T * 2`, float32, percent of the HBM
+            # peak with the default tile / the fitted one: (n, 3): 5 / 38, (3, n): 8 / 44,
+            # (n, 4): 6 / 75, (n, 8): 12 / 64, (8, n): 17 / 74, (n, 16): 21 / 73, (16, n):
+            # 24 / 76, (32, n): 28 / 74; float64 (n, 6): 42 / 61, (6, n): 43 / 63.
+            def fitted(extent):
+                p2 = 4
+                while p2 < extent:
+                    p2 *= 2
+                return p2
+            if mshape[tp] <= 16:
+                t_r, t_c = fitted(mshape[tp]), 256
+            elif mshape[last] <= 32:
+                t_c = fitted(mshape[last])
+                t_r = 256 if 257 * t_c * widest <= 48 * 1024 else 128
         lds_bytes = sum((t_r + 1) * t_c * cg.ITEMSIZE[c]
                         for c, k in zip(prog.leaves, kinds) if k[0] == "t")
         if lds_bytes > 64 * 1024:

@@ -1923,3 +1923,25 @@ def test_element_wise_work_on_short_rows_takes_the_row_kernel():
     dst[:, 4:52] = da * dr.array(c[:64])                                         # its own pitch
     ref = np.zeros((64, 60)); ref[:, 4:52] = a * c[:64]
     assert bits_equal(dst.get(), ref)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32])
+def test_transposes_of_matrices_with_one_short_side(dtype):
+    """Points as rows of a few coordinates and the coordinate vectors (`pts.T`): the
+    transposing tiles are fitted to the short side (4 to 16 rows of the operand by 256, or
+    256 by 4 to 32 columns).  Bit-equal to NumPy for every short extent, also when it is no
+    power of two, with a second operand and with a batch in front."""
+    rs = np.random.RandomState(18)
+    for n, R in ((100003, 2), (100003, 3), (70001, 4), (30011, 7), (20000, 8), (9973, 12), (5000, 16),
+                 (4099, 24), (3001, 32)):
+        x = (rs.standard_normal((n, R)) * 50).astype(dtype)
+        other = (rs.standard_normal((R, n)) * 50).astype(dtype)
+        dx, do = dr.array(x), dr.array(other)
+        low, _ = hip.lower_only(dx.T * 2)
+        assert low.kind == "tile2dt", (n, R)
+        assert bits_equal((dx.T * 2).get(), x.T * 2)
+        assert bits_equal((dx.T + do).get(), x.T + other)            # with an operand read directly
+        assert bits_equal((do.T * 2).get(), other.T * 2)             # the short side first
+        assert bits_equal((do.T - dx).get(), other.T - x)
+    b = (rs.standard_normal((5, 4001, 3)) * 50).astype(dtype)
+    assert bits_equal((dr.transpose(dr.array(b), (0, 2, 1)) * 2).get(), b.transpose(0, 2, 1) * 2)
