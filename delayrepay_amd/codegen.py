@@ -2862,7 +2862,11 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
         if not recompute:
             return f"v{g}"
         ct = CTYPE[prog.ops[g][2]]
-        L.append(f'{pad}{ct} v{g}_{tag} = v{g}; asm volatile("" : "+v"(v{g}_{tag}));')
+        if ITEMSIZE[prog.ops[g][2]] < 4:    # a byte (a mask) has no register class of its own
+            L.append(f'{pad}{ct} v{g}_{tag}; {{ int w_ = v{g}; asm volatile("" : "+v"(w_)); '
+                     f'v{g}_{tag} = ({ct})w_; }}')
+        else:
+            L.append(f'{pad}{ct} v{g}_{tag} = v{g}; asm volatile("" : "+v"(v{g}_{tag}));')
         return f"v{g}_{tag}"
     if not rotate:
         for j in range(steps):

@@ -284,10 +284,17 @@ int drhip_matmul(int is_double, const void* a, const void* b, void* c, int64_t m
     if (m < 0 || n < 0 || k < 0 || lda < k || ldb < n || ldc < n)
         return fail(DRHIP_EINVAL, "drhip_matmul", "bad dimensions");
     if (m == 0 || n == 0) return 0;
-    if ((m + 63) / 64 > 65535) return fail(DRHIP_EINVAL, "drhip_matmul", "too many rows");
-    drhip_k_launch_matmul(is_double, a, b, c, m, n, k, lda, ldb, ldc, g_stream);
-    HIP_TRY(hipGetLastError());
-    g_cnt.n_launches++;
+    // the launch counts 64-row tiles in the grid's second dimension (at most 65535):
+    // taller products go in slabs of rows
+    const int64_t slab = 65535LL * 64;
+    const size_t item = is_double ? sizeof(double) : sizeof(float);
+    for (int64_t r0 = 0; r0 < m; r0 += slab) {
+        const int64_t rows = m - r0 < slab ? m - r0 : slab;
+        drhip_k_launch_matmul(is_double, (const char*)a + (size_t)r0 * lda * item, b,
+                              (char*)c + (size_t)r0 * ldc * item, rows, n, k, lda, ldb, ldc, g_stream);
+        HIP_TRY(hipGetLastError());
+        g_cnt.n_launches++;
+    }
     return 0;
 }
 

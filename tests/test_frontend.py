@@ -682,3 +682,18 @@ def test_reductions_along_rows_of_a_batch_with_a_shared_operand_keep_the_row_wis
         hip.compile_source(src)
         plain, src1 = hip.lower_only(ReduceEx(np.add, leaf((B, N, R)) * 2.0, (2,)))
         assert plain.kind == kind and "dr_row_at" not in src1
+
+
+def test_masks_that_are_the_same_along_a_row_compile_in_the_row_kernel():
+    """A comparison of per-row values (`row maximum > 0`, a mask per row from a column) is
+    a byte that is computed once per row and handed on; bytes have no vector register class
+    of their own, so they are passed through a word where the kernel hides a value from
+    the optimiser."""
+    a = leaf((1000, 300))
+    mx = a.max(axis=1, keepdims=True)
+    for ex in (np.where(mx > 0, a / mx, a),
+               np.where(a.sum(axis=1, keepdims=True) > mx, a, -a) * (mx > 1),
+               np.where((leaf((1 << 20,)) > 0)[:, None], leaf((1 << 20, 3)), 0.0)):
+        low, src = hip.lower_only(ex)
+        assert low.kind == "rows" and "unsigned char" in src
+        hip.compile_source(src)

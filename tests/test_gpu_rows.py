@@ -476,3 +476,21 @@ def test_operands_repeated_over_a_batch_stay_in_the_row_kernel(dtype):
     dy, dm2 = dr.array(y), dr.array(m2)
     got = ((dy + dm2) - (dy + dm2).max(axis=-1, keepdims=True)).get()
     assert bits_equal(got, (y + m2) - (y + m2).max(axis=-1, keepdims=True))
+
+
+def test_masks_that_are_the_same_along_a_row():
+    """`where(row maximum > 0, a / maximum, a)`, a mask per row from a vector: the per-row
+    comparison is a byte computed once per row; bit-equal to NumPy."""
+    rs = np.random.RandomState(19)
+    a = rs.standard_normal((500, 300)).astype(np.float32)
+    a[::7] -= 10.0                                         # rows whose maximum is negative
+    da = dr.array(a)
+    mx, hmx = da.max(axis=1, keepdims=True), a.max(axis=1, keepdims=True)
+    got, n = launches(lambda: np.where(mx > 0, da / mx, da).get())
+    assert n == 1 and bits_equal(got, np.where(hmx > 0, a / hmx, a))
+    got, n = launches(lambda: (np.where(da.min(axis=1, keepdims=True) < -3, da, -da) * (mx > 1)).get())
+    assert n == 1 and bits_equal(got, np.where(a.min(axis=1, keepdims=True) < -3, a, -a) * (hmx > 1))
+    w = rs.standard_normal(100003).astype(np.float32)
+    x = rs.standard_normal((100003, 3)).astype(np.float32)
+    got, n = launches(lambda: np.where((dr.array(w) > 0)[:, None], dr.array(x), 0.0).get())
+    assert n == 1 and bits_equal(got, np.where((w > 0)[:, None], x, np.float32(0.0)))

@@ -591,3 +591,18 @@ def test_writes_by_hand_aliasing_out_and_stretched_views():
         wide[0, 0] = 5.0
     with pytest.raises(ValueError, match="read-only"):
         wide[...] = dr.array(np.ones((3, 4))) * 2.0
+
+
+def test_matrix_product_with_more_rows_than_one_launch_takes():
+    """Points times a 3 x 3 matrix: 5 million rows are more 64-row tiles than the second
+    grid dimension holds (65535), so the library multiplies slabs of rows."""
+    rs = np.random.RandomState(20)
+    pts = rs.standard_normal((5_000_000, 3)).astype(np.float32)
+    rot = rs.standard_normal((3, 3)).astype(np.float32)
+    got = (dr.array(pts) @ dr.array(rot)).get()
+    ref = pts.astype(np.float64) @ rot.astype(np.float64)
+    assert got.shape == ref.shape and got.dtype == np.float32
+    np.testing.assert_allclose(got[::997], ref[::997], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(got[-3:], ref[-3:], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(got[65535 * 64 - 2:65535 * 64 + 2], ref[65535 * 64 - 2:65535 * 64 + 2],
+                               rtol=1e-5, atol=1e-5)
