@@ -599,6 +599,7 @@ def test_matrix_product_with_more_rows_than_one_launch_takes():
     rs = np.random.RandomState(20)
     pts = rs.standard_normal((5_000_000, 3)).astype(np.float32)
     rot = rs.standard_normal((3, 3)).astype(np.float32)
+    import delayrepay_amd as dr
     got = (dr.array(pts) @ dr.array(rot)).get()
     ref = pts.astype(np.float64) @ rot.astype(np.float64)
     assert got.shape == ref.shape and got.dtype == np.float32
