@@ -2541,7 +2541,7 @@ def row_vector(prog, leaf_kind, out_dtypes, out_uniform):
 
 def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt_store=False,
                    fence=True, recompute=True, pipeline=True, carry_values=True, wave_map=False,
-                   nt_load=False, hoist=True, outer2=False):
+                   nt_load=False, hoist=True, outer2=False, restrict=True):
     """Rows that are reduced and used again: `a - max(a, axis=-1)`, softmax, the variance,
     layer normalisation.  A group of G lanes (1..64: part of a wave; 256 or 512: the block) owns a
     row of R elements (a compile-time constant, unit stride); lane j takes the 16-byte
@@ -2675,8 +2675,9 @@ def emit_row_fused(prog, leaf_kind, out_dtypes, out_uniform, R, G, keep=None, nt
         body.append("}")
         src.append("\n".join(body))
 
-    params = [f"const {CTYPE[dt]}* __restrict__ a{i}" for i, dt in enumerate(prog.leaves)]
-    params += [f"{CTYPE[dt]}* __restrict__ o{n}" for n, dt in enumerate(out_dtypes)]
+    rq = "__restrict__ " if restrict else ""      # (not when a result is written over an operand)
+    params = [f"const {CTYPE[dt]}* {rq}a{i}" for i, dt in enumerate(prog.leaves)]
+    params += [f"{CTYPE[dt]}* {rq}o{n}" for n, dt in enumerate(out_dtypes)]
     params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
     params.append("const long long K")
     params += [f"const long long sk{i}" for i in range(nl)]

@@ -352,7 +352,8 @@ def _row_steps_max(G):
     return cg.ROW_STEPS_LONG if G > cg.BLOCK else cg.ROW_STEPS_MAX
 
 
-def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False):
+def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False, out_strides=None,
+               in_place=False):
     """Expression with reductions along its last axis inside it (`codegen.emit_row_fused`):
     every row is read once, reduced, used again and written once.  `shape` is the shape the
     expression is evaluated at, rows along its last axis; outputs are new dense arrays, of
@@ -371,19 +372,29 @@ def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False):
     dense = [1] * len(shape)             # a new array of `shape`
     for k in range(len(shape) - 2, -1, -1):
         dense[k] = dense[k + 1] * shape[k + 1]
-    mshape, msets = merge_dims(shape[:-1], [st[:-1] for st in strides] + [dense[:-1]])
+    # the results: new dense arrays, or (element-wise work written into existing arrays)
+    # views whose rows lie one pitch apart
+    outs = [dense] * len(out_codes) if out_strides is None else [list(st) for st in out_strides]
+    if any(st[-1] != 1 for st in outs if shape[-1] > 1):
+        raise cg.RowFusionUnsupported("a destination without unit stride along the row")
+    mshape, msets = merge_dims(shape[:-1], [st[:-1] for st in strides] + [st[:-1] for st in outs])
+    nl_ = len(strides)
+    if len(mshape) == 2 and any(st[0] != st[1] * mshape[1] for st in msets[nl_:]):
+        raise cg.RowFusionUnsupported("a destination whose rows do not form one sequence")
     sj = None
     if len(mshape) == 2 and mshape[0] * mshape[1] < 2 ** 31:
         # two levels of rows (a matrix added to every item of a batch before the rows are
         # normalised): the kernel splits the row number
         K, K1 = mshape[0] * mshape[1], mshape[1]
-        sk = [st[0] for st in msets[:-1]]
-        sj = [st[1] for st in msets[:-1]]
+        sk = [st[0] for st in msets[:nl_]]
+        sj = [st[1] for st in msets[:nl_]]
+        so = [st[1] for st in msets[nl_:]]
     elif len(mshape) > 1:
         raise cg.RowFusionUnsupported("rows that do not form one sequence in every operand")
     else:
         K = mshape[0] if mshape else 1
-        sk = [st[0] if st else 0 for st in msets[:-1]]
+        sk = [st[0] if st else 0 for st in msets[:nl_]]
+        so = [st[0] if st else R for st in msets[nl_:]]
     level, uniform, stages = cg.row_analysis(prog, kinds)
     row_out = []
     for (kind, j), _ in prog.roots:
@@ -423,12 +434,13 @@ def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False):
     hoist = bool(TUNE["row_hoist"])
     low.key = ("rows", prog.key(), tuple(kinds), tuple(out_codes), low.row_out, R, G, keep, nts,
                fence, recompute, pipe, carry, wmap, ntl) + (() if hoist else ("per element",)) \
-        + (("two levels",) if sj else ())
+        + (("two levels",) if sj else ()) + (("over an operand",) if in_place else ())
 
     def emit():
         return cg.emit_row_fused(prog, kinds, out_codes, row_out, R, G, keep=keep, nt_store=nts,
                                  fence=fence, recompute=recompute, pipeline=pipe, carry_values=carry,
-                                 wave_map=wmap, nt_load=ntl, hoist=hoist, outer2=bool(sj))
+                                 wave_map=wmap, nt_load=ntl, hoist=hoist, outer2=bool(sj),
+                                 restrict=not in_place)
     low.emit = emit
     if G >= cg.BLOCK:
         blocks = K
@@ -444,7 +456,7 @@ def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False):
         + "q" * (1 + len(leaves) + len(out_codes)) + ("I" + "q" * len(leaves) if sj else "")
     low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
     low.scal = list(scalars)
-    low.tail = [K] + sk + [1 if u else R for u in row_out] + ([K1] + sj if sj else [])
+    low.tail = [K] + sk + [1 if u else p for u, p in zip(row_out, so)] + ([K1] + sj if sj else [])
     return low
 
 
@@ -634,21 +646,18 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     # columns leaves most lanes idle (x * v, percent of the HBM peak, tiled / row kernel:
     # rows of 3 float32: 4 / 71, of 16: 10 / 78, of 64: 38 / 77, of 200: 65 / 73, of 300:
     # 55 / 67, of 1024: 76 / 79; of 2000: 72 / 69, of 4096: 77 / 76).  The row kernel without
-    # reductions gives each row to a group of lanes sized to it; results go to dense arrays.
-    if (TUNE["rows_elem"] and not reduce_op and not in_place and ndim >= 2 and out_codes
+    # reductions gives each row to a group of lanes sized to it.  Results go to new arrays
+    # or into views whose rows lie one pitch apart, also over an operand (`x[...] = x * v`:
+    # every element is read before it is written, by the lane that writes it).
+    if (TUNE["rows_elem"] and not reduce_op and ndim >= 2 and out_codes
             and out_shape[-1] * max(cg.ITEMSIZE[c] for c in out_codes) <= TUNE["rows_elem"]
             and all(s[-1] in (0, 1) for s in m_leaf)
             and len({id(a.buf) for a in leaves}) == len(leaves)):     # no shifted views: those share an LDS window
-        dense = []
-        step = 1
-        for d in reversed(out_shape):
-            dense.insert(0, step)
-            step *= d
-        if all(list(st) == dense for st in out_strides):
-            try:
-                return lower_rows(prog, leaves, scalars, tuple(out_shape), out_codes, whole_rows=True)
-            except cg.RowFusionUnsupported:
-                pass
+        try:
+            return lower_rows(prog, leaves, scalars, tuple(out_shape), out_codes, whole_rows=True,
+                              out_strides=out_strides, in_place=in_place)
+        except cg.RowFusionUnsupported:
+            pass
 
     # Tiled family: the last merged dimension is walked with unit stride by every output
     # and with stride 1 or 0 by every operand; the dimensions in front of it are the

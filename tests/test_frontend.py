@@ -296,7 +296,11 @@ def test_strided_and_broadcast_operands_use_nd():
     finally:
         lowering.TUNE["rows_elem"] = 4096
     dst = hip.placeholder((64, 32), np.float32, strides=(64, 1))           # a destination with
-    assert hip.lower_only(leaf((64, 32)) * col, dst=dst)[0].kind == "tile2d"   # its own pitch
+    low, src = hip.lower_only(leaf((64, 32)) * col, dst=dst)               # its own pitch
+    assert low.kind == "rows" and low.tail[:4] == [64, 32, 1, 64]
+    hip.compile_source(src)
+    dst3 = hip.placeholder((4, 16, 32), np.float32, strides=(2048, 64, 1))  # rows on two levels
+    assert hip.lower_only(leaf((4, 16, 32)) * 2.0, dst=dst3)[0].kind == "tile2d"
     m = hip.placeholder((100, 200), np.float32)
     low, src = hip.lower_only(NPArray(m.T) * 2.0)           # transposed operand: through LDS
     assert low.kind == "tile2dt" and "__shared__ float tt0[" in src

@@ -1945,3 +1945,39 @@ def test_transposes_of_matrices_with_one_short_side(dtype):
         assert bits_equal((do.T - dx).get(), other.T - x)
     b = (rs.standard_normal((5, 4001, 3)) * 50).astype(dtype)
     assert bits_equal((dr.transpose(dr.array(b), (0, 2, 1)) * 2).get(), b.transpose(0, 2, 1) * 2)
+
+
+def test_element_wise_work_on_short_rows_written_into_existing_arrays():
+    """`x[...] = x * v + c` over its own operand, a destination that is a view with a pitch
+    (`y[:, :2] = ...`), a dense preallocated result: the row kernel writes them as it writes
+    new arrays; a destination whose rows are on two levels keeps the tiled kernel.  Bit-equal
+    to NumPy, repeated so that every sweep reads what the one before wrote."""
+    rs = np.random.RandomState(21)
+    for dtype in (np.float32, np.float64):
+        for n, R in ((100003, 3), (4099, 33), (1000, 64), (513, 200)):
+            x = rs.standard_normal((n, R)).astype(dtype)
+            v = rs.uniform(0.5, 1.5, R).astype(dtype)
+            c = rs.standard_normal((n, 1)).astype(dtype)
+            dx, dv, dc = dr.array(x), dr.array(v), dr.array(c)
+            for _ in range(3):
+                before = hip.STATS["launches"]
+                dx[...] = dx * dv + dc
+                assert hip.STATS["launches"] == before + 1
+                x[...] = x * v + c
+            assert bits_equal(dx.get(), x)
+            y, dy = np.zeros((n, R + 5), dtype), dr.zeros((n, R + 5), dtype=dtype)
+            dy[:, 2:R + 2] = dx * dv
+            y[:, 2:R + 2] = x * v
+            assert bits_equal(dy.get(), y)
+            k = max(1, R // 2)
+            dy[:, :k] = dy[:, :k] * 2 + dc                      # a view over itself
+            y[:, :k] = y[:, :k] * 2 + c
+            assert bits_equal(dy.get(), y)
+            dy[1:, 1:R + 1] = dx[:-1] - dv                     # rows shifted against the operand
+            y[1:, 1:R + 1] = x[:-1] - v
+            assert bits_equal(dy.get(), y)
+    cube, dcube = np.zeros((4, 20, 40)), dr.zeros((4, 20, 40))
+    src = rs.standard_normal((4, 16, 32))
+    dcube[:, 2:18, 4:36] = dr.array(src) * 2.0                   # rows on two levels
+    cube[:, 2:18, 4:36] = src * 2.0
+    assert bits_equal(dcube.get(), cube)
