@@ -1702,7 +1702,8 @@ def emit_narrow_cols(prog, leaf_kind, acc_dt, op, K):
     [w LW, (w+1) LW), so lane l always sees columns (l mod KC) V ... + V - 1.  A wave
     takes four consecutive chunks at a time.
 
-    leaf_kind  per leaf 'd' (dense R x K), 'w' (one row of K for all), 'b' (one element)
+    leaf_kind  per leaf 'd' (dense R x K), 'w' (one row of K for all), 'c' (one value per
+               row: the weights of a weighted sum of the rows), 'b' (one element)
     Parameters: leaf pointers, partials pointer, scalars, U (units in the matrix).
     Output: one partial per block and column, [block][K]."""
     ct = CTYPE[acc_dt]
@@ -1750,6 +1751,9 @@ def emit_narrow_cols(prog, leaf_kind, acc_dt, op, K):
                 else:
                     L.append(f"        {CTYPE[dt]} X{i}_{j} = 0;")
                     L.append(f"        if (ok{j}) X{i}_{j} = a{i}[u{j}];")
+            elif kind == "c":       # the row of unit u: neighbouring lanes share it
+                L.append(f"        {CTYPE[dt]} C{i}_{j} = 0;")
+                L.append(f"        if (ok{j}) C{i}_{j} = a{i}[u{j} / {KC}];")
     for j in range(UN):
         L.append(f"        if (ok{j}) {{")
         for e in range(V):
@@ -1759,6 +1763,8 @@ def emit_narrow_cols(prog, leaf_kind, acc_dt, op, K):
                     args.append(f"X{i}_{j}[{e}]" if V > 1 else f"X{i}_{j}")
                 elif kind == "w":
                     args.append(f"w{i}_{e}")
+                elif kind == "c":
+                    args.append(f"C{i}_{j}")
                 else:
                     args.append(f"b{i}")
             L.append(f"            {{ {ct} t0; dr_body({', '.join(args + call_tail)}); "

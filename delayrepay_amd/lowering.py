@@ -1019,10 +1019,12 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
     if (strategy == "col" and slices in (None, 1) and 2 <= K <= TUNE["ax_narrow"]
             and (R >= 4096 or slices == 1)
             and len(kmerged) == 1 and len(rmerged) == 1 and R * K < 2 ** 40
-            and all((k[0], r[0]) in ((1, K), (1, 0), (0, 0)) for k, r in zip(ksets, rsets))
+            and all((k[0], r[0]) in ((1, K), (1, 0), (0, 0), (0, 1)) for k, r in zip(ksets, rsets))
             and any((k[0], r[0]) == (1, K) for k, r in zip(ksets, rsets))):
         # a dense matrix with few columns, summed over its rows: read it as one stream
-        kinds = tuple("d" if r[0] == K else "w" if k[0] == 1 else "b" for k, r in zip(ksets, rsets))
+        # (beside it: a row of weights for the columns, a dense vector of weights for the rows)
+        kinds = tuple("d" if r[0] == K else "w" if k[0] == 1 else "c" if r[0] == 1 else "b"
+                      for k, r in zip(ksets, rsets))
         low = Lowered()
         low.lds = 0
         low.fin_count = 0

@@ -1981,3 +1981,26 @@ def test_element_wise_work_on_short_rows_written_into_existing_arrays():
     dcube[:, 2:18, 4:36] = dr.array(src) * 2.0                   # rows on two levels
     cube[:, 2:18, 4:36] = src * 2.0
     assert bits_equal(dcube.get(), cube)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_weighted_sums_of_the_rows_of_a_narrow_matrix(dtype):
+    """`(points * w[:, None]).sum(axis=0)`: a centroid, a weighted mean of a few features.
+    The matrix is read as one stream (`axis_narrow`) with the weight of each row beside
+    it, instead of a lane per column walking rows a pitch apart."""
+    rs = np.random.RandomState(22)
+    for n, R in ((200003, 3), (100000, 2), (50001, 8), (30000, 16), (9000, 33), (5000, 64)):
+        x = rs.standard_normal((n, R)).astype(dtype)
+        w = rs.uniform(0, 1, n).astype(dtype)
+        v = rs.standard_normal(R).astype(dtype)
+        dx, dw, dv = dr.array(x), dr.array(w), dr.array(v)
+        low, _ = hip.lower_only(ReduceEx(np.add, dx * dw[:, None], (0,)))
+        assert low.kind == "axis_narrow" and "c" in low.key[2], (n, R, low.kind)
+        tol = dict(rtol=2e-4, atol=2e-2) if dtype == np.float32 else dict(rtol=1e-11, atol=1e-9)
+        np.testing.assert_allclose(dr.sum(dx * dw[:, None], axis=0).get(), (x * w[:, None]).sum(axis=0), **tol)
+        np.testing.assert_allclose(dr.sum((dx - dv) * dw.reshape(n, 1) + dv, axis=0).get(),
+                                   ((x - v) * w.reshape(n, 1) + v).sum(axis=0), **tol)
+        assert np.array_equal(dr.max(dx * dw[:, None], axis=0).get(), (x * w[:, None]).max(axis=0))
+        mean = dr.sum(dx * dw[:, None], axis=0) / dr.sum(dw)
+        np.testing.assert_allclose(np.asarray(mean.get()), (x * w[:, None]).sum(axis=0) / w.sum(),
+                                   rtol=1e-3 if dtype == np.float32 else 1e-10, atol=1e-3 if dtype == np.float32 else 1e-10)
