@@ -353,7 +353,7 @@ def _row_steps_max(G):
 
 
 def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False, out_strides=None,
-               in_place=False):
+               in_place=False, leaf_strides=None):
     """Expression with reductions along its last axis inside it (`codegen.emit_row_fused`):
     every row is read once, reduced, used again and written once.  `shape` is the shape the
     expression is evaluated at, rows along its last axis; outputs are new dense arrays, of
@@ -363,7 +363,10 @@ def lower_rows(prog, leaves, scalars, shape, out_codes, whole_rows=False, out_st
     if not TUNE["rowfuse"] or len(shape) < 2 or shape[-1] < 2:
         raise cg.RowFusionUnsupported("not a matrix of rows")
     R = shape[-1]
-    strides = [broadcast_strides(a, shape) for a in leaves]
+    # (`leaf_strides`: the operands' strides at `shape` where the caller has merged
+    # dimensions already, so that a row is the longest run every operand walks as one)
+    strides = [list(st) for st in leaf_strides] if leaf_strides is not None \
+        else [broadcast_strides(a, shape) for a in leaves]
     kinds = []
     for st in strides:
         if st[-1] not in (0, 1):
@@ -650,12 +653,12 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     # or into views whose rows lie one pitch apart, also over an operand (`x[...] = x * v`:
     # every element is read before it is written, by the lane that writes it).
     if (TUNE["rows_elem"] and not reduce_op and ndim >= 2 and out_codes
-            and out_shape[-1] * max(cg.ITEMSIZE[c] for c in out_codes) <= TUNE["rows_elem"]
+            and mshape[-1] * max(cg.ITEMSIZE[c] for c in out_codes) <= TUNE["rows_elem"]
             and all(s[-1] in (0, 1) for s in m_leaf)
             and len({id(a.buf) for a in leaves}) == len(leaves)):     # no shifted views: those share an LDS window
         try:
-            return lower_rows(prog, leaves, scalars, tuple(out_shape), out_codes, whole_rows=True,
-                              out_strides=out_strides, in_place=in_place)
+            return lower_rows(prog, leaves, scalars, tuple(mshape), out_codes, whole_rows=True,
+                              out_strides=m_out, in_place=in_place, leaf_strides=m_leaf)
         except cg.RowFusionUnsupported:
             pass
 

@@ -1904,6 +1904,13 @@ def test_element_wise_work_on_short_rows_takes_the_row_kernel():
     dx, dm, dw = dr.array(x), dr.array(m), dr.array(w)
     assert hip.lower_only(dx * dw + dm)[0].kind == "rows"
     assert bits_equal((dx * dw + dm).get(), x * w + m)
+    # images with few pixels per channel: a value per channel, rows of 7 x 7 merged
+    img = rs.standard_normal((6, 20, 7, 7)).astype(np.float32)
+    g, b = rs.standard_normal((1, 20, 1, 1)).astype(np.float32), rs.standard_normal((20, 1, 1)).astype(np.float32)
+    di, dg, db = dr.array(img), dr.array(g), dr.array(b)
+    low = hip.lower_only(np.maximum(di * dg + db, 0.0))[0]
+    assert low.kind == "rows" and low.tail[0] == 120 and low.key[5] == 49
+    assert bits_equal(np.maximum(di * dg + db, 0.0).get(), np.maximum(img * g + b, np.float32(0.0)))
     # what stays with the tiled kernels
     c = rs.standard_normal((300, 1))
     dc = dr.array(c)
