@@ -695,6 +695,8 @@ def _compile_together(entries):
         kern.func = hiprt.get_function(module, name)
         kern.finalize = hiprt.get_function(module, name + "_fin") if fin else None
         kern.packer = struct.Struct(low.fmt)
+        if _block_lanes(low) != cg.BLOCK:
+            _BLOCK_OF[kern.func] = _block_lanes(low)
         _KERNELS[low.key] = kern
 
 
