@@ -69,6 +69,9 @@ TUNE = {
     "softdiv": 2,     # quotients and square roots that only inexact functions read: to one ulp, in
                       # fewer operations (1: float64 only, 2: float32 too, in packed bodies; 0: never)
                       # (2: float32 quotients as well, 4 operations; measured slower)
+    "rows_stencil": 384,      # ... shifted views of one matrix among them: rows of at most this many bytes
+                      # (5-point stencil, float32, tiled / row kernel: rows of 16: 10 / 36 % of the
+                      # HBM peak, of 64: 28 / 40, of 128: 46 / 42, of 256: 66 / 44)
     "rows_elem": 4096,    # element-wise work on rows of at most this many bytes with repeated
                       # operands takes the row kernel (0: the tiled kernel)
     "rowfuse": 1,     # reductions along the last axis inside an expression: one kernel per row
@@ -655,7 +658,10 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
     if (TUNE["rows_elem"] and not reduce_op and ndim >= 2 and out_codes
             and mshape[-1] * max(cg.ITEMSIZE[c] for c in out_codes) <= TUNE["rows_elem"]
             and all(s[-1] in (0, 1) for s in m_leaf)
-            and len({id(a.buf) for a in leaves}) == len(leaves)):     # no shifted views: those share an LDS window
+            and (len({id(a.buf) for a in leaves}) == len(leaves) or (
+                ndim == 2 and mshape[-1] * max(cg.ITEMSIZE[c] for c in out_codes) <= TUNE["rows_stencil"]))):    # (shifted views of a
+        # volume share the 3-D kernel's LDS window; of a matrix with short rows, `x[:, 1:] - x[:, :-1]`,
+        # they are read one by one, from the caches: the tiled kernel's window is 256 columns wide)
         try:
             return lower_rows(prog, leaves, scalars, tuple(mshape), out_codes, whole_rows=True,
                               out_strides=m_out, in_place=in_place, leaf_strides=m_leaf)

@@ -2011,3 +2011,25 @@ def test_weighted_sums_of_the_rows_of_a_narrow_matrix(dtype):
         mean = dr.sum(dx * dw[:, None], axis=0) / dr.sum(dw)
         np.testing.assert_allclose(np.asarray(mean.get()), (x * w[:, None]).sum(axis=0) / w.sum(),
                                    rtol=1e-3 if dtype == np.float32 else 1e-10, atol=1e-3 if dtype == np.float32 else 1e-10)
+
+
+def test_shifted_views_of_a_matrix_with_short_rows():
+    """`x[:, 1:] - x[:, :-1]` and a 5-point stencil on rows of at most 384 bytes: the tiled
+    kernel's LDS window is 256 columns wide, so the row kernel reads the views one by one
+    from the caches instead; wider rows and volumes keep their LDS windows.  Bit-equal."""
+    rs = np.random.RandomState(23)
+    for n, R, kind in ((100003, 3, "rows"), (20011, 16, "rows"), (5003, 64, "rows"), (3001, 96, "rows"),
+                       (2000, 200, "tile2d")):
+        x = rs.standard_normal((n, R)).astype(np.float32)
+        dx = dr.array(x)
+        d = dx[:, 1:] - dx[:, :-1]
+        assert hip.lower_only(d)[0].kind == kind, (n, R)
+        assert bits_equal(d.get(), x[:, 1:] - x[:, :-1])
+        if R >= 3:
+            lap = 0.25 * (dx[:-2, 1:-1] + dx[2:, 1:-1] + dx[1:-1, :-2] + dx[1:-1, 2:])
+            ref = np.float32(0.25) * (((x[:-2, 1:-1] + x[2:, 1:-1]) + x[1:-1, :-2]) + x[1:-1, 2:])
+            assert bits_equal(lap.get(), ref)
+        for _ in range(2):                       # written back over the matrix: a hazard, not in place
+            dx[:, 1:] = dx[:, 1:] - dx[:, :-1]
+            x[:, 1:] = x[:, 1:] - x[:, :-1]
+        assert bits_equal(dx.get(), x)
