@@ -1662,6 +1662,19 @@ def stack(arrays, axis=0, **kwargs):
     if builtins.any(p.shape != parts[0].shape for p in parts):
         raise ValueError("all input arrays must have the same shape")
     axis = _axis(axis, parts[0].ndim + 1)
+    if (axis == parts[0].ndim >= 1 and 2 <= len(parts) <= 8 and not kwargs
+            and builtins.all(p.dtype.kind in "fiu" and p.dtype.itemsize in (4, 8) for p in parts)):
+        # A few vectors side by side as the columns of a matrix (coordinates into points):
+        # one expression, `where(column == 0, a, where(column == 1, b, c))`, that a single
+        # kernel writes row by row (and that fuses with what reads it), instead of one
+        # strided write per column.
+        dtype = np.result_type(*[p.dtype for p in parts])
+        column = array(np.arange(len(parts), dtype=np.int32 if dtype.itemsize == 4 else np.int64))
+        cols = [expand_dims(p if p.dtype == dtype else p.astype(dtype), axis) for p in parts]
+        out = cols[-1]
+        for k in range(len(parts) - 2, -1, -1):
+            out = where(column == k, cols[k], out)
+        return out
     return concatenate([expand_dims(p, axis) for p in parts], axis=axis, **kwargs)
 
 
