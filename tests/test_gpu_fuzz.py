@@ -313,3 +313,70 @@ def test_random_geometry_with_flips_and_masks(seed):
             dst_h[key] = h
             got, ref = dst_d.get(), dst_h
     assert got.dtype == np.asarray(ref).dtype and bits_equal(got, np.asarray(ref)), (seed, shape, mode)
+
+
+def test_short_rows_with_repeated_operands_into_every_kind_of_destination():
+    """Random element-wise expressions over a matrix or a batch of matrices with short rows
+    and operands that repeat along or across them (a row, a column, a matrix per batch, a
+    vector per item, a scalar), evaluated into a new array, an existing dense array, a view
+    with a pitch, and over the first operand: bit-equal to NumPy in all of them."""
+    bad = 0
+    kinds = {}
+    for seed in range(160):
+        rs = np.random.RandomState(1000 + seed)
+        dtype = [np.float32, np.float64, np.int32, np.int64][rs.randint(4)]
+        R = int(rs.choice([1, 2, 3, 5, 8, 16, 33, 64, 70, 200, 500, 1000, 1024]))
+        three = rs.randint(3) == 0
+        lead = (int(rs.choice([1, 2, 5])), int(rs.choice([1, 7, 40]))) if three else (int(rs.choice([1, 3, 100, 1001])),)
+        shape = lead + (R,)
+        def mk(s):
+            if np.dtype(dtype).kind == "f":
+                return (rs.standard_normal(s) * 4).astype(dtype)
+            return rs.randint(-20, 20, s).astype(dtype)
+        ops = {"x": mk(shape), "v": mk((R,)), "c": mk(lead + (1,)), "s": mk(())}
+        if three:
+            ops["m"] = mk(lead[1:] + (R,)); ops["b"] = mk((lead[0], 1, R))
+        names = list(ops)
+        dev = {k: dr.array(v) for k, v in ops.items()}
+        def build(env, xp):
+            e = env["x"]
+            for _ in range(rs_local.randint(1, 5)):
+                o = env[names[rs_local.randint(len(names))]]
+                k = rs_local.randint(6)
+                if k == 0: e = e + o
+                elif k == 1: e = e - o
+                elif k == 2: e = e * o
+                elif k == 3: e = xp.maximum(e, o)
+                elif k == 4: e = xp.where(e > o, e, o)
+                else: e = xp.minimum(e, o) - e
+            return e
+        st = rs.randint(1 << 30)
+        rs_local = np.random.RandomState(st); ref = build(ops, np)
+        rs_local = np.random.RandomState(st); ex = build(dev, dr)
+        mode = rs.randint(4)
+        try:
+            if mode == 0:
+                k = hip.lower_only(ex)[0].kind
+                got = ex.get()
+            elif mode == 1:                       # dense existing destination
+                dst = dr.zeros(shape, dtype=ref.dtype); k = "w"; dst[...] = ex; got = dst.get()
+            elif mode == 2:                       # pitched view
+                big = dr.zeros(lead + (R + 7,), dtype=ref.dtype); k = "p"; big[..., 3:R + 3] = ex
+                got = big.get()[..., 3:R + 3]
+                assert not big.get()[..., :3].any() and not big.get()[..., R + 3:].any()
+            else:                                 # over the operand
+                k = "i"
+                if ref.dtype == ops["x"].dtype and ref.shape == shape:
+                    dev["x"][...] = ex; got = dev["x"].get()
+                else:
+                    got = ex.get()
+            kinds[k] = kinds.get(k, 0) + 1
+            ok = got.dtype == ref.dtype and got.shape == ref.shape and got.tobytes() == np.ascontiguousarray(ref).tobytes()
+        except Exception as e:
+            ok = False; print("seed", seed, "raised", type(e).__name__, str(e)[:100])
+        if not ok:
+            bad += 1; print("MISMATCH seed", seed, np.dtype(dtype).name, shape, "mode", mode, flush=True)
+
+
+    print("destinations and kernels:", kinds)
+    assert bad == 0
