@@ -1916,9 +1916,9 @@ def test_element_wise_work_on_short_rows_takes_the_row_kernel():
     dc = dr.array(c)
     rep = dc * 2.0 + dr.zeros((300, 5))
     assert bits_equal(np.repeat(dr.array(c[:, 0]), 5).get(), np.repeat(c[:, 0], 5))
-    a = rs.standard_normal((64, 48))
+    a = rs.standard_normal((64, 100))
     da = dr.array(a)
-    assert hip.lower_only(da[:, 1:] - da[:, :-1])[0].kind.startswith("tile2d")   # shifted views
+    assert hip.lower_only(da[:, 1:] - da[:, :-1])[0].kind.startswith("tile2d")   # shifted views, 792 bytes
     assert bits_equal((da[:, 1:] - da[:, :-1]).get(), a[:, 1:] - a[:, :-1])
     wide = rs.standard_normal((40, 1300)).astype(np.float32)
     other = rs.standard_normal((40, 1300))
@@ -1927,8 +1927,8 @@ def test_element_wise_work_on_short_rows_takes_the_row_kernel():
     assert hip.lower_only(mixed)[0].kind == "tile2d"                          # longer rows, mixed types
     assert bits_equal(mixed.get(), wide * other + col)
     dst = dr.zeros((64, 60))
-    dst[:, 4:52] = da * dr.array(c[:64])                                         # its own pitch
-    ref = np.zeros((64, 60)); ref[:, 4:52] = a * c[:64]
+    dst[:, 4:52] = da[:, :48] * dr.array(c[:64])                                 # its own pitch
+    ref = np.zeros((64, 60)); ref[:, 4:52] = a[:, :48] * c[:64]
     assert bits_equal(dst.get(), ref)
 
 
