@@ -1693,7 +1693,8 @@ def emit_axis_reduce(prog, kdim, rdim, acc_dt, op, strategy, row_vec=None):
 
 def emit_narrow_cols(prog, leaf_kind, acc_dt, op, K):
     """Reduction over the rows of a dense row-major matrix with few columns (K is a
-    compile-time constant, K <= 64): the matrix is read as one contiguous stream, each
+    compile-time constant; at most 64 units of 16 bytes, or 64 elements when K is no
+    multiple of a unit): the matrix is read as one contiguous stream, each
     lane keeps the columns it meets in its own accumulators, and lanes holding the
     same columns are combined once at the end.
 

@@ -26,7 +26,9 @@ TUNE = {
     "ax_blocks": 4096,   # axis reductions: blocks ('col') / waves ('row') worth of work to
     "ax_waves": 32768,   # aim for before the reduced extent is cut into slices
     "ax_rows": 4,        # 'row' strategy: outputs per wave (grid-stride), to amortise set-up
-    "ax_narrow": 64,     # kept unit-stride extents up to this many columns: stream the matrix
+    "ax_narrow": 128,    # kept unit-stride extents up to this many columns: stream the matrix
+                         # (sum over the rows, float32, percent of the HBM peak, a lane per column /
+                         # the stream: 96 columns 52 / 68, 128: 64 / 71, 200: 52 / 51, 256: 64 / 56)
     "ax_short": 28,      # reduced unit-stride extents up to this length: a lane per output
     "ax_group": 2048,    # ... and up to this length: a group of 8 to 64 lanes per output
     "ax_group_lanes": 0,  # force the group size (0: the one that wastes the fewest unit slots)
@@ -1025,7 +1027,14 @@ def lower_axis_reduce(prog, leaves, scalars, shape, axes, acc, reduce_op, slices
     inner_kept = any(ksets[i][-1] == 1 for i in heavy)
     inner_red = any(rsets[i][-1] == 1 for i in heavy)
     strategy = "col" if (inner_kept and not inner_red) else "row"
+    def narrow_units():
+        """16-byte units per row of the narrow matrix, as `codegen.emit_narrow_cols` counts them
+        (a wave's lanes must hold at least one row of them)."""
+        widths = {cg.ITEMSIZE[c] for c, r in zip(prog.leaves, rsets) if r[0] == K}
+        V = 16 // next(iter(widths)) if len(widths) == 1 and widths <= {4, 8} else 1
+        return K // V if K % V == 0 else K
     if (strategy == "col" and slices in (None, 1) and 2 <= K <= TUNE["ax_narrow"]
+            and narrow_units() <= cg.WAVE
             and (R >= 4096 or slices == 1)
             and len(kmerged) == 1 and len(rmerged) == 1 and R * K < 2 ** 40
             and all((k[0], r[0]) in ((1, K), (1, 0), (0, 0), (0, 1)) for k, r in zip(ksets, rsets))

@@ -1996,7 +1996,8 @@ def test_weighted_sums_of_the_rows_of_a_narrow_matrix(dtype):
     The matrix is read as one stream (`axis_narrow`) with the weight of each row beside
     it, instead of a lane per column walking rows a pitch apart."""
     rs = np.random.RandomState(22)
-    for n, R in ((200003, 3), (100000, 2), (50001, 8), (30000, 16), (9000, 33), (5000, 64)):
+    for n, R in ((200003, 3), (100000, 2), (50001, 8), (30000, 16), (9000, 33), (5000, 64), (4100, 96),
+                 (4100, 128)):
         x = rs.standard_normal((n, R)).astype(dtype)
         w = rs.uniform(0, 1, n).astype(dtype)
         v = rs.standard_normal(R).astype(dtype)
