@@ -1654,6 +1654,9 @@ def concatenate(arrays, axis=0, **kwargs):
     return out
 
 
+_COLUMN_NUMBERS = {}        # (count, integer type) -> the leaf 0, 1, ... count - 1 that `stack` compares with
+
+
 @implements(np.stack)
 def stack(arrays, axis=0, **kwargs):
     parts = [arg_to_numpy_ex(a) for a in arrays]
@@ -1669,7 +1672,10 @@ def stack(arrays, axis=0, **kwargs):
         # kernel writes row by row (and that fuses with what reads it), instead of one
         # strided write per column.
         dtype = np.result_type(*[p.dtype for p in parts])
-        column = array(np.arange(len(parts), dtype=np.int32 if dtype.itemsize == 4 else np.int64))
+        kind = (len(parts), np.int32 if dtype.itemsize == 4 else np.int64)
+        column = _COLUMN_NUMBERS.get(kind)
+        if column is None:          # uploaded once: the same leaf every time, so plans are found again
+            column = _COLUMN_NUMBERS[kind] = array(np.arange(kind[0], dtype=kind[1]))
         cols = [expand_dims(p if p.dtype == dtype else p.astype(dtype), axis) for p in parts]
         out = cols[-1]
         for k in range(len(parts) - 2, -1, -1):
