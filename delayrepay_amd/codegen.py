@@ -2384,6 +2384,60 @@ def emit_tile_transpose(prog, leaf_kind, out_dtypes, restrict=True, vec=0, nt_lo
     return "\n".join(src) + "\n"
 
 
+def emit_thin_transpose(prog, leaf_kind, out_dtypes, short, short_rows, restrict=True):
+    """Transposed operands in a matrix with one side of a few elements (`short`, a compile-time
+    constant): points as rows of coordinates and the coordinate vectors.  No tile and no LDS: a
+    lane takes one index of the long side and all `short` indices of the other.
+
+    short_rows  the output has `short` rows (and the 't' operands rows of `short` contiguous
+                elements): a lane reads those elements one after the other and stores one
+                element into each output row, the wave's stores covering 256 contiguous bytes
+                of it; otherwise the output has `short` columns: the lane reads one element of
+                each of the operand's `short` rows (the wave 256 contiguous bytes) and stores
+                its output row
+    leaf_kind   per leaf ('t',) unit stride along the output's rows, ('d',) along its columns,
+                ('b',) one element
+    Parameters: leaf pointers, output pointers, scalars, n (the long extent), per 't' leaf its
+    stride along output columns, per 'd' leaf its row stride, per output its row stride."""
+    rs = "__restrict__ " if restrict else ""
+    n_out = len(out_dtypes)
+    src = [PREAMBLE, emit_body(prog, out_dtypes)]
+    params = [f"const {CTYPE[dt]}* {rs}a{i}" for i, dt in enumerate(prog.leaves)]
+    params += [f"{CTYPE[dt]}* {rs}o{i}" for i, dt in enumerate(out_dtypes)]
+    params += [f"const {CTYPE[dt]} s{i}" for i, dt in enumerate(prog.scalars)]
+    params.append("const long long n")
+    params += [f"const long long cs{i}" for i, k in enumerate(leaf_kind) if k[0] == "t"]
+    params += [f"const long long rs{i}" for i, k in enumerate(leaf_kind) if k[0] == "d"]
+    params += [f"const long long ors{o}" for o in range(n_out)]
+    L = [f'extern "C" __global__ __launch_bounds__({BLOCK})',
+         f"void dr_kernel({', '.join(params)})", "{",
+         f"    const long long i = (long long)blockIdx.x * {BLOCK} + threadIdx.x;",
+         "    if (i >= n) return;"]
+    # element (row, column) of the output: (r, i) with short rows, (i, r) with short columns
+    row, col = ("r", "i") if short_rows else ("i", "r")
+    for i, (dt, k) in enumerate(zip(prog.leaves, leaf_kind)):
+        if k[0] == "b":
+            L.append(f"    const {CTYPE[dt]} x{i} = a{i}[0];")
+        else:
+            L.append(f"    {CTYPE[dt]} x{i}[{short}];")
+    L += ["#pragma unroll", f"    for (int r = 0; r < {short}; ++r) {{"]
+    for i, k in enumerate(leaf_kind):
+        if k[0] == "t":
+            L.append(f"        x{i}[r] = a{i}[{col} * cs{i} + {row}];")
+        elif k[0] == "d":
+            L.append(f"        x{i}[r] = a{i}[{row} * rs{i} + {col}];")
+    L += ["    }", "#pragma unroll", f"    for (int r = 0; r < {short}; ++r) {{"]
+    args = [f"x{i}" if k[0] == "b" else f"x{i}[r]" for i, k in enumerate(leaf_kind)]
+    args += [f"s{i}" for i in range(len(prog.scalars))] + [f"t{o}" for o in range(n_out)]
+    L.append("        " + " ".join(f"{CTYPE[dt]} t{o};" for o, dt in enumerate(out_dtypes)))
+    L.append(f"        dr_body({', '.join(args)});")
+    for o in range(n_out):
+        L.append(f"        o{o}[{row} * ors{o} + {col}] = t{o};")
+    L += ["    }", "}"]
+    src.append("\n".join(L))
+    return "\n".join(src) + "\n"
+
+
 # Rows counted over two levels, K = K0 * K1, that some operand does not walk as one sequence
 # (a matrix repeated for every item of a batch): row k of operand i starts at
 # (k / K1) * sk_i + (k % K1) * sj_i.  Kernels that take such rows have the parameters K1 and

@@ -343,6 +343,13 @@ def _row_lanes(prog, leaves, kinds, sk, out_codes, row_out, R, V, uniform=None):
     return best[1] if best else cg.BLOCK
 
 
+# Transposes of a matrix with one side of at most this many elements take a lane per index of
+# the long side (`codegen.emit_thin_transpose`) when that side is no power of two; powers of
+# two have tiles that fit them and move 16 bytes per lane.
+THIN_TRANSPOSE = 16
+THIN_TRANSPOSE_ALL = False
+
+
 def block_lanes(low):
     """Lanes per block that the kernel of `low` is launched with: `codegen.BLOCK`, except
     for a row kernel whose block of 512 lanes holds one long row (read from the cache key,
@@ -871,6 +878,28 @@ def lower(prog, leaves, scalars, out_shape, out_codes, out_ptrs, out_strides, re
         # array) puts every column of a tile on another page: fewer, longer columns then
         # (512 x 512 x 1024 float32 reversed: 32 x 256: 59, 64 x 64: 64, 128 x 64: 67,
         # 128 x 32: 66, 256 x 32: 65).
+        short = min(mshape[tp], mshape[last])
+        if (not batch and short <= THIN_TRANSPOSE and (short & (short - 1) or THIN_TRANSPOSE_ALL)
+                and max(mshape[tp], mshape[last]) >= 4096):
+            # one side of a few elements, no power of two (rows of three coordinates): the tiles
+            # move single elements on that side; a lane per index of the long side needs no tile
+            short_rows = mshape[tp] == short
+            n_long = mshape[last] if short_rows else mshape[tp]
+            low.kind = "thin_t"
+            low.key = ("thin_t", prog.key(), kinds, tuple(out_codes), in_place, short, short_rows)
+
+            def emit_thin():
+                return cg.emit_thin_transpose(prog, kinds, out_codes, short, short_rows,
+                                              restrict=not in_place)
+            low.emit = emit_thin
+            low.grid = -(-n_long // cg.BLOCK)
+            low.fmt = "@" + "P" * (len(leaves) + len(out_ptrs)) + scal_fmt + "q" \
+                + "q" * (sum(k[0] in ("t", "d") for k in kinds) + len(out_ptrs))
+            low.srcs = [(a.buf, a.offset * a.dtype.itemsize) for a in leaves]
+            low.scal = scal_vals
+            low.tail = [n_long] + [st[last] for st, k in zip(m_leaf, kinds) if k[0] == "t"] \
+                + [st[tp] for st, k in zip(m_leaf, kinds) if k[0] == "d"] + [st[tp] for st in m_out]
+            return low
         widest = max(cg.ITEMSIZE[c] for c in list(prog.leaves) + list(out_codes))
         far = max(abs(st[last]) * cg.ITEMSIZE[c] for st, c, k in zip(m_leaf, prog.leaves, kinds)
                   if k[0] == "t") >= 1 << 20

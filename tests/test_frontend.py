@@ -701,3 +701,17 @@ def test_masks_that_are_the_same_along_a_row_compile_in_the_row_kernel():
         low, src = hip.lower_only(ex)
         assert low.kind == "rows" and "unsigned char" in src
         hip.compile_source(src)
+
+
+def test_thin_transposes_are_a_lane_per_index_of_the_long_side():
+    """A transposed operand in a matrix with a side of at most 16 elements that is no power of
+    two: no tile; both orientations, a directly read operand beside the transposed one."""
+    for shape, short_rows in (((1 << 20, 3), True), ((3, 1 << 20), False), ((1 << 18, 12), True)):
+        x, o = leaf(shape), leaf(shape[::-1])
+        low, src = hip.lower_only(x.T * 2.0 + o)
+        assert low.kind == "thin_t" and low.key[-2:] == (min(shape), short_rows)
+        assert "__shared__" not in src and low.tail[0] == max(shape) and low.grid == max(shape) // 256
+        hip.compile_source(src)
+    assert hip.lower_only(leaf((1 << 20, 4)).T * 2.0)[0].kind == "tile2dt"      # a power of two
+    assert hip.lower_only(leaf((1000, 3)).T * 2.0)[0].kind == "tile2dt"         # a short long side
+    assert hip.lower_only(leaf((1 << 20, 24)).T * 2.0)[0].kind == "tile2dt"
